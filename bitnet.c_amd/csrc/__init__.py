@@ -1,0 +1,1 @@
+"""HIP sources of the gfx950 kernels and the driver that compiles them."""

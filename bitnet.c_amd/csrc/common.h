@@ -1,0 +1,70 @@
+// Shared device helpers for the gfx950 kernels of this library.
+// Wavefronts are 64 lanes wide; every reduction below assumes that.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+
+#define BN_WAVE 64
+#define BN_PAGE 64            // tokens per cache page; the Python side uses the same number
+
+// error codes returned by the extern "C" entry points (0 = ok, >0 = hipError_t)
+#define BN_ERR_ARG   (-1)     // an argument the kernel cannot take (size, alignment)
+#define BN_ERR_DTYPE (-2)
+
+#define BN_DT_F32  0
+#define BN_DT_BF16 1
+
+typedef __hip_bfloat16 bf16;
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16 v) { return __bfloat162float(v); }
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16 from_f32<bf16>(float v) { return __float2bfloat16(v); }
+
+// bf16 bits <-> float without going through the class type (for packed loads)
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
+    return __uint_as_float(((uint32_t)b) << 16);
+}
+__device__ __forceinline__ float bf16lo_to_f32(uint32_t two) { return __uint_as_float(two << 16); }
+__device__ __forceinline__ float bf16hi_to_f32(uint32_t two) { return __uint_as_float(two & 0xffff0000u); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, BN_WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, BN_WAVE));
+    return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.
+// `scratch` holds at least 16 floats of shared memory.  The order of the additions is
+// fixed by the block size alone.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    const int lane = threadIdx.x & (BN_WAVE - 1), w = threadIdx.x / BN_WAVE;
+    const int nw = (blockDim.x + BN_WAVE - 1) / BN_WAVE;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) scratch[w] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nw; ++i) t += scratch[i];
+    return t;
+}
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+    const int lane = threadIdx.x & (BN_WAVE - 1), w = threadIdx.x / BN_WAVE;
+    const int nw = (blockDim.x + BN_WAVE - 1) / BN_WAVE;
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) scratch[w] = v;
+    __syncthreads();
+    float t = scratch[0];
+    for (int i = 1; i < nw; ++i) t = fmaxf(t, scratch[i]);
+    return t;
+}
+
+static inline int bn_launch_status() { return (int)hipGetLastError(); }

@@ -1,0 +1,153 @@
+// Row-wise kernels around the matrix products: embedding gather, residual add fused with
+// RMSNorm, SwiGLU, bias add, row gather.  The residual stream is float32; `T` is the
+// activation type (float or bf16) that the matrix products read and write.
+#include "common.h"
+
+// x[t, :] = float(E[token[t], :]).  A token outside [0, vocab) gives a zero row, as the
+// reference's embedding does (src/model_embed.c:6-28, test/test_safety.c:278-315); the
+// step function rejects such tokens before it launches anything.
+template <typename T>
+__global__ void embed_gather_kernel(float* __restrict__ x, const T* __restrict__ table,
+                                    const int* __restrict__ tokens, int dim, int vocab) {
+    const int t = blockIdx.x;
+    const int tok = tokens[t];
+    float* row = x + (size_t)t * dim;
+    if (tok < 0 || tok >= vocab) {
+        for (int i = threadIdx.x; i < dim; i += blockDim.x) row[i] = 0.f;
+        return;
+    }
+    const T* src = table + (size_t)tok * dim;
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) row[i] = to_f32(src[i]);
+}
+
+// One block per output row r.  src row = rows ? rows[r] : r.
+//   s = x[src] (+ delta[src])          float32; written back to x[src] when delta && !rows
+//   out[r] = s * rsqrt(mean(s^2) + eps) * w     (src/transformer/rmsnorm_scalar.c:4-13;
+//   the fused add is the reference's residual_rmsnorm, src/gpu_cuda.cu:5077)
+// The sum of squares is float32: per thread in index order, then a fixed tree.
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta,
+                                   const float* __restrict__ w, T* __restrict__ out,
+                                   const int* __restrict__ rows, int dim, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int src = rows ? rows[r] : r;
+    float* xr = x + (size_t)src * dim;
+    const T* dr = delta ? delta + (size_t)src * dim : nullptr;
+    const bool write_back = (dr != nullptr) && (rows == nullptr);
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+        float v = xr[i];
+        if (dr) v += to_f32(dr[i]);
+        if (write_back) xr[i] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)dim + eps);
+    T* o = out + (size_t)r * dim;
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+        float v = xr[i];
+        if (dr && !write_back) v += to_f32(dr[i]);
+        o[i] = from_f32<T>(v * scale * w[i]);
+    }
+}
+
+// x[t, :] += delta[t, :]   (src/transformer/cpu_backend.c:252-256)
+template <typename T>
+__global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__ delta, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] += to_f32(delta[i]);
+}
+
+// out[t, f] = silu(gu[t, f]) * gu[t, F + f], silu(g) = g / (1 + exp(-g))
+// (src/transformer/cpu_backend.c:385-391, exact exponential)
+template <typename T>
+__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gu, int F, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    size_t t = i / F;
+    int f = (int)(i - t * F);
+    float g = to_f32(gu[t * 2 * F + f]);
+    float u = to_f32(gu[t * 2 * F + F + f]);
+    out[i] = from_f32<T>((g / (1.0f + expf(-g))) * u);
+}
+
+// y[t, n] += b[n]   (src/gpu_cuda.cu:5161-5166)
+template <typename T>
+__global__ void bias_add_kernel(T* __restrict__ y, const float* __restrict__ b, int N, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = from_f32<T>(to_f32(y[i]) + b[i % N]);
+}
+
+template <typename T>
+static int embed_gather_t(void* x, const void* table, const int* tokens, int n_tokens, int dim,
+                          int vocab, hipStream_t s) {
+    hipLaunchKernelGGL(embed_gather_kernel<T>, dim3(n_tokens), dim3(256), 0, s, (float*)x,
+                       (const T*)table, tokens, dim, vocab);
+    return bn_launch_status();
+}
+
+extern "C" int bn_embed_gather(int dtype, void* x, const void* table, const int* tokens, int n_tokens,
+                               int dim, int vocab, hipStream_t s) {
+    if (n_tokens <= 0 || dim <= 0 || vocab <= 0) return BN_ERR_ARG;
+    if (dtype == BN_DT_F32) return embed_gather_t<float>(x, table, tokens, n_tokens, dim, vocab, s);
+    if (dtype == BN_DT_BF16) return embed_gather_t<bf16>(x, table, tokens, n_tokens, dim, vocab, s);
+    return BN_ERR_DTYPE;
+}
+
+extern "C" int bn_add_rmsnorm(int dtype, void* x, const void* delta, const float* w, void* out,
+                              const int* rows, int n_rows, int dim, float eps, hipStream_t s) {
+    if (n_rows <= 0 || dim <= 0) return BN_ERR_ARG;
+    const int threads = dim >= 2048 ? 512 : 256;
+    if (dtype == BN_DT_F32)
+        hipLaunchKernelGGL(add_rmsnorm_kernel<float>, dim3(n_rows), dim3(threads), 0, s, (float*)x,
+                           (const float*)delta, w, (float*)out, rows, dim, eps);
+    else if (dtype == BN_DT_BF16)
+        hipLaunchKernelGGL(add_rmsnorm_kernel<bf16>, dim3(n_rows), dim3(threads), 0, s, (float*)x,
+                           (const bf16*)delta, w, (bf16*)out, rows, dim, eps);
+    else
+        return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+extern "C" int bn_residual_add(int dtype, void* x, const void* delta, long long n, hipStream_t s) {
+    if (n <= 0) return BN_ERR_ARG;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (dtype == BN_DT_F32)
+        hipLaunchKernelGGL(residual_add_kernel<float>, dim3(blocks), dim3(256), 0, s, (float*)x,
+                           (const float*)delta, (size_t)n);
+    else if (dtype == BN_DT_BF16)
+        hipLaunchKernelGGL(residual_add_kernel<bf16>, dim3(blocks), dim3(256), 0, s, (float*)x,
+                           (const bf16*)delta, (size_t)n);
+    else
+        return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+extern "C" int bn_swiglu(int dtype, void* out, const void* gu, int n_rows, int F, hipStream_t s) {
+    if (n_rows <= 0 || F <= 0) return BN_ERR_ARG;
+    const size_t n = (size_t)n_rows * F;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (dtype == BN_DT_F32)
+        hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, s, (float*)out,
+                           (const float*)gu, F, n);
+    else if (dtype == BN_DT_BF16)
+        hipLaunchKernelGGL(swiglu_kernel<bf16>, dim3(blocks), dim3(256), 0, s, (bf16*)out,
+                           (const bf16*)gu, F, n);
+    else
+        return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+extern "C" int bn_bias_add(int dtype, void* y, const float* b, int n_rows, int N, hipStream_t s) {
+    if (n_rows <= 0 || N <= 0) return BN_ERR_ARG;
+    const size_t n = (size_t)n_rows * N;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (dtype == BN_DT_F32)
+        hipLaunchKernelGGL(bias_add_kernel<float>, dim3(blocks), dim3(256), 0, s, (float*)y, b, N, n);
+    else if (dtype == BN_DT_BF16)
+        hipLaunchKernelGGL(bias_add_kernel<bf16>, dim3(blocks), dim3(256), 0, s, (bf16*)y, b, N, n);
+    else
+        return BN_ERR_DTYPE;
+    return bn_launch_status();
+}

@@ -1,0 +1,143 @@
+// Decode-phase matrix product for bf16: Y[M, N] = X[M, K] . W[N, K]^T with M <= 64 rows
+// of activations, on the matrix cores (v_mfma_f32_16x16x32_bf16).  The weights are
+// streamed once from HBM with 16-byte loads, each lane reading 128 contiguous bytes of
+// one weight row per 256-element K chunk; K is split over the waves of a workgroup and
+// the partial sums are added through shared memory in wave order, so the result does
+// not depend on timing.  It plays the part of the reference's matvec kernels
+// (src/gpu_cuda.cu:3976-4010, one warp per output row) and of its stacked gate/up
+// matvec followed by the activation (src/gpu_cuda.cu:4176, :8971), written for 64-wide
+// waves and MFMA instead.
+//
+// DUAL: W holds two row blocks (gate rows n, up rows up_off + n); the epilogue writes
+// silu(gate) * up, silu(g) = g / (1 + exp(-g)) (src/transformer/cpu_backend.c:385-391).
+//
+// Needs K % 8 == 0 and 16-byte aligned rows; other shapes go to the tiled kernel.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+#define SK_CHUNK 256          // K elements per wave iteration
+
+__device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+template <int MT, bool DUAL, typename TO>
+__global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
+                                                           TO* __restrict__ Y, int M, int N, int K, int ldx,
+                                                           int ldw, int ldy, int up_off) {
+    constexpr int NA = DUAL ? 2 * MT : MT;            // accumulator tiles per wave
+    extern __shared__ __align__(16) float red[];      // [n_waves][NA][64][4]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n_waves = blockDim.x >> 6;
+    const int i = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int n = min(n0 + i, N - 1);                 // clamp: rows past N are computed and dropped
+    const bf16* wrow = W + (size_t)n * ldw;
+    const bf16* urow = DUAL ? W + (size_t)(up_off + n) * ldw : nullptr;
+
+    f32x4 acc[NA];
+#pragma unroll
+    for (int a = 0; a < NA; ++a) acc[a] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    for (int kc = wave * SK_CHUNK; kc < K; kc += n_waves * SK_CHUNK) {
+        const int kb = kc + g * 64;                   // this lane's 64 elements of the chunk
+        uint4 wv[8], uv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int k = kb + j * 8;
+            wv[j] = (k < K) ? *reinterpret_cast<const uint4*>(wrow + k) : make_uint4(0, 0, 0, 0);
+            if (DUAL) uv[j] = (k < K) ? *reinterpret_cast<const uint4*>(urow + k) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + i;
+            const bf16* xrow = X + (size_t)m * ldx;
+            uint4 xv[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int k = kb + j * 8;
+                xv[j] = (m < M && k < K) ? *reinterpret_cast<const uint4*>(xrow + k) : make_uint4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xv[j]), as_bf16x8(wv[j]), acc[mt], 0, 0, 0);
+                if (DUAL)
+                    acc[MT + mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xv[j]), as_bf16x8(uv[j]),
+                                                                          acc[MT + mt], 0, 0, 0);
+            }
+        }
+    }
+    // partial sums of every wave -> shared memory
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+        *reinterpret_cast<f32x4*>(red + (((size_t)wave * NA + a) * 64 + lane) * 4) = acc[a];
+    __syncthreads();
+    // thread (l, r): C row 4*(l/16)+r of each tile, column l%16; sums over waves in wave order
+    for (int idx = threadIdx.x; idx < MT * 256; idx += blockDim.x) {
+        const int mt = idx >> 8, rem = idx & 255;
+        const int l = rem & 63, r = rem >> 6;
+        float v = 0.f, u = 0.f;
+        for (int w = 0; w < n_waves; ++w) {
+            v += red[(((size_t)w * NA + mt) * 64 + l) * 4 + r];
+            if (DUAL) u += red[(((size_t)w * NA + MT + mt) * 64 + l) * 4 + r];
+        }
+        const int m = mt * 16 + 4 * (l >> 4) + r;
+        const int nn = n0 + (l & 15);
+        if (m < M && nn < N) {
+            const float y = DUAL ? (v / (1.0f + expf(-v))) * u : v;
+            Y[(size_t)m * ldy + nn] = from_f32<TO>(y);
+        }
+    }
+}
+
+template <int MT, bool DUAL, typename TO>
+static int launch(const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw, int ldy,
+                  int up_off, int n_waves, hipStream_t s) {
+    constexpr int NA = DUAL ? 2 * MT : MT;
+    const size_t smem = (size_t)n_waves * NA * 64 * 4 * sizeof(float);
+    hipLaunchKernelGGL((skinny_gemm_kernel<MT, DUAL, TO>), dim3((N + 15) / 16), dim3(n_waves * 64), smem, s,
+                       (const bf16*)X, (const bf16*)W, (TO*)Y, M, N, K, ldx, ldw, ldy, up_off);
+    return bn_launch_status();
+}
+
+template <bool DUAL, typename TO>
+static int launch_mt(int MT, const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw,
+                     int ldy, int up_off, int n_waves, hipStream_t s) {
+    switch (MT) {
+        case 1: return launch<1, DUAL, TO>(X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s);
+        case 2: return launch<2, DUAL, TO>(X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s);
+        case 3: return launch<3, DUAL, TO>(X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s);
+        case 4: return launch<4, DUAL, TO>(X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s);
+    }
+    return BN_ERR_ARG;
+}
+
+// 1 if the kernel takes the shape, 0 if the caller must use the tiled kernel.
+extern "C" int bn_skinny_gemm_supports(int M, int N, int K, int ldx, int ldw) {
+    return (M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0) ? 1 : 0;
+}
+
+// out_dtype: type of Y (bf16 or float32).  dual != 0: N is the width of the result and W has
+// the gate rows at [0, N) and the up rows at [up_off, up_off + N).
+extern "C" int bn_skinny_gemm(int out_dtype, const void* X, const void* W, void* Y, int M, int N, int K,
+                              int ldx, int ldw, int ldy, int dual, int up_off, hipStream_t s) {
+    if (!bn_skinny_gemm_supports(M, N, K, ldx, ldw) || ldy < N) return BN_ERR_ARG;
+    if (((uintptr_t)X | (uintptr_t)W) & 15) return BN_ERR_ARG;
+    const int MT = (M + 15) / 16;
+    const int NA = dual ? 2 * MT : MT;
+    // waves per workgroup: enough loads in flight when there are few column tiles, bounded by
+    // the K chunks there are and by 48 KB of shared memory for the partial sums
+    const int tiles = (N + 15) / 16;
+    int n_waves = tiles >= 2048 ? 4 : (tiles >= 1024 ? 8 : 16);
+    const int k_chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
+    while (n_waves > 1 && n_waves / 2 >= k_chunks) n_waves >>= 1;
+    while (n_waves > 1 && n_waves * NA > 48) n_waves >>= 1;
+    if (dual && MT >= 3 && n_waves > 8) n_waves = 8;      // that variant is built for 512 threads
+    if (out_dtype == BN_DT_BF16)
+        return dual ? launch_mt<true, bf16>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s)
+                    : launch_mt<false, bf16>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s);
+    if (out_dtype == BN_DT_F32)
+        return dual ? launch_mt<true, float>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s)
+                    : launch_mt<false, float>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s);
+    return BN_ERR_DTYPE;
+}

@@ -1,0 +1,465 @@
+"""Checked Python entry points of the HIP kernels.
+
+Every function here validates shapes, dtypes, devices and strides on the host before it
+launches anything: a kernel is never handed operands that its indexing does not expect.
+There is no other implementation behind these functions: without a GPU, or when the
+kernels cannot be compiled, they raise.  Kernels run on torch's current stream, so a
+step can be captured into a HIP graph.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_longlong, c_void_p
+
+import torch
+
+from .csrc import build as _build
+
+PAGE = 64                     # tokens per cache page (BN_PAGE in csrc/common.h)
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_SIGNATURES = {
+    "elementwise": {
+        "bn_embed_gather": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "bn_add_rmsnorm": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p],
+        "bn_residual_add": [c_int, c_void_p, c_void_p, c_longlong, c_void_p],
+        "bn_swiglu": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+        "bn_bias_add": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    },
+    "rope_kv": {
+        "bn_rope_kv_write": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                             c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    },
+    "attn_rows": {
+        "bn_attn_rows_key_tile": [c_int, c_int, c_int],
+        "bn_attn_rows": [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                         c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
+                         c_void_p, c_void_p, c_void_p],
+    },
+    "gemm_tiled": {
+        "bn_gemm_tiled": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                          c_void_p],
+    },
+    "skinny_gemm": {
+        "bn_skinny_gemm_supports": [c_int, c_int, c_int, c_int, c_int],
+        "bn_skinny_gemm": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                           c_int, c_void_p],
+    },
+    "sampling": {
+        "bn_argmax": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p],
+        "bn_repeat_penalty": [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_float, c_void_p],
+        "bn_sample": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p],
+    },
+}
+_fns = {}
+
+
+def _fn(lib: str, name: str):
+    f = _fns.get(name)
+    if f is None:
+        handle = _build.load(lib)
+        f = getattr(handle, name)
+        f.argtypes = _SIGNATURES[lib][name]
+        f.restype = c_int
+        _fns[name] = f
+    return f
+
+
+def require_gpu() -> None:
+    if not torch.cuda.is_available():
+        raise KernelError("no GPU: the kernels of this library are HIP code for gfx950 and there is "
+                          "no CPU implementation behind them")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(rc: int, what: str) -> None:
+    if rc == 0:
+        return
+    if rc == -1:
+        raise KernelError(f"{what}: the kernel refuses these sizes or this alignment")
+    if rc == -2:
+        raise KernelError(f"{what}: unsupported dtype")
+    raise KernelError(f"{what}: HIP error {rc}")
+
+
+def _dev(t: torch.Tensor, name: str, dtype=None, dims=None) -> None:
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise KernelError(f"{name}: expected a GPU tensor")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: expected {dtype}, got {t.dtype}")
+    if dims is not None and t.dim() != dims:
+        raise KernelError(f"{name}: expected {dims} dimensions, got shape {tuple(t.shape)}")
+
+
+def _rows(t: torch.Tensor, name: str) -> int:
+    """Row stride of a 2-D tensor whose rows are contiguous."""
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise KernelError(f"{name}: expected a 2-D tensor with contiguous rows, got shape "
+                          f"{tuple(t.shape)} strides {t.stride()}")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+def _code(dtype) -> int:
+    if dtype not in _DT:
+        raise KernelError(f"unsupported dtype {dtype}")
+    return _DT[dtype]
+
+
+# --------------------------------------------------------------------------------------
+# row-wise kernels
+# --------------------------------------------------------------------------------------
+
+def embed_gather(table: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
+    """float32 rows of the embedding table for int32 token ids."""
+    require_gpu()
+    _dev(table, "table", dims=2)
+    _dev(tokens, "tokens", torch.int32, 1)
+    if not table.is_contiguous() or not tokens.is_contiguous():
+        raise KernelError("embed_gather: table and tokens must be contiguous")
+    n, dim = tokens.numel(), table.shape[1]
+    x = torch.empty((n, dim), dtype=torch.float32, device=table.device)
+    _check(_fn("elementwise", "bn_embed_gather")(_code(table.dtype), x.data_ptr(), table.data_ptr(),
+                                                 tokens.data_ptr(), n, dim, table.shape[0], _stream()),
+           "embed_gather")
+    return x
+
+
+def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor, eps: float, out_dtype,
+                rows=None) -> torch.Tensor:
+    """x (float32, [T, D]) += delta (if given), and the RMS-normed rows in out_dtype.
+    With `rows` (int32 indices) only those rows are normed and x is left as it is."""
+    require_gpu()
+    _dev(x, "x", torch.float32, 2)
+    _dev(weight, "weight", torch.float32, 1)
+    T, D = x.shape
+    if not x.is_contiguous() or weight.numel() != D or not weight.is_contiguous():
+        raise KernelError(f"add_rmsnorm: x {tuple(x.shape)} must be contiguous and weight have {D} elements")
+    if delta is not None:
+        _dev(delta, "delta", out_dtype, 2)
+        if delta.shape != x.shape or not delta.is_contiguous():
+            raise KernelError(f"add_rmsnorm: delta {tuple(delta.shape)} does not match x {tuple(x.shape)}")
+    n = T
+    if rows is not None:
+        _dev(rows, "rows", torch.int32, 1)
+        if not rows.is_contiguous():
+            raise KernelError("add_rmsnorm: rows must be contiguous")
+        n = rows.numel()
+    out = torch.empty((n, D), dtype=out_dtype, device=x.device)
+    if n == 0:
+        return out
+    _check(_fn("elementwise", "bn_add_rmsnorm")(_code(out_dtype), x.data_ptr(),
+                                                delta.data_ptr() if delta is not None else None,
+                                                weight.data_ptr(), out.data_ptr(),
+                                                rows.data_ptr() if rows is not None else None,
+                                                n, D, float(eps), _stream()), "add_rmsnorm")
+    return out
+
+
+def residual_add(x: torch.Tensor, delta: torch.Tensor) -> None:
+    require_gpu()
+    _dev(x, "x", torch.float32)
+    _dev(delta, "delta")
+    if x.shape != delta.shape or not x.is_contiguous() or not delta.is_contiguous():
+        raise KernelError("residual_add: shapes differ or tensors are not contiguous")
+    _check(_fn("elementwise", "bn_residual_add")(_code(delta.dtype), x.data_ptr(), delta.data_ptr(),
+                                                 x.numel(), _stream()), "residual_add")
+
+
+def swiglu(gu: torch.Tensor) -> torch.Tensor:
+    """[T, 2F] (gate | up) -> silu(gate) * up, [T, F]."""
+    require_gpu()
+    _dev(gu, "gu", dims=2)
+    if not gu.is_contiguous() or gu.shape[1] % 2:
+        raise KernelError(f"swiglu: expected a contiguous [T, 2F] tensor, got {tuple(gu.shape)}")
+    T, F = gu.shape[0], gu.shape[1] // 2
+    out = torch.empty((T, F), dtype=gu.dtype, device=gu.device)
+    _check(_fn("elementwise", "bn_swiglu")(_code(gu.dtype), out.data_ptr(), gu.data_ptr(), T, F, _stream()),
+           "swiglu")
+    return out
+
+
+def bias_add(y: torch.Tensor, bias: torch.Tensor) -> None:
+    require_gpu()
+    _dev(y, "y", dims=2)
+    _dev(bias, "bias", torch.float32, 1)
+    if not y.is_contiguous() or bias.numel() != y.shape[1] or not bias.is_contiguous():
+        raise KernelError("bias_add: y must be contiguous [T, N] and bias have N elements")
+    _check(_fn("elementwise", "bn_bias_add")(_code(y.dtype), y.data_ptr(), bias.data_ptr(), y.shape[0],
+                                             y.shape[1], _stream()), "bias_add")
+
+
+# --------------------------------------------------------------------------------------
+# matrix products
+# --------------------------------------------------------------------------------------
+
+def _tiled(x, w, out_dtype):
+    M, K = x.shape
+    N = w.shape[0]
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    _check(_fn("gemm_tiled", "bn_gemm_tiled")(_code(x.dtype), _code(out_dtype), x.data_ptr(), w.data_ptr(),
+                                              y.data_ptr(), M, N, K, _rows(x, "x"), _rows(w, "w"), N,
+                                              _stream()), "gemm_tiled")
+    return y
+
+
+def skinny_supported(M: int, N: int, K: int, ldx: int, ldw: int) -> bool:
+    return bool(_fn("skinny_gemm", "bn_skinny_gemm_supports")(M, N, K, ldx, ldw))
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, *, allow_library: bool = True) -> torch.Tensor:
+    """y[M, N] = x[M, K] . w[N, K]^T.
+
+    float32: the tiled kernel (plain fmaf, a fixed order of summation).
+    bf16: up to 64 rows the matrix-core kernel that streams the weights once; above
+    that the library's matrix product (as the reference hands its batched prompt
+    products to a library, src/gpu_cuda.cu:11571); shapes neither takes go to the
+    tiled kernel."""
+    require_gpu()
+    _dev(x, "x", dims=2)
+    _dev(w, "w", x.dtype, 2)
+    M, K = x.shape
+    N = w.shape[0]
+    if w.shape[1] != K:
+        raise KernelError(f"linear: x {tuple(x.shape)} and w {tuple(w.shape)} do not agree")
+    out_dtype = out_dtype or x.dtype
+    if M == 0:
+        return torch.empty((0, N), dtype=out_dtype, device=x.device)
+    ldx, ldw = _rows(x, "x"), _rows(w, "w")
+    if x.dtype == torch.float32:
+        if out_dtype != torch.float32:
+            raise KernelError("linear: float32 inputs give float32 outputs")
+        return _tiled(x, w, torch.float32)
+    if x.dtype != torch.bfloat16:
+        raise KernelError(f"linear: unsupported dtype {x.dtype}")
+    aligned = (x.data_ptr() % 16 == 0) and (w.data_ptr() % 16 == 0)
+    if M <= 64 and aligned and skinny_supported(M, N, K, ldx, ldw):
+        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        _check(_fn("skinny_gemm", "bn_skinny_gemm")(_code(out_dtype), x.data_ptr(), w.data_ptr(), y.data_ptr(),
+                                                    M, N, K, ldx, ldw, N, 0, 0, _stream()), "skinny_gemm")
+        return y
+    if M > 64 and allow_library and out_dtype == torch.bfloat16:
+        return torch.matmul(x, w.t())
+    if M > 64 and out_dtype == torch.float32 and aligned and skinny_supported(64, N, K, ldx, ldw):
+        # float32 results from bf16 operands (logits at many positions): 64 rows at a time
+        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        f = _fn("skinny_gemm", "bn_skinny_gemm")
+        for m0 in range(0, M, 64):
+            m = min(64, M - m0)
+            _check(f(_code(out_dtype), x[m0:].data_ptr(), w.data_ptr(), y[m0:].data_ptr(), m, N, K, ldx, ldw,
+                     N, 0, 0, _stream()), "skinny_gemm")
+        return y
+    return _tiled(x, w, out_dtype)
+
+
+def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(x.Wg^T) * (x.Wu^T) for w_gate_up = [Wg; Wu] ([2F, K]).  The decode-sized bf16
+    case is one kernel; every other case is the product followed by the SwiGLU kernel."""
+    require_gpu()
+    _dev(x, "x", dims=2)
+    _dev(w_gate_up, "w_gate_up", x.dtype, 2)
+    M, K = x.shape
+    if w_gate_up.shape[0] % 2 or w_gate_up.shape[1] != K:
+        raise KernelError(f"linear_swiglu: x {tuple(x.shape)} and w {tuple(w_gate_up.shape)} do not agree")
+    F = w_gate_up.shape[0] // 2
+    if M == 0:
+        return torch.empty((0, F), dtype=x.dtype, device=x.device)
+    ldx, ldw = _rows(x, "x"), _rows(w_gate_up, "w_gate_up")
+    if (x.dtype == torch.bfloat16 and M <= 64 and x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0
+            and skinny_supported(M, F, K, ldx, ldw)):
+        y = torch.empty((M, F), dtype=x.dtype, device=x.device)
+        _check(_fn("skinny_gemm", "bn_skinny_gemm")(_code(x.dtype), x.data_ptr(), w_gate_up.data_ptr(),
+                                                    y.data_ptr(), M, F, K, ldx, ldw, F, 1, F, _stream()),
+               "skinny_gemm(dual)")
+        return y
+    return swiglu(linear(x, w_gate_up))
+
+
+# --------------------------------------------------------------------------------------
+# position encoding + cache write, attention
+# --------------------------------------------------------------------------------------
+
+def _check_pages(k_pages, v_pages, Hkv, hs, dtype):
+    for t, nm in ((k_pages, "k_pages"), (v_pages, "v_pages")):
+        _dev(t, nm, dtype, 4)
+        if tuple(t.shape[1:]) != (Hkv, PAGE, hs) or not t.is_contiguous():
+            raise KernelError(f"{nm}: expected contiguous [pages, {Hkv}, {PAGE}, {hs}], got {tuple(t.shape)}")
+    if k_pages.shape != v_pages.shape:
+        raise KernelError("k_pages and v_pages differ in shape")
+
+
+def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, hs: int, *,
+                  inv_freq=None, rope_dims: int = 0, seq_index=None, block_table=None,
+                  k_pages=None, v_pages=None) -> None:
+    """Rotate the Q heads of qkv ([T, (H+2Hkv)*hs]) in place, rotate the K heads and store
+    them and the V heads at each token's position of its sequence's pages.
+    k_pages None: rotate Q only.  rope_dims 0: no rotation.  positions < 0: padding rows."""
+    require_gpu()
+    _dev(qkv, "qkv", dims=2)
+    _dev(positions, "positions", torch.int32, 1)
+    T = qkv.shape[0]
+    stride = _rows(qkv, "qkv")
+    if qkv.shape[1] < (H + 2 * Hkv) * hs or positions.numel() != T or not positions.is_contiguous():
+        raise KernelError(f"rope_kv_write: qkv {tuple(qkv.shape)} / positions {tuple(positions.shape)} do not "
+                          f"fit H={H} Hkv={Hkv} hs={hs}")
+    if rope_dims:
+        _dev(inv_freq, "inv_freq", torch.float32, 1)
+        if rope_dims % 2 or rope_dims > hs or inv_freq.numel() != rope_dims // 2 or not inv_freq.is_contiguous():
+            raise KernelError(f"rope_kv_write: rope_dims {rope_dims} does not fit hs={hs} / inv_freq "
+                              f"{tuple(inv_freq.shape)}")
+    bt_stride = 0
+    if k_pages is not None:
+        _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype)
+        _dev(seq_index, "seq_index", torch.int32, 1)
+        _dev(block_table, "block_table", torch.int32, 2)
+        if seq_index.numel() != T or not seq_index.is_contiguous() or not block_table.is_contiguous():
+            raise KernelError("rope_kv_write: seq_index must have one entry per token; tables contiguous")
+        bt_stride = block_table.shape[1]
+    if T == 0:
+        return
+    _check(_fn("rope_kv", "bn_rope_kv_write")(
+        _code(qkv.dtype), qkv.data_ptr(), stride, positions.data_ptr(),
+        seq_index.data_ptr() if k_pages is not None else None,
+        block_table.data_ptr() if k_pages is not None else None, bt_stride,
+        k_pages.data_ptr() if k_pages is not None else None,
+        v_pages.data_ptr() if k_pages is not None else None,
+        inv_freq.data_ptr() if rope_dims else None, rope_dims, T, H, Hkv, hs, _stream()), "rope_kv_write")
+
+
+def _pow2_at_least(n: int) -> int:
+    p = 1
+    while p < n:
+        p *= 2
+    return p
+
+
+def attention_row_shape(H: int, Hkv: int, decode: bool):
+    """(RT, GT, QT): rows of a workgroup = QT query tokens x GT heads of one kv group."""
+    G = H // Hkv
+    GT = min(_pow2_at_least(G), 16)
+    RT = GT if decode else 16
+    return RT, GT, RT // GT
+
+
+def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int):
+    """(n_splits, chunk): how the keys of a decode step are cut so that the launch fills the
+    chip.  A function of the batch's shape and of max_len alone."""
+    RT, GT, _ = attention_row_shape(H, Hkv, True)
+    G = H // Hkv
+    wgs = max(1, n_seqs * Hkv * ((G + GT - 1) // GT))
+    pages = max(1, (max_len + PAGE - 1) // PAGE)
+    want = max(1, min(pages, 64, (512 + wgs - 1) // wgs))
+    chunk = ((pages + want - 1) // want) * PAGE
+    n_splits = (pages * PAGE + chunk - 1) // chunk
+    return n_splits, chunk
+
+
+def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+              block_table: torch.Tensor, H: int, Hkv: int, hs: int, scale: float, *, window: int = 0,
+              tiles=None, qt: int = 0, seq_lens=None, n_splits: int = 1, chunk: int = 0) -> None:
+    """Causal attention of the (rotated) Q heads in qkv over the paged cache.
+
+    Prompt form: `tiles` [n, 4] int32 = (sequence, first token row, tokens (<= qt), position of
+    the first), qt = the QT of attention_row_shape(H, Hkv, False).
+    Decode form: tiles None, seq_lens [B] int32 (keys in the cache, the new one included; 0 for a
+    padding row); row b of qkv is sequence b's token; n_splits/chunk from decode_splits."""
+    require_gpu()
+    _dev(qkv, "qkv", dims=2)
+    _dev(out, "out", qkv.dtype, 2)
+    _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype)
+    _dev(block_table, "block_table", torch.int32, 2)
+    T = qkv.shape[0]
+    if H % Hkv or qkv.shape[1] < H * hs or out.shape != (T, H * hs) or not out.is_contiguous():
+        raise KernelError(f"attention: qkv {tuple(qkv.shape)} / out {tuple(out.shape)} do not fit H={H} hs={hs}")
+    if hs % 8 or hs > 256:
+        raise KernelError(f"attention: head size {hs} is not supported (a multiple of 8, at most 256)")
+    if not block_table.is_contiguous():
+        raise KernelError("attention: block_table must be contiguous")
+    decode = tiles is None
+    RT, GT, QT = attention_row_shape(H, Hkv, decode)
+    if decode:
+        _dev(seq_lens, "seq_lens", torch.int32, 1)
+        if seq_lens.numel() != T or block_table.shape[0] < T or not seq_lens.is_contiguous():
+            raise KernelError("attention(decode): one seq_lens entry and one block_table row per token")
+        n_tiles = T
+    else:
+        _dev(tiles, "tiles", torch.int32, 2)
+        if tiles.shape[1] != 4 or not tiles.is_contiguous() or qt != QT:
+            raise KernelError(f"attention(prompt): tiles must be [n, 4] built for qt={QT}")
+        n_tiles = tiles.shape[0]
+        n_splits, chunk = 1, 0
+    if T == 0 or n_tiles == 0:
+        return
+    part_o = part_ml = None
+    if n_splits > 1:
+        if chunk <= 0 or chunk % PAGE:
+            raise KernelError(f"attention: chunk {chunk} must be a positive multiple of {PAGE}")
+        part_o = torch.empty((T * H * n_splits, hs), dtype=torch.float32, device=qkv.device)
+        part_ml = torch.empty((T * H * n_splits, 2), dtype=torch.float32, device=qkv.device)
+    _check(_fn("attn_rows", "bn_attn_rows")(
+        _code(qkv.dtype), qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * hs,
+        k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+        seq_lens.data_ptr() if decode else None, tiles.data_ptr() if not decode else None,
+        n_tiles, T, H, Hkv, hs, RT, GT, int(window), float(scale), int(n_splits), int(chunk),
+        part_o.data_ptr() if part_o is not None else None,
+        part_ml.data_ptr() if part_ml is not None else None, _stream()), "attention")
+
+
+# --------------------------------------------------------------------------------------
+# sampling
+# --------------------------------------------------------------------------------------
+
+def _logits_ok(logits):
+    _dev(logits, "logits", torch.float32, 2)
+    return _rows(logits, "logits")
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    require_gpu()
+    ld = _logits_ok(logits)
+    B, V = logits.shape
+    out = torch.empty((B,), dtype=torch.int32, device=logits.device)
+    if B:
+        _check(_fn("sampling", "bn_argmax")(logits.data_ptr(), ld, B, V, out.data_ptr(), _stream()), "argmax")
+    return out
+
+
+def repeat_penalty_(logits: torch.Tensor, recent: torch.Tensor, penalty: float) -> None:
+    """In place: every distinct token id of a row of `recent` (int32, -1 = none) is penalised once."""
+    require_gpu()
+    ld = _logits_ok(logits)
+    _dev(recent, "recent", torch.int32, 2)
+    if recent.shape[0] != logits.shape[0] or not recent.is_contiguous():
+        raise KernelError("repeat_penalty: one contiguous row of recent tokens per row of logits")
+    if logits.shape[0] and recent.shape[1]:
+        _check(_fn("sampling", "bn_repeat_penalty")(logits.data_ptr(), ld, logits.shape[0], logits.shape[1],
+                                                    recent.data_ptr(), recent.shape[1], float(penalty),
+                                                    _stream()), "repeat_penalty")
+
+
+def sample(logits: torch.Tensor, temperature: float, top_p: float, uniforms=None) -> torch.Tensor:
+    """One token id per row.  temperature 0: argmax.  uniforms: float32 [B] in [0, 1)."""
+    require_gpu()
+    ld = _logits_ok(logits)
+    B, V = logits.shape
+    out = torch.empty((B,), dtype=torch.int32, device=logits.device)
+    if B == 0:
+        return out
+    probs = None
+    if temperature != 0.0:
+        _dev(uniforms, "uniforms", torch.float32, 1)
+        if uniforms.numel() != B or not uniforms.is_contiguous():
+            raise KernelError("sample: one uniform number per row")
+        probs = torch.empty((B, V), dtype=torch.float32, device=logits.device)
+    _check(_fn("sampling", "bn_sample")(logits.data_ptr(), ld, B, V,
+                                        probs.data_ptr() if probs is not None else None,
+                                        uniforms.data_ptr() if probs is not None else None,
+                                        float(temperature), float(top_p), out.data_ptr(), _stream()), "sample")
+    return out
