@@ -1,0 +1,174 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the Llama-3.1-8B shape with random bf16 weights on one
+MI355X.  One JSON line on stdout.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
+
+A step is one decode step of the whole batch: the step function, greedy sampling on the
+device and the read-back of the tokens, as generation does it.  `value` is decoded
+tokens a second at the default batch.  The same line carries the prefill of 2,048
+tokens, the decode roofline (bytes the step has to read: every weight once plus the
+cache of the live requests, over its time, against 8 TB/s) and decode at batch 1 and 64.
+"""
+import argparse
+import json
+import os
+import random
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+HBM_GBS = 8000.0
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "fp32": 157.3}
+
+# The Llama-3.1-8B shape (the benchmark configuration): context 4,096, prompts of 128..2048 tokens
+SHAPE = dict(model_type="llama", vocab_size=128256, hidden_size=4096, intermediate_size=14336,
+             num_hidden_layers=32, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+             max_position_embeddings=131072, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+             rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                               original_max_position_embeddings=8192))
+CONTEXT = 4096
+PREFILL_TOKENS = 2048
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=SHAPE["num_hidden_layers"],
+                    help="fewer layers than the configuration has (named in the record)")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+
+    import bitnet_c_amd as bn
+    from bitnet_c_amd import ops
+    from bitnet_c_amd.config import architecture_for
+    from bitnet_c_amd.engine import DecoderModel
+    from bitnet_c_amd.weights import random_tensors
+
+    dev = "cuda:0"
+    raw = dict(SHAPE, num_hidden_layers=args.layers)
+    cfg = bn.LlamaConfig.from_dict(raw)
+    plan = architecture_for(raw).build_plan(cfg)
+    t0 = time.time()
+    model = DecoderModel(plan, torch.bfloat16, dev)
+    tensors = random_tensors(plan.expected_tensors(), args.seed, torch.bfloat16, device=dev)
+    model.load(tensors)
+    del tensors
+    torch.cuda.empty_cache()
+    print(f"[bench] model built in {time.time() - t0:.1f} s, weights {model.weight_bytes() / 1e9:.2f} GB",
+          file=sys.stderr, flush=True)
+
+    max_batch = max(args.batch, 1 if args.no_points else 64)
+    per_seq = ((2048 + args.steps + args.warmup + 64 + 63) // 64) * 64
+    engine = bn.Engine(model, max_tokens=max(max_batch * per_seq, 4096), max_seq_len=CONTEXT)
+    L, H, Hkv, hs = cfg.num_hidden_layers, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    kv_bytes_per_token = 2 * L * Hkv * hs * 2
+    weight_bytes = model.weight_bytes() - (0 if cfg.tie_word_embeddings else model.embedding.numel() * 2)
+    rnd = random.Random(args.seed + 1)
+
+    def sync():
+        torch.cuda.synchronize()
+
+    # ---- prefill of 2,048 tokens ------------------------------------------------------
+    def prefill_once(n):
+        toks = [rnd.randrange(cfg.vocab_size) for _ in range(n)]
+        s = engine.new_sequence()
+        sync()
+        t = time.perf_counter()
+        lg = engine.step([bn.StepEntry(s, toks, [n - 1])])
+        ops.argmax(lg).cpu()
+        sync()
+        dt = time.perf_counter() - t
+        engine.release(s)
+        return dt
+
+    prefill_once(PREFILL_TOKENS)
+    prefill_once(PREFILL_TOKENS)
+    p_ms = sorted(prefill_once(PREFILL_TOKENS) for _ in range(5))[2] * 1e3
+    T = PREFILL_TOKENS
+    lin_params = L * (cfg.hidden_size * (cfg.q_dim + 2 * cfg.kv_dim) + cfg.q_dim * cfg.hidden_size
+                      + 3 * cfg.hidden_size * cfg.intermediate_size)
+    flops = 2.0 * T * lin_params + 4.0 * T * T * hs * H * L / 2 + 2.0 * cfg.vocab_size * cfg.hidden_size
+    prefill = {"value": round(T / (p_ms / 1e3), 1), "tokens": T, "ms": round(p_ms, 3),
+               "frac": round(flops / (p_ms / 1e3) / (PEAK_TFLOPS["bf16"] * 1e12), 4)}
+    print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
+
+    # ---- decode -----------------------------------------------------------------------
+    def decode(batch, steps, warmup):
+        lens = [rnd.randint(128, 2048) for _ in range(batch)]
+        slots = [engine.new_sequence() for _ in range(batch)]
+        # the prompts, a few sequences a step to bound the activations
+        last = [0] * batch
+        for i in range(0, batch, 8):
+            ent = [bn.StepEntry(slots[j], [rnd.randrange(cfg.vocab_size) for _ in range(lens[j])], [lens[j] - 1])
+                   for j in range(i, min(batch, i + 8))]
+            toks = ops.argmax(engine.step(ent)).cpu().tolist()
+            for j, t in zip(range(i, min(batch, i + 8)), toks):
+                last[j] = t
+
+        def one():
+            nonlocal last
+            lg = engine.step([bn.StepEntry(slots[j], [last[j]], [0]) for j in range(batch)])
+            last = ops.argmax(lg).cpu().tolist()
+
+        for _ in range(warmup):
+            one()
+        sync()
+        t = time.perf_counter()
+        for _ in range(steps):
+            one()
+        sync()
+        dt = time.perf_counter() - t
+        ctx_mid = sum(lens) + batch * (warmup + steps / 2.0)          # cached tokens read by a mid step
+        for s in slots:
+            engine.release(s)
+        return dt / steps, ctx_mid
+
+    step_s, ctx_tokens = decode(args.batch, args.steps, args.warmup)
+    value = args.batch / step_s
+    bytes_step = weight_bytes + ctx_tokens * kv_bytes_per_token
+    achieved = bytes_step / step_s / 1e9
+    print(f"[bench] decode b{args.batch}: {step_s * 1e3:.3f} ms/step, {value:.1f} tok/s, {achieved:.0f} GB/s",
+          file=sys.stderr, flush=True)
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            s_b, _ = decode(b, max(16, args.steps // 2), args.warmup)
+            points[f"decode_b{b}"] = round(b / s_b, 1)
+            print(f"[bench] decode b{b}: {s_b * 1e3:.3f} ms/step, {b / s_b:.1f} tok/s", file=sys.stderr, flush=True)
+
+    rec = {
+        "metric": "decode tok/s @ batch 8 (Llama-3.1-8B shape, bf16)", "value": round(value, 1), "unit": "tok/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic: random N(0,0.02) weights, uniform random token ids, prompts of 128..2048 tokens",
+        "config": {"model": "llama-3.1-8b-shape", "layers": cfg.num_hidden_layers,
+                   "layers_of_config": SHAPE["num_hidden_layers"], "hidden": cfg.hidden_size,
+                   "heads": H, "kv_heads": Hkv, "head_dim": hs, "intermediate": cfg.intermediate_size,
+                   "vocab": cfg.vocab_size, "rope_theta": cfg.rope_theta, "rope_scaling": "llama3 f8 l1 h4 o8192",
+                   "rms_norm_eps": cfg.rms_norm_eps, "tied": cfg.tie_word_embeddings,
+                   "global_batch": args.batch, "seq_len": CONTEXT, "prompt_lens": "U[128,2048]",
+                   "prefill_tokens": PREFILL_TOKENS, "parallelism": "none (1 GPU)"},
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(rec), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

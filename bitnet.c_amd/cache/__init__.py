@@ -1,0 +1,1 @@
+from .paged import PAGE, CacheError, CacheFull, PagePool, PagedCache

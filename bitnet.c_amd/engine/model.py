@@ -1,0 +1,80 @@
+"""The model: parts built from a plan, weights loaded into them, one forward over the
+tokens of a step.  It owns the uploaded device tensors (the reference's backend model
+holds them apart from the immutable host weights, include/backend_model.h:14-108).
+"""
+from __future__ import annotations
+
+from typing import Dict, List
+
+import torch
+
+from .. import ops
+from ..parts import BLOCKS, NORMS, CacheNeed, ResidualStream
+from .plan import ModelPlan
+
+
+class DecoderModel:
+    def __init__(self, plan: ModelPlan, dtype=torch.bfloat16, device="cuda:0"):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"compute dtype must be bfloat16 or float32, got {dtype}")
+        plan.validate()
+        self.plan, self.dtype, self.device = plan, dtype, torch.device(device)
+        self.blocks = [BLOCKS.build(lp.block) for lp in plan.layers]
+        self.final_norm = NORMS.build(plan.final_norm)
+        self.embedding = None            # [V, D] in the compute dtype
+        self.lm_head = None              # [V, D]; the embedding itself when tied
+
+    # ---- weights --------------------------------------------------------------------
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        """tensors: folder name -> host tensor (every name of plan.expected_tensors())."""
+        p = self.plan
+        for lp, blk in zip(p.layers, self.blocks):
+            local = {ln: tensors[fn] for ln, fn in lp.names.items() if fn in tensors and ln in blk.tensors()}
+            blk.load(local, self.device, self.dtype)
+        self.final_norm.load({ln: tensors[fn] for ln, fn in p.final_norm_names.items()}, self.device, self.dtype)
+        self.embedding = tensors[p.embedding_name].to(self.dtype).to(self.device).contiguous()
+        if p.lm_head_name is None:
+            self.lm_head = self.embedding
+        else:
+            self.lm_head = tensors[p.lm_head_name].to(self.dtype).to(self.device).contiguous()
+
+    def weight_bytes(self) -> int:
+        """Bytes of every weight a decode step reads once (the embedding table only when it is
+        also the output matrix)."""
+        seen, total = set(), 0
+
+        def add(t):
+            nonlocal total
+            if t is not None and t.data_ptr() not in seen:
+                seen.add(t.data_ptr())
+                total += t.numel() * t.element_size()
+
+        def walk(obj, depth=0):
+            if isinstance(obj, torch.Tensor):
+                add(obj)
+            elif depth < 4 and hasattr(obj, "__dict__"):
+                for v in vars(obj).values():
+                    walk(v, depth + 1)
+
+        for blk in self.blocks:
+            walk(blk)
+        walk(self.final_norm)
+        add(self.lm_head)
+        return total
+
+    # ---- cache needs -------------------------------------------------------------------
+    def cache_needs(self):
+        needs: List[CacheNeed] = [self.blocks[e.layer].cache_need() for e in self.plan.schedule]
+        return needs, [e.kv_from for e in self.plan.schedule]
+
+    # ---- forward -----------------------------------------------------------------------
+    def forward(self, ctx, views) -> torch.Tensor:
+        """ctx: the step's StepContext; views[i]: the KVView of schedule entry i.
+        Returns float32 logits [len(ctx.want_rows), vocab]."""
+        x = ops.embed_gather(self.embedding, ctx.tokens)          # src/model_embed.c:6-28
+        stream = ResidualStream(x)
+        for i, e in enumerate(self.plan.schedule):
+            self.blocks[e.layer].forward(stream, ctx, views[i])
+        # final norm on the wanted rows only, then the output matrix (src/transformer/logits.c:249-314)
+        h = stream.normed(self.final_norm, self.dtype, rows=ctx.want_rows)
+        return ops.linear(h, self.lm_head, torch.float32)

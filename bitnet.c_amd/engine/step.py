@@ -1,0 +1,293 @@
+"""The step function and what it needs: the description of a step's batch and the engine
+that runs it against the cache.
+
+One step takes a batch of sequences that start together, with unequal lengths: their
+prompts in one step, then one token each.  It runs only the tokens it is given, all
+sequences as one flattened batch without padding between them, reads everything earlier
+from the cache, and returns the float32 logits at the wanted places.  The reference has
+five single-sequence entry points for this (include/transformer.h:9-30: one token with or
+without logits; n tokens with last, no or all logits) and validates tokens and positions
+before it touches state (src/transformer/prefill.c:1228-1237, src/transformer.c:60-70);
+all new keys and values are in the cache before any new token attends
+(src/transformer/prefill.c:1836-1875 before :1962).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from .. import ops
+from ..cache import PAGE, CacheError, CacheFull, PagedCache
+from ..config import load_config
+from ..weights import load_tensors
+from .model import DecoderModel
+
+
+class StepError(ValueError):
+    """A step that cannot run; nothing was changed."""
+
+
+@dataclass
+class StepEntry:
+    slot: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()          # places among `tokens` whose logits are wanted
+
+
+class StepContext:
+    """Device-side description of one step, shared by all parts."""
+
+    def __init__(self, device, act_dtype, tokens, positions, seq_index, seq_lens, want_rows, slots_dev,
+                 is_decode, slots, n_new, pos0):
+        self.device, self.act_dtype = device, act_dtype
+        self.tokens, self.positions, self.seq_index = tokens, positions, seq_index
+        self.seq_lens, self.want_rows, self.slot_ids = seq_lens, want_rows, slots_dev
+        self.is_decode = is_decode
+        self.slots, self.n_new, self.pos0 = list(slots), list(n_new), list(pos0)   # host copies
+        self.n_rows = int(tokens.numel())
+        self.n_seqs = len(self.slots)
+        self._tiles: Dict[int, torch.Tensor] = {}
+
+    def row_ranges(self):
+        """(first row, rows) of every sequence in the flattened batch."""
+        out, r = [], 0
+        for n in self.n_new:
+            out.append((r, n))
+            r += n
+        return out
+
+    def tiles(self, qt: int) -> torch.Tensor:
+        """[n, 4] int32: (sequence, first row, rows <= qt, position of the first) covering all new
+        tokens, for the prompt form of the attention kernel."""
+        t = self._tiles.get(qt)
+        if t is None:
+            rows, r = [], 0
+            for s, (n, p0) in enumerate(zip(self.n_new, self.pos0)):
+                for i in range(0, n, qt):
+                    rows.append((s, r + i, min(qt, n - i), p0 + i))
+                r += n
+            t = torch.tensor(rows, dtype=torch.int32).reshape(-1, 4).to(self.device)
+            self._tiles[qt] = t
+        return t
+
+
+def _bucket(n: int) -> int:
+    b = 1
+    while b < n:
+        b *= 2
+    return b
+
+
+class _DecodeGraph:
+    """A captured decode step for up to `rows` sequences whose block tables have `width`
+    columns.  Inputs live in one int32 buffer that is refilled before every replay."""
+
+    def __init__(self, engine: "Engine", rows: int, width: int):
+        self.rows, self.width = rows, width
+        dev = engine.device
+        n_groups = len(engine.cache.groups)
+        self.n_ints = 5 * rows + n_groups * rows * width
+        self.host = torch.zeros(self.n_ints, dtype=torch.int32).pin_memory()
+        self.dev = torch.zeros(self.n_ints, dtype=torch.int32, device=dev)
+        self.copied = torch.cuda.Event()
+        self.copied.record()
+        o = 0
+
+        def take(n):
+            nonlocal o
+            v = self.dev[o:o + n]
+            o += n
+            return v
+
+        self.tokens, self.positions, self.seq_index = take(rows), take(rows), take(rows)
+        self.seq_lens, self.want = take(rows), take(rows)
+        self.tables = {g: take(rows * width).view(rows, width) for g in range(n_groups)}
+        views = [engine.cache.view(i, self.tables, width * PAGE) for i in range(len(engine.model.plan.schedule))]
+        self.ctx = StepContext(dev, engine.model.dtype, self.tokens, self.positions, self.seq_index, self.seq_lens,
+                               self.want, None, True, [-1] * rows, [1] * rows, [0] * rows)
+        # padding rows everywhere: the warm-up and the capture run touch no sequence's pages
+        self.fill([-1] * rows, [0] * rows, [0] * rows, engine)
+        self.upload()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            engine.model.forward(self.ctx, views)              # loads every kernel before the capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits = engine.model.forward(self.ctx, views)
+
+    def fill(self, slots, tokens, lens_after, engine):
+        rows, h = self.rows, self.host
+        self.copied.synchronize()
+        n = len(slots)
+        h.zero_()
+        h[0:n] = torch.tensor(tokens, dtype=torch.int32)
+        h[rows:rows + n] = torch.tensor([l - 1 for l in lens_after], dtype=torch.int32)
+        h[rows + n:2 * rows] = -1                                     # padding rows: position -1
+        for i, s in enumerate(slots):
+            if s < 0:
+                h[rows + i] = -1
+        h[2 * rows:3 * rows] = torch.arange(rows, dtype=torch.int32)  # row b is sequence b
+        h[3 * rows:3 * rows + n] = torch.tensor([max(l, 0) for l in lens_after], dtype=torch.int32)
+        h[4 * rows:5 * rows] = torch.arange(rows, dtype=torch.int32)
+        o = 5 * rows
+        for g in range(len(engine.cache.groups)):
+            bt = engine.cache.block_table(g, list(slots) + [-1] * (rows - n), self.width)
+            h[o:o + rows * self.width] = bt[:, :self.width].reshape(-1)
+            o += rows * self.width
+
+    def upload(self):
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+
+    def run(self):
+        self.graph.replay()
+        return self.logits
+
+
+class Engine:
+    """A model, its cache and the step function over both."""
+
+    def __init__(self, model: DecoderModel, max_tokens: int, max_seq_len: int = 0, max_slots: int = 0,
+                 use_graphs: bool = True):
+        ops.require_gpu()
+        self.model, self.device = model, model.device
+        needs, kv_from = model.cache_needs()
+        self.cache = PagedCache(needs, kv_from, max_tokens, dtype=model.dtype, device=self.device,
+                                max_slots=max_slots or None)
+        limit = self.cache.n_pages * PAGE
+        if model.plan.max_positions:
+            limit = min(limit, model.plan.max_positions)
+        self.max_seq_len = min(limit, max_seq_len) if max_seq_len else limit
+        self.vocab_size = model.plan.vocab_size
+        # a mixer that keeps a state addresses it by the host's slot list, which a replayed graph
+        # cannot see: such models run their decode steps eagerly
+        self.use_graphs = use_graphs and all(n.state is None for n in needs)
+        self._graphs: Dict[tuple, _DecodeGraph] = {}
+        self.steps_run = 0
+
+    # ---- construction ---------------------------------------------------------------
+    @staticmethod
+    def from_folder(folder: str, dtype=torch.bfloat16, max_tokens: int = 4096, device="cuda:0",
+                    max_seq_len: int = 0, max_slots: int = 0, use_graphs: bool = True) -> "Engine":
+        ops.require_gpu()
+        arch, config = load_config(folder)
+        plan = arch.build_plan(config)
+        tensors = load_tensors(folder, plan.expected_tensors())
+        model = DecoderModel(plan, dtype, device)
+        model.load(tensors)
+        eng = Engine(model, max_tokens, max_seq_len, max_slots, use_graphs)
+        eng.config = config
+        return eng
+
+    # ---- sequences ------------------------------------------------------------------
+    def new_sequence(self) -> int:
+        return self.cache.alloc_slot()
+
+    def release(self, slot: int) -> None:
+        self.cache.free_slot(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    # ---- the step -------------------------------------------------------------------
+    def _validate(self, entries: Sequence[StepEntry]):
+        if not entries:
+            raise StepError("a step needs at least one sequence")
+        seen = set()
+        for e in entries:
+            if e.slot in seen:
+                raise StepError(f"slot {e.slot} appears twice in one step")
+            seen.add(e.slot)
+            try:
+                have = self.cache.length(e.slot)
+            except CacheError as err:
+                raise StepError(str(err)) from None
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"slot {e.slot}: no tokens in this step")
+            for t in e.tokens:
+                if not (0 <= int(t) < self.vocab_size):
+                    raise StepError(f"slot {e.slot}: token {t} is outside [0, {self.vocab_size})")
+            if have + n > self.max_seq_len:
+                raise StepError(f"slot {e.slot}: {have} + {n} tokens exceed the sequence limit {self.max_seq_len}")
+            for w in e.want:
+                if not (0 <= int(w) < n):
+                    raise StepError(f"slot {e.slot}: wanted place {w} is outside its {n} tokens")
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Runs the entries' tokens as one batch; returns float32 logits [wanted, vocab] in the
+        order of the entries and of each entry's `want`.  On an error nothing has changed."""
+        entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        self._validate(entries)
+        slots = [e.slot for e in entries]
+        n_new = [len(e.tokens) for e in entries]
+        pos0 = [self.cache.length(s) for s in slots]
+        try:
+            self.cache.reserve(slots, n_new)
+        except CacheFull as err:
+            raise StepError(str(err)) from None
+        is_decode = all(n == 1 for n in n_new)
+        if is_decode and self.use_graphs and len(entries) <= 64:
+            logits = self._step_graph(entries, slots, pos0)
+        else:
+            logits = self._step_eager(entries, slots, n_new, pos0, is_decode)
+        self.cache.commit(slots, n_new)
+        self.steps_run += 1
+        return logits
+
+    def _step_eager(self, entries, slots, n_new, pos0, is_decode):
+        dev = self.device
+        tokens, positions, seq_index, want = [], [], [], []
+        row = 0
+        for s, e in enumerate(entries):
+            tokens += [int(t) for t in e.tokens]
+            positions += list(range(pos0[s], pos0[s] + n_new[s]))
+            seq_index += [s] * n_new[s]
+            want += [row + int(w) for w in e.want]
+            row += n_new[s]
+        T, B = row, len(entries)
+        lens_after = [p + n for p, n in zip(pos0, n_new)]
+        tables = {g: self.cache.block_table(g, slots) for g in range(len(self.cache.groups))}
+        # one upload for all integer inputs of the step
+        parts = [tokens, positions, seq_index, lens_after, want, slots] + [tables[g].reshape(-1).tolist()
+                                                                            for g in sorted(tables)]
+        flat = torch.tensor([v for p in parts for v in p], dtype=torch.int32)
+        devbuf = flat.to(dev)
+        o = 0
+
+        def take(n):
+            nonlocal o
+            v = devbuf[o:o + n]
+            o += n
+            return v
+
+        d_tokens, d_pos, d_seq, d_lens, d_want, d_slots = take(T), take(T), take(T), take(B), take(len(want)), take(B)
+        d_tables = {g: take(tables[g].numel()).view(tables[g].shape) for g in sorted(tables)}
+        ctx = StepContext(dev, self.model.dtype, d_tokens, d_pos, d_seq, d_lens, d_want, d_slots, is_decode,
+                          slots, n_new, pos0)
+        max_len = max(lens_after)
+        views = [self.cache.view(i, d_tables, max_len) for i in range(len(self.model.plan.schedule))]
+        return self.model.forward(ctx, views)
+
+    def _step_graph(self, entries, slots, pos0):
+        B = len(entries)
+        lens_after = [p + 1 for p in pos0]
+        width = _bucket(max((l + PAGE - 1) // PAGE for l in lens_after))
+        key = (_bucket(B), width)
+        g = self._graphs.get(key)
+        if g is None:
+            g = _DecodeGraph(self, key[0], width)
+            self._graphs[key] = g
+        g.fill(slots, [int(e.tokens[0]) for e in entries], lens_after, self)
+        g.upload()
+        logits = g.run()
+        rows = [i for i, e in enumerate(entries) for _ in e.want]
+        if rows == list(range(B)):
+            return logits[:B].clone()
+        idx = torch.tensor(rows, dtype=torch.long, device=self.device)
+        return logits.index_select(0, idx)

@@ -401,6 +401,9 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     if n_splits > 1:
         if chunk <= 0 or chunk % PAGE:
             raise KernelError(f"attention: chunk {chunk} must be a positive multiple of {PAGE}")
+        if n_splits * chunk < block_table.shape[1] * PAGE:
+            raise KernelError(f"attention: {n_splits} splits of {chunk} keys do not cover the "
+                              f"{block_table.shape[1]} pages of the block table")
         part_o = torch.empty((T * H * n_splits, hs), dtype=torch.float32, device=qkv.device)
         part_ml = torch.empty((T * H * n_splits, 2), dtype=torch.float32, device=qkv.device)
     _check(_fn("attn_rows", "bn_attn_rows")(

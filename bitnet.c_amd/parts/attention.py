@@ -1,0 +1,87 @@
+"""Attention mixer: grouped-query attention over the paged cache.
+
+Order of the reference's layer (src/transformer/cpu.c:770-939): Q, K, V projections
+(+ bias when the tensors exist) -> position encoding of Q and K -> K, V into the cache
+-> for head h, kv head h / (H/Hkv): scores (q.k) * scale over the visible keys, softmax,
+weighted sum of values -> output projection.  scale is a parameter (1/sqrt(head_dim)
+for this architecture, src/model_arch.c:141-145); `window` > 0 limits the visible keys
+to the last `window` positions.
+
+The three projections are stored stacked ([Wq; Wk; Wv], as the reference's GPU upload
+stacks them, include/backend_model.h:21-22) so that one product computes them.
+A schedule entry that reads another entry's cache computes Q only.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from .base import MIXERS, POSITION_ENCODINGS, CacheNeed, KVNeed, ParamSpec, Part, PartSpec
+from .linear import Linear
+
+
+@MIXERS.register("attention")
+class Attention(Part):
+    def __init__(self, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
+                 position: PartSpec, window: int = 0, bias: bool = False):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} kv heads")
+        if head_dim % 8 or head_dim > 256:
+            raise ValueError(f"attention: head_dim {head_dim} is not supported by the kernels "
+                             f"(a multiple of 8, at most 256)")
+        self.hidden, self.H, self.Hkv, self.hs = int(hidden), int(n_heads), int(n_kv_heads), int(head_dim)
+        self.scale, self.window, self.has_bias = float(scale), int(window), bool(bias)
+        self.position = POSITION_ENCODINGS.build(position)
+        self.qkv, self.o = Linear(), Linear()
+
+    @property
+    def q_dim(self):
+        return self.H * self.hs
+
+    @property
+    def kv_dim(self):
+        return self.Hkv * self.hs
+
+    def tensors(self):
+        t = {"wq": ParamSpec((self.q_dim, self.hidden)), "wk": ParamSpec((self.kv_dim, self.hidden)),
+             "wv": ParamSpec((self.kv_dim, self.hidden)), "wo": ParamSpec((self.hidden, self.q_dim))}
+        if self.has_bias:
+            t.update({"bq": ParamSpec((self.q_dim,), "zeros"), "bk": ParamSpec((self.kv_dim,), "zeros"),
+                      "bv": ParamSpec((self.kv_dim,), "zeros"), "bo": ParamSpec((self.hidden,), "zeros")})
+        return t
+
+    def load(self, tensors, device, dtype):
+        w = torch.cat([tensors["wq"].to(dtype), tensors["wk"].to(dtype), tensors["wv"].to(dtype)], dim=0)
+        b = None
+        if self.has_bias:
+            b = torch.cat([tensors["bq"].float(), tensors["bk"].float(), tensors["bv"].float()])
+        self.qkv.load(w, b, device, dtype)
+        self.o.load(tensors["wo"], tensors.get("bo") if self.has_bias else None, device, dtype)
+        self.position.prepare(device)
+
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed(kv=KVNeed(self.Hkv, self.hs, self.window))
+
+    def forward(self, h, ctx, kv):
+        H, Hkv, hs = self.H, self.Hkv, self.hs
+        if kv.writes:
+            qkv = self.qkv(h)                                   # [T, (H + 2 Hkv) hs]
+        else:
+            qkv = self.qkv(h, rows=slice(0, self.q_dim))        # Q alone
+            pad = torch.empty((h.shape[0], (H + 2 * Hkv) * hs), dtype=h.dtype, device=h.device)
+            pad[:, :self.q_dim] = qkv
+            qkv = pad
+        self.position.encode_and_store(qkv, ctx, H, Hkv, hs, kv)
+        out = torch.empty((h.shape[0], self.q_dim), dtype=h.dtype, device=h.device)
+        if ctx.is_decode:
+            if self.window:                   # a window is short; its keys are not split
+                n_splits, chunk = 1, 0
+            else:
+                n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len)
+            ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
+                          window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk)
+        else:
+            _, _, qt = ops.attention_row_shape(H, Hkv, False)
+            ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
+                          window=self.window, tiles=ctx.tiles(qt), qt=qt)
+        return self.o(out)

@@ -1,0 +1,161 @@
+"""What a layer is put together from: a mixer (attention here), a feed-forward, norms, a
+position encoding, and the arrangement of these in a block.  Each kind of part has its
+own registry from a name to a class; a plan names parts by (kind, params) and a layer is
+built from the plan alone, so one model can hold different mixers and feed-forwards in
+different layers.  No part knows which model it is in: sizes and constants arrive as
+parameters, tensors under local names ("wq", "weight"), and the architecture maps the
+local names to the names of the model folder.
+
+Interfaces (a new part implements the one of its kind and registers itself):
+
+  every part     tensors() -> {local name: TensorSpec-like (shape, init, optional)}
+                 load(tensors: {local name: host tensor}, device, dtype) -> None
+
+  norm           apply(x_f32 [T, D], delta or None, out_dtype, rows=None) -> [T or len(rows), D]
+                 (adds delta into x in place when rows is None, then norms)
+
+  position       prepare(device) -> None
+                 encode_and_store(qkv, ctx, H, Hkv, hs, kv) -> None
+                 (encodes Q in place, encodes K and stores K, V into kv when kv.writes)
+
+  mixer          cache_need() -> CacheNeed (what it keeps per sequence: keys/values and/or a
+                 state of fixed size)
+                 forward(h [T, D], ctx, kv) -> delta [T, D]
+
+  feed-forward   forward(h [T, D], ctx) -> delta [T, D]
+
+  block          forward(stream: ResidualStream, ctx, kv) -> None
+
+The reference decides the same things per call with per-layer plan structs
+(include/transformer_plan_internal.h:12-185, src/transformer/plan.c:315-342, 705-863);
+here the decision is made once, when the model is built.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """A part named by its registry key and its constants."""
+    kind: str
+    params: Tuple[Tuple[str, object], ...] = ()
+
+    @staticmethod
+    def of(kind: str, **params) -> "PartSpec":
+        return PartSpec(kind, tuple(sorted(params.items())))
+
+    def kwargs(self) -> dict:
+        return dict(self.params)
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    shape: Tuple[int, ...]
+    init: str = "normal"        # how the random-weights mode fills it: normal | ones | zeros
+    optional: bool = False
+
+
+@dataclass(frozen=True)
+class KVNeed:
+    """Keys and values of every position (window 0) or of the last `window` positions."""
+    n_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """A state of fixed size per sequence, zero when the sequence starts."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    kv: Optional[KVNeed] = None
+    state: Optional[StateNeed] = None
+
+
+class Registry:
+    def __init__(self, what: str):
+        self.what = what
+        self._items: Dict[str, type] = {}
+
+    def register(self, name: str, cls: type = None, *, replace: bool = False):
+        def put(c):
+            if name in self._items and not replace:
+                raise ValueError(f"{self.what} {name!r} is already registered")
+            self._items[name] = c
+            return c
+        return put(cls) if cls is not None else put
+
+    def build(self, spec: PartSpec, **extra):
+        if spec.kind not in self._items:
+            raise KeyError(f"unknown {self.what} {spec.kind!r}; registered: {sorted(self._items)}")
+        return self._items[spec.kind](**spec.kwargs(), **extra)
+
+    def names(self):
+        return sorted(self._items)
+
+    def __contains__(self, name):
+        return name in self._items
+
+
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+NORMS = Registry("norm")
+POSITION_ENCODINGS = Registry("position encoding")
+BLOCKS = Registry("block")
+
+
+class Part:
+    """Base of all parts: no tensors, nothing to load."""
+
+    def tensors(self) -> Dict[str, ParamSpec]:
+        return {}
+
+    def load(self, tensors: Dict[str, torch.Tensor], device, dtype) -> None:
+        pass
+
+
+@dataclass
+class KVView:
+    """What a mixer sees of the cache for one entry of the schedule in one step."""
+    k_pages: Optional[torch.Tensor] = None      # [pages, Hkv, PAGE, hs]
+    v_pages: Optional[torch.Tensor] = None
+    block_table: Optional[torch.Tensor] = None  # [B, W] int32, this step's sequences
+    writes: bool = True                         # False: the entry reads another entry's cache
+    state: Optional[torch.Tensor] = None        # [max_slots, *shape] fixed-size state, by slot
+    max_len: int = 0                            # bound of the key count in this step (sizes the splits)
+
+
+class ResidualStream:
+    """The float32 residual stream of a step.  A part's output is held back as `pending` and
+    is added by the kernel of the next norm, so the sum is formed once, in float32, without a
+    pass of its own."""
+
+    def __init__(self, x: torch.Tensor):
+        self.x = x
+        self.pending: Optional[torch.Tensor] = None
+
+    def add(self, delta: torch.Tensor) -> None:
+        if self.pending is not None:
+            self.flush()
+        self.pending = delta
+
+    def flush(self) -> torch.Tensor:
+        if self.pending is not None:
+            from .. import ops
+            ops.residual_add(self.x, self.pending)
+            self.pending = None
+        return self.x
+
+    def normed(self, norm, out_dtype, rows=None) -> torch.Tensor:
+        h = norm.apply(self.x, self.pending, out_dtype, rows)
+        if rows is None:
+            self.pending = None
+        return h

@@ -1,0 +1,40 @@
+"""Dense gated feed-forward: down(silu(gate(x)) * up(x)), silu(g) = g / (1 + exp(-g))
+(src/transformer/cpu.c:1270-1303, src/transformer/cpu_backend.c:385-391).  Gate and up
+are stored stacked ([Wg; Wu], as the reference's GPU upload stacks them,
+include/backend_model.h:22) so that one product computes both; at decode sizes the
+activation is part of that kernel."""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from .base import FEED_FORWARDS, ParamSpec, Part
+from .linear import Linear
+
+
+@FEED_FORWARDS.register("swiglu")
+class SwiGLU(Part):
+    def __init__(self, hidden: int, intermediate: int, bias: bool = False):
+        self.hidden, self.F, self.has_bias = int(hidden), int(intermediate), bool(bias)
+        self.gate_up, self.down = Linear(), Linear()
+
+    def tensors(self):
+        t = {"w_gate": ParamSpec((self.F, self.hidden)), "w_up": ParamSpec((self.F, self.hidden)),
+             "w_down": ParamSpec((self.hidden, self.F))}
+        if self.has_bias:
+            t.update({"b_gate": ParamSpec((self.F,), "zeros"), "b_up": ParamSpec((self.F,), "zeros"),
+                      "b_down": ParamSpec((self.hidden,), "zeros")})
+        return t
+
+    def load(self, tensors, device, dtype):
+        w = torch.cat([tensors["w_gate"].to(dtype), tensors["w_up"].to(dtype)], dim=0)
+        b = torch.cat([tensors["b_gate"].float(), tensors["b_up"].float()]) if self.has_bias else None
+        self.gate_up.load(w, b, device, dtype)
+        self.down.load(tensors["w_down"], tensors.get("b_down") if self.has_bias else None, device, dtype)
+
+    def forward(self, h, ctx):
+        if self.has_bias:
+            act = ops.swiglu(self.gate_up(h))
+        else:
+            act = ops.linear_swiglu(h, self.gate_up.weight)
+        return self.down(act)

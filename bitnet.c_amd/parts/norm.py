@@ -1,0 +1,25 @@
+"""RMSNorm: out = x * 1/sqrt(mean(x^2) + eps) * w, eps inside the root
+(src/transformer/rmsnorm_scalar.c:4-13).  Computed in float32 whatever the activation
+type; the weight is kept in float32."""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from .base import NORMS, ParamSpec, Part
+
+
+@NORMS.register("rmsnorm")
+class RMSNorm(Part):
+    def __init__(self, dim: int, eps: float):
+        self.dim, self.eps = int(dim), float(eps)
+        self.weight = None
+
+    def tensors(self):
+        return {"weight": ParamSpec((self.dim,), init="ones")}
+
+    def load(self, tensors, device, dtype):
+        self.weight = tensors["weight"].to(torch.float32).to(device).contiguous()
+
+    def apply(self, x, delta, out_dtype, rows=None):
+        return ops.add_rmsnorm(x, delta, self.weight, self.eps, out_dtype, rows)

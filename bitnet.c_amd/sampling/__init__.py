@@ -1,0 +1,1 @@
+from .sampler import SamplingParams, SequenceSampler, XorShift64Star, sample_batch

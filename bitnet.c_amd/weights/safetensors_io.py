@@ -79,10 +79,8 @@ class SafetensorsFile:
         a, b = self._spans[name]
         if a == b:
             return torch.empty(shape, dtype=dt)
-        buf = memoryview(self._mm)[self._base + a:self._base + b]
-        t = torch.frombuffer(buf, dtype=dt).reshape(shape).clone()
-        buf.release()
-        return t
+        owned = bytearray(self._mm[self._base + a:self._base + b])     # one copy out of the map
+        return torch.frombuffer(owned, dtype=dt).reshape(shape)
 
     def close(self) -> None:
         if self._mm is not None:

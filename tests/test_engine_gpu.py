@@ -1,0 +1,254 @@
+"""The engine against the plain implementation, in float32 and in bfloat16: each request
+alone and whole; with the last 32 tokens one by one; in batches of unequal lengths whose
+shorter requests end earlier, one batch after another so that slots and pages are used
+again; long decoding; the first tokens of a sequence; with and without HIP graphs."""
+import functools
+import random
+
+import pytest
+import torch
+
+import plain_llama as pl
+from conftest import TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+NAMES = ["A", "B", "C"]
+
+
+def _requests(vocab, seed, lengths):
+    rnd = random.Random(seed)
+    return [[rnd.randrange(vocab) for _ in range(n)] for n in lengths]
+
+
+@functools.lru_cache(maxsize=None)
+def _plain_cached(folder, tokens, rounded):
+    c, W = pl.read_config(folder), pl.read_weights(folder)
+    return pl.forward(c, W, list(tokens), torch.bfloat16 if rounded else None)
+
+
+def plain_logits(folder, tokens, dtype):
+    return _plain_cached(folder, tuple(tokens), dtype == torch.bfloat16)
+
+
+def make_engine(folder, dtype, max_tokens=1024, **kw):
+    from bitnet_c_amd import Engine
+    return Engine.from_folder(folder, dtype=dtype, max_tokens=max_tokens, **kw)
+
+
+LENGTHS = [1, 5, 33, 64, 65, 100, 150]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_whole_requests_alone(model_folders, name, dtype):
+    from bitnet_c_amd import StepEntry
+    folder = model_folders(name, dtype)
+    eng = make_engine(folder, dtype)
+    for toks in _requests(eng.vocab_size, 11, LENGTHS):
+        s = eng.new_sequence()
+        got = eng.step([StepEntry(s, toks, list(range(len(toks))))])
+        eng.release(s)
+        assert rel_err(got, plain_logits(folder, toks, dtype)) < TOL[dtype], len(toks)
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_last_32_tokens_one_by_one(model_folders, name, dtype, graphs):
+    from bitnet_c_amd import StepEntry
+    folder = model_folders(name, dtype)
+    eng = make_engine(folder, dtype, use_graphs=graphs)
+    for toks in _requests(eng.vocab_size, 12, [33, 70, 129, 160]):
+        ref = plain_logits(folder, toks, dtype)
+        s = eng.new_sequence()
+        n0 = len(toks) - 32
+        got = [eng.step([StepEntry(s, toks[:n0], list(range(n0)))])]
+        for t in toks[n0:]:
+            got.append(eng.step([StepEntry(s, [t], [0])]))
+        eng.release(s)
+        got = torch.cat(got)
+        assert rel_err(got, ref) < TOL[dtype], len(toks)
+        # the first wrong token, if any, names the place
+        per_row = (got.cpu().double() - ref.double()).abs().max(dim=1).values / ref.double().pow(2).mean().sqrt()
+        assert int((per_row > TOL[dtype]).sum()) == 0, per_row.argmax()
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_unequal_batches_with_slot_reuse(model_folders, name, dtype, graphs):
+    """Three batches one after another in a cache that holds just one of them.  In a batch the
+    prompts (unequal) run in one step, then every request goes on one token a step until its own
+    end; ended requests give their slots back while the others go on."""
+    from bitnet_c_amd import StepEntry
+    folder = model_folders(name, dtype)
+    eng = make_engine(folder, dtype, max_tokens=64 * 9, use_graphs=graphs)
+    rnd = random.Random(13)
+    batches = [[(5, 3), (70, 40), (17, 20), (1, 9)], [(64, 1), (3, 66), (128, 5)], [(30, 30), (2, 2), (63, 2), (65, 10), (9, 31)]]
+    for bi, batch in enumerate(batches):
+        reqs = [[rnd.randrange(eng.vocab_size) for _ in range(p + d)] for p, d in batch]
+        slots = [eng.new_sequence() for _ in batch]
+        got = [[] for _ in batch]
+        out = eng.step([StepEntry(slots[i], reqs[i][:p], list(range(p))) for i, (p, d) in enumerate(batch)])
+        o = 0
+        for i, (p, d) in enumerate(batch):
+            got[i].append(out[o:o + p])
+            o += p
+        fed = [p for p, d in batch]
+        live = list(range(len(batch)))
+        while live:
+            out = eng.step([StepEntry(slots[i], [reqs[i][fed[i]]], [0]) for i in live])
+            for r, i in enumerate(live):
+                got[i].append(out[r:r + 1])
+                fed[i] += 1
+            for i in [i for i in live if fed[i] == len(reqs[i])]:
+                eng.release(slots[i])
+            live = [i for i in live if fed[i] < len(reqs[i])]
+        eng.cache.check()
+        assert not eng.cache.live_slots()
+        for i, toks in enumerate(reqs):
+            assert rel_err(torch.cat(got[i]), plain_logits(folder, toks, dtype)) < TOL[dtype], (bi, i)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_batch_and_cut_do_not_change_logits_beyond_rounding(model_folders, dtype):
+    """The same request alone, in a batch with partners, and cut into uneven pieces: float32 logits
+    agree to float32 rounding, far below the tolerance against the plain implementation."""
+    from bitnet_c_amd import StepEntry
+    folder = model_folders("A", dtype)
+    eng = make_engine(folder, dtype, max_tokens=2048)
+    toks, p1, p2 = _requests(eng.vocab_size, 14, [90, 31, 140])
+    s = eng.new_sequence()
+    alone = eng.step([StepEntry(s, toks, list(range(90)))])
+    eng.release(s)
+    a, b, c = eng.new_sequence(), eng.new_sequence(), eng.new_sequence()
+    out = eng.step([StepEntry(a, p1, []), StepEntry(b, toks, list(range(90))), StepEntry(c, p2, [139])])
+    batched = out[:90]
+    for x in (a, b, c):
+        eng.release(x)
+    s = eng.new_sequence()
+    pieces = [eng.step([StepEntry(s, toks[i:j], list(range(j - i)))]) for i, j in ((0, 1), (1, 64), (64, 65), (65, 90))]
+    eng.release(s)
+    tight = 2e-6 if dtype == torch.float32 else 2e-2
+    assert rel_err(batched, alone) < tight
+    assert rel_err(torch.cat(pieces), alone) < tight
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(model_folders, dtype):
+    """300 tokens decoded one by one after a short prompt, across several pages and split
+    plans, in a batch whose partner is much shorter."""
+    from bitnet_c_amd import StepEntry
+    folder = model_folders("A", dtype)
+    eng = make_engine(folder, dtype, max_tokens=1024)
+    long_req, short_req = _requests(eng.vocab_size, 15, [310, 12])
+    a, b = eng.new_sequence(), eng.new_sequence()
+    got = [eng.step([StepEntry(a, long_req[:10], list(range(10))), StepEntry(b, short_req[:2], [])])[:10]]
+    for i in range(10, 310):
+        ent = [StepEntry(a, [long_req[i]], [0])]
+        j = i - 10 + 2
+        if j < len(short_req):
+            ent.append(StepEntry(b, [short_req[j]], []))
+        elif j == len(short_req):
+            eng.release(b)
+        got.append(eng.step(ent)[:1])
+    eng.release(a)
+    assert rel_err(torch.cat(got), plain_logits(folder, long_req, dtype)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_first_tokens_of_a_sequence(model_folders, dtype):
+    """A sequence that starts with one token and grows by one: positions 0, 1, 2 are the places
+    where an off-by-one in lengths or in the first page shows."""
+    from bitnet_c_amd import StepEntry
+    folder = model_folders("B", dtype)
+    eng = make_engine(folder, dtype)
+    toks = _requests(eng.vocab_size, 16, [6])[0]
+    s = eng.new_sequence()
+    got = torch.cat([eng.step([StepEntry(s, [t], [0])]) for t in toks])
+    eng.release(s)
+    ref = plain_logits(folder, toks, dtype)
+    for i in range(6):
+        assert rel_err(got[i:i + 1], ref[i:i + 1]) < TOL[dtype], i
+
+
+def test_errors_change_nothing(model_folders):
+    from bitnet_c_amd import StepEntry
+    from bitnet_c_amd.engine import StepError
+    folder = model_folders("A", torch.float32)
+    eng = make_engine(folder, torch.float32, max_tokens=128)
+    s = eng.new_sequence()
+    ref = eng.step([StepEntry(s, [1, 2, 3], [2])])
+    for bad in ([StepEntry(s, [256], [0])], [StepEntry(s, [-1], [0])], [StepEntry(s, [], [])],
+                [StepEntry(s, [1], [1])], [StepEntry(s, [1] * 200, [])], [StepEntry(99, [1], [0])],
+                [StepEntry(s, [1], [0]), StepEntry(s, [2], [0])], []):
+        with pytest.raises(StepError):
+            eng.step(bad)
+        assert eng.length(s) == 3
+    eng.release(s)
+    s2 = eng.new_sequence()
+    again = eng.step([StepEntry(s2, [1, 2, 3], [2])])
+    assert torch.equal(again, ref)
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_far_key_through_the_engine(model_folders, dtype, tmp_path):
+    """Weights made so that a fault shows: in a one-layer model whose q and k projections pick out
+    one embedding dimension and whose positions are not rotated there (the lowest frequency at a
+    huge theta), token `mark` at a far position takes all the attention of a later `probe` token;
+    moving the marked token changes the logits, and they match the plain implementation."""
+    import json, os
+    from bitnet_c_amd import StepEntry
+    from bitnet_c_amd.config import LlamaConfig
+    from bitnet_c_amd.weights import write_file, random_tensors
+    from bitnet_c_amd.config import load_config
+    cfg = dict(model_type="llama", vocab_size=50, hidden_size=32, intermediate_size=48, num_hidden_layers=1,
+               num_attention_heads=2, num_key_value_heads=1, head_dim=16, max_position_embeddings=2048,
+               rope_theta=1e12, rms_norm_eps=1e-5, tie_word_embeddings=False)
+    c = LlamaConfig.from_dict(cfg)
+    folder = str(tmp_path / "far")
+    os.makedirs(folder)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(c.to_dict(), f)
+    arch, _ = load_config(folder)
+    t = random_tensors(arch.build_plan(c).expected_tensors(), 21, torch.float32)
+    mark, probe = 7, 9
+    E = t["model.embed_tokens.weight"]
+    E[:, 0] = 0
+    E[mark, 0] = 1.0
+    E[probe, 0] = 1.0
+    # dimension 7 of a head is paired with 15 and turns at theta^(-14/16): no rotation over 1000 positions
+    wq = torch.zeros_like(t["model.layers.0.self_attn.q_proj.weight"])
+    wk = torch.zeros_like(t["model.layers.0.self_attn.k_proj.weight"])
+    wq[7, 0] = wq[16 + 7, 0] = 60.0
+    wk[7, 0] = 60.0
+    t["model.layers.0.self_attn.q_proj.weight"], t["model.layers.0.self_attn.k_proj.weight"] = wq, wk
+    t["model.layers.0.self_attn.v_proj.weight"] *= 20.0
+    t["model.layers.0.self_attn.o_proj.weight"] *= 20.0
+    if dtype == torch.bfloat16:
+        t = {k: (v.to(torch.bfloat16) if v.dim() == 2 else v) for k, v in t.items()}
+    write_file(os.path.join(folder, "model.safetensors"), t)
+    eng = make_engine(folder, dtype, max_tokens=2048)
+    rnd = random.Random(22)
+    outs = {}
+    for far in (0, 63, 64, 500, 958):
+        toks = [rnd.choice([x for x in range(50) if x not in (mark, probe)]) for _ in range(960)]
+        toks[far] = mark
+        toks[959] = probe
+        s = eng.new_sequence()
+        eng.step([StepEntry(s, toks[:900], [])])
+        for tk in toks[900:959]:
+            eng.step([StepEntry(s, [tk], [])])
+        got = eng.step([StepEntry(s, [probe], [0])])
+        eng.release(s)
+        ref = plain_logits(folder, toks, dtype)[959:960]
+        assert rel_err(got, ref) < TOL[dtype], far
+        outs[far] = got
+        # and the marked key matters: without it the logits differ by far more than the tolerance
+        toks2 = list(toks)
+        toks2[far] = 3
+        assert rel_err(plain_logits(folder, toks2, dtype)[959:960], ref) > 20 * TOL[dtype], far

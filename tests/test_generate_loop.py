@@ -1,0 +1,136 @@
+"""The generation loop's decisions with a stand-in engine and sampler (no GPU), and the
+host side of the sampler."""
+import pytest
+import torch
+
+import plain_llama as pl
+from bitnet_c_amd.engine.generate import Request, generate, plan_batches
+from bitnet_c_amd.sampling import SamplingParams, SequenceSampler, XorShift64Star
+
+
+class FakeCache:
+    def __init__(self, n_pages):
+        self.n_pages = n_pages
+
+
+class FakeEngine:
+    """Logits whose argmax is (last token + 1) % vocab; records every step."""
+
+    def __init__(self, vocab=50, max_seq_len=1000, n_pages=64):
+        self.vocab, self.max_seq_len, self.cache = vocab, max_seq_len, FakeCache(n_pages)
+        self.free, self.live, self.steps, self.released = list(range(100)), {}, [], []
+
+    def new_sequence(self):
+        s = self.free.pop(0)
+        self.live[s] = 0
+        return s
+
+    def release(self, s):
+        assert s in self.live, "released twice"
+        del self.live[s]
+        self.released.append(s)
+        self.free.insert(0, s)
+
+    def step(self, entries):
+        self.steps.append([(e.slot, list(e.tokens)) for e in entries])
+        rows = []
+        for e in entries:
+            assert e.slot in self.live
+            self.live[e.slot] += len(e.tokens)
+            for w in e.want:
+                lg = torch.zeros(self.vocab)
+                lg[(e.tokens[w] + 1) % self.vocab] = 1.0
+                rows.append(lg)
+        return torch.stack(rows) if rows else torch.zeros(0, self.vocab)
+
+
+def greedy(logits, samplers):
+    return [int(t) for t in logits.argmax(dim=1)]
+
+
+def test_unequal_prompts_stop_tokens_and_early_ends():
+    eng = FakeEngine()
+    reqs = [Request([1, 2, 3], 5), Request([10], 2), Request([20, 21], 10, stop_ids=(24,)), Request([30], 0)]
+    res = generate(eng, reqs, greedy, batch_size=8)
+    assert res[0].tokens == [4, 5, 6, 7, 8] and res[0].finish == "length"
+    assert res[1].tokens == [11, 12] and res[1].finish == "length"
+    assert res[2].tokens == [22, 23] and res[2].finish == "stop"          # the stop token is not emitted
+    assert res[3].tokens == [] and res[3].finish == "length"              # -n 0: the prompt only
+    # one step for all prompts, then one token each for the live ones
+    assert [len(s) for s in eng.steps] == [4, 3, 2, 1, 1]
+    assert eng.steps[1] == [(0, [4]), (1, [11]), (2, [22])]
+    # after the budget is reached no further step runs for that sequence
+    assert sum(len(t) for st in eng.steps[1:] for _, t in st) == (5 - 1) + (2 - 1) + 2
+    assert not eng.live and sorted(eng.released) == [0, 1, 2, 3]
+
+
+def test_batches_one_after_another_reuse_slots():
+    eng = FakeEngine()
+    reqs = [Request([i], 1 + i % 3) for i in range(7)]
+    res = generate(eng, reqs, greedy, batch_size=3)
+    assert [r.tokens for r in res] == [[(i + 1 + k) % 50 for k in range(1 + i % 3)] for i in range(7)]
+    firsts = [s for s in eng.steps if len(s[0][1]) == 1 and s[0][1][0] < 7 and len(s) > 1 or s[0][1] == [6]]
+    assert [len(s) for s in eng.steps if s[0][1][0] in (0, 3, 6) and len(s[0][1]) == 1][:3] == [3, 3, 1]
+    assert max(max(sl for sl, _ in s) for s in eng.steps) <= 2             # three slots serve seven requests
+    assert not eng.live
+    del firsts
+
+
+def test_batch_planning_respects_the_cache():
+    reqs = [Request([0] * 100, 28), Request([0] * 10, 10), Request([0] * 200, 0), Request([0] * 5000, 1),
+            Request([], 3), Request([0] * 60, 600)]
+    batches, errors = plan_batches(reqs, batch_size=8, max_tokens=64 * 5, max_seq_len=1024)
+    # needs (rounded to pages): 128, 64, 256, -, -, 704 > 320
+    assert batches == [[0, 1], [2]] and set(errors) == {3, 4, 5}
+    assert "sequence limit" in errors[3] and "empty" in errors[4] and "cache holds" in errors[5]
+    b2, _ = plan_batches([Request([1], 1)] * 5, batch_size=2, max_tokens=10 ** 6, max_seq_len=100)
+    assert b2 == [[0, 1], [2, 3], [4]]
+
+
+def test_sequence_limit_and_cancel():
+    eng = FakeEngine(max_seq_len=6)
+    res = generate(eng, [Request([1, 2, 3, 4], 10)], greedy)
+    assert res[0].finish == "limit" and res[0].tokens == [5, 6, 7]         # positions 4, 5 fed; the 7th has no room
+    eng = FakeEngine()
+    seen = []
+    res = generate(eng, [Request([1], 10), Request([5], 3)], greedy, on_token=lambda i, t: seen.append((i, t)) or i == 0)
+    assert res[0].tokens == [2] and res[0].finish == "cancelled"           # the callback stops after one token
+    assert res[1].tokens == [6, 7, 8]
+    assert (0, 2) in seen and not eng.live
+
+
+def test_an_error_in_a_step_gives_the_slots_back():
+    class Broken(FakeEngine):
+        def step(self, entries):
+            if len(self.steps) == 2:
+                raise RuntimeError("boom")
+            return super().step(entries)
+    eng = Broken()
+    with pytest.raises(RuntimeError):
+        generate(eng, [Request([1], 5), Request([2], 5)], greedy)
+    assert not eng.live
+
+
+def test_host_rng_and_recent_ring_follow_the_plain_sampler():
+    a, b = XorShift64Star(0), pl.XorShift64Star(42)
+    assert [a.next_float() for _ in range(50)] == [b.next_float() for _ in range(50)]
+    s = SequenceSampler(SamplingParams(repeat_penalty=1.1, repeat_window=4), prompt=[1, 2, 3, 4, 5])
+    s.accept(6)
+    assert s.recent == [3, 4, 5, 6]
+    off = SequenceSampler(SamplingParams(), prompt=[1, 2, 3])
+    off.accept(9)
+    assert off.recent == []
+    with pytest.raises(ValueError):
+        SamplingParams(temperature=-1.0)
+
+
+def test_same_seed_same_stream_whatever_the_batch():
+    # every sequence owns its generator: the k-th draw of a sequence is the same alone or among others
+    def draws(n_partners):
+        ss = [SequenceSampler(SamplingParams(temperature=0.8, seed=42 + i)) for i in range(1 + n_partners)]
+        out = []
+        for _ in range(5):
+            vals = [s.rng.next_float() for s in ss]
+            out.append(vals[0])
+        return out
+    assert draws(0) == draws(3)

@@ -1,0 +1,388 @@
+"""Each HIP kernel alone against the plain implementation (or the formula written out in
+float64), at other sizes than the engine tests use."""
+import math
+import random
+
+import pytest
+import torch
+
+import plain_llama as pl
+from conftest import rel_err
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+KTOL = {torch.float32: 2e-5}      # float32 kernels differ from the formula by summation order only
+
+
+def close(got, ref, dtype) -> bool:
+    """A kernel computes in float32 and rounds its result once to `dtype`.  float32: the largest
+    difference is below 2e-5 of the reference's rms.  bfloat16: every element is within one
+    rounding (2^-8 of its own size) of the reference, plus the float32 slack."""
+    got, ref = got.detach().double().cpu(), ref.detach().double().cpu()
+    assert got.shape == ref.shape, (got.shape, ref.shape)
+    rms = float(ref.pow(2).mean().sqrt()) if ref.numel() else 0.0
+    slack = 2e-5 * max(rms, 1e-30)
+    if dtype == torch.float32:
+        return bool(((got - ref).abs() <= slack).all())
+    return bool(((got - ref).abs() <= ref.abs() * 2.0 ** -8 + slack).all())
+
+
+def _ops():
+    from bitnet_c_amd import ops
+    return ops
+
+
+def _rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dim,vocab", [(40, 19), (4096, 33), (1003, 7)])
+def test_embed_gather(dtype, dim, vocab):
+    ops = _ops()
+    table = _rand((vocab, dim), dtype, 1)
+    toks = torch.tensor([0, vocab - 1, 3, 3, 1], dtype=torch.int32)
+    x = ops.embed_gather(table.cuda(), toks.cuda())
+    assert x.dtype == torch.float32
+    assert torch.equal(x.cpu(), table[toks.long()].float())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dim", [24, 100, 4096, 5123])
+def test_add_rmsnorm(dtype, dim):
+    ops = _ops()
+    T, eps = 5, 1e-3
+    x = _rand((T, dim), torch.float32, 2, 3.0)
+    d = _rand((T, dim), dtype, 3)
+    w = _rand((dim,), torch.float32, 4) + 1.0
+    # without delta
+    xg = x.cuda()
+    h = ops.add_rmsnorm(xg, None, w.cuda(), eps, dtype)
+    assert torch.equal(xg.cpu(), x)
+    assert close(h.float(), pl.rmsnorm(x, w, eps), dtype)
+    # with delta: x is updated in place in float32, the norm is of the sum
+    xg = x.clone().cuda()
+    h = ops.add_rmsnorm(xg, d.cuda(), w.cuda(), eps, dtype)
+    s = x + d.float()
+    assert torch.equal(xg.cpu(), s)
+    assert close(h.float(), pl.rmsnorm(s, w, eps), dtype)
+    # selected rows: x stays, the selected rows are normed with the delta added
+    rows = torch.tensor([4, 0, 0], dtype=torch.int32)
+    xg = x.clone().cuda()
+    h = ops.add_rmsnorm(xg, d.cuda(), w.cuda(), eps, dtype, rows=rows.cuda())
+    assert torch.equal(xg.cpu(), x)
+    assert close(h.float(), pl.rmsnorm(s[rows.long()], w, eps), dtype)
+
+
+def test_rmsnorm_eps_inside_root_on_device():
+    ops = _ops()
+    x = torch.full((1, 8), 1e-4)
+    h = ops.add_rmsnorm(x.cuda(), None, torch.ones(8).cuda(), 1e-2, torch.float32)
+    assert torch.allclose(h.cpu(), x / math.sqrt(1e-8 + 1e-2), rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu_bias_residual(dtype):
+    ops = _ops()
+    T, F = 7, 173
+    gu = _rand((T, 2 * F), dtype, 5, 2.0)
+    out = ops.swiglu(gu.cuda())
+    want = pl.swiglu(gu[:, :F].float(), gu[:, F:].float())
+    assert close(out.float(), want, dtype)
+    # the reference's own vector (test/test_transformer.c:645-677)
+    g = torch.tensor([-2.0, -1.0, -0.25, 0.0, 0.25, 1.0, 2.0, 4.0])
+    u = torch.tensor([1.0, 0.5, 2.0, 3.0, -1.0, 1.5, -0.5, 2.0])
+    o = ops.swiglu(torch.cat([g, u]).view(1, 16).cuda())
+    assert torch.allclose(o.cpu()[0], (g / (1 + torch.exp(-g))) * u, atol=1e-6)
+    y = _rand((T, 50), dtype, 6)
+    b = _rand((50,), torch.float32, 7)
+    yg = y.clone().cuda()
+    ops.bias_add(yg, b.cuda())
+    assert close(yg.float(), y.float() + b, dtype)
+    x = _rand((T, 50), torch.float32, 8)
+    xg = x.clone().cuda()
+    ops.residual_add(xg, y.cuda())
+    assert torch.equal(xg.cpu(), x + y.float())
+
+
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (3, 70, 172), (17, 130, 65), (70, 33, 300), (130, 257, 64)])
+def test_gemm_tiled_float32(M, N, K):
+    ops = _ops()
+    x, w = _rand((M, K), torch.float32, 9), _rand((N, K), torch.float32, 10)
+    y = ops.linear(x.cuda(), w.cuda())
+    assert rel_err(y, (x.double() @ w.double().t()).float()) < 2e-6
+    # a row's result does not depend on its batch: bit-equal alone and among others
+    y1 = ops.linear(x[:1].contiguous().cuda(), w.cuda())
+    assert torch.equal(y1.cpu()[0], y.cpu()[0])
+
+
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(16, 8), (100, 64), (48, 1000), (4104, 4096), (31, 264)])
+def test_skinny_gemm_bf16(M, N, K):
+    ops = _ops()
+    x, w = _rand((M, K), torch.bfloat16, 11), _rand((N, K), torch.bfloat16, 12, 0.05)
+    ref = x.double() @ w.double().t()
+    y32 = ops.linear(x.cuda(), w.cuda(), torch.float32)
+    assert rel_err(y32, ref.float()) < 1e-5                       # bf16 products are exact in float32
+    y16 = ops.linear(x.cuda(), w.cuda())
+    assert y16.dtype == torch.bfloat16 and close(y16.float(), ref.float(), torch.bfloat16)
+
+
+@pytest.mark.parametrize("M,F,K", [(1, 24, 64), (8, 172, 64), (20, 100, 264), (64, 1000, 512), (40, 14336, 256)])
+def test_skinny_gemm_dual_swiglu(M, F, K):
+    ops = _ops()
+    x, w = _rand((M, K), torch.bfloat16, 13), _rand((2 * F, K), torch.bfloat16, 14, 0.1)
+    y = ops.linear_swiglu(x.cuda(), w.cuda())
+    g = x.double() @ w[:F].double().t()
+    u = x.double() @ w[F:].double().t()
+    assert close(y.float(), ((g / (1 + torch.exp(-g))) * u).float(), torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_linear_odd_shapes_and_many_rows(dtype):
+    ops = _ops()
+    for M, N, K in [(3, 50, 172), (100, 70, 172), (200, 96, 64), (130, 40, 100)]:
+        x, w = _rand((M, K), dtype, 15), _rand((N, K), dtype, 16, 0.05)
+        y = ops.linear(x.cuda(), w.cuda())
+        assert close(y.float(), (x.double() @ w.double().t()).float(), dtype), (M, N, K)
+        y32 = ops.linear(x.cuda(), w.cuda(), torch.float32)
+        assert y32.dtype == torch.float32
+        assert rel_err(y32, (x.double() @ w.double().t()).float()) < 1e-5, (M, N, K)
+        # float32 logits of a bf16 model at many rows agree with the same rows taken alone
+        if dtype == torch.bfloat16 and K % 8 == 0:
+            y1 = ops.linear(x[:1].contiguous().cuda(), w.cuda(), torch.float32)
+            assert rel_err(y1, y32[:1]) < 1e-6
+
+
+# ---------------------------------------------------------------------------------------
+def _paged(seqs_k, seqs_v, dtype, n_pages, seed):
+    """Random distinct pages for every sequence; returns k_pages, v_pages, block_table."""
+    Hkv, hs = seqs_k[0].shape[1], seqs_k[0].shape[2]
+    rnd = random.Random(seed)
+    free = list(range(n_pages))
+    rnd.shuffle(free)
+    # unused pages hold NaN: a kernel that reads a key it must not see shows it
+    k_pages = torch.full((n_pages, Hkv, 64, hs), float("nan"), dtype=dtype)
+    v_pages = torch.full((n_pages, Hkv, 64, hs), float("nan"), dtype=dtype)
+    width = max((k.shape[0] + 63) // 64 for k in seqs_k)
+    bt = torch.zeros((len(seqs_k), width), dtype=torch.int32)
+    for s, (k, v) in enumerate(zip(seqs_k, seqs_v)):
+        for i in range((k.shape[0] + 63) // 64):
+            p = free.pop()
+            bt[s, i] = p
+            n = min(64, k.shape[0] - 64 * i)
+            k_pages[p, :, :n] = k[64 * i:64 * i + n].transpose(0, 1).to(dtype)
+            v_pages[p, :, :n] = v[64 * i:64 * i + n].transpose(0, 1).to(dtype)
+    return k_pages, v_pages, bt
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,hs,rope_dims", [(4, 2, 16, 16), (6, 3, 40, 24), (5, 5, 24, 24), (8, 1, 128, 128),
+                                                 (2, 2, 256, 64)])
+def test_rope_kv_write(dtype, H, Hkv, hs, rope_dims):
+    ops = _ops()
+    lens_before, n_new = [0, 70, 130], [5, 1, 66]
+    T = sum(n_new)
+    qkv = _rand((T, (H + 2 * Hkv) * hs), dtype, 17)
+    inv_freq = pl.rope_inv_freq(hs, 10000.0, None, rope_dims)
+    positions, seq_index = [], []
+    for s, (p0, n) in enumerate(zip(lens_before, n_new)):
+        positions += list(range(p0, p0 + n))
+        seq_index += [s] * n
+    pos = torch.tensor(positions, dtype=torch.int32)
+    n_pages = 12
+    bt = torch.tensor([[3, 0, 0, 0], [7, 1, 0, 0], [2, 9, 5, 11]], dtype=torch.int32)
+    kp = torch.zeros((n_pages, Hkv, 64, hs), dtype=dtype).cuda()
+    vp = torch.zeros_like(kp)
+    q_in = qkv.clone()
+    g = qkv.cuda()
+    ops.rope_kv_write(g, pos.cuda(), H, Hkv, hs, inv_freq=inv_freq.cuda(), rope_dims=rope_dims,
+                      seq_index=torch.tensor(seq_index, dtype=torch.int32).cuda(), block_table=bt.cuda(),
+                      k_pages=kp, v_pages=vp)
+    q_ref = pl.apply_rope(q_in[:, :H * hs].float().view(T, H, hs), pos, inv_freq)
+    k_ref = pl.apply_rope(q_in[:, H * hs:(H + Hkv) * hs].float().view(T, Hkv, hs), pos, inv_freq)
+    v_ref = q_in[:, (H + Hkv) * hs:].float().view(T, Hkv, hs)
+    assert close(g[:, :H * hs].float().view(T, H, hs), q_ref, dtype)
+    assert torch.equal(g[:, H * hs:].cpu(), q_in[:, H * hs:])            # K, V of the input stay as they are
+    kp, vp = kp.cpu().float(), vp.cpu().float()
+    written = torch.zeros((n_pages, 64), dtype=torch.bool)
+    for t in range(T):
+        page, off = int(bt[seq_index[t], positions[t] // 64]), positions[t] % 64
+        written[page, off] = True
+        assert close(kp[page, :, off], k_ref[t], dtype), t
+        assert torch.equal(vp[page, :, off], v_ref[t].to(dtype).float())
+    assert float(kp.transpose(1, 2)[~written].abs().sum()) == 0.0
+    assert float(vp.transpose(1, 2)[~written].abs().sum()) == 0.0
+    # position -1 is a padding row: nothing is rotated or written; Q-only form leaves the cache alone
+    g2 = q_in.clone().cuda()
+    kp2 = torch.zeros((n_pages, Hkv, 64, hs), dtype=dtype).cuda()
+    ops.rope_kv_write(g2, torch.full((T,), -1, dtype=torch.int32).cuda(), H, Hkv, hs, inv_freq=inv_freq.cuda(),
+                      rope_dims=rope_dims, seq_index=torch.zeros(T, dtype=torch.int32).cuda(), block_table=bt.cuda(),
+                      k_pages=kp2, v_pages=kp2.clone())
+    assert torch.equal(g2.cpu(), q_in) and float(kp2.abs().sum()) == 0.0
+    g3 = q_in.clone().cuda()
+    ops.rope_kv_write(g3, pos.cuda(), H, Hkv, hs, inv_freq=inv_freq.cuda(), rope_dims=rope_dims)
+    assert torch.equal(g3.cpu(), g.cpu())
+
+
+def test_rope_reference_vector_on_device():
+    # test/test_transformer.c:636-643 through the kernel: angles pi/2 and 0
+    ops = _ops()
+    H, hs = 2, 8                                        # rope_dims 4 of head size 8: the rest passes through
+    qkv = torch.tensor([1.0, 2, 3, 4, 9, 9, 9, 9, -1, -2, -3, -4, 7, 7, 7, 7]).view(1, 16)
+    g = qkv.clone().cuda()
+    ops.rope_kv_write(g, torch.tensor([1], dtype=torch.int32).cuda(), H, 0, hs,
+                      inv_freq=torch.tensor([math.pi / 2, 0.0]).cuda(), rope_dims=4)
+    want = torch.tensor([-3.0, 2, 1, 4, 9, 9, 9, 9, 3, -2, -1, -4, 7, 7, 7, 7])
+    assert torch.allclose(g.cpu()[0], want, atol=1e-6)
+
+
+def _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, seed):
+    """Random sequences; returns the kernel's output and the plain implementation's, rows in
+    batch order."""
+    ops = _ops()
+    seqs_q, seqs_k, seqs_v = [], [], []
+    for s, (p0, n) in enumerate(zip(lens_before, n_new)):
+        L = p0 + n
+        seqs_q.append(_rand((L, H, hs), dtype, seed + 3 * s))
+        seqs_k.append(_rand((L, Hkv, hs), dtype, seed + 3 * s + 1))
+        seqs_v.append(_rand((L, Hkv, hs), dtype, seed + 3 * s + 2))
+    n_pages = sum((p0 + n + 63) // 64 for p0, n in zip(lens_before, n_new)) + 3
+    kp, vp, bt = _paged(seqs_k, seqs_v, dtype, n_pages, seed)
+    scale = 1.0 / math.sqrt(hs)
+    qrows, ref = [], []
+    for s, (p0, n) in enumerate(zip(lens_before, n_new)):
+        full = pl.attention(seqs_q[s].float(), seqs_k[s].float(), seqs_v[s].float(), scale, window or None)
+        ref.append(full[p0:].reshape(n, H * hs))
+        qrows.append(seqs_q[s][p0:].reshape(n, H * hs))
+    q = torch.cat(qrows).contiguous()
+    # the kernel takes the Q heads out of a qkv buffer: give it a wider row to test the stride
+    qkv = torch.cat([q, torch.full((q.shape[0], 2 * Hkv * hs), float("nan"), dtype=dtype)], dim=1).contiguous()
+    return ops, qkv.cuda(), kp.cuda(), vp.cuda(), bt.cuda(), torch.cat(ref), scale
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,hs,window", [(4, 2, 16, 0), (5, 5, 24, 0), (6, 2, 32, 0), (8, 2, 128, 0), (32, 1, 64, 0),
+                                             (2, 1, 256, 0), (4, 2, 16, 7), (4, 4, 64, 100), (20, 1, 40, 0)])
+def test_attention_prompt_form(dtype, H, Hkv, hs, window):
+    lens_before, n_new = [0, 0, 64, 130, 5], [1, 37, 64, 3, 70]
+    ops, qkv, kp, vp, bt, ref, scale = _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, 100)
+    _, _, qt = ops.attention_row_shape(H, Hkv, False)
+    tiles, r = [], 0
+    for s, (p0, n) in enumerate(zip(lens_before, n_new)):
+        for i in range(0, n, qt):
+            tiles.append((s, r + i, min(qt, n - i), p0 + i))
+        r += n
+    out = torch.full((qkv.shape[0], H * hs), float("nan"), dtype=dtype).cuda()
+    ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, scale, window=window,
+                  tiles=torch.tensor(tiles, dtype=torch.int32).cuda(), qt=qt)
+    assert close(out.float(), ref, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,hs,window", [(4, 2, 16, 0), (5, 5, 24, 0), (8, 2, 128, 0), (12, 4, 64, 0),
+                                             (16, 1, 32, 0), (4, 2, 16, 50), (8, 8, 64, 129)])
+@pytest.mark.parametrize("force_splits", [1, 0, 5])
+def test_attention_decode_form(dtype, H, Hkv, hs, window, force_splits):
+    lens_before, n_new = [0, 63, 64, 700, 129, 300], [1] * 6
+    ops, qkv, kp, vp, bt, ref, scale = _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, 200)
+    B = len(n_new)
+    # two padding rows at the end: length 0, their output is zero and nothing else changes
+    qkv = torch.cat([qkv, torch.zeros((2, qkv.shape[1]), dtype=dtype).cuda()])
+    bt = torch.cat([bt, torch.zeros((2, bt.shape[1]), dtype=torch.int32).cuda()])
+    lens = torch.tensor([p + 1 for p in lens_before] + [0, 0], dtype=torch.int32).cuda()
+    max_len = bt.shape[1] * 64
+    if force_splits == 0:
+        n_splits, chunk = ops.decode_splits(B + 2, H, Hkv, max_len)
+    elif force_splits == 1:
+        n_splits, chunk = 1, 0
+    else:
+        chunk = ((max_len + force_splits - 1) // force_splits + 63) // 64 * 64
+        n_splits = (max_len + chunk - 1) // chunk
+    if window:
+        n_splits, chunk = 1, 0
+    out = torch.full((B + 2, H * hs), float("nan"), dtype=dtype).cuda()
+    ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, scale, window=window, seq_lens=lens,
+                  n_splits=n_splits, chunk=chunk)
+    assert close(out[:B].float(), ref, dtype)
+    assert float(out[B:].float().abs().sum()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_a_far_key(dtype):
+    """One key among 900 has a large score with the query: the output must be its value row,
+    wherever it lies (first page, a page's edge, the last position)."""
+    ops = _ops()
+    H, Hkv, hs, L = 4, 2, 32, 900
+    for far in (0, 63, 64, 449, 898, 899):
+        k = _rand((L, Hkv, hs), dtype, 300, 0.1)
+        v = _rand((L, Hkv, hs), dtype, 301)
+        q = _rand((1, H, hs), dtype, 302, 0.1)
+        k[far] = 0
+        k[far, :, 0] = 16.0
+        q[0, :, 0] = 16.0                                   # score 256 * scale at `far`, about 0 elsewhere
+        kp, vp, bt = _paged([k], [v], dtype, 20, far)
+        qkv = q.reshape(1, H * hs).contiguous().cuda()
+        for n_splits, chunk in ((1, 0), (4, 256), (15, 64)):
+            out = torch.empty((1, H * hs), dtype=dtype).cuda()
+            ops.attention(qkv, out, kp.cuda(), vp.cuda(), bt.cuda(), H, Hkv, hs, 1 / math.sqrt(hs),
+                          seq_lens=torch.tensor([L], dtype=torch.int32).cuda(), n_splits=n_splits, chunk=chunk)
+            want = v[far].float().repeat_interleave(H // Hkv, dim=0).reshape(1, H * hs)
+            assert rel_err(out.float(), want) < 1e-3, (far, n_splits)
+
+
+# ---------------------------------------------------------------------------------------
+def test_argmax_ties_and_odd_vocab():
+    ops = _ops()
+    x = _rand((5, 1009), torch.float32, 400)
+    x[1, 17] = x[1, 900] = 50.0                    # a tie: the lower index wins
+    x[2, 1008] = 60.0
+    x[3, 0] = 70.0
+    got = ops.argmax(x.cuda()).cpu().tolist()
+    assert got == torch.argmax(x, dim=1).tolist() and got[1] == 17 and got[2] == 1008 and got[3] == 0
+    assert ops.argmax(torch.tensor([[1.0, 3.0, 2.0, 0.5]]).cuda()).item() == 1        # test/test_safety.c:208-211
+
+
+@pytest.mark.parametrize("vocab", [4, 389, 128256])
+@pytest.mark.parametrize("temperature,top_p", [(0.8, 1.0), (1.0, 0.0), (0.7, 0.9), (1.3, 0.5)])
+def test_sample_matches_the_plain_sampler(vocab, temperature, top_p):
+    ops = _ops()
+    B = 6
+    logits = _rand((B, vocab), torch.float32, 500, 3.0)
+    rng = pl.XorShift64Star(99)
+    rs = [rng.next_float() for _ in range(B)]
+    got = ops.sample(logits.cuda(), temperature, top_p, torch.tensor(rs, dtype=torch.float32).cuda()).cpu().tolist()
+
+    class Fixed:
+        def __init__(self, r): self.r = r
+        def next_float(self): return self.r
+    want = [pl.sample(logits[i], temperature, top_p, Fixed(rs[i])) for i in range(B)]
+    # the two may differ when r falls within rounding of a boundary of the cdf; with 6 draws from a
+    # continuous r that has probability ~1e-6, so equality is demanded
+    assert got == want
+
+
+def test_sample_reference_cases_on_device():
+    ops = _ops()
+    # top-p 0.5 with a dominant logit: always token 0 (test/test_safety.c:256-272)
+    lg = torch.tensor([[10.0, 0.0, 0.0, 0.0]] * 64).cuda()
+    rng = pl.XorShift64Star(42)
+    r = torch.tensor([rng.next_float() for _ in range(64)], dtype=torch.float32).cuda()
+    assert sum(t == 0 for t in ops.sample(lg, 1.0, 0.5, r).cpu().tolist()) > 51
+    assert ops.sample(torch.tensor([[5.0]]).cuda(), 0.5, 0.9, torch.tensor([0.3]).cuda()).item() == 0   # vocab 1
+    # temperature 0 ignores the uniforms
+    assert ops.sample(torch.tensor([[1.0, 3.0, 2.0, 0.5]]).cuda(), 0.0, 0.9).item() == 1
+
+
+def test_repeat_penalty_on_device():
+    ops = _ops()
+    lg = torch.tensor([[2.0, 2.1, 2.0, 2.0], [1.0, -1.0, 0.5, 3.0]]).cuda()
+    recent = torch.tensor([[1, 1, 1, -1], [1, 3, 3, 1]], dtype=torch.int32).cuda()
+    ops.repeat_penalty_(lg, recent, 1.5)
+    want = torch.tensor([[2.0, 2.1 / 1.5, 2.0, 2.0], [1.0, -1.5, 0.5, 2.0]])
+    assert torch.allclose(lg.cpu(), want, atol=1e-6)
+    assert ops.argmax(lg).cpu().tolist()[0] != 1           # test/test_safety.c:229-238
