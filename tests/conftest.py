@@ -76,3 +76,15 @@ def rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
 # summation order only; bfloat16 by the rounding of activations to 8 bits of mantissa at
 # every part's boundary (the plain implementation rounds at the same places).
 TOL = {torch.float32: 1e-4, torch.bfloat16: 3e-2}
+
+
+def part_close(got: torch.Tensor, want: torch.Tensor, dtype) -> bool:
+    """For a part whose output is stored in `dtype`.  float32: as for logits.  bfloat16: the two
+    sides round their results on their own, so an element may differ by one unit in the last place
+    (2^-7 of its size), plus what the rounding of the part's inner tensors brings (1e-2 of the rms)."""
+    if dtype == torch.float32:
+        return rel_err(got, want) < TOL[dtype]
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    assert got.shape == want.shape, (got.shape, want.shape)
+    rms = float(want.pow(2).mean().sqrt())
+    return bool(((got - want).abs() <= want.abs() * 2.0 ** -7 + 1e-2 * rms).all())

@@ -198,9 +198,10 @@ def test_errors_change_nothing(model_folders):
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_far_key_through_the_engine(model_folders, dtype, tmp_path):
     """Weights made so that a fault shows: in a one-layer model whose q and k projections pick out
-    one embedding dimension and whose positions are not rotated there (the lowest frequency at a
-    huge theta), token `mark` at a far position takes all the attention of a later `probe` token;
-    moving the marked token changes the logits, and they match the plain implementation."""
+    one embedding dimension each and whose positions are not rotated there (the lowest frequency at
+    a huge theta), token `mark` at a far position takes all the attention of the last token `probe`;
+    without the marked token the logits differ by several times their size, and with it they match
+    the plain implementation wherever it lies (first position, a page's edge, the decoded part)."""
     import json, os
     from bitnet_c_amd import StepEntry
     from bitnet_c_amd.config import LlamaConfig
@@ -219,12 +220,13 @@ def test_far_key_through_the_engine(model_folders, dtype, tmp_path):
     mark, probe = 7, 9
     E = t["model.embed_tokens.weight"]
     E[:, 0] = 0
-    E[mark, 0] = 1.0
-    E[probe, 0] = 1.0
+    E[:, 1] = 0
+    E[mark, 0] = 1.0            # the key of `mark` comes from embedding dimension 0,
+    E[probe, 1] = 1.0           # the query of `probe` from dimension 1: the probe does not see itself
     # dimension 7 of a head is paired with 15 and turns at theta^(-14/16): no rotation over 1000 positions
     wq = torch.zeros_like(t["model.layers.0.self_attn.q_proj.weight"])
     wk = torch.zeros_like(t["model.layers.0.self_attn.k_proj.weight"])
-    wq[7, 0] = wq[16 + 7, 0] = 60.0
+    wq[7, 1] = wq[16 + 7, 1] = 60.0
     wk[7, 0] = 60.0
     t["model.layers.0.self_attn.q_proj.weight"], t["model.layers.0.self_attn.k_proj.weight"] = wq, wk
     t["model.layers.0.self_attn.v_proj.weight"] *= 20.0

@@ -65,15 +65,17 @@ def test_unequal_prompts_stop_tokens_and_early_ends():
 
 
 def test_batches_one_after_another_reuse_slots():
-    eng = FakeEngine()
-    reqs = [Request([i], 1 + i % 3) for i in range(7)]
+    eng = FakeEngine(vocab=1000)
+    reqs = [Request([100 + 10 * i], 1 + i % 3) for i in range(7)]     # prompts are multiples of 10, new tokens never
     res = generate(eng, reqs, greedy, batch_size=3)
-    assert [r.tokens for r in res] == [[(i + 1 + k) % 50 for k in range(1 + i % 3)] for i in range(7)]
-    firsts = [s for s in eng.steps if len(s[0][1]) == 1 and s[0][1][0] < 7 and len(s) > 1 or s[0][1] == [6]]
-    assert [len(s) for s in eng.steps if s[0][1][0] in (0, 3, 6) and len(s[0][1]) == 1][:3] == [3, 3, 1]
+    assert [r.tokens for r in res] == [[101 + 10 * i + k for k in range(1 + i % 3)] for i in range(7)]
+    prompts = [[t[0] for _, t in s] for s in eng.steps if s[0][1][0] % 10 == 0]
+    assert prompts == [[100, 110, 120], [130, 140, 150], [160]]           # as many batches as the requests need
+    # a batch starts only when the one before it has ended
+    starts = [k for k, s in enumerate(eng.steps) if s[0][1][0] % 10 == 0]
+    assert starts == [0, 3, 6]
     assert max(max(sl for sl, _ in s) for s in eng.steps) <= 2             # three slots serve seven requests
     assert not eng.live
-    del firsts
 
 
 def test_batch_planning_respects_the_cache():

@@ -1,0 +1,324 @@
+"""Each part alone against the plain implementation; the order of layers as data (a layer named
+twice, a layer that reads another layer's cache); and a toy mixer with a state of its own,
+defined here, registered, built and stepped without a change to the library's files."""
+import json
+import math
+import os
+import random
+from dataclasses import asdict, dataclass
+
+import pytest
+import torch
+
+import plain_llama as pl
+from conftest import TOL, part_close, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _rand(shape, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * scale
+
+
+def _ctx(cache, slots, n_new, dtype, tokens=None):
+    """A StepContext and block tables for hand-driven parts, the way the engine makes them."""
+    from bitnet_c_amd.engine.step import StepContext
+    pos0 = [cache.length(s) for s in slots]
+    cache.reserve(slots, n_new)
+    positions, seq_index = [], []
+    for i, (p, n) in enumerate(zip(pos0, n_new)):
+        positions += list(range(p, p + n))
+        seq_index += [i] * n
+    T = sum(n_new)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    ctx = StepContext(torch.device(DEV), dtype, i32(tokens or [0] * T), i32(positions), i32(seq_index),
+                      i32([p + n for p, n in zip(pos0, n_new)]), i32(list(range(T))), i32(slots),
+                      all(n == 1 for n in n_new), slots, n_new, pos0)
+    tables = {g: cache.block_table(g, slots).to(DEV) for g in range(len(cache.groups))}
+    return ctx, tables, max(p + n for p, n in zip(pos0, n_new))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_and_feed_forward_parts(dtype):
+    from bitnet_c_amd.parts import FEED_FORWARDS, NORMS, PartSpec
+    norm = NORMS.build(PartSpec.of("rmsnorm", dim=72, eps=1e-4))
+    w = _rand((72,), 1) + 1.0
+    norm.load({"weight": w}, DEV, dtype)
+    x = _rand((9, 72), 2, 2.0)
+    assert part_close(norm.apply(x.to(DEV), None, dtype).float(), pl.rmsnorm(x, w, 1e-4), dtype)
+    ffn = FEED_FORWARDS.build(PartSpec.of("swiglu", hidden=72, intermediate=100))
+    assert {k: v.shape for k, v in ffn.tensors().items()} == {"w_gate": (100, 72), "w_up": (100, 72), "w_down": (72, 100)}
+    t = {"w_gate": _rand((100, 72), 3, 0.1).to(dtype), "w_up": _rand((100, 72), 4, 0.1).to(dtype),
+         "w_down": _rand((72, 100), 5, 0.1).to(dtype)}
+    ffn.load(t, DEV, dtype)
+    rt = None if dtype == torch.float32 else dtype
+    for T in (1, 9, 70):                                        # decode-sized and prompt-sized products
+        h = _rand((T, 72), 6).to(dtype)
+        got = ffn.forward(h.to(DEV), None)
+        want = pl.feed_forward(h.float(), t["w_gate"].float(), t["w_up"].float(), t["w_down"].float(), rt)
+        assert part_close(got.float(), want, dtype), T
+    # a feed-forward with biases
+    fb = FEED_FORWARDS.build(PartSpec.of("swiglu", hidden=72, intermediate=100, bias=True))
+    tb = dict(t, b_gate=_rand((100,), 7, 0.1), b_up=_rand((100,), 8, 0.1), b_down=_rand((72,), 9, 0.1))
+    fb.load(tb, DEV, dtype)
+    h = _rand((5, 72), 10).to(dtype)
+    g = pl.linear(h.float(), t["w_gate"]) + tb["b_gate"]
+    u = pl.linear(h.float(), t["w_up"]) + tb["b_up"]
+    want = pl.linear(pl.swiglu(g, u), t["w_down"]) + tb["b_down"]
+    assert part_close(fb.forward(h.to(DEV), None).float(), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,Hkv,hs,window,pos_kind", [(6, 2, 32, 0, "rope"), (4, 4, 16, 40, "rope"), (3, 1, 24, 0, "none")])
+def test_attention_part_alone(dtype, H, Hkv, hs, window, pos_kind):
+    """The mixer with its own cache entry: prompts of unequal lengths, then tokens one by one,
+    against plain attention over the whole sequences."""
+    from bitnet_c_amd.cache import PagedCache
+    from bitnet_c_amd.parts import MIXERS, PartSpec
+    hidden, scale = 48, 0.2
+    pos = PartSpec.of("rope", head_dim=hs, theta=5000.0, rope_dims=hs // 2) if pos_kind == "rope" else PartSpec.of("none")
+    att = MIXERS.build(PartSpec.of("attention", hidden=hidden, n_heads=H, n_kv_heads=Hkv, head_dim=hs, scale=scale,
+                                   position=pos, window=window))
+    t = {k: _rand(v.shape, 20 + i, 0.15).to(dtype) for i, (k, v) in enumerate(att.tensors().items())}
+    att.load(t, DEV, dtype)
+    cache = PagedCache([att.cache_need()], [None], 64 * 8, dtype=dtype, device=DEV)
+    lens = [70, 5, 130]
+    hs_in = [_rand((n, hidden), 30 + i).to(dtype) for i, n in enumerate(lens)]
+    slots = [cache.alloc_slot() for _ in lens]
+    got = [[] for _ in lens]
+    fed = [n - 3 for n in lens]
+    ctx, tables, max_len = _ctx(cache, slots, fed, dtype)
+    out = att.forward(torch.cat([h[:f] for h, f in zip(hs_in, fed)]).to(DEV), ctx, cache.view(0, tables, max_len))
+    cache.commit(slots, fed)
+    o = 0
+    for i, f in enumerate(fed):
+        got[i].append(out[o:o + f])
+        o += f
+    for step in range(3):
+        ctx, tables, max_len = _ctx(cache, slots, [1] * 3, dtype)
+        out = att.forward(torch.stack([h[f + step] for h, f in zip(hs_in, fed)]).to(DEV), ctx,
+                          cache.view(0, tables, max_len))
+        cache.commit(slots, [1] * 3)
+        for i in range(3):
+            got[i].append(out[i:i + 1])
+    rt = (lambda x: x) if dtype == torch.float32 else (lambda x: x.to(dtype).float())
+    inv = pl.rope_inv_freq(hs, 5000.0, None, hs // 2) if pos_kind == "rope" else torch.zeros(0)
+    for i, n in enumerate(lens):
+        h = hs_in[i].float()
+        p = torch.arange(n)
+        q = rt(pl.apply_rope(rt(pl.linear(h, t["wq"])).view(n, H, hs), p, inv))
+        k = rt(pl.apply_rope(rt(pl.linear(h, t["wk"])).view(n, Hkv, hs), p, inv))
+        v = rt(pl.linear(h, t["wv"])).view(n, Hkv, hs)
+        a = rt(pl.attention(q, k, v, scale, window or None).reshape(n, H * hs))
+        want = rt(pl.linear(a, t["wo"]))
+        assert part_close(torch.cat(got[i]).float(), want, dtype), i
+
+
+def _tiny_folder(tmp_path, dtype=torch.float32):
+    from bitnet_c_amd.config import LlamaConfig
+    from bitnet_c_amd.weights import write_model_folder
+    from conftest import TINY_A
+    d = str(tmp_path / "m")
+    write_model_folder(d, LlamaConfig.from_dict(dict(TINY_A, num_hidden_layers=3)), 3, dtype)
+    return d
+
+
+def test_the_order_of_layers_is_data(tmp_path):
+    """A schedule that names a layer twice (shared weights, a cache entry each) equals the plain
+    model with that layer's weights copied; an entry that reads an earlier entry's cache attends
+    over that entry's keys and values with its own queries."""
+    from bitnet_c_amd import Engine, StepEntry
+    from bitnet_c_amd.config import load_config
+    from bitnet_c_amd.engine import DecoderModel, ScheduleEntry
+    from bitnet_c_amd.weights import load_tensors
+    from dataclasses import replace
+    folder = _tiny_folder(tmp_path)
+    arch, cfg = load_config(folder)
+    plan = arch.build_plan(cfg)
+    tensors = load_tensors(folder, plan.expected_tensors())
+    c, W = pl.read_config(folder), pl.read_weights(folder)
+    toks = [random.Random(5).randrange(256) for _ in range(80)]
+
+    def run(schedule):
+        model = DecoderModel(replace(plan, schedule=schedule), torch.float32, DEV)
+        model.load(tensors)
+        eng = Engine(model, max_tokens=256)
+        s = eng.new_sequence()
+        a = eng.step([StepEntry(s, toks[:70], list(range(70)))])
+        b = [eng.step([StepEntry(s, [t], [0])]) for t in toks[70:]]
+        return torch.cat([a] + b), eng
+
+    # layers 0, 1, 1, 2
+    got, eng = run([ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(1), ScheduleEntry(2)])
+    assert eng.cache.groups[0].k.shape[0] == 4                   # four cache entries for three layers
+    W4 = {k: v for k, v in W.items() if ".layers." not in k}
+    for new, old in enumerate([0, 1, 1, 2]):
+        for k, v in W.items():
+            if f".layers.{old}." in k:
+                W4[k.replace(f".layers.{old}.", f".layers.{new}.")] = v
+    assert rel_err(got, pl.forward(dict(c, layers=4), W4, toks)) < TOL[torch.float32]
+
+    # layer 2 reads the cache of entry 0: plain version written out here
+    got, eng = run([ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2, kv_from=0)])
+    assert eng.cache.groups[0].k.shape[0] == 2                   # the third entry has no storage
+    x = W["model.embed_tokens.weight"][toks]
+    pos = torch.arange(len(toks))
+    inv = pl.rope_inv_freq(c["head_dim"], c["theta"])
+    keep = {}
+    for l in range(3):
+        p = f"model.layers.{l}."
+        xb = pl.rmsnorm(x, W[p + "input_layernorm.weight"], c["eps"])
+        q = pl.apply_rope(pl.linear(xb, W[p + "self_attn.q_proj.weight"]).view(-1, 4, 16), pos, inv)
+        if l < 2:
+            k = pl.apply_rope(pl.linear(xb, W[p + "self_attn.k_proj.weight"]).view(-1, 2, 16), pos, inv)
+            v = pl.linear(xb, W[p + "self_attn.v_proj.weight"]).view(-1, 2, 16)
+            keep[l] = (k, v)
+        else:
+            k, v = keep[0]
+        o = pl.attention(q, k, v, 0.25).reshape(len(toks), 64)
+        x = x + pl.linear(o, W[p + "self_attn.o_proj.weight"])
+        xb = pl.rmsnorm(x, W[p + "post_attention_layernorm.weight"], c["eps"])
+        x = x + pl.feed_forward(xb, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"], W[p + "mlp.down_proj.weight"])
+    want = pl.linear(pl.rmsnorm(x, W["model.norm.weight"], c["eps"]), W["lm_head.weight"])
+    assert rel_err(got, want) < TOL[torch.float32]
+
+
+# ---------------------------------------------------------------------------------------
+# a toy architecture, defined here: layers alternate between attention and a mixer that keeps
+# a running decayed sum of its inputs per sequence; nothing of it lives in the library
+# ---------------------------------------------------------------------------------------
+
+def _register_toy():
+    from bitnet_c_amd.config import Architecture, register_architecture
+    from bitnet_c_amd.config.base import _ARCHITECTURES
+    from bitnet_c_amd.engine import LayerPlan, ModelPlan, ScheduleEntry
+    from bitnet_c_amd.parts import MIXERS, CacheNeed, ParamSpec, Part, PartSpec, StateNeed
+
+    if "decay_sum" not in MIXERS:
+        @MIXERS.register("decay_sum")
+        class DecaySum(Part):
+            """s_t = decay * s_{t-1} + h_t ;  out_t = W s_t."""
+
+            def __init__(self, hidden, decay):
+                self.hidden, self.decay = hidden, decay
+
+            def tensors(self):
+                return {"w": ParamSpec((self.hidden, self.hidden))}
+
+            def load(self, tensors, device, dtype):
+                self.w = tensors["w"].to(dtype).to(device)
+
+            def cache_need(self):
+                return CacheNeed(state=StateNeed((self.hidden,), torch.float32))
+
+            def forward(self, h, ctx, kv):
+                out = torch.empty_like(h)
+                for slot, (r0, n) in zip(ctx.slots, ctx.row_ranges()):
+                    s = kv.state[slot]
+                    for t in range(r0, r0 + n):                 # strictly in order inside a sequence
+                        s = self.decay * s + h[t].float()
+                        out[t] = (self.w.float() @ s).to(h.dtype)
+                    kv.state[slot] = s
+                return out
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int
+        hidden_size: int
+        n_layers: int
+        decay: float
+        model_type: str = "toy_decay"
+
+        @staticmethod
+        def from_dict(raw):
+            return ToyConfig(raw["vocab_size"], raw["hidden_size"], raw["n_layers"], raw["decay"])
+
+        def to_dict(self):
+            return asdict(self)
+
+    def build(c):
+        norm = PartSpec.of("rmsnorm", dim=c.hidden_size, eps=1e-5)
+        ffn = PartSpec.of("swiglu", hidden=c.hidden_size, intermediate=2 * c.hidden_size)
+        att = PartSpec.of("attention", hidden=c.hidden_size, n_heads=2, n_kv_heads=1, head_dim=c.hidden_size // 2,
+                          scale=(c.hidden_size // 2) ** -0.5,
+                          position=PartSpec.of("rope", head_dim=c.hidden_size // 2, theta=100.0))
+        dec = PartSpec.of("decay_sum", hidden=c.hidden_size, decay=c.decay)
+        layers = []
+        for i in range(c.n_layers):
+            mixer = att if i % 2 == 0 else dec
+            blk = PartSpec.of("prenorm", mixer=mixer, ffn=ffn, mixer_norm=norm, ffn_norm=norm)
+            from bitnet_c_amd.parts import BLOCKS
+            names = {local: f"layers.{i}.{local}" for local in BLOCKS.build(blk).tensors()}
+            layers.append(LayerPlan(block=blk, names=names))
+        return ModelPlan(vocab_size=c.vocab_size, hidden_size=c.hidden_size, layers=layers,
+                         schedule=[ScheduleEntry(i) for i in range(c.n_layers)], final_norm=norm,
+                         embedding_name="embed.weight", final_norm_names={"weight": "norm.weight"},
+                         lm_head_name="head.weight")
+
+    if "toy_decay" not in _ARCHITECTURES:
+        register_architecture(Architecture("toy_decay", ToyConfig, build))
+    return ToyConfig
+
+
+def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
+    from bitnet_c_amd import Engine, StepEntry
+    from bitnet_c_amd.weights import write_model_folder
+    ToyConfig = _register_toy()
+    cfg = ToyConfig(vocab_size=40, hidden_size=32, n_layers=3, decay=0.9)
+    folder = write_model_folder(str(tmp_path / "toy"), cfg, 11, torch.float32)
+    assert json.load(open(os.path.join(folder, "config.json")))["model_type"] == "toy_decay"
+    eng = Engine.from_folder(folder, dtype=torch.float32, max_tokens=512)       # chosen by config.json
+    assert not eng.use_graphs and list(eng.cache.states) == [1]
+    assert eng.cache.states[1].shape[1:] == (32,) and len(eng.cache.groups) == 1
+
+    # the plain version of the toy model
+    from safetensors.torch import load_file
+    W = load_file(os.path.join(folder, "model.safetensors"))
+
+    def plain(toks):
+        x = W["embed.weight"][toks]
+        n = len(toks)
+        pos = torch.arange(n)
+        for l in range(3):
+            p = f"layers.{l}."
+            xb = pl.rmsnorm(x, W[p + "mixer_norm.weight"], 1e-5)
+            if l % 2 == 0:
+                inv = pl.rope_inv_freq(16, 100.0)
+                q = pl.apply_rope(pl.linear(xb, W[p + "mixer.wq"]).view(n, 2, 16), pos, inv)
+                k = pl.apply_rope(pl.linear(xb, W[p + "mixer.wk"]).view(n, 1, 16), pos, inv)
+                v = pl.linear(xb, W[p + "mixer.wv"]).view(n, 1, 16)
+                x = x + pl.linear(pl.attention(q, k, v, 0.25).reshape(n, 32), W[p + "mixer.wo"])
+            else:
+                s, rows = torch.zeros(32), []
+                for t in range(n):
+                    s = 0.9 * s + xb[t]
+                    rows.append(W[p + "mixer.w"] @ s)
+                x = x + torch.stack(rows)
+            xb = pl.rmsnorm(x, W[p + "ffn_norm.weight"], 1e-5)
+            x = x + pl.feed_forward(xb, W[p + "ffn.w_gate"], W[p + "ffn.w_up"], W[p + "ffn.w_down"])
+        return pl.linear(pl.rmsnorm(x, W["norm.weight"], 1e-5), W["head.weight"])
+
+    rnd = random.Random(12)
+    reqs = [[rnd.randrange(40) for _ in range(n)] for n in (20, 7, 33)]
+    # a batch of unequal prompts, then one token each; the state is carried from step to step
+    slots = [eng.new_sequence() for _ in reqs]
+    fed = [len(r) - 4 for r in reqs]
+    out = eng.step([StepEntry(s, r[:f], list(range(f))) for s, r, f in zip(slots, reqs, fed)])
+    got, o = [[] for _ in reqs], 0
+    for i, f in enumerate(fed):
+        got[i].append(out[o:o + f])
+        o += f
+    for k in range(4):
+        out = eng.step([StepEntry(s, [r[f + k]], [0]) for s, r, f in zip(slots, reqs, fed)])
+        for i in range(3):
+            got[i].append(out[i:i + 1])
+    for i, r in enumerate(reqs):
+        assert rel_err(torch.cat(got[i]), plain(r)) < TOL[torch.float32], i
+    # a slot that is used again starts from a zero state
+    eng.release(slots[0])
+    s = eng.new_sequence()
+    assert s == slots[0]
+    again = eng.step([StepEntry(s, reqs[1], list(range(7)))])
+    assert rel_err(again, plain(reqs[1])) < TOL[torch.float32]
