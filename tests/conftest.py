@@ -78,13 +78,31 @@ def rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
 TOL = {torch.float32: 1e-4, torch.bfloat16: 3e-2}
 
 
-def part_close(got: torch.Tensor, want: torch.Tensor, dtype) -> bool:
-    """For a part whose output is stored in `dtype`.  float32: as for logits.  bfloat16: the two
-    sides round their results on their own, so an element may differ by one unit in the last place
-    (2^-7 of its size), plus what the rounding of the part's inner tensors brings (1e-2 of the rms)."""
+def part_close(got: torch.Tensor, want: torch.Tensor, dtype, exact: torch.Tensor = None) -> bool:
+    """For a part whose output is stored in `dtype`; `want` is the plain implementation with its
+    tensors rounded to `dtype` where a part stores them.
+    float32: as for logits.
+    bfloat16, short paths (one or two roundings): an element may differ from `want` by one unit in
+    the last place (2^-7 of its size) plus 1e-2 of the rms for the inner roundings.
+    bfloat16 with `exact` (the plain implementation without any rounding): the two sides round at
+    different places (a fused kernel keeps float32 where the plain one stores bfloat16), so they are
+    compared by their distance to the exact result: the part is at most twice as far from it as the
+    rounded plain implementation is, plus one rounding of the largest element."""
     if dtype == torch.float32:
         return rel_err(got, want) < TOL[dtype]
+    if exact is not None:
+        e_got, e_want = rel_err(got, exact), rel_err(want, exact)
+        ok = e_got <= 2.0 * e_want + 2.0 ** -8
+        if not ok:
+            print(f"part_close: part is {e_got} from the exact result, the rounded plain one {e_want}")
+        return ok
     got, want = got.detach().double().cpu(), want.detach().double().cpu()
     assert got.shape == want.shape, (got.shape, want.shape)
     rms = float(want.pow(2).mean().sqrt())
-    return bool(((got - want).abs() <= want.abs() * 2.0 ** -7 + 1e-2 * rms).all())
+    excess = (got - want).abs() - (want.abs() * 2.0 ** -7 + 1e-2 * rms)
+    if bool((excess > 0).any()):
+        i = int(excess.argmax())
+        print(f"part_close: worst element {i}: got {float(got.flatten()[i])} want {float(want.flatten()[i])} "
+              f"rms {rms} excess {float(excess.max())}")
+        return False
+    return True

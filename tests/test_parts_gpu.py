@@ -58,7 +58,8 @@ def test_norm_and_feed_forward_parts(dtype):
         h = _rand((T, 72), 6).to(dtype)
         got = ffn.forward(h.to(DEV), None)
         want = pl.feed_forward(h.float(), t["w_gate"].float(), t["w_up"].float(), t["w_down"].float(), rt)
-        assert part_close(got.float(), want, dtype), T
+        exact = pl.feed_forward(h.float(), t["w_gate"].float(), t["w_up"].float(), t["w_down"].float())
+        assert part_close(got.float(), want, dtype, exact), T
     # a feed-forward with biases
     fb = FEED_FORWARDS.build(PartSpec.of("swiglu", hidden=72, intermediate=100, bias=True))
     tb = dict(t, b_gate=_rand((100,), 7, 0.1), b_up=_rand((100,), 8, 0.1), b_down=_rand((72,), 9, 0.1))
@@ -67,7 +68,7 @@ def test_norm_and_feed_forward_parts(dtype):
     g = pl.linear(h.float(), t["w_gate"]) + tb["b_gate"]
     u = pl.linear(h.float(), t["w_up"]) + tb["b_up"]
     want = pl.linear(pl.swiglu(g, u), t["w_down"]) + tb["b_down"]
-    assert part_close(fb.forward(h.to(DEV), None).float(), want, dtype)
+    assert part_close(fb.forward(h.to(DEV), None).float(), want, dtype, want)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
