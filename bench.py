@@ -43,6 +43,8 @@ def main() -> int:
                     help="fewer layers than the configuration has (named in the record)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points")
+    ap.add_argument("--only", choices=["prefill", "decode"], default=None,
+                    help="for profiling: run one phase alone (the record then lacks the other)")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -94,9 +96,12 @@ def main() -> int:
         engine.release(s)
         return dt
 
-    prefill_once(PREFILL_TOKENS)
-    prefill_once(PREFILL_TOKENS)
-    p_ms = sorted(prefill_once(PREFILL_TOKENS) for _ in range(5))[2] * 1e3
+    if args.only == "decode":
+        p_ms = float("nan")
+    else:
+        prefill_once(PREFILL_TOKENS)
+        prefill_once(PREFILL_TOKENS)
+        p_ms = sorted(prefill_once(PREFILL_TOKENS) for _ in range(5))[2] * 1e3
     T = PREFILL_TOKENS
     lin_params = L * (cfg.hidden_size * (cfg.q_dim + 2 * cfg.kv_dim) + cfg.q_dim * cfg.hidden_size
                       + 3 * cfg.hidden_size * cfg.intermediate_size)
@@ -136,6 +141,9 @@ def main() -> int:
             engine.release(s)
         return dt / steps, ctx_mid
 
+    if args.only == "prefill":
+        print(json.dumps({"prefill": prefill}), flush=True)
+        return 0
     step_s, ctx_tokens = decode(args.batch, args.steps, args.warmup)
     value = args.batch / step_s
     bytes_step = weight_bytes + ctx_tokens * kv_bytes_per_token

@@ -76,7 +76,7 @@ class _Group:
     pool: PagePool
     pages: Dict[int, List[int]]              # slot -> page of each PAGE positions (-1: given back)
     k: Optional[torch.Tensor] = None         # [entries, pages, Hkv, PAGE, hs]
-    v: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None         # the same; in bfloat16 [entries, pages, Hkv, hs, PAGE]
 
 
 class PagedCache:
@@ -122,6 +122,8 @@ class PagedCache:
             for g in self.groups:
                 shape = (len(g.entries), self.n_pages, g.need.n_kv_heads, PAGE, g.need.head_dim)
                 g.k = torch.zeros(shape, dtype=dtype, device=device)
+                if dtype == torch.bfloat16:     # V transposed inside a page: [.., head_dim, PAGE]
+                    shape = shape[:3] + (g.need.head_dim, PAGE)
                 g.v = torch.zeros(shape, dtype=dtype, device=device)
             for i, sn in self._state_needs.items():
                 self.states[i] = torch.zeros((self.max_slots,) + tuple(sn.shape), dtype=sn.dtype, device=device)

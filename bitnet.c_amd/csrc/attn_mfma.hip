@@ -1,0 +1,375 @@
+// Attention over the paged bf16 cache on the matrix cores (v_mfma_f32_16x16x32_bf16), for
+// head sizes 64 and 128, both phases.  Formulas as in attn_rows.hip (reference:
+// src/transformer/gqa_scalar.c:61-207, src/transformer/batched_attn_scalar.c:97-245):
+// kv head of head h is h / (H/Hkv); score = (q.k) * scale over the keys at positions <= the
+// query's (and inside the window); online softmax; out = sum_t p_t V_t.  Scores, maxima,
+// sums and the output accumulate in float32; p is rounded to bf16 for the second product.
+//
+// A wave works on "columns": a column is one (query token, query head) pair of one kv head,
+// 16 columns per MFMA tile.  Everything stays in registers:
+//   S^T[key, col]  = K[key, :] . Q[col, :]          A = 16 key rows of K,   B = Q^T
+//   O^T[dim, col] += V^T[dim, keys] . P^T[keys, col]  A = 16 rows of V^T,   B = P^T
+// The S^T tile leaves lane (col, g) with 4 keys per 16-key tile; the key rows fed to the two
+// tiles of a 32-key block are permuted (row i of tile sb is key 8*(i/4) + 4*sb + i%4) so
+// that each lane group g ends up with the 8 consecutive keys 8g..8g+7, which is exactly what
+// the B operand of the second product wants and what one 16-byte load of a V^T row holds.
+// Hence V is kept transposed in bf16 caches: K pages [page, kv_head, 64, hs], V pages
+// [page, kv_head, hs, 64].
+//
+// Prompt form: a workgroup of 4 waves owns 64*NT columns = consecutive query tokens x GT heads;
+// every wave walks the keys of its own columns, no shared memory, no barriers.
+// Decode form: the 16 columns are the heads of one kv group for the sequence's one new token;
+// the 4 waves take 32-key blocks in turn and merge through shared memory; long contexts are
+// also split over gridDim.z and merged by attn_mfma_combine_kernel in a fixed order.
+#include "common.h"
+#include <math.h>
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+#define LOG2E 1.4426950408889634f
+#define LN2 0.6931471805599453f
+
+struct MfmaArgs {
+    const bf16* q;            // [n_tokens, q_stride], head h at h*HS, rotated
+    bf16* out;                // [n_tokens, out_stride]
+    const bf16* k_pages;      // [pages, Hkv, 64, HS]
+    const bf16* vt_pages;     // [pages, Hkv, HS, 64]
+    const int* block_table;   // [n_seqs, bt_stride]
+    const int* seq_lens;      // decode: keys in the cache, the new one included; 0 = padding row
+    const int* tiles;         // prompt: [n, 4] = seq, first token row, tokens, position of the first
+    float* part_o;            // [n_tokens*H, n_splits, HS]
+    float* part_ml;           // [n_tokens*H, n_splits, 2]   (max in natural-log units, sum)
+    int q_stride, out_stride, bt_stride;
+    int H, Hkv, GT;           // GT: heads of a kv group per column tile row (power of two <= 16)
+    int window;
+    int n_splits, chunk;
+    float scale;
+};
+
+__device__ __forceinline__ bf16x8 ld16(const bf16* p) {
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
+}
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+    // round to nearest even, as __float2bfloat16 does
+    uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b);
+    ua += 0x7fffu + ((ua >> 16) & 1u);
+    ub += 0x7fffu + ((ub >> 16) & 1u);
+    return (ua >> 16) | (ub & 0xffff0000u);
+}
+
+// One 32-key block for NT column tiles.  kbase/vbase point at the block's first key inside its
+// page.  qpos/lo: per tile, this lane's column's position and first visible key (qpos < 0: no
+// such column).  key_hi: keys >= key_hi do not exist (decode: split end / length).
+template <int HS, int NT>
+__device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, const bf16* __restrict__ vbase,
+                                             int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
+                                             float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
+                                             const int (&lo)[NT], int key_hi, bool need_mask, float scale2,
+                                             int lane) {
+    constexpr int DC = HS / 32, DT = HS / 16;
+    const int i = lane & 15, g = lane >> 4;
+    const int krow0 = 8 * (i >> 2) + (i & 3);        // key row of tile 0; tile 1 is 4 further
+    f32x4 st[NT][2];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) { st[nt][0] = (f32x4){0.f, 0.f, 0.f, 0.f}; st[nt][1] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
+    bf16x8 ka[DC][2];
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+        ka[c][0] = ld16(kbase + (size_t)krow0 * HS + c * 32 + g * 8);
+        ka[c][1] = ld16(kbase + (size_t)(krow0 + 4) * HS + c * 32 + g * 8);
+    }
+    bf16x8 va[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) va[t] = ld16(vbase + (size_t)(t * 16 + i) * BN_PAGE + 8 * g);
+#pragma unroll
+    for (int c = 0; c < DC; ++c)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            st[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c][0], q[nt][c], st[nt][0], 0, 0, 0);
+            st[nt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c][1], q[nt][c], st[nt][1], 0, 0, 0);
+        }
+    if (need_mask) {
+        // keys that do not exist may hold anything, NaN included: clear them in V^T (0 * NaN is NaN)
+        const int first = kb + 8 * g;                 // this lane's 8 keys are first .. first+7
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            uint4 v = __builtin_bit_cast(uint4, va[t]);
+            if (first + 0 >= key_hi) v.x &= 0xffff0000u;
+            if (first + 1 >= key_hi) v.x &= 0x0000ffffu;
+            if (first + 2 >= key_hi) v.y &= 0xffff0000u;
+            if (first + 3 >= key_hi) v.y &= 0x0000ffffu;
+            if (first + 4 >= key_hi) v.z &= 0xffff0000u;
+            if (first + 5 >= key_hi) v.z &= 0x0000ffffu;
+            if (first + 6 >= key_hi) v.w &= 0xffff0000u;
+            if (first + 7 >= key_hi) v.w &= 0x0000ffffu;
+            va[t] = __builtin_bit_cast(bf16x8, v);
+        }
+    }
+    bf16x8 pb[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        float s[8];
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float v = st[nt][sb][r] * scale2;
+                if (need_mask) {
+                    const int key = kb + 8 * g + 4 * sb + r;
+                    if (key > qpos[nt] || key < lo[nt] || key >= key_hi) v = -INFINITY;
+                }
+                s[sb * 4 + r] = v;
+            }
+        float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, BN_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, BN_WAVE));
+        const float m_new = fmaxf(m[nt], mx);
+        float alpha = 1.f, rs = 0.f;
+        if (m_new == -INFINITY) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s[e] = 0.f;
+        } else {
+            alpha = exp2f(m[nt] - m_new);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { s[e] = exp2f(s[e] - m_new); rs += s[e]; }
+        }
+        rs += __shfl_xor(rs, 16, BN_WAVE);
+        rs += __shfl_xor(rs, 32, BN_WAVE);
+        l[nt] = l[nt] * alpha + rs;
+        m[nt] = m_new;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) acc[nt][t] *= alpha;
+        uint4 pk;
+        pk.x = pack2(s[0], s[1]); pk.y = pack2(s[2], s[3]); pk.z = pack2(s[4], s[5]); pk.w = pack2(s[6], s[7]);
+        pb[nt] = __builtin_bit_cast(bf16x8, pk);
+    }
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+            acc[nt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[t], pb[nt], acc[nt][t], 0, 0, 0);
+}
+
+// ---------------------------------------------------------------------------------------
+// prompt form
+// ---------------------------------------------------------------------------------------
+template <int HS, int NT>
+__global__ __launch_bounds__(256) void attn_mfma_prompt_kernel(MfmaArgs a) {
+    constexpr int DC = HS / 32, DT = HS / 16;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = lane & 15, g = lane >> 4;
+    const int G = a.H / a.Hkv, GT = a.GT;
+    const int n_head_tiles = (G + GT - 1) / GT;
+    const int kvh = blockIdx.y / n_head_tiles, ht = blockIdx.y - kvh * n_head_tiles;
+    const int* tl = a.tiles + 4 * blockIdx.x;
+    const int seq = tl[0], tok0 = tl[1], n_tok = tl[2], pos0 = tl[3];
+
+    bf16x8 q[NT][DC];
+    int qpos[NT], lo[NT], head[NT], tok[NT];
+    int w_hi = -1, w_lo = 0x7fffffff, all_hi = 0x7fffffff, all_lo = 0;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int c = (wave * NT + nt) * 16 + n;            // column within the workgroup
+        const int ti = c / GT, hg = ht * GT + (c - ti * GT);
+        const bool ok = ti < n_tok && hg < G;
+        head[nt] = kvh * G + hg;
+        tok[nt] = tok0 + ti;
+        qpos[nt] = ok ? pos0 + ti : -1;
+        lo[nt] = (ok && a.window > 0) ? max(0, qpos[nt] + 1 - a.window) : 0;
+#pragma unroll
+        for (int c2 = 0; c2 < DC; ++c2) {
+            uint4 z = make_uint4(0, 0, 0, 0);
+            if (ok) z = *reinterpret_cast<const uint4*>(a.q + (size_t)tok[nt] * a.q_stride + (size_t)head[nt] * HS + c2 * 32 + g * 8);
+            q[nt][c2] = __builtin_bit_cast(bf16x8, z);
+        }
+        if (ok) { w_hi = max(w_hi, qpos[nt]); w_lo = min(w_lo, lo[nt]); all_hi = min(all_hi, qpos[nt]); all_lo = max(all_lo, lo[nt]); }
+    }
+    // the wave's key range and the range that every one of its columns sees
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        w_hi = max(w_hi, __shfl_xor(w_hi, o, BN_WAVE));
+        w_lo = min(w_lo, __shfl_xor(w_lo, o, BN_WAVE));
+        all_hi = min(all_hi, __shfl_xor(all_hi, o, BN_WAVE));
+        all_lo = max(all_lo, __shfl_xor(all_lo, o, BN_WAVE));
+    }
+    // columns that do not exist have q = 0 and are never written; they need no masking
+    f32x4 acc[NT][DT];
+    float m[NT], l[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        m[nt] = -INFINITY; l[nt] = 0.f;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) acc[nt][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
+    const float scale2 = a.scale * LOG2E;
+    if (w_hi >= 0) {
+        const size_t bt_row = (size_t)seq * a.bt_stride;
+        for (int kb = (w_lo / 32) * 32; kb <= w_hi; kb += 32) {
+            const int page = a.block_table[bt_row + kb / BN_PAGE];
+            const int koff = kb % BN_PAGE;
+            const bf16* kbase = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS;
+            const bf16* vbase = a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff;
+            const bool need_mask = (kb + 31 > all_hi) || (kb < all_lo);
+            attend_block<HS, NT>(kbase, vbase, kb, q, acc, m, l, qpos, lo, w_hi + 1, need_mask, scale2, lane);
+        }
+    }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        if (qpos[nt] < 0) continue;
+        const float inv = l[nt] > 0.f ? 1.0f / l[nt] : 0.f;
+        bf16* o = a.out + (size_t)tok[nt] * a.out_stride + (size_t)head[nt] * HS + 4 * g;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            uint2 w;
+            w.x = pack2(acc[nt][t][0] * inv, acc[nt][t][1] * inv);
+            w.y = pack2(acc[nt][t][2] * inv, acc[nt][t][3] * inv);
+            *reinterpret_cast<uint2*>(o + t * 16) = w;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// decode form
+// ---------------------------------------------------------------------------------------
+template <int HS>
+__global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
+    constexpr int DC = HS / 32, DT = HS / 16;
+    __shared__ float m_s[4][16], l_s[4][16];
+    __shared__ float o_s[4][HS][17];                    // [wave][dim][col], padded
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = lane & 15, g = lane >> 4;
+    const int G = a.H / a.Hkv, GT = a.GT;
+    const int n_head_tiles = (G + GT - 1) / GT;
+    const int kvh = blockIdx.y / n_head_tiles, ht = blockIdx.y - kvh * n_head_tiles;
+    const int seq = blockIdx.x, split = blockIdx.z;
+    const int L = a.seq_lens[seq];
+    const int hg = ht * GT + n;
+    const bool ok = n < GT && hg < G && L > 0;
+    const int head = kvh * G + hg;
+
+    bf16x8 q[1][DC];
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+        uint4 z = make_uint4(0, 0, 0, 0);
+        if (ok) z = *reinterpret_cast<const uint4*>(a.q + (size_t)seq * a.q_stride + (size_t)head * HS + c * 32 + g * 8);
+        q[0][c] = __builtin_bit_cast(bf16x8, z);
+    }
+    int qpos[1] = {ok ? L - 1 : -1};
+    int lo_key = a.window > 0 ? max(0, L - a.window) : 0;
+    int lo[1] = {lo_key};
+    int k_lo = max(lo_key, split * a.chunk), k_hi = min(L, (split + 1) * a.chunk);   // [k_lo, k_hi)
+
+    f32x4 acc[1][DT];
+    float m[1] = {-INFINITY}, l[1] = {0.f};
+#pragma unroll
+    for (int t = 0; t < DT; ++t) acc[0][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    const float scale2 = a.scale * LOG2E;
+    if (k_lo < k_hi) {
+        const size_t bt_row = (size_t)seq * a.bt_stride;
+        for (int kb = (k_lo / 32) * 32 + 32 * wave; kb < k_hi; kb += 128) {
+            const int page = a.block_table[bt_row + kb / BN_PAGE];
+            const int koff = kb % BN_PAGE;
+            const bf16* kbase = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS;
+            const bf16* vbase = a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff;
+            const bool need_mask = (kb + 32 > k_hi) || (kb < k_lo);
+            attend_block<HS, 1>(kbase, vbase, kb, q, acc, m, l, qpos, lo, k_hi, need_mask, scale2, lane);
+        }
+    }
+    // merge the four waves: every wave's (m, l, O^T) through shared memory, in wave order
+    if (g == 0) { m_s[wave][n] = m[0]; l_s[wave][n] = l[0]; }
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o_s[wave][t * 16 + 4 * g + r][n] = acc[0][t][r];
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < HS * GT; idx += 256) {
+        const int col = idx / HS, dim = idx - col * HS;      // consecutive threads: consecutive dims
+        const int hg2 = ht * GT + col;
+        if (hg2 >= G) continue;
+        float M = fmaxf(fmaxf(m_s[0][col], m_s[1][col]), fmaxf(m_s[2][col], m_s[3][col]));
+        float num = 0.f, den = 0.f;
+        if (M != -INFINITY) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const float e = exp2f(m_s[w][col] - M);
+                num = fmaf(e, o_s[w][dim][col], num);
+                den = fmaf(e, l_s[w][col], den);
+            }
+        }
+        const int hd = kvh * G + hg2;
+        if (a.n_splits == 1) {
+            a.out[(size_t)seq * a.out_stride + (size_t)hd * HS + dim] = __float2bfloat16(den > 0.f ? num / den : 0.f);
+        } else {
+            const size_t row = ((size_t)seq * a.H + hd) * a.n_splits + split;
+            a.part_o[row * HS + dim] = num;
+            if (dim == 0) { a.part_ml[row * 2] = (M == -INFINITY) ? -INFINITY : M * LN2; a.part_ml[row * 2 + 1] = den; }
+        }
+    }
+}
+
+// out[row, d] = sum_s e^{m_s - m} o_s[d] / sum_s e^{m_s - m} l_s: one wave per row, the weights
+// of all splits computed at once (one lane per split), the sums in split order.
+__global__ __launch_bounds__(64) void attn_mfma_combine_kernel(bf16* __restrict__ out, int out_stride,
+                                                               const float* __restrict__ part_o,
+                                                               const float* __restrict__ part_ml, int H, int hs,
+                                                               int n_splits) {
+    const int row = blockIdx.x, lane = threadIdx.x;
+    const int tok = row / H, head = row - tok * H;
+    const float* ml = part_ml + (size_t)row * n_splits * 2;
+    float ms = -INFINITY, ls = 0.f;
+    if (lane < n_splits) { ms = ml[2 * lane]; ls = ml[2 * lane + 1]; }
+    const float M = wave_max(ms);
+    const float w = (M == -INFINITY || ms == -INFINITY) ? 0.f : expf(ms - M);
+    float den = 0.f;
+    for (int s = 0; s < n_splits; ++s) den = fmaf(__shfl(w, s, BN_WAVE), __shfl(ls, s, BN_WAVE), den);
+    const float inv = den > 0.f ? 1.0f / den : 0.f;
+    for (int d = lane; d < hs; d += 64) {
+        float num = 0.f;
+        for (int s = 0; s < n_splits; ++s)
+            num = fmaf(__shfl(w, s, BN_WAVE), part_o[((size_t)row * n_splits + s) * hs + d], num);
+        out[(size_t)tok * out_stride + (size_t)head * hs + d] = __float2bfloat16(num * inv);
+    }
+}
+
+// 1 when the matrix-core kernels take this shape
+extern "C" int bn_attn_mfma_supports(int hs) { return (hs == 64 || hs == 128) ? 1 : 0; }
+
+// query tokens per tile of the prompt form, for GT heads per group
+extern "C" int bn_attn_mfma_prompt_tokens(int hs, int GT) { return (hs == 64 ? 256 : 128) / GT; }
+
+extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
+                            const void* vt_pages, const int* block_table, int bt_stride, const int* seq_lens,
+                            const int* tiles, int n_tiles, int n_tokens, int H, int Hkv, int hs, int GT,
+                            int window, float scale, int n_splits, int chunk, float* part_o, float* part_ml,
+                            hipStream_t s) {
+    if (!bn_attn_mfma_supports(hs) || n_tiles <= 0 || n_tokens <= 0 || H <= 0 || Hkv <= 0 || H % Hkv) return BN_ERR_ARG;
+    if (GT <= 0 || GT > 16 || (GT & (GT - 1)) || window < 0 || n_splits < 1 || n_splits > 64) return BN_ERR_ARG;
+    if (n_splits > 1 && (chunk <= 0 || chunk % BN_PAGE || !part_o || !part_ml)) return BN_ERR_ARG;
+    if (!tiles && !seq_lens) return BN_ERR_ARG;
+    if (q_stride % 8 || out_stride % 4 || (((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)vt_pages) & 15) ||
+        ((uintptr_t)out & 7))
+        return BN_ERR_ARG;
+    MfmaArgs a;
+    a.q = (const bf16*)q; a.out = (bf16*)out; a.k_pages = (const bf16*)k_pages; a.vt_pages = (const bf16*)vt_pages;
+    a.block_table = block_table; a.seq_lens = seq_lens; a.tiles = tiles; a.part_o = part_o; a.part_ml = part_ml;
+    a.q_stride = q_stride; a.out_stride = out_stride; a.bt_stride = bt_stride;
+    a.H = H; a.Hkv = Hkv; a.GT = GT; a.window = window; a.scale = scale;
+    a.n_splits = n_splits; a.chunk = n_splits > 1 ? chunk : 0x40000000;
+    const int G = H / Hkv;
+    const int n_head_tiles = (G + GT - 1) / GT;
+    if (tiles) {
+        const dim3 grid(n_tiles, Hkv * n_head_tiles);
+        if (hs == 64) hipLaunchKernelGGL((attn_mfma_prompt_kernel<64, 4>), grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((attn_mfma_prompt_kernel<128, 2>), grid, dim3(256), 0, s, a);
+        return bn_launch_status();
+    }
+    const dim3 grid(n_tiles, Hkv * n_head_tiles, n_splits);
+    if (hs == 64) hipLaunchKernelGGL(attn_mfma_decode_kernel<64>, grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(attn_mfma_decode_kernel<128>, grid, dim3(256), 0, s, a);
+    int rc = bn_launch_status();
+    if (rc != 0 || n_splits == 1) return rc;
+    hipLaunchKernelGGL(attn_mfma_combine_kernel, dim3(n_tokens * H), dim3(64), 0, s, (bf16*)out, out_stride, part_o,
+                       part_ml, H, hs, n_splits);
+    return bn_launch_status();
+}

@@ -33,6 +33,7 @@ struct AttnArgs {
     int KT;                   // keys per tile: 16, 32 or 64
     int window;               // 0 = all earlier keys, else the last `window` of them
     int n_splits, chunk;      // keys per split, a multiple of BN_PAGE
+    int v_transposed;         // V pages are [page, kv_head, hs, BN_PAGE]
     float scale;
 };
 
@@ -135,9 +136,18 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
             for (int idx = tid; idx < KT * vec_per_row; idx += ATT_THREADS) {
                 const int j = idx / vec_per_row, c = idx - j * vec_per_row;
                 uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
-                if (j0 + j < hi) { kv = kg[idx]; vv = vg[idx]; }   // rows not yet written stay zero
+                if (j0 + j < hi) { kv = kg[idx]; if (!a.v_transposed) vv = vg[idx]; }   // rows not yet written stay zero
                 *reinterpret_cast<uint4*>(reinterpret_cast<unsigned char*>(k_s + j * kstride) + c * 16) = kv;
-                *reinterpret_cast<uint4*>(reinterpret_cast<unsigned char*>(v_s + j * kstride) + c * 16) = vv;
+                if (!a.v_transposed)
+                    *reinterpret_cast<uint4*>(reinterpret_cast<unsigned char*>(v_s + j * kstride) + c * 16) = vv;
+            }
+            if (a.v_transposed) {
+                const T* vt = reinterpret_cast<const T*>(a.v_pages) + ((size_t)page * a.Hkv + kvh) * hs * BN_PAGE +
+                              (j0 % BN_PAGE);
+                for (int idx = tid; idx < KT * hs; idx += ATT_THREADS) {
+                    const int d = idx / KT, j = idx - d * KT;
+                    v_s[j * kstride + d] = (j0 + j < hi) ? vt[(size_t)d * BN_PAGE + j] : from_f32<T>(0.f);
+                }
             }
         }
         __syncthreads();
@@ -326,7 +336,7 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
                             int bt_stride, const int* seq_lens, const int* tiles, int n_tiles,
                             int n_tokens, int H, int Hkv, int hs, int RT, int GT, int window,
                             float scale, int n_splits, int chunk, float* part_o, float* part_ml,
-                            hipStream_t s) {
+                            int v_transposed, hipStream_t s) {
     if (n_tiles <= 0 || n_tokens <= 0 || H <= 0 || Hkv <= 0 || H % Hkv) return BN_ERR_ARG;
     if (hs < 8 || hs > 256 || hs % 8) return BN_ERR_ARG;
     if (GT <= 0 || GT > RT || (GT & (GT - 1)) || RT > 16 || (RT & (RT - 1))) return BN_ERR_ARG;
@@ -341,6 +351,7 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
     a.H = H; a.Hkv = Hkv; a.hs = hs; a.GT = GT; a.window = window;
     a.n_splits = n_splits; a.chunk = n_splits > 1 ? chunk : 0x40000000;
     a.scale = scale;
+    a.v_transposed = v_transposed;
     a.KT = bn_attn_rows_key_tile(dtype, RT, hs);
     if (a.KT == 0) return BN_ERR_ARG;
     int rc;

@@ -5,7 +5,8 @@
 // (src/transformer/cpu_backend.c:283-296).  angle = float(pos) * inv_freq[i], cos/sin
 // at full float32 accuracy (src/transformer.c:143-162 uses cosf/sinf).  The cache
 // holds rotated keys (src/transformer/cpu.c:893-898 rotates the cached row).
-// Cache layout per layer: [page, kv_head, BN_PAGE, head_dim].
+// Cache layout per layer: K [page, kv_head, BN_PAGE, head_dim]; V the same, or transposed
+// [page, kv_head, head_dim, BN_PAGE] (v_transposed) for the matrix-core attention kernels.
 #include "common.h"
 
 template <typename T>
@@ -15,7 +16,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
                                      const int* __restrict__ block_table, int bt_stride,
                                      T* __restrict__ k_pages, T* __restrict__ v_pages,
                                      const float* __restrict__ inv_freq, int rope_dims,
-                                     int H, int Hkv, int hs) {
+                                     int H, int Hkv, int hs, int v_transposed) {
     extern __shared__ float cs[];            // cos[half], sin[half]
     const int t = blockIdx.x;
     const int pos = positions[t];
@@ -58,7 +59,10 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
         }
         const size_t dst = (((size_t)page * Hkv + kh) * BN_PAGE + off) * hs + d;
         k_pages[dst] = from_f32<T>(o);
-        v_pages[dst] = vrow[idx];
+        if (v_transposed)       // V pages [page, kv_head, head_dim, BN_PAGE]
+            v_pages[(((size_t)page * Hkv + kh) * hs + d) * BN_PAGE + off] = vrow[idx];
+        else
+            v_pages[dst] = vrow[idx];
     }
 }
 
@@ -68,7 +72,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
 extern "C" int bn_rope_kv_write(int dtype, void* qkv, int row_stride, const int* positions,
                                 const int* seq_index, const int* block_table, int bt_stride,
                                 void* k_pages, void* v_pages, const float* inv_freq, int rope_dims,
-                                int n_tokens, int H, int Hkv, int hs, hipStream_t s) {
+                                int n_tokens, int H, int Hkv, int hs, int v_transposed, hipStream_t s) {
     if (n_tokens <= 0 || H <= 0 || Hkv < 0 || hs <= 0 || rope_dims < 0 || rope_dims > hs ||
         (rope_dims & 1) || row_stride < (H + 2 * Hkv) * hs)
         return BN_ERR_ARG;
@@ -78,11 +82,11 @@ extern "C" int bn_rope_kv_write(int dtype, void* qkv, int row_stride, const int*
     if (dtype == BN_DT_F32)
         hipLaunchKernelGGL(rope_kv_write_kernel<float>, dim3(n_tokens), dim3(256), smem, s,
                            (float*)qkv, row_stride, positions, seq_index, block_table, bt_stride,
-                           (float*)k_pages, (float*)v_pages, inv_freq, rope_dims, H, Hkv, hs);
+                           (float*)k_pages, (float*)v_pages, inv_freq, rope_dims, H, Hkv, hs, v_transposed);
     else if (dtype == BN_DT_BF16)
         hipLaunchKernelGGL(rope_kv_write_kernel<bf16>, dim3(n_tokens), dim3(256), smem, s,
                            (bf16*)qkv, row_stride, positions, seq_index, block_table, bt_stride,
-                           (bf16*)k_pages, (bf16*)v_pages, inv_freq, rope_dims, H, Hkv, hs);
+                           (bf16*)k_pages, (bf16*)v_pages, inv_freq, rope_dims, H, Hkv, hs, v_transposed);
     else
         return BN_ERR_DTYPE;
     return bn_launch_status();

@@ -1,7 +1,7 @@
 // Decode-phase matrix product for bf16: Y[M, N] = X[M, K] . W[N, K]^T with M <= 64 rows
 // of activations, on the matrix cores (v_mfma_f32_16x16x32_bf16).  The weights are
-// streamed once from HBM with 16-byte loads, each lane reading 128 contiguous bytes of
-// one weight row per 256-element K chunk; K is split over the waves of a workgroup and
+// streamed once from HBM with 16-byte loads, four lanes covering 64 contiguous bytes of
+// one weight row per load and a wave 512 bytes of 16 rows per 256-element K chunk; K is split over the waves of a workgroup and
 // the partial sums are added through shared memory in wave order, so the result does
 // not depend on timing.  It plays the part of the reference's matvec kernels
 // (src/gpu_cuda.cu:3976-4010, one warp per output row) and of its stacked gate/up
@@ -40,11 +40,11 @@ __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_ke
     for (int a = 0; a < NA; ++a) acc[a] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     for (int kc = wave * SK_CHUNK; kc < K; kc += n_waves * SK_CHUNK) {
-        const int kb = kc + g * 64;                   // this lane's 64 elements of the chunk
+        const int kb = kc + g * 8;                    // lane group g: 8 elements of every 32 (64 contiguous bytes per row and load)
         uint4 wv[8], uv[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const int k = kb + j * 8;
+            const int k = kb + j * 32;
             wv[j] = (k < K) ? *reinterpret_cast<const uint4*>(wrow + k) : make_uint4(0, 0, 0, 0);
             if (DUAL) uv[j] = (k < K) ? *reinterpret_cast<const uint4*>(urow + k) : make_uint4(0, 0, 0, 0);
         }
@@ -55,7 +55,7 @@ __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_ke
             uint4 xv[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const int k = kb + j * 8;
+                const int k = kb + j * 32;
                 xv[j] = (m < M && k < K) ? *reinterpret_cast<const uint4*>(xrow + k) : make_uint4(0, 0, 0, 0);
             }
 #pragma unroll
@@ -112,6 +112,10 @@ static int launch_mt(int MT, const void* X, const void* W, void* Y, int M, int N
     return BN_ERR_ARG;
 }
 
+// Tuning hook: > 0 fixes the waves per workgroup (still bounded by the K chunks and by shared memory).
+static int g_force_waves = 0;
+extern "C" void bn_skinny_gemm_force_waves(int n) { g_force_waves = n; }
+
 // 1 if the kernel takes the shape, 0 if the caller must use the tiled kernel.
 extern "C" int bn_skinny_gemm_supports(int M, int N, int K, int ldx, int ldw) {
     return (M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0) ? 1 : 0;
@@ -129,6 +133,7 @@ extern "C" int bn_skinny_gemm(int out_dtype, const void* X, const void* W, void*
     // the K chunks there are and by 48 KB of shared memory for the partial sums
     const int tiles = (N + 15) / 16;
     int n_waves = tiles >= 2048 ? 4 : (tiles >= 1024 ? 8 : 16);
+    if (g_force_waves > 0) n_waves = g_force_waves;
     const int k_chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
     while (n_waves > 1 && n_waves / 2 >= k_chunks) n_waves >>= 1;
     while (n_waves > 1 && n_waves * NA > 48) n_waves >>= 1;

@@ -33,13 +33,20 @@ _SIGNATURES = {
     },
     "rope_kv": {
         "bn_rope_kv_write": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                             c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                             c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "attn_rows": {
         "bn_attn_rows_key_tile": [c_int, c_int, c_int],
         "bn_attn_rows": [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
-                         c_void_p, c_void_p, c_void_p],
+                         c_void_p, c_void_p, c_int, c_void_p],
+    },
+    "attn_mfma": {
+        "bn_attn_mfma_supports": [c_int],
+        "bn_attn_mfma_prompt_tokens": [c_int, c_int],
+        "bn_attn_mfma": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                         c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p,
+                         c_void_p],
     },
     "gemm_tiled": {
         "bn_gemm_tiled": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
@@ -286,13 +293,22 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
 # position encoding + cache write, attention
 # --------------------------------------------------------------------------------------
 
+def v_transposed_for(dtype) -> bool:
+    """bf16 caches keep V transposed ([pages, Hkv, hs, PAGE]) for the matrix-core attention
+    kernels; float32 caches keep V like K ([pages, Hkv, PAGE, hs])."""
+    return dtype == torch.bfloat16
+
+
 def _check_pages(k_pages, v_pages, Hkv, hs, dtype):
-    for t, nm in ((k_pages, "k_pages"), (v_pages, "v_pages")):
+    """Checks both page tensors; returns whether V is transposed."""
+    vt = v_transposed_for(dtype)
+    for t, nm, shape in ((k_pages, "k_pages", (Hkv, PAGE, hs)), (v_pages, "v_pages", (Hkv, hs, PAGE) if vt else (Hkv, PAGE, hs))):
         _dev(t, nm, dtype, 4)
-        if tuple(t.shape[1:]) != (Hkv, PAGE, hs) or not t.is_contiguous():
-            raise KernelError(f"{nm}: expected contiguous [pages, {Hkv}, {PAGE}, {hs}], got {tuple(t.shape)}")
-    if k_pages.shape != v_pages.shape:
-        raise KernelError("k_pages and v_pages differ in shape")
+        if tuple(t.shape[1:]) != shape or not t.is_contiguous():
+            raise KernelError(f"{nm}: expected contiguous [pages, {', '.join(map(str, shape))}], got {tuple(t.shape)}")
+    if k_pages.shape[0] != v_pages.shape[0]:
+        raise KernelError("k_pages and v_pages differ in their number of pages")
+    return vt
 
 
 def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, hs: int, *,
@@ -315,8 +331,9 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
             raise KernelError(f"rope_kv_write: rope_dims {rope_dims} does not fit hs={hs} / inv_freq "
                               f"{tuple(inv_freq.shape)}")
     bt_stride = 0
+    vt = False
     if k_pages is not None:
-        _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype)
+        vt = _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype)
         _dev(seq_index, "seq_index", torch.int32, 1)
         _dev(block_table, "block_table", torch.int32, 2)
         if seq_index.numel() != T or not seq_index.is_contiguous() or not block_table.is_contiguous():
@@ -330,7 +347,7 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
         block_table.data_ptr() if k_pages is not None else None, bt_stride,
         k_pages.data_ptr() if k_pages is not None else None,
         v_pages.data_ptr() if k_pages is not None else None,
-        inv_freq.data_ptr() if rope_dims else None, rope_dims, T, H, Hkv, hs, _stream()), "rope_kv_write")
+        inv_freq.data_ptr() if rope_dims else None, rope_dims, T, H, Hkv, hs, int(vt), _stream()), "rope_kv_write")
 
 
 def _pow2_at_least(n: int) -> int:
@@ -340,12 +357,22 @@ def _pow2_at_least(n: int) -> int:
     return p
 
 
-def attention_row_shape(H: int, Hkv: int, decode: bool):
-    """(RT, GT, QT): rows of a workgroup = QT query tokens x GT heads of one kv group."""
+def mfma_attention(dtype, hs: int) -> bool:
+    """Whether the matrix-core attention kernels take this cache type and head size."""
+    return dtype == torch.bfloat16 and bool(_fn("attn_mfma", "bn_attn_mfma_supports")(int(hs)))
+
+
+def attention_row_shape(H: int, Hkv: int, decode: bool, dtype=None, hs: int = 0):
+    """(RT, GT, QT): what one workgroup covers: QT query tokens x GT heads of one kv group
+    (RT = QT * GT rows for the vector kernel)."""
     G = H // Hkv
     GT = min(_pow2_at_least(G), 16)
-    RT = GT if decode else 16
-    return RT, GT, RT // GT
+    if decode:
+        return GT, GT, 1
+    if dtype is not None and mfma_attention(dtype, hs):
+        qt = _fn("attn_mfma", "bn_attn_mfma_prompt_tokens")(int(hs), GT)
+        return qt * GT, GT, qt
+    return 16, GT, 16 // GT
 
 
 def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int):
@@ -355,7 +382,7 @@ def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int):
     G = H // Hkv
     wgs = max(1, n_seqs * Hkv * ((G + GT - 1) // GT))
     pages = max(1, (max_len + PAGE - 1) // PAGE)
-    want = max(1, min(pages, 64, (512 + wgs - 1) // wgs))
+    want = max(1, min(pages, 64, (1024 + wgs - 1) // wgs))
     chunk = ((pages + want - 1) // want) * PAGE
     n_splits = (pages * PAGE + chunk - 1) // chunk
     return n_splits, chunk
@@ -363,17 +390,21 @@ def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int):
 
 def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
               block_table: torch.Tensor, H: int, Hkv: int, hs: int, scale: float, *, window: int = 0,
-              tiles=None, qt: int = 0, seq_lens=None, n_splits: int = 1, chunk: int = 0) -> None:
+              tiles=None, qt: int = 0, seq_lens=None, n_splits: int = 1, chunk: int = 0,
+              force_vector: bool = False) -> None:
     """Causal attention of the (rotated) Q heads in qkv over the paged cache.
 
     Prompt form: `tiles` [n, 4] int32 = (sequence, first token row, tokens (<= qt), position of
-    the first), qt = the QT of attention_row_shape(H, Hkv, False).
+    the first), qt = the QT of attention_row_shape(H, Hkv, False, dtype, hs).
     Decode form: tiles None, seq_lens [B] int32 (keys in the cache, the new one included; 0 for a
-    padding row); row b of qkv is sequence b's token; n_splits/chunk from decode_splits."""
+    padding row); row b of qkv is sequence b's token; n_splits/chunk from decode_splits.
+    bf16 with head size 64 or 128 runs on the matrix cores, everything else on the vector ALUs
+    (force_vector: the vector kernel also where the other would run; its qt then is that of
+    attention_row_shape without dtype)."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(out, "out", qkv.dtype, 2)
-    _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype)
+    vt = _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype)
     _dev(block_table, "block_table", torch.int32, 2)
     T = qkv.shape[0]
     if H % Hkv or qkv.shape[1] < H * hs or out.shape != (T, H * hs) or not out.is_contiguous():
@@ -383,7 +414,8 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     if not block_table.is_contiguous():
         raise KernelError("attention: block_table must be contiguous")
     decode = tiles is None
-    RT, GT, QT = attention_row_shape(H, Hkv, decode)
+    use_mfma = mfma_attention(qkv.dtype, hs) and not force_vector
+    RT, GT, QT = attention_row_shape(H, Hkv, decode, qkv.dtype if use_mfma else None, hs)
     if decode:
         _dev(seq_lens, "seq_lens", torch.int32, 1)
         if seq_lens.numel() != T or block_table.shape[0] < T or not seq_lens.is_contiguous():
@@ -392,7 +424,7 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     else:
         _dev(tiles, "tiles", torch.int32, 2)
         if tiles.shape[1] != 4 or not tiles.is_contiguous() or qt != QT:
-            raise KernelError(f"attention(prompt): tiles must be [n, 4] built for qt={QT}")
+            raise KernelError(f"attention(prompt): tiles must be [n, 4] built for qt={QT}, got qt={qt}")
         n_tiles = tiles.shape[0]
         n_splits, chunk = 1, 0
     if T == 0 or n_tiles == 0:
@@ -404,15 +436,25 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
         if n_splits * chunk < block_table.shape[1] * PAGE:
             raise KernelError(f"attention: {n_splits} splits of {chunk} keys do not cover the "
                               f"{block_table.shape[1]} pages of the block table")
+        if n_splits > 64:
+            raise KernelError("attention: at most 64 splits")
         part_o = torch.empty((T * H * n_splits, hs), dtype=torch.float32, device=qkv.device)
         part_ml = torch.empty((T * H * n_splits, 2), dtype=torch.float32, device=qkv.device)
+    po = part_o.data_ptr() if part_o is not None else None
+    pm = part_ml.data_ptr() if part_ml is not None else None
+    sl = seq_lens.data_ptr() if decode else None
+    tl = tiles.data_ptr() if not decode else None
+    if use_mfma:
+        _check(_fn("attn_mfma", "bn_attn_mfma")(
+            qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * hs, k_pages.data_ptr(), v_pages.data_ptr(),
+            block_table.data_ptr(), block_table.shape[1], sl, tl, n_tiles, T, H, Hkv, hs, GT, int(window),
+            float(scale), int(n_splits), int(chunk), po, pm, _stream()), "attention(mfma)")
+        return
     _check(_fn("attn_rows", "bn_attn_rows")(
         _code(qkv.dtype), qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * hs,
         k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1],
-        seq_lens.data_ptr() if decode else None, tiles.data_ptr() if not decode else None,
-        n_tiles, T, H, Hkv, hs, RT, GT, int(window), float(scale), int(n_splits), int(chunk),
-        part_o.data_ptr() if part_o is not None else None,
-        part_ml.data_ptr() if part_ml is not None else None, _stream()), "attention")
+        sl, tl, n_tiles, T, H, Hkv, hs, RT, GT, int(window), float(scale), int(n_splits), int(chunk),
+        po, pm, int(vt), _stream()), "attention")
 
 
 # --------------------------------------------------------------------------------------

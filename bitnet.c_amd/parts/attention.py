@@ -81,7 +81,7 @@ class Attention(Part):
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
                           window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk)
         else:
-            _, _, qt = ops.attention_row_shape(H, Hkv, False)
+            _, _, qt = ops.attention_row_shape(H, Hkv, False, h.dtype, hs)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
                           window=self.window, tiles=ctx.tiles(qt), qt=qt)
         return self.o(out)

@@ -102,6 +102,9 @@ def test_groups_by_need_and_shared_entries():
     assert len(c.groups) == 2
     assert c.groups[0].entries == [0, 2] and c.groups[1].entries == [1]     # storage of their own
     assert c.groups[0].k.shape == (2, 8, 2, PAGE, 16) and c.groups[1].k.shape == (1, 8, 2, PAGE, 16)
+    assert c.groups[0].v.shape == (2, 8, 2, PAGE, 16)
+    cb = PagedCache(needs, [None, None, None, 0, None], 64 * 8, dtype=torch.bfloat16, device="cpu")
+    assert cb.groups[0].v.shape == (2, 8, 2, 16, PAGE)          # bfloat16: V transposed inside a page
     tables = {0: torch.zeros(1, 1, dtype=torch.int32), 1: torch.zeros(1, 1, dtype=torch.int32)}
     v0, v3, v4 = c.view(0, tables, 64), c.view(3, tables, 64), c.view(4, tables, 64)
     assert v3.k_pages.data_ptr() == v0.k_pages.data_ptr() and v0.writes and not v3.writes

@@ -168,6 +168,7 @@ def _paged(seqs_k, seqs_v, dtype, n_pages, seed):
     # unused pages hold NaN: a kernel that reads a key it must not see shows it
     k_pages = torch.full((n_pages, Hkv, 64, hs), float("nan"), dtype=dtype)
     v_pages = torch.full((n_pages, Hkv, 64, hs), float("nan"), dtype=dtype)
+    vt = dtype == torch.bfloat16                      # bf16 caches keep V transposed inside a page
     width = max((k.shape[0] + 63) // 64 for k in seqs_k)
     bt = torch.zeros((len(seqs_k), width), dtype=torch.int32)
     for s, (k, v) in enumerate(zip(seqs_k, seqs_v)):
@@ -177,6 +178,8 @@ def _paged(seqs_k, seqs_v, dtype, n_pages, seed):
             n = min(64, k.shape[0] - 64 * i)
             k_pages[p, :, :n] = k[64 * i:64 * i + n].transpose(0, 1).to(dtype)
             v_pages[p, :, :n] = v[64 * i:64 * i + n].transpose(0, 1).to(dtype)
+    if vt:
+        v_pages = v_pages.transpose(2, 3).contiguous()
     return k_pages, v_pages, bt
 
 
@@ -196,8 +199,9 @@ def test_rope_kv_write(dtype, H, Hkv, hs, rope_dims):
     pos = torch.tensor(positions, dtype=torch.int32)
     n_pages = 12
     bt = torch.tensor([[3, 0, 0, 0], [7, 1, 0, 0], [2, 9, 5, 11]], dtype=torch.int32)
+    vt = dtype == torch.bfloat16
     kp = torch.zeros((n_pages, Hkv, 64, hs), dtype=dtype).cuda()
-    vp = torch.zeros_like(kp)
+    vp = torch.zeros((n_pages, Hkv, hs, 64) if vt else (n_pages, Hkv, 64, hs), dtype=dtype).cuda()
     q_in = qkv.clone()
     g = qkv.cuda()
     ops.rope_kv_write(g, pos.cuda(), H, Hkv, hs, inv_freq=inv_freq.cuda(), rope_dims=rope_dims,
@@ -209,6 +213,8 @@ def test_rope_kv_write(dtype, H, Hkv, hs, rope_dims):
     assert close(g[:, :H * hs].float().view(T, H, hs), q_ref, dtype)
     assert torch.equal(g[:, H * hs:].cpu(), q_in[:, H * hs:])            # K, V of the input stay as they are
     kp, vp = kp.cpu().float(), vp.cpu().float()
+    if vt:
+        vp = vp.transpose(2, 3)
     written = torch.zeros((n_pages, 64), dtype=torch.bool)
     for t in range(T):
         page, off = int(bt[seq_index[t], positions[t] // 64]), positions[t] % 64
@@ -222,7 +228,8 @@ def test_rope_kv_write(dtype, H, Hkv, hs, rope_dims):
     kp2 = torch.zeros((n_pages, Hkv, 64, hs), dtype=dtype).cuda()
     ops.rope_kv_write(g2, torch.full((T,), -1, dtype=torch.int32).cuda(), H, Hkv, hs, inv_freq=inv_freq.cuda(),
                       rope_dims=rope_dims, seq_index=torch.zeros(T, dtype=torch.int32).cuda(), block_table=bt.cuda(),
-                      k_pages=kp2, v_pages=kp2.clone())
+                      k_pages=kp2,
+                      v_pages=torch.zeros((n_pages, Hkv, hs, 64) if vt else (n_pages, Hkv, 64, hs), dtype=dtype).cuda())
     assert torch.equal(g2.cpu(), q_in) and float(kp2.abs().sum()) == 0.0
     g3 = q_in.clone().cuda()
     ops.rope_kv_write(g3, pos.cuda(), H, Hkv, hs, inv_freq=inv_freq.cuda(), rope_dims=rope_dims)
@@ -239,6 +246,15 @@ def test_rope_reference_vector_on_device():
                       inv_freq=torch.tensor([math.pi / 2, 0.0]).cuda(), rope_dims=4)
     want = torch.tensor([-3.0, 2, 1, 4, 9, 9, 9, 9, 3, -2, -1, -4, 7, 7, 7, 7])
     assert torch.allclose(g.cpu()[0], want, atol=1e-6)
+
+
+def mfma_close(got, ref) -> bool:
+    """The matrix-core attention rounds the softmax weights to bf16 before the second product
+    (8 bits: each weight is off by at most 2^-9 of itself, so a weighted mean of values is off by
+    at most 2^-9 of the largest |value| it mixes, here below 2^-9 * 5 for unit normal values),
+    and its result once more."""
+    got, ref = got.detach().double().cpu(), ref.detach().double().cpu()
+    return bool(((got - ref).abs() <= ref.abs() * 2.0 ** -8 + 5 * 2.0 ** -9).all())
 
 
 def _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, seed):
@@ -267,11 +283,15 @@ def _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, seed):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,Hkv,hs,window", [(4, 2, 16, 0), (5, 5, 24, 0), (6, 2, 32, 0), (8, 2, 128, 0), (32, 1, 64, 0),
-                                             (2, 1, 256, 0), (4, 2, 16, 7), (4, 4, 64, 100), (20, 1, 40, 0)])
-def test_attention_prompt_form(dtype, H, Hkv, hs, window):
-    lens_before, n_new = [0, 0, 64, 130, 5], [1, 37, 64, 3, 70]
+                                             (2, 1, 256, 0), (4, 2, 16, 7), (4, 4, 64, 100), (20, 1, 40, 0),
+                                             (32, 8, 128, 0), (8, 8, 128, 33), (6, 2, 64, 0), (40, 2, 64, 0)])
+@pytest.mark.parametrize("force_vector", [False, True])
+def test_attention_prompt_form(dtype, H, Hkv, hs, window, force_vector):
+    lens_before, n_new = [0, 0, 64, 130, 5, 0], [1, 37, 64, 3, 70, 300]
     ops, qkv, kp, vp, bt, ref, scale = _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, 100)
-    _, _, qt = ops.attention_row_shape(H, Hkv, False)
+    if force_vector and not ops.mfma_attention(dtype, hs):
+        pytest.skip("the vector kernel is what runs anyway")
+    _, _, qt = ops.attention_row_shape(H, Hkv, False, None if force_vector else dtype, hs)
     tiles, r = [], 0
     for s, (p0, n) in enumerate(zip(lens_before, n_new)):
         for i in range(0, n, qt):
@@ -279,17 +299,21 @@ def test_attention_prompt_form(dtype, H, Hkv, hs, window):
         r += n
     out = torch.full((qkv.shape[0], H * hs), float("nan"), dtype=dtype).cuda()
     ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, scale, window=window,
-                  tiles=torch.tensor(tiles, dtype=torch.int32).cuda(), qt=qt)
-    assert close(out.float(), ref, dtype)
+                  tiles=torch.tensor(tiles, dtype=torch.int32).cuda(), qt=qt, force_vector=force_vector)
+    assert mfma_close(out.float(), ref) if ops.mfma_attention(dtype, hs) and not force_vector else close(out.float(), ref, dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,Hkv,hs,window", [(4, 2, 16, 0), (5, 5, 24, 0), (8, 2, 128, 0), (12, 4, 64, 0),
-                                             (16, 1, 32, 0), (4, 2, 16, 50), (8, 8, 64, 129)])
+                                             (16, 1, 32, 0), (4, 2, 16, 50), (8, 8, 64, 129), (32, 8, 128, 0),
+                                             (40, 2, 128, 0), (6, 6, 128, 70)])
 @pytest.mark.parametrize("force_splits", [1, 0, 5])
-def test_attention_decode_form(dtype, H, Hkv, hs, window, force_splits):
+@pytest.mark.parametrize("force_vector", [False, True])
+def test_attention_decode_form(dtype, H, Hkv, hs, window, force_splits, force_vector):
     lens_before, n_new = [0, 63, 64, 700, 129, 300], [1] * 6
     ops, qkv, kp, vp, bt, ref, scale = _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, 200)
+    if force_vector and not ops.mfma_attention(dtype, hs):
+        pytest.skip("the vector kernel is what runs anyway")
     B = len(n_new)
     # two padding rows at the end: length 0, their output is zero and nothing else changes
     qkv = torch.cat([qkv, torch.zeros((2, qkv.shape[1]), dtype=dtype).cuda()])
@@ -307,8 +331,11 @@ def test_attention_decode_form(dtype, H, Hkv, hs, window, force_splits):
         n_splits, chunk = 1, 0
     out = torch.full((B + 2, H * hs), float("nan"), dtype=dtype).cuda()
     ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, scale, window=window, seq_lens=lens,
-                  n_splits=n_splits, chunk=chunk)
-    assert close(out[:B].float(), ref, dtype)
+                  n_splits=n_splits, chunk=chunk, force_vector=force_vector)
+    if ops.mfma_attention(dtype, hs) and not force_vector:
+        assert mfma_close(out[:B].float(), ref)
+    else:
+        assert close(out[:B].float(), ref, dtype)
     assert float(out[B:].float().abs().sum()) == 0.0
 
 
@@ -317,8 +344,8 @@ def test_attention_finds_a_far_key(dtype):
     """One key among 900 has a large score with the query: the output must be its value row,
     wherever it lies (first page, a page's edge, the last position)."""
     ops = _ops()
-    H, Hkv, hs, L = 4, 2, 32, 900
-    for far in (0, 63, 64, 449, 898, 899):
+    for H, Hkv, hs, L in ((4, 2, 32, 900), (8, 2, 128, 900)):
+      for far in (0, 63, 64, 449, 898, 899):
         k = _rand((L, Hkv, hs), dtype, 300, 0.1)
         v = _rand((L, Hkv, hs), dtype, 301)
         q = _rand((1, H, hs), dtype, 302, 0.1)

@@ -65,10 +65,13 @@ def test_norm_and_feed_forward_parts(dtype):
     tb = dict(t, b_gate=_rand((100,), 7, 0.1), b_up=_rand((100,), 8, 0.1), b_down=_rand((72,), 9, 0.1))
     fb.load(tb, DEV, dtype)
     h = _rand((5, 72), 10).to(dtype)
-    g = pl.linear(h.float(), t["w_gate"]) + tb["b_gate"]
-    u = pl.linear(h.float(), t["w_up"]) + tb["b_up"]
-    want = pl.linear(pl.swiglu(g, u), t["w_down"]) + tb["b_down"]
-    assert part_close(fb.forward(h.to(DEV), None).float(), want, dtype, want)
+    def with_bias(r):
+        g = r(r(pl.linear(h.float(), t["w_gate"])) + tb["b_gate"])
+        u = r(r(pl.linear(h.float(), t["w_up"])) + tb["b_up"])
+        return r(r(pl.linear(r(pl.swiglu(g, u)), t["w_down"])) + tb["b_down"])
+    exact = with_bias(lambda x: x)
+    want = with_bias((lambda x: x) if dtype == torch.float32 else (lambda x: x.to(dtype).float()))
+    assert part_close(fb.forward(h.to(DEV), None).float(), want, dtype, exact)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
