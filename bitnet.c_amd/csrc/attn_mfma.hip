@@ -326,8 +326,14 @@ __global__ __launch_bounds__(64) void attn_mfma_combine_kernel(bf16* __restrict_
     const float inv = den > 0.f ? 1.0f / den : 0.f;
     for (int d = lane; d < hs; d += 64) {
         float num = 0.f;
-        for (int s = 0; s < n_splits; ++s)
-            num = fmaf(__shfl(w, s, BN_WAVE), part_o[((size_t)row * n_splits + s) * hs + d], num);
+        const float* po = part_o + (size_t)row * n_splits * hs + d;
+        for (int s0 = 0; s0 < n_splits; s0 += 8) {
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = (s0 + j < n_splits) ? po[(size_t)(s0 + j) * hs] : 0.f;   // loads first
+#pragma unroll
+            for (int j = 0; j < 8; ++j) num = fmaf(__shfl(w, min(s0 + j, 63), BN_WAVE), v[j], num);      // then split order
+        }
         out[(size_t)tok * out_stride + (size_t)head * hs + d] = __float2bfloat16(num * inv);
     }
 }
