@@ -45,6 +45,14 @@ struct MfmaArgs {
     int window;
     int n_splits, chunk;
     float scale;
+    // decode form only.  rotate != 0: q (and the new key) arrive unrotated and are rotated here,
+    // angle = position * inv_freq[i], pairs (i, i + HS/2).  write_kv != 0: the workgroup whose keys
+    // include the new position stores the new key (rotated) and value into the pages first.
+    // counters != null: the last workgroup of a (sequence, kv head) to finish merges the splits
+    // itself (no combine launch); the counters are zero between launches.
+    const float* inv_freq;
+    int rotate, write_kv;
+    int* counters;
 };
 
 __device__ __forceinline__ bf16x8 ld16(const bf16* p) {
@@ -232,11 +240,27 @@ __global__ __launch_bounds__(256) void attn_mfma_prompt_kernel(MfmaArgs a) {
 // ---------------------------------------------------------------------------------------
 // decode form
 // ---------------------------------------------------------------------------------------
+__device__ __forceinline__ void rotate8(uint4& lo, uint4& hi, const float* __restrict__ cs, const float* __restrict__ sn) {
+    // lo/hi: 8 bf16 each, element e of lo pairs with element e of hi; cs/sn: their 8 cos/sin
+    uint32_t* pl = reinterpret_cast<uint32_t*>(&lo);
+    uint32_t* ph = reinterpret_cast<uint32_t*>(&hi);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float a0 = bf16lo_to_f32(pl[k]), a1 = bf16hi_to_f32(pl[k]);
+        const float b0 = bf16lo_to_f32(ph[k]), b1 = bf16hi_to_f32(ph[k]);
+        const float c0 = cs[2 * k], c1 = cs[2 * k + 1], s0 = sn[2 * k], s1 = sn[2 * k + 1];
+        pl[k] = pack2(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
+        ph[k] = pack2(a0 * s0 + b0 * c0, a1 * s1 + b1 * c1);
+    }
+}
+
 template <int HS>
 __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
-    constexpr int DC = HS / 32, DT = HS / 16;
+    constexpr int DC = HS / 32, DT = HS / 16, HALF = HS / 2;
     __shared__ float m_s[4][16], l_s[4][16];
     __shared__ float o_s[4][HS][17];                    // [wave][dim][col], padded
+    __shared__ float cos_s[HALF], sin_s[HALF];
+    __shared__ int ticket_s;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
     const int G = a.H / a.Hkv, GT = a.GT;
@@ -247,18 +271,63 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
     const int hg = ht * GT + n;
     const bool ok = n < GT && hg < G && L > 0;
     const int head = kvh * G + hg;
+    const int lo_key = a.window > 0 ? max(0, L - a.window) : 0;
+    const int k_lo = max(lo_key, split * a.chunk), k_hi = min(L, (split + 1) * a.chunk);   // [k_lo, k_hi)
+    const bf16* row = a.q + (size_t)seq * a.q_stride;
+
+    if (a.rotate && L > 0) {
+        for (int i = threadIdx.x; i < HALF; i += 256) {
+            float sv, cv;
+            sincosf((float)(L - 1) * a.inv_freq[i], &sv, &cv);
+            cos_s[i] = cv; sin_s[i] = sv;
+        }
+        __syncthreads();
+    }
+    // the new token's key and value go into the cache before anyone reads them: the workgroup
+    // that owns the new position does it (there is one per kv head: write_kv needs n_head_tiles == 1)
+    if (a.write_kv && L > 0 && L - 1 >= k_lo && L - 1 < k_hi) {
+        const int pos = L - 1;
+        const int page = a.block_table[(size_t)seq * a.bt_stride + pos / BN_PAGE], off = pos % BN_PAGE;
+        bf16* kdst = const_cast<bf16*>(a.k_pages) + (((size_t)page * a.Hkv + kvh) * BN_PAGE + off) * HS;
+        bf16* vdst = const_cast<bf16*>(a.vt_pages) + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + off;
+        const bf16* kraw = row + (size_t)(a.H + kvh) * HS;
+        const bf16* vraw = row + (size_t)(a.H + a.Hkv + kvh) * HS;
+        const int t = threadIdx.x;
+        if (t < HALF) {
+            float k0 = __bfloat162float(kraw[t]), k1 = __bfloat162float(kraw[t + HALF]);
+            if (a.rotate) {
+                const float c = cos_s[t], sv = sin_s[t];
+                const float r0 = k0 * c - k1 * sv, r1 = k0 * sv + k1 * c;
+                k0 = r0; k1 = r1;
+            }
+            kdst[t] = __float2bfloat16(k0);
+            kdst[t + HALF] = __float2bfloat16(k1);
+        } else if (t < HALF + HS) {
+            const int d = t - HALF;
+            vdst[(size_t)d * BN_PAGE] = vraw[d];
+        }
+        __threadfence();
+        __syncthreads();
+    }
 
     bf16x8 q[1][DC];
+    {
+        uint4 z[DC];
 #pragma unroll
-    for (int c = 0; c < DC; ++c) {
-        uint4 z = make_uint4(0, 0, 0, 0);
-        if (ok) z = *reinterpret_cast<const uint4*>(a.q + (size_t)seq * a.q_stride + (size_t)head * HS + c * 32 + g * 8);
-        q[0][c] = __builtin_bit_cast(bf16x8, z);
+        for (int c = 0; c < DC; ++c) {
+            z[c] = make_uint4(0, 0, 0, 0);
+            if (ok) z[c] = *reinterpret_cast<const uint4*>(row + (size_t)head * HS + c * 32 + g * 8);
+        }
+        if (a.rotate && L > 0) {
+#pragma unroll
+            for (int c = 0; c < DC / 2; ++c)      // chunk c holds pair indices c*32 + g*8 .. +7, its partners are in chunk c + DC/2
+                rotate8(z[c], z[c + DC / 2], cos_s + c * 32 + g * 8, sin_s + c * 32 + g * 8);
+        }
+#pragma unroll
+        for (int c = 0; c < DC; ++c) q[0][c] = __builtin_bit_cast(bf16x8, z[c]);
     }
     int qpos[1] = {ok ? L - 1 : -1};
-    int lo_key = a.window > 0 ? max(0, L - a.window) : 0;
     int lo[1] = {lo_key};
-    int k_lo = max(lo_key, split * a.chunk), k_hi = min(L, (split + 1) * a.chunk);   // [k_lo, k_hi)
 
     f32x4 acc[1][DT];
     float m[1] = {-INFINITY}, l[1] = {0.f};
@@ -301,10 +370,50 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
         if (a.n_splits == 1) {
             a.out[(size_t)seq * a.out_stride + (size_t)hd * HS + dim] = __float2bfloat16(den > 0.f ? num / den : 0.f);
         } else {
-            const size_t row = ((size_t)seq * a.H + hd) * a.n_splits + split;
-            a.part_o[row * HS + dim] = num;
-            if (dim == 0) { a.part_ml[row * 2] = (M == -INFINITY) ? -INFINITY : M * LN2; a.part_ml[row * 2 + 1] = den; }
+            const size_t prow = ((size_t)seq * a.H + hd) * a.n_splits + split;
+            a.part_o[prow * HS + dim] = num;
+            if (dim == 0) { a.part_ml[prow * 2] = (M == -INFINITY) ? -INFINITY : M * LN2; a.part_ml[prow * 2 + 1] = den; }
         }
+    }
+    if (a.n_splits == 1 || a.counters == nullptr) return;
+    // the last workgroup of this (sequence, kv head, head tile) to arrive merges all splits, in split order
+    __threadfence();
+    __syncthreads();
+    int* counter = a.counters + ((size_t)seq * gridDim.y + blockIdx.y);
+    if (threadIdx.x == 0) ticket_s = atomicAdd(counter, 1);
+    __syncthreads();
+    if (ticket_s != a.n_splits - 1) return;
+    __threadfence();
+    if (threadIdx.x == 0) *counter = 0;                     // ready for the next launch
+    for (int idx = threadIdx.x; idx < HS * GT; idx += 256) {
+        const int col = idx / HS, dim = idx - col * HS;
+        const int hg2 = ht * GT + col;
+        if (hg2 >= G) continue;
+        const int hd = kvh * G + hg2;
+        const size_t prow = ((size_t)seq * a.H + hd) * a.n_splits;
+        const float* ml = a.part_ml + prow * 2;
+        float M = -INFINITY;
+        for (int sp = 0; sp < a.n_splits; ++sp) M = fmaxf(M, ml[2 * sp]);
+        float num = 0.f, den = 0.f;
+        if (M != -INFINITY) {
+            for (int s0 = 0; s0 < a.n_splits; s0 += 8) {
+                float v[8], wgt[8], ls[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const bool in = s0 + j < a.n_splits;
+                    v[j] = in ? a.part_o[(prow + s0 + j) * HS + dim] : 0.f;
+                    wgt[j] = in ? ml[2 * (s0 + j)] : -INFINITY;
+                    ls[j] = in ? ml[2 * (s0 + j) + 1] : 0.f;
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float e = wgt[j] == -INFINITY ? 0.f : expf(wgt[j] - M);
+                    num = fmaf(e, v[j], num);
+                    den = fmaf(e, ls[j], den);
+                }
+            }
+        }
+        a.out[(size_t)seq * a.out_stride + (size_t)hd * HS + dim] = __float2bfloat16(den > 0.f ? num / den : 0.f);
     }
 }
 
@@ -348,7 +457,7 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
                             const void* vt_pages, const int* block_table, int bt_stride, const int* seq_lens,
                             const int* tiles, int n_tiles, int n_tokens, int H, int Hkv, int hs, int GT,
                             int window, float scale, int n_splits, int chunk, float* part_o, float* part_ml,
-                            hipStream_t s) {
+                            const float* inv_freq, int rotate, int write_kv, int* counters, hipStream_t s) {
     if (!bn_attn_mfma_supports(hs) || n_tiles <= 0 || n_tokens <= 0 || H <= 0 || Hkv <= 0 || H % Hkv) return BN_ERR_ARG;
     if (GT <= 0 || GT > 16 || (GT & (GT - 1)) || window < 0 || n_splits < 1 || n_splits > 64) return BN_ERR_ARG;
     if (n_splits > 1 && (chunk <= 0 || chunk % BN_PAGE || !part_o || !part_ml)) return BN_ERR_ARG;
@@ -356,14 +465,18 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
     if (q_stride % 8 || out_stride % 4 || (((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)vt_pages) & 15) ||
         ((uintptr_t)out & 7))
         return BN_ERR_ARG;
+    const int G = H / Hkv;
+    const int n_head_tiles = (G + GT - 1) / GT;
+    if ((rotate || write_kv) && tiles) return BN_ERR_ARG;                 // decode form only
+    if (rotate && !inv_freq) return BN_ERR_ARG;
+    if (write_kv && (n_head_tiles != 1 || q_stride < (H + 2 * Hkv) * hs)) return BN_ERR_ARG;
     MfmaArgs a;
     a.q = (const bf16*)q; a.out = (bf16*)out; a.k_pages = (const bf16*)k_pages; a.vt_pages = (const bf16*)vt_pages;
     a.block_table = block_table; a.seq_lens = seq_lens; a.tiles = tiles; a.part_o = part_o; a.part_ml = part_ml;
     a.q_stride = q_stride; a.out_stride = out_stride; a.bt_stride = bt_stride;
     a.H = H; a.Hkv = Hkv; a.GT = GT; a.window = window; a.scale = scale;
     a.n_splits = n_splits; a.chunk = n_splits > 1 ? chunk : 0x40000000;
-    const int G = H / Hkv;
-    const int n_head_tiles = (G + GT - 1) / GT;
+    a.inv_freq = inv_freq; a.rotate = rotate; a.write_kv = write_kv; a.counters = counters;
     if (tiles) {
         const dim3 grid(n_tiles, Hkv * n_head_tiles);
         if (hs == 64) hipLaunchKernelGGL((attn_mfma_prompt_kernel<64, 4>), grid, dim3(256), 0, s, a);
@@ -374,7 +487,7 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
     if (hs == 64) hipLaunchKernelGGL(attn_mfma_decode_kernel<64>, grid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL(attn_mfma_decode_kernel<128>, grid, dim3(256), 0, s, a);
     int rc = bn_launch_status();
-    if (rc != 0 || n_splits == 1) return rc;
+    if (rc != 0 || n_splits == 1 || counters != nullptr) return rc;
     hipLaunchKernelGGL(attn_mfma_combine_kernel, dim3(n_tokens * H), dim3(64), 0, s, (bf16*)out, out_stride, part_o,
                        part_ml, H, hs, n_splits);
     return bn_launch_status();

@@ -52,6 +52,75 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ 
     }
 }
 
+// The same for rows of up to 256*4*NV elements (a multiple of 4): every load of the row is
+// issued before anything waits, the row stays in registers, one block reduction, one store.
+// Each thread's partial sum runs over its elements in index order; the tree is the same as above.
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void add_rmsnorm_row_kernel(float* __restrict__ x, const T* __restrict__ delta,
+                                                              const float* __restrict__ w, T* __restrict__ out,
+                                                              const int* __restrict__ rows, int dim, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int src = rows ? rows[r] : r;
+    float* xr = x + (size_t)src * dim;
+    const T* dr = delta ? delta + (size_t)src * dim : nullptr;
+    const bool write_back = (dr != nullptr) && (rows == nullptr);
+    float4 v[NV], wv[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int i = (k * 256 + threadIdx.x) * 4;
+        v[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+        wv[k] = v[k];
+        if (i < dim) {
+            v[k] = *reinterpret_cast<const float4*>(xr + i);
+            wv[k] = *reinterpret_cast<const float4*>(w + i);
+        }
+    }
+    if (dr) {
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int i = (k * 256 + threadIdx.x) * 4;
+            if (i < dim) {
+                float d[4];
+                if (sizeof(T) == 2) {
+                    const uint2 t = *reinterpret_cast<const uint2*>(dr + i);
+                    d[0] = bf16lo_to_f32(t.x); d[1] = bf16hi_to_f32(t.x); d[2] = bf16lo_to_f32(t.y); d[3] = bf16hi_to_f32(t.y);
+                } else {
+                    const float4 t = *reinterpret_cast<const float4*>(dr + i);
+                    d[0] = t.x; d[1] = t.y; d[2] = t.z; d[3] = t.w;
+                }
+                v[k].x += d[0]; v[k].y += d[1]; v[k].z += d[2]; v[k].w += d[3];
+            }
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int i = (k * 256 + threadIdx.x) * 4;
+        if (i < dim) {
+            if (write_back) *reinterpret_cast<float4*>(xr + i) = v[k];
+            ss += v[k].x * v[k].x; ss += v[k].y * v[k].y; ss += v[k].z * v[k].z; ss += v[k].w * v[k].w;
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)dim + eps);
+    T* o = out + (size_t)r * dim;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int i = (k * 256 + threadIdx.x) * 4;
+        if (i < dim) {
+            const float a = v[k].x * scale * wv[k].x, b = v[k].y * scale * wv[k].y;
+            const float c = v[k].z * scale * wv[k].z, d = v[k].w * scale * wv[k].w;
+            if (sizeof(T) == 2) {
+                bf16 t[4] = {from_f32<bf16>(a), from_f32<bf16>(b), from_f32<bf16>(c), from_f32<bf16>(d)};
+                *reinterpret_cast<uint2*>(o + i) = *reinterpret_cast<const uint2*>(t);
+            } else {
+                *reinterpret_cast<float4*>(o + i) = make_float4(a, b, c, d);
+            }
+        }
+    }
+}
+
 // x[t, :] += delta[t, :]   (src/transformer/cpu_backend.c:252-256)
 template <typename T>
 __global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__ delta, size_t n) {
@@ -70,6 +139,28 @@ __global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gu, int
     float g = to_f32(gu[t * 2 * F + f]);
     float u = to_f32(gu[t * 2 * F + F + f]);
     out[i] = from_f32<T>((g / (1.0f + expf(-g))) * u);
+}
+
+// the same, 8 bf16 values a thread (F a multiple of 8, 16-byte aligned rows)
+__global__ void swiglu_bf16x8_kernel(bf16* __restrict__ out, const bf16* __restrict__ gu, int F, size_t n8) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n8) return;
+    const int f8 = F / 8;
+    const size_t t = i / f8;
+    const int f = (int)(i - t * f8) * 8;
+    const uint4 g = *reinterpret_cast<const uint4*>(gu + t * 2 * F + f);
+    const uint4 u = *reinterpret_cast<const uint4*>(gu + t * 2 * F + F + f);
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float g0 = bf16lo_to_f32(gw[k]), g1 = bf16hi_to_f32(gw[k]);
+        const float r0 = (g0 / (1.0f + expf(-g0))) * bf16lo_to_f32(uw[k]);
+        const float r1 = (g1 / (1.0f + expf(-g1))) * bf16hi_to_f32(uw[k]);
+        const bf16 b0 = __float2bfloat16(r0), b1 = __float2bfloat16(r1);
+        ow[k] = (uint32_t)(*reinterpret_cast<const uint16_t*>(&b0)) | ((uint32_t)(*reinterpret_cast<const uint16_t*>(&b1)) << 16);
+    }
+    *reinterpret_cast<uint4*>(out + t * F + f) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
 }
 
 // y[t, n] += b[n]   (src/gpu_cuda.cu:5161-5166)
@@ -95,18 +186,33 @@ extern "C" int bn_embed_gather(int dtype, void* x, const void* table, const int*
     return BN_ERR_DTYPE;
 }
 
+template <typename T>
+static void launch_add_rmsnorm(float* x, const void* delta, const float* w, void* out, const int* rows, int n_rows,
+                               int dim, float eps, hipStream_t s) {
+    const bool aligned = dim % 4 == 0 && !(((uintptr_t)x | (uintptr_t)w | (uintptr_t)out | (uintptr_t)delta) & 15);
+    const int nv = (dim + 1023) / 1024;
+    if (aligned && nv <= 8) {
+#define ROW_CASE(NV) hipLaunchKernelGGL((add_rmsnorm_row_kernel<T, NV>), dim3(n_rows), dim3(256), 0, s, x, (const T*)delta, w, (T*)out, rows, dim, eps)
+        switch (nv) {
+            case 1: ROW_CASE(1); break;
+            case 2: ROW_CASE(2); break;
+            case 3: case 4: ROW_CASE(4); break;
+            default: ROW_CASE(8); break;
+        }
+#undef ROW_CASE
+        return;
+    }
+    const int threads = dim >= 2048 ? 512 : 256;
+    hipLaunchKernelGGL(add_rmsnorm_kernel<T>, dim3(n_rows), dim3(threads), 0, s, x, (const T*)delta, w, (T*)out, rows,
+                       dim, eps);
+}
+
 extern "C" int bn_add_rmsnorm(int dtype, void* x, const void* delta, const float* w, void* out,
                               const int* rows, int n_rows, int dim, float eps, hipStream_t s) {
     if (n_rows <= 0 || dim <= 0) return BN_ERR_ARG;
-    const int threads = dim >= 2048 ? 512 : 256;
-    if (dtype == BN_DT_F32)
-        hipLaunchKernelGGL(add_rmsnorm_kernel<float>, dim3(n_rows), dim3(threads), 0, s, (float*)x,
-                           (const float*)delta, w, (float*)out, rows, dim, eps);
-    else if (dtype == BN_DT_BF16)
-        hipLaunchKernelGGL(add_rmsnorm_kernel<bf16>, dim3(n_rows), dim3(threads), 0, s, (float*)x,
-                           (const bf16*)delta, w, (bf16*)out, rows, dim, eps);
-    else
-        return BN_ERR_DTYPE;
+    if (dtype == BN_DT_F32) launch_add_rmsnorm<float>((float*)x, delta, w, out, rows, n_rows, dim, eps, s);
+    else if (dtype == BN_DT_BF16) launch_add_rmsnorm<bf16>((float*)x, delta, w, out, rows, n_rows, dim, eps, s);
+    else return BN_ERR_DTYPE;
     return bn_launch_status();
 }
 
@@ -131,6 +237,9 @@ extern "C" int bn_swiglu(int dtype, void* out, const void* gu, int n_rows, int F
     if (dtype == BN_DT_F32)
         hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, s, (float*)out,
                            (const float*)gu, F, n);
+    else if (dtype == BN_DT_BF16 && F % 8 == 0 && !(((uintptr_t)out | (uintptr_t)gu) & 15))
+        hipLaunchKernelGGL(swiglu_bf16x8_kernel, dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0, s, (bf16*)out,
+                           (const bf16*)gu, F, n / 8);
     else if (dtype == BN_DT_BF16)
         hipLaunchKernelGGL(swiglu_kernel<bf16>, dim3(blocks), dim3(256), 0, s, (bf16*)out,
                            (const bf16*)gu, F, n);

@@ -164,6 +164,7 @@ class Engine:
             limit = min(limit, model.plan.max_positions)
         self.max_seq_len = min(limit, max_seq_len) if max_seq_len else limit
         self.vocab_size = model.plan.vocab_size
+        ops.attention_counters(self.device)          # made before any graph capture
         # a mixer that keeps a state addresses it by the host's slot list, which a replayed graph
         # cannot see: such models run their decode steps eagerly
         self.use_graphs = use_graphs and all(n.state is None for n in needs)

@@ -46,7 +46,7 @@ _SIGNATURES = {
         "bn_attn_mfma_prompt_tokens": [c_int, c_int],
         "bn_attn_mfma": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p,
-                         c_void_p],
+                         c_void_p, c_int, c_int, c_void_p, c_void_p],
     },
     "gemm_tiled": {
         "bn_gemm_tiled": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
@@ -388,10 +388,32 @@ def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int):
     return n_splits, chunk
 
 
+_COUNTERS = {}
+_N_COUNTERS = 65536
+
+
+def attention_counters(device) -> torch.Tensor:
+    """Zeroed int32 counters that the decode attention kernel uses to find the last workgroup of a
+    (sequence, kv head); the kernel leaves them zero.  One buffer per device: attention launches
+    that overlap on one device (two streams) would race on it.  Create it outside a graph capture."""
+    device = torch.device(device)
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    t = _COUNTERS.get(key)
+    if t is None:
+        t = torch.zeros(_N_COUNTERS, dtype=torch.int32, device=device)
+        _COUNTERS[key] = t
+    return t
+
+
+def can_fuse_decode(dtype, H: int, Hkv: int, hs: int) -> bool:
+    """Whether decode attention can rotate Q and K and store the new K, V itself."""
+    return mfma_attention(dtype, hs) and H // Hkv <= 16
+
+
 def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
               block_table: torch.Tensor, H: int, Hkv: int, hs: int, scale: float, *, window: int = 0,
               tiles=None, qt: int = 0, seq_lens=None, n_splits: int = 1, chunk: int = 0,
-              force_vector: bool = False) -> None:
+              force_vector: bool = False, fused_rotate=None, fused_write: bool = False) -> None:
     """Causal attention of the (rotated) Q heads in qkv over the paged cache.
 
     Prompt form: `tiles` [n, 4] int32 = (sequence, first token row, tokens (<= qt), position of
@@ -400,7 +422,10 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     padding row); row b of qkv is sequence b's token; n_splits/chunk from decode_splits.
     bf16 with head size 64 or 128 runs on the matrix cores, everything else on the vector ALUs
     (force_vector: the vector kernel also where the other would run; its qt then is that of
-    attention_row_shape without dtype)."""
+    attention_row_shape without dtype).
+    Decode on the matrix cores can do the work of rope_kv_write itself (can_fuse_decode):
+    fused_rotate = inv_freq [hs/2]: qkv arrives unrotated, Q and the new K are rotated inside;
+    fused_write: the new K, V of every row (from qkv) are stored at position seq_lens - 1 first."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(out, "out", qkv.dtype, 2)
@@ -444,11 +469,27 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     pm = part_ml.data_ptr() if part_ml is not None else None
     sl = seq_lens.data_ptr() if decode else None
     tl = tiles.data_ptr() if not decode else None
+    fused = fused_rotate is not None or fused_write
+    if fused and not (use_mfma and decode and can_fuse_decode(qkv.dtype, H, Hkv, hs)):
+        raise KernelError("attention: rotation / cache write inside the kernel needs the decode form on the "
+                          "matrix cores with at most 16 heads per kv head")
+    if fused_rotate is not None:
+        _dev(fused_rotate, "fused_rotate", torch.float32, 1)
+        if fused_rotate.numel() != hs // 2 or not fused_rotate.is_contiguous():
+            raise KernelError(f"attention: fused rotation needs {hs // 2} frequencies (full rotary)")
+    if fused_write and qkv.shape[1] < (H + 2 * Hkv) * hs:
+        raise KernelError("attention: fused cache write needs the K and V heads in qkv")
     if use_mfma:
+        counters = None
+        if decode and n_splits > 1 and T * Hkv * ((H // Hkv + GT - 1) // GT) <= _N_COUNTERS:
+            counters = attention_counters(qkv.device)
         _check(_fn("attn_mfma", "bn_attn_mfma")(
             qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * hs, k_pages.data_ptr(), v_pages.data_ptr(),
             block_table.data_ptr(), block_table.shape[1], sl, tl, n_tiles, T, H, Hkv, hs, GT, int(window),
-            float(scale), int(n_splits), int(chunk), po, pm, _stream()), "attention(mfma)")
+            float(scale), int(n_splits), int(chunk), po, pm,
+            fused_rotate.data_ptr() if fused_rotate is not None else None, int(fused_rotate is not None),
+            int(bool(fused_write)), counters.data_ptr() if counters is not None else None, _stream()),
+            "attention(mfma)")
         return
     _check(_fn("attn_rows", "bn_attn_rows")(
         _code(qkv.dtype), qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * hs,

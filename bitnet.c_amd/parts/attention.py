@@ -71,8 +71,19 @@ class Attention(Part):
             pad = torch.empty((h.shape[0], (H + 2 * Hkv) * hs), dtype=h.dtype, device=h.device)
             pad[:, :self.q_dim] = qkv
             qkv = pad
-        self.position.encode_and_store(qkv, ctx, H, Hkv, hs, kv)
         out = torch.empty((h.shape[0], self.q_dim), dtype=h.dtype, device=h.device)
+        fuse_ok, inv_freq = self.position.fusable(hs)
+        if ctx.is_decode and fuse_ok and ops.can_fuse_decode(h.dtype, H, Hkv, hs):
+            # one kernel: rotation of Q and the new K, the cache write, attention, merge of the splits
+            if self.window:
+                n_splits, chunk = 1, 0
+            else:
+                n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len)
+            ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
+                          window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
+                          fused_rotate=inv_freq, fused_write=kv.writes)
+            return self.o(out)
+        self.position.encode_and_store(qkv, ctx, H, Hkv, hs, kv)
         if ctx.is_decode:
             if self.window:                   # a window is short; its keys are not split
                 n_splits, chunk = 1, 0

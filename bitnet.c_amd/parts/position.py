@@ -47,6 +47,13 @@ class PositionEncoding(Part):
     def prepare(self, device) -> None:
         pass
 
+    def fusable(self, hs: int):
+        """(ok, inv_freq or None): whether a decode attention kernel may do this encoding and the
+        cache write itself: a rotation of the whole head with these frequencies, or none."""
+        if self.rope_dims == 0:
+            return True, None
+        return self.rope_dims == hs, self.inv_freq
+
     def encode_and_store(self, qkv, ctx, H, Hkv, hs, kv) -> None:
         ops.rope_kv_write(qkv, ctx.positions, H, Hkv, hs, inv_freq=self.inv_freq, rope_dims=self.rope_dims,
                           seq_index=ctx.seq_index if kv.writes else None,

@@ -51,7 +51,7 @@ def test_embed_gather(dtype, dim, vocab):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("dim", [24, 100, 4096, 5123])
+@pytest.mark.parametrize("dim", [24, 100, 4096, 5123, 8192, 9000])
 def test_add_rmsnorm(dtype, dim):
     ops = _ops()
     T, eps = 5, 1e-3
@@ -87,11 +87,12 @@ def test_rmsnorm_eps_inside_root_on_device():
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_swiglu_bias_residual(dtype):
     ops = _ops()
-    T, F = 7, 173
-    gu = _rand((T, 2 * F), dtype, 5, 2.0)
-    out = ops.swiglu(gu.cuda())
-    want = pl.swiglu(gu[:, :F].float(), gu[:, F:].float())
-    assert close(out.float(), want, dtype)
+    for T, F in ((7, 173), (5, 176), (300, 1024)):
+        gu = _rand((T, 2 * F), dtype, 5, 2.0)
+        out = ops.swiglu(gu.cuda())
+        want = pl.swiglu(gu[:, :F].float(), gu[:, F:].float())
+        assert close(out.float(), want, dtype), (T, F)
+    T = 7
     # the reference's own vector (test/test_transformer.c:645-677)
     g = torch.tensor([-2.0, -1.0, -0.25, 0.0, 0.25, 1.0, 2.0, 4.0])
     u = torch.tensor([1.0, 0.5, 2.0, 3.0, -1.0, 1.5, -0.5, 2.0])
@@ -413,3 +414,52 @@ def test_repeat_penalty_on_device():
     want = torch.tensor([[2.0, 2.1 / 1.5, 2.0, 2.0], [1.0, -1.5, 0.5, 2.0]])
     assert torch.allclose(lg.cpu(), want, atol=1e-6)
     assert ops.argmax(lg).cpu().tolist()[0] != 1           # test/test_safety.c:229-238
+
+
+@pytest.mark.parametrize("H,Hkv,hs,window", [(32, 8, 128, 0), (8, 2, 64, 0), (16, 1, 128, 0), (6, 6, 64, 90), (4, 4, 128, 0)])
+@pytest.mark.parametrize("force_splits", [1, 0, 7])
+def test_decode_attention_that_rotates_and_stores_itself(H, Hkv, hs, window, force_splits):
+    """The decode kernel doing rope_kv_write's work: unrotated qkv in, the new key and value stored,
+    against rope_kv_write followed by the same attention; run twice in a row, since it leaves its
+    counters behind for the next launch."""
+    ops = _ops()
+    dtype = torch.bfloat16
+    lens_before = [0, 63, 64, 700, 129, 300, 31]
+    B = len(lens_before)
+    seqs_k = [_rand((p + 1, Hkv, hs), dtype, 700 + i) for i, p in enumerate(lens_before)]
+    seqs_v = [_rand((p + 1, Hkv, hs), dtype, 800 + i) for i, p in enumerate(lens_before)]
+    kp, vp, bt = _paged(seqs_k, seqs_v, dtype, sum((p + 64) // 64 for p in lens_before) + 2, 7)
+    inv_freq = pl.rope_inv_freq(hs, 10000.0)
+    qkv = _rand((B + 1, (H + 2 * Hkv) * hs), dtype, 900)
+    lens = torch.tensor([p + 1 for p in lens_before] + [0], dtype=torch.int32)
+    pos = lens - 1
+    bt = torch.cat([bt, torch.zeros((1, bt.shape[1]), dtype=torch.int32)])
+    max_len = bt.shape[1] * 64
+    if window or force_splits == 1:
+        n_splits, chunk = 1, 0
+    elif force_splits == 0:
+        n_splits, chunk = ops.decode_splits(B + 1, H, Hkv, max_len)
+    else:
+        chunk = ((max_len + force_splits - 1) // force_splits + 63) // 64 * 64
+        n_splits = (max_len + chunk - 1) // chunk
+    scale = hs ** -0.5
+    # reference: the two kernels one after the other
+    q1, k1, v1 = qkv.clone().cuda(), kp.clone().cuda(), vp.clone().cuda()
+    ops.rope_kv_write(q1, pos.cuda(), H, Hkv, hs, inv_freq=inv_freq.cuda(), rope_dims=hs,
+                      seq_index=torch.arange(B + 1, dtype=torch.int32).cuda(), block_table=bt.cuda(), k_pages=k1, v_pages=v1)
+    want = torch.empty((B + 1, H * hs), dtype=dtype).cuda()
+    ops.attention(q1, want, k1, v1, bt.cuda(), H, Hkv, hs, scale, window=window, seq_lens=lens.cuda(),
+                  n_splits=n_splits, chunk=chunk)
+    for _ in range(2):
+        q2, k2, v2 = qkv.clone().cuda(), kp.clone().cuda(), vp.clone().cuda()
+        got = torch.full((B + 1, H * hs), float("nan"), dtype=dtype).cuda()
+        ops.attention(q2, got, k2, v2, bt.cuda(), H, Hkv, hs, scale, window=window, seq_lens=lens.cuda(),
+                      n_splits=n_splits, chunk=chunk, fused_rotate=inv_freq.cuda(), fused_write=True)
+        torch.cuda.synchronize()
+        assert torch.equal(q2.cpu(), qkv)                            # the input stays unrotated
+        # the stored key and value are the ones rope_kv_write stores (NaN marks untouched places in both)
+        assert torch.equal(torch.nan_to_num(k2.float(), nan=-7.0).cpu(), torch.nan_to_num(k1.float(), nan=-7.0).cpu())
+        assert torch.equal(torch.nan_to_num(v2.float(), nan=-7.0).cpu(), torch.nan_to_num(v1.float(), nan=-7.0).cpu())
+        assert mfma_close(got[:B].float(), want[:B].float())
+        assert float(got[B:].float().abs().sum()) == 0.0
+        assert int(ops.attention_counters("cuda:0").abs().sum()) == 0
