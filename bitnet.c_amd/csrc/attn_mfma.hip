@@ -306,7 +306,8 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
             const int d = t - HALF;
             vdst[(size_t)d * BN_PAGE] = vraw[d];
         }
-        __threadfence();
+        // only this workgroup reads what it has just stored: a fence of workgroup scope is enough
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
         __syncthreads();
     }
 

@@ -390,6 +390,10 @@ def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int):
 
 _COUNTERS = {}
 _N_COUNTERS = 65536
+# Merging the splits inside the decode kernel (the last workgroup to arrive does it) saves a launch
+# but needs fences of device scope in every workgroup, which on this chip write back and
+# invalidate a whole L2 each; measured slower than the separate combine launch, so it is off.
+MERGE_SPLITS_IN_KERNEL = False
 
 
 def attention_counters(device) -> torch.Tensor:
@@ -481,7 +485,8 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
         raise KernelError("attention: fused cache write needs the K and V heads in qkv")
     if use_mfma:
         counters = None
-        if decode and n_splits > 1 and T * Hkv * ((H // Hkv + GT - 1) // GT) <= _N_COUNTERS:
+        if (MERGE_SPLITS_IN_KERNEL and decode and n_splits > 1
+                and T * Hkv * ((H // Hkv + GT - 1) // GT) <= _N_COUNTERS):
             counters = attention_counters(qkv.device)
         _check(_fn("attn_mfma", "bn_attn_mfma")(
             qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * hs, k_pages.data_ptr(), v_pages.data_ptr(),

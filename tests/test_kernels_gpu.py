@@ -418,11 +418,13 @@ def test_repeat_penalty_on_device():
 
 @pytest.mark.parametrize("H,Hkv,hs,window", [(32, 8, 128, 0), (8, 2, 64, 0), (16, 1, 128, 0), (6, 6, 64, 90), (4, 4, 128, 0)])
 @pytest.mark.parametrize("force_splits", [1, 0, 7])
-def test_decode_attention_that_rotates_and_stores_itself(H, Hkv, hs, window, force_splits):
+@pytest.mark.parametrize("merge_in_kernel", [False, True])
+def test_decode_attention_that_rotates_and_stores_itself(H, Hkv, hs, window, force_splits, merge_in_kernel, monkeypatch):
     """The decode kernel doing rope_kv_write's work: unrotated qkv in, the new key and value stored,
     against rope_kv_write followed by the same attention; run twice in a row, since it leaves its
     counters behind for the next launch."""
     ops = _ops()
+    monkeypatch.setattr(ops, "MERGE_SPLITS_IN_KERNEL", merge_in_kernel)
     dtype = torch.bfloat16
     lens_before = [0, 63, 64, 700, 129, 300, 31]
     B = len(lens_before)
