@@ -130,26 +130,28 @@ __global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__
 
 // out[t, f] = silu(gu[t, f]) * gu[t, F + f], silu(g) = g / (1 + exp(-g))
 // (src/transformer/cpu_backend.c:385-391, exact exponential)
+// il8: gate and up interleaved in blocks of 8 columns (gate f at 16*(f/8) + f%8, up 8 further)
 template <typename T>
-__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gu, int F, size_t n) {
+__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gu, int F, size_t n, int il8) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     size_t t = i / F;
     int f = (int)(i - t * F);
-    float g = to_f32(gu[t * 2 * F + f]);
-    float u = to_f32(gu[t * 2 * F + F + f]);
+    const size_t gi = il8 ? t * 2 * F + 16 * (f / 8) + (f % 8) : t * 2 * F + f;
+    float g = to_f32(gu[gi]);
+    float u = to_f32(gu[il8 ? gi + 8 : gi + F]);
     out[i] = from_f32<T>((g / (1.0f + expf(-g))) * u);
 }
 
 // the same, 8 bf16 values a thread (F a multiple of 8, 16-byte aligned rows)
-__global__ void swiglu_bf16x8_kernel(bf16* __restrict__ out, const bf16* __restrict__ gu, int F, size_t n8) {
+__global__ void swiglu_bf16x8_kernel(bf16* __restrict__ out, const bf16* __restrict__ gu, int F, size_t n8, int il8) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n8) return;
     const int f8 = F / 8;
     const size_t t = i / f8;
     const int f = (int)(i - t * f8) * 8;
-    const uint4 g = *reinterpret_cast<const uint4*>(gu + t * 2 * F + f);
-    const uint4 u = *reinterpret_cast<const uint4*>(gu + t * 2 * F + F + f);
+    const uint4 g = *reinterpret_cast<const uint4*>(gu + t * 2 * F + (il8 ? 2 * f : f));
+    const uint4 u = *reinterpret_cast<const uint4*>(gu + t * 2 * F + (il8 ? 2 * f + 8 : F + f));
     const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
     uint32_t ow[4];
 #pragma unroll
@@ -230,19 +232,19 @@ extern "C" int bn_residual_add(int dtype, void* x, const void* delta, long long 
     return bn_launch_status();
 }
 
-extern "C" int bn_swiglu(int dtype, void* out, const void* gu, int n_rows, int F, hipStream_t s) {
-    if (n_rows <= 0 || F <= 0) return BN_ERR_ARG;
+extern "C" int bn_swiglu(int dtype, void* out, const void* gu, int n_rows, int F, int il8, hipStream_t s) {
+    if (n_rows <= 0 || F <= 0 || (il8 && F % 8)) return BN_ERR_ARG;
     const size_t n = (size_t)n_rows * F;
     const unsigned blocks = (unsigned)((n + 255) / 256);
     if (dtype == BN_DT_F32)
         hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, s, (float*)out,
-                           (const float*)gu, F, n);
+                           (const float*)gu, F, n, il8);
     else if (dtype == BN_DT_BF16 && F % 8 == 0 && !(((uintptr_t)out | (uintptr_t)gu) & 15))
         hipLaunchKernelGGL(swiglu_bf16x8_kernel, dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0, s, (bf16*)out,
-                           (const bf16*)gu, F, n / 8);
+                           (const bf16*)gu, F, n / 8, il8);
     else if (dtype == BN_DT_BF16)
         hipLaunchKernelGGL(swiglu_kernel<bf16>, dim3(blocks), dim3(256), 0, s, (bf16*)out,
-                           (const bf16*)gu, F, n);
+                           (const bf16*)gu, F, n, il8);
     else
         return BN_ERR_DTYPE;
     return bn_launch_status();

@@ -10,6 +10,9 @@
 //
 // DUAL: W holds two row blocks (gate rows n, up rows up_off + n); the epilogue writes
 // silu(gate) * up, silu(g) = g / (1 + exp(-g)) (src/transformer/cpu_backend.c:385-391).
+// GLU8: the same product with gate and up rows interleaved in blocks of 8 (rows 16t..16t+7 are
+// gate rows 8t..8t+7, rows 16t+8..16t+15 the up rows of the same columns): every 16-row tile holds
+// both halves of 8 result columns, so the plain kernel does it with half the loads in flight.
 //
 // Needs K % 8 == 0 and 16-byte aligned rows; other shapes go to the tiled kernel.
 #include "common.h"
@@ -21,7 +24,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
 
-template <int MT, bool DUAL, typename TO>
+template <int MT, bool DUAL, typename TO, bool GLU8 = false>
 __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                            TO* __restrict__ Y, int M, int N, int K, int ldx,
                                                            int ldw, int ldy, int up_off) {
@@ -83,21 +86,38 @@ __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_ke
         }
         const int m = mt * 16 + 4 * (l >> 4) + r;
         const int nn = n0 + (l & 15);
-        if (m < M && nn < N) {
+        if (GLU8) {
+            // columns 0..7 of the tile are gates, 8..15 the ups of the same result columns
+            const float up = __shfl_xor(v, 8, BN_WAVE);
+            if ((l & 8) == 0 && m < M && nn < N)
+                Y[(size_t)m * ldy + (n0 >> 1) + (l & 7)] = from_f32<TO>((v / (1.0f + expf(-v))) * up);
+        } else if (m < M && nn < N) {
             const float y = DUAL ? (v / (1.0f + expf(-v))) * u : v;
             Y[(size_t)m * ldy + nn] = from_f32<TO>(y);
         }
     }
 }
 
-template <int MT, bool DUAL, typename TO>
+template <int MT, bool DUAL, typename TO, bool GLU8 = false>
 static int launch(const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw, int ldy,
                   int up_off, int n_waves, hipStream_t s) {
     constexpr int NA = DUAL ? 2 * MT : MT;
     const size_t smem = (size_t)n_waves * NA * 64 * 4 * sizeof(float);
-    hipLaunchKernelGGL((skinny_gemm_kernel<MT, DUAL, TO>), dim3((N + 15) / 16), dim3(n_waves * 64), smem, s,
+    hipLaunchKernelGGL((skinny_gemm_kernel<MT, DUAL, TO, GLU8>), dim3((N + 15) / 16), dim3(n_waves * 64), smem, s,
                        (const bf16*)X, (const bf16*)W, (TO*)Y, M, N, K, ldx, ldw, ldy, up_off);
     return bn_launch_status();
+}
+
+template <typename TO>
+static int launch_glu8(int MT, const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw,
+                       int ldy, int n_waves, hipStream_t s) {
+    switch (MT) {
+        case 1: return launch<1, false, TO, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, n_waves, s);
+        case 2: return launch<2, false, TO, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, n_waves, s);
+        case 3: return launch<3, false, TO, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, n_waves, s);
+        case 4: return launch<4, false, TO, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, n_waves, s);
+    }
+    return BN_ERR_ARG;
 }
 
 template <bool DUAL, typename TO>
@@ -121,14 +141,19 @@ extern "C" int bn_skinny_gemm_supports(int M, int N, int K, int ldx, int ldw) {
     return (M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0) ? 1 : 0;
 }
 
-// out_dtype: type of Y (bf16 or float32).  dual != 0: N is the width of the result and W has
-// the gate rows at [0, N) and the up rows at [up_off, up_off + N).
+// out_dtype: type of Y (bf16 or float32).  dual == 1: N is the width of the result and W has
+// the gate rows at [0, N) and the up rows at [up_off, up_off + N).  dual == 2: W has 2N rows, gate
+// and up interleaved in blocks of 8 (N a multiple of 8); the result has N columns.
 extern "C" int bn_skinny_gemm(int out_dtype, const void* X, const void* W, void* Y, int M, int N, int K,
                               int ldx, int ldw, int ldy, int dual, int up_off, hipStream_t s) {
     if (!bn_skinny_gemm_supports(M, N, K, ldx, ldw) || ldy < N) return BN_ERR_ARG;
     if (((uintptr_t)X | (uintptr_t)W) & 15) return BN_ERR_ARG;
+    if (dual == 2) {
+        if (N % 8) return BN_ERR_ARG;
+        N *= 2;                                   // rows of W; the kernel halves the column index itself
+    }
     const int MT = (M + 15) / 16;
-    const int NA = dual ? 2 * MT : MT;
+    const int NA = dual == 1 ? 2 * MT : MT;
     // waves per workgroup: enough loads in flight when there are few column tiles, bounded by
     // the K chunks there are and by 48 KB of shared memory for the partial sums
     const int tiles = (N + 15) / 16;
@@ -137,7 +162,12 @@ extern "C" int bn_skinny_gemm(int out_dtype, const void* X, const void* W, void*
     const int k_chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
     while (n_waves > 1 && n_waves / 2 >= k_chunks) n_waves >>= 1;
     while (n_waves > 1 && n_waves * NA > 48) n_waves >>= 1;
-    if (dual && MT >= 3 && n_waves > 8) n_waves = 8;      // that variant is built for 512 threads
+    if (dual == 1 && MT >= 3 && n_waves > 8) n_waves = 8;      // that variant is built for 512 threads
+    if (dual == 2) {
+        if (out_dtype == BN_DT_BF16) return launch_glu8<bf16>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, n_waves, s);
+        if (out_dtype == BN_DT_F32) return launch_glu8<float>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, n_waves, s);
+        return BN_ERR_DTYPE;
+    }
     if (out_dtype == BN_DT_BF16)
         return dual ? launch_mt<true, bf16>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s)
                     : launch_mt<false, bf16>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s);

@@ -28,7 +28,7 @@ _SIGNATURES = {
         "bn_embed_gather": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "bn_add_rmsnorm": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p],
         "bn_residual_add": [c_int, c_void_p, c_void_p, c_longlong, c_void_p],
-        "bn_swiglu": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+        "bn_swiglu": [c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "bn_bias_add": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
     },
     "rope_kv": {
@@ -180,16 +180,19 @@ def residual_add(x: torch.Tensor, delta: torch.Tensor) -> None:
                                                  x.numel(), _stream()), "residual_add")
 
 
-def swiglu(gu: torch.Tensor) -> torch.Tensor:
-    """[T, 2F] (gate | up) -> silu(gate) * up, [T, F]."""
+def swiglu(gu: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
+    """[T, 2F] (gate | up) -> silu(gate) * up, [T, F].  interleaved: gate and up columns
+    alternate in blocks of 8 (see interleave_gate_up)."""
     require_gpu()
     _dev(gu, "gu", dims=2)
     if not gu.is_contiguous() or gu.shape[1] % 2:
         raise KernelError(f"swiglu: expected a contiguous [T, 2F] tensor, got {tuple(gu.shape)}")
     T, F = gu.shape[0], gu.shape[1] // 2
     out = torch.empty((T, F), dtype=gu.dtype, device=gu.device)
-    _check(_fn("elementwise", "bn_swiglu")(_code(gu.dtype), out.data_ptr(), gu.data_ptr(), T, F, _stream()),
-           "swiglu")
+    if interleaved and F % 8:
+        raise KernelError("swiglu: the interleaved layout needs F to be a multiple of 8")
+    _check(_fn("elementwise", "bn_swiglu")(_code(gu.dtype), out.data_ptr(), gu.data_ptr(), T, F, int(interleaved),
+                                           _stream()), "swiglu")
     return out
 
 
@@ -266,9 +269,20 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, *, allow_library: b
     return _tiled(x, w, out_dtype)
 
 
-def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
-    """silu(x.Wg^T) * (x.Wu^T) for w_gate_up = [Wg; Wu] ([2F, K]).  The decode-sized bf16
-    case is one kernel; every other case is the product followed by the SwiGLU kernel."""
+def interleave_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor) -> torch.Tensor:
+    """[2F, K] with gate and up rows alternating in blocks of 8 (F a multiple of 8): rows
+    16t..16t+7 are gate rows 8t..8t+7, rows 16t+8..16t+15 the up rows of the same columns.  A
+    16-row tile of the decode kernel then holds both halves of 8 result columns."""
+    F, K = w_gate.shape
+    if F % 8 or w_up.shape != w_gate.shape:
+        raise KernelError("interleave_gate_up: F must be a multiple of 8 and the shapes equal")
+    return torch.stack([w_gate.reshape(F // 8, 8, K), w_up.reshape(F // 8, 8, K)], dim=1).reshape(2 * F, K).contiguous()
+
+
+def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
+    """silu(x.Wg^T) * (x.Wu^T) for w_gate_up = [Wg; Wu] ([2F, K]), or the two interleaved in
+    blocks of 8 rows (interleave_gate_up).  The decode-sized bf16 case is one kernel; every other
+    case is the product followed by the SwiGLU kernel."""
     require_gpu()
     _dev(x, "x", dims=2)
     _dev(w_gate_up, "w_gate_up", x.dtype, 2)
@@ -276,6 +290,8 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     if w_gate_up.shape[0] % 2 or w_gate_up.shape[1] != K:
         raise KernelError(f"linear_swiglu: x {tuple(x.shape)} and w {tuple(w_gate_up.shape)} do not agree")
     F = w_gate_up.shape[0] // 2
+    if interleaved and F % 8:
+        raise KernelError("linear_swiglu: the interleaved layout needs F to be a multiple of 8")
     if M == 0:
         return torch.empty((0, F), dtype=x.dtype, device=x.device)
     ldx, ldw = _rows(x, "x"), _rows(w_gate_up, "w_gate_up")
@@ -283,10 +299,10 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
             and skinny_supported(M, F, K, ldx, ldw)):
         y = torch.empty((M, F), dtype=x.dtype, device=x.device)
         _check(_fn("skinny_gemm", "bn_skinny_gemm")(_code(x.dtype), x.data_ptr(), w_gate_up.data_ptr(),
-                                                    y.data_ptr(), M, F, K, ldx, ldw, F, 1, F, _stream()),
-               "skinny_gemm(dual)")
+                                                    y.data_ptr(), M, F, K, ldx, ldw, F, 2 if interleaved else 1, F,
+                                                    _stream()), "skinny_gemm(glu)")
         return y
-    return swiglu(linear(x, w_gate_up))
+    return swiglu(linear(x, w_gate_up), interleaved)
 
 
 # --------------------------------------------------------------------------------------

@@ -1,8 +1,9 @@
 """Dense gated feed-forward: down(silu(gate(x)) * up(x)), silu(g) = g / (1 + exp(-g))
 (src/transformer/cpu.c:1270-1303, src/transformer/cpu_backend.c:385-391).  Gate and up
-are stored stacked ([Wg; Wu], as the reference's GPU upload stacks them,
-include/backend_model.h:22) so that one product computes both; at decode sizes the
-activation is part of that kernel."""
+are stored stacked (as the reference's GPU upload stacks them, include/backend_model.h:22)
+so that one product computes both, with gate and up rows alternating in blocks of 8 when the
+width allows it, so that the decode kernel finds both halves of a result column in one tile;
+at decode sizes the activation is part of that kernel."""
 from __future__ import annotations
 
 import torch
@@ -27,14 +28,22 @@ class SwiGLU(Part):
         return t
 
     def load(self, tensors, device, dtype):
-        w = torch.cat([tensors["w_gate"].to(dtype), tensors["w_up"].to(dtype)], dim=0)
-        b = torch.cat([tensors["b_gate"].float(), tensors["b_up"].float()]) if self.has_bias else None
+        self.interleaved = self.F % 8 == 0
+        if self.interleaved:
+            w = ops.interleave_gate_up(tensors["w_gate"].to(dtype), tensors["w_up"].to(dtype))
+        else:
+            w = torch.cat([tensors["w_gate"].to(dtype), tensors["w_up"].to(dtype)], dim=0)
+        b = None
+        if self.has_bias:
+            bg, bu = tensors["b_gate"].float(), tensors["b_up"].float()
+            b = (torch.stack([bg.reshape(-1, 8), bu.reshape(-1, 8)], dim=1).reshape(-1) if self.interleaved
+                 else torch.cat([bg, bu]))
         self.gate_up.load(w, b, device, dtype)
         self.down.load(tensors["w_down"], tensors.get("b_down") if self.has_bias else None, device, dtype)
 
     def forward(self, h, ctx):
         if self.has_bias:
-            act = ops.swiglu(self.gate_up(h))
+            act = ops.swiglu(self.gate_up(h), self.interleaved)
         else:
-            act = ops.linear_swiglu(h, self.gate_up.weight)
+            act = ops.linear_swiglu(h, self.gate_up.weight, self.interleaved)
         return self.down(act)

@@ -92,6 +92,9 @@ def test_swiglu_bias_residual(dtype):
         out = ops.swiglu(gu.cuda())
         want = pl.swiglu(gu[:, :F].float(), gu[:, F:].float())
         assert close(out.float(), want, dtype), (T, F)
+        if F % 8 == 0:
+            gi = torch.stack([gu[:, :F].reshape(T, F // 8, 8), gu[:, F:].reshape(T, F // 8, 8)], dim=2).reshape(T, 2 * F)
+            assert torch.equal(ops.swiglu(gi.contiguous().cuda(), True).cpu(), out.cpu()), (T, F)
     T = 7
     # the reference's own vector (test/test_transformer.c:645-677)
     g = torch.tensor([-2.0, -1.0, -0.25, 0.0, 0.25, 1.0, 2.0, 4.0])
@@ -133,14 +136,24 @@ def test_skinny_gemm_bf16(M, N, K):
     assert y16.dtype == torch.bfloat16 and close(y16.float(), ref.float(), torch.bfloat16)
 
 
-@pytest.mark.parametrize("M,F,K", [(1, 24, 64), (8, 172, 64), (20, 100, 264), (64, 1000, 512), (40, 14336, 256)])
+@pytest.mark.parametrize("M,F,K", [(1, 24, 64), (8, 172, 64), (20, 100, 264), (64, 1000, 512), (40, 14336, 256), (33, 8, 8), (17, 328, 120)])
 def test_skinny_gemm_dual_swiglu(M, F, K):
     ops = _ops()
     x, w = _rand((M, K), torch.bfloat16, 13), _rand((2 * F, K), torch.bfloat16, 14, 0.1)
     y = ops.linear_swiglu(x.cuda(), w.cuda())
     g = x.double() @ w[:F].double().t()
     u = x.double() @ w[F:].double().t()
-    assert close(y.float(), ((g / (1 + torch.exp(-g))) * u).float(), torch.bfloat16)
+    want = ((g / (1 + torch.exp(-g))) * u).float()
+    assert close(y.float(), want, torch.bfloat16)
+    if F % 8 == 0:          # gate and up rows interleaved in blocks of 8
+        wi = ops.interleave_gate_up(w[:F].cuda(), w[F:].cuda())
+        assert torch.equal(wi[:8].cpu(), w[:8]) and torch.equal(wi[8:16].cpu(), w[F:F + 8])
+        assert close(ops.linear_swiglu(x.cuda(), wi, True).float(), want, torch.bfloat16)
+        xl = _rand((100, K), torch.bfloat16, 15)                    # more than 64 rows: product, then the kernel
+        yl = ops.linear(xl.cuda(), wi).float().cpu().reshape(100, F // 8, 2, 8)
+        gl, ul = yl[:, :, 0].reshape(100, F), yl[:, :, 1].reshape(100, F)
+        assert close(ops.linear_swiglu(xl.cuda(), wi, True).float(), pl.swiglu(gl, ul), torch.bfloat16)
+        assert close(gl, (xl.double() @ w[:F].double().t()).float(), torch.bfloat16)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
