@@ -17,7 +17,7 @@
 // [page, kv_head, hs, 64].
 //
 // Prompt form: a workgroup of 4 waves owns 64*NT columns = consecutive query tokens x GT heads;
-// every wave walks the keys of its own columns, no shared memory, no barriers.
+// the keys and values it walks are staged through shared memory once for all four waves.
 // Decode form: the 16 columns are the heads of one kv group for the sequence's one new token;
 // the 4 waves take 32-key blocks in turn and merge through shared memory; long contexts are
 // also split over gridDim.z and merged by attn_mfma_combine_kernel in a fixed order.
@@ -58,6 +58,12 @@ struct MfmaArgs {
 __device__ __forceinline__ bf16x8 ld16(const bf16* p) {
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
+typedef __attribute__((ext_vector_type(8))) float f32x8;
+// eight floats to eight bf16, round to nearest even (gfx950 converts two a time in hardware)
+__device__ __forceinline__ bf16x8 pack8(const float (&s)[8]) {
+    const f32x8 v = {s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7]};
+    return __builtin_convertvector(v, bf16x8);
+}
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
     // round to nearest even, as __float2bfloat16 does
     uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b);
@@ -67,62 +73,76 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
 }
 
 // One 32-key block for NT column tiles.  kbase/vbase point at the block's first key inside its
-// page.  qpos/lo: per tile, this lane's column's position and first visible key (qpos < 0: no
+// page (row strides HS and BN_PAGE) or inside a staged copy in shared memory (KSTRIDE, VSTRIDE).  qpos/lo: per tile, this lane's column's position and first visible key (qpos < 0: no
 // such column).  key_hi: keys >= key_hi do not exist (decode: split end / length).
-template <int HS, int NT>
+template <int HS, int NT, int KSTRIDE = HS, int VSTRIDE = BN_PAGE, bool STREAM = false>
 __device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, const bf16* __restrict__ vbase,
                                              int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
                                              float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
                                              const int (&lo)[NT], int key_hi, bool need_mask, float scale2,
                                              int lane) {
+    // STREAM: the operands come from shared memory (short latency): fetch each one right before its
+    // products instead of all of them up front, which keeps fewer registers live.
     constexpr int DC = HS / 32, DT = HS / 16;
     const int i = lane & 15, g = lane >> 4;
     const int krow0 = 8 * (i >> 2) + (i & 3);        // key row of tile 0; tile 1 is 4 further
     f32x4 st[NT][2];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) { st[nt][0] = (f32x4){0.f, 0.f, 0.f, 0.f}; st[nt][1] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
-    bf16x8 ka[DC][2];
+    bf16x8 ka[STREAM ? 1 : DC][2];
+    bf16x8 va[STREAM ? 1 : DT];
+    if (!STREAM) {
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+            ka[c][0] = ld16(kbase + (size_t)krow0 * KSTRIDE + c * 32 + g * 8);
+            ka[c][1] = ld16(kbase + (size_t)(krow0 + 4) * KSTRIDE + c * 32 + g * 8);
+        }
+#pragma unroll
+        for (int t = 0; t < DT; ++t) va[t] = ld16(vbase + (size_t)(t * 16 + i) * VSTRIDE + 8 * g);
+    }
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
-        ka[c][0] = ld16(kbase + (size_t)krow0 * HS + c * 32 + g * 8);
-        ka[c][1] = ld16(kbase + (size_t)(krow0 + 4) * HS + c * 32 + g * 8);
-    }
-    bf16x8 va[DT];
-#pragma unroll
-    for (int t = 0; t < DT; ++t) va[t] = ld16(vbase + (size_t)(t * 16 + i) * BN_PAGE + 8 * g);
-#pragma unroll
-    for (int c = 0; c < DC; ++c)
+        if (STREAM) {
+            // staged keys are stored with their 16-byte chunks swizzled by (row / 8): the four rows
+            // r, r+8, r+16, r+24 that one load touches would otherwise share their banks
+            const int chunk = ((c * 4 + g) ^ (i >> 2)) * 8;
+            ka[0][0] = ld16(kbase + (size_t)krow0 * KSTRIDE + chunk);
+            ka[0][1] = ld16(kbase + (size_t)(krow0 + 4) * KSTRIDE + chunk);
+        }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            st[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c][0], q[nt][c], st[nt][0], 0, 0, 0);
-            st[nt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c][1], q[nt][c], st[nt][1], 0, 0, 0);
+            st[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[STREAM ? 0 : c][0], q[nt][c], st[nt][0], 0, 0, 0);
+            st[nt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[STREAM ? 0 : c][1], q[nt][c], st[nt][1], 0, 0, 0);
         }
-    if (need_mask) {
-        // keys that do not exist may hold anything, NaN included: clear them in V^T (0 * NaN is NaN)
-        const int first = kb + 8 * g;                 // this lane's 8 keys are first .. first+7
+    }
+    // keys that do not exist may hold anything, NaN included: they are cleared in V^T (0 * NaN is NaN)
+    const int first = kb + 8 * g;                     // this lane's 8 keys are first .. first+7
+    auto clear_missing = [&](bf16x8 x) {
+        uint4 v = __builtin_bit_cast(uint4, x);
+        if (first + 0 >= key_hi) v.x &= 0xffff0000u;
+        if (first + 1 >= key_hi) v.x &= 0x0000ffffu;
+        if (first + 2 >= key_hi) v.y &= 0xffff0000u;
+        if (first + 3 >= key_hi) v.y &= 0x0000ffffu;
+        if (first + 4 >= key_hi) v.z &= 0xffff0000u;
+        if (first + 5 >= key_hi) v.z &= 0x0000ffffu;
+        if (first + 6 >= key_hi) v.w &= 0xffff0000u;
+        if (first + 7 >= key_hi) v.w &= 0x0000ffffu;
+        return __builtin_bit_cast(bf16x8, v);
+    };
+    if (!STREAM && need_mask) {
 #pragma unroll
-        for (int t = 0; t < DT; ++t) {
-            uint4 v = __builtin_bit_cast(uint4, va[t]);
-            if (first + 0 >= key_hi) v.x &= 0xffff0000u;
-            if (first + 1 >= key_hi) v.x &= 0x0000ffffu;
-            if (first + 2 >= key_hi) v.y &= 0xffff0000u;
-            if (first + 3 >= key_hi) v.y &= 0x0000ffffu;
-            if (first + 4 >= key_hi) v.z &= 0xffff0000u;
-            if (first + 5 >= key_hi) v.z &= 0x0000ffffu;
-            if (first + 6 >= key_hi) v.w &= 0xffff0000u;
-            if (first + 7 >= key_hi) v.w &= 0x0000ffffu;
-            va[t] = __builtin_bit_cast(bf16x8, v);
-        }
+        for (int t = 0; t < DT; ++t) va[t] = clear_missing(va[t]);
     }
     bf16x8 pb[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
+        // raw scores; the scale (with log2 e folded in) is applied inside the exponent's fma
         float s[8];
 #pragma unroll
         for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                float v = st[nt][sb][r] * scale2;
+                float v = st[nt][sb][r];
                 if (need_mask) {
                     const int key = kb + 8 * g + 4 * sb + r;
                     if (key > qpos[nt] || key < lo[nt] || key >= key_hi) v = -INFINITY;
@@ -132,45 +152,64 @@ __device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, con
         float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
         mx = fmaxf(mx, __shfl_xor(mx, 16, BN_WAVE));
         mx = fmaxf(mx, __shfl_xor(mx, 32, BN_WAVE));
-        const float m_new = fmaxf(m[nt], mx);
-        float alpha = 1.f, rs = 0.f;
+        mx *= scale2;                                  // scale2 > 0: the maximum of the scaled scores
+        // The reference point of the exponents moves only when the maximum has grown by more than
+        // 2^8: until then p = 2^(s - m) may exceed 1 (at most 256), which float32 sums and bf16
+        // weights hold as well, and the accumulators need no rescaling.  The result is the same.
+        float m_new = m[nt];
+        if (mx > m[nt] + 8.0f || m[nt] == -INFINITY) m_new = mx;
+        float rs = 0.f;
         if (m_new == -INFINITY) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) s[e] = 0.f;
         } else {
-            alpha = exp2f(m[nt] - m_new);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) { s[e] = exp2f(s[e] - m_new); rs += s[e]; }
+            for (int e = 0; e < 8; ++e) { s[e] = __builtin_amdgcn_exp2f(fmaf(s[e], scale2, -m_new)); rs += s[e]; }
         }
         rs += __shfl_xor(rs, 16, BN_WAVE);
         rs += __shfl_xor(rs, 32, BN_WAVE);
-        l[nt] = l[nt] * alpha + rs;
-        m[nt] = m_new;
+        const bool moved = m_new != m[nt];
+        if (__any(moved)) {
+            const float alpha = (moved && m[nt] != -INFINITY) ? __builtin_amdgcn_exp2f(m[nt] - m_new) : (moved ? 0.f : 1.f);
+            l[nt] *= alpha;
 #pragma unroll
-        for (int t = 0; t < DT; ++t) acc[nt][t] *= alpha;
-        uint4 pk;
-        pk.x = pack2(s[0], s[1]); pk.y = pack2(s[2], s[3]); pk.z = pack2(s[4], s[5]); pk.w = pack2(s[6], s[7]);
-        pb[nt] = __builtin_bit_cast(bf16x8, pk);
+            for (int t = 0; t < DT; ++t) acc[nt][t] *= alpha;
+        }
+        l[nt] += rs;
+        m[nt] = m_new;
+        pb[nt] = pack8(s);
     }
 #pragma unroll
-    for (int t = 0; t < DT; ++t)
+    for (int t = 0; t < DT; ++t) {
+        if (STREAM) {
+            va[0] = ld16(vbase + (size_t)(t * 16 + i) * VSTRIDE + 8 * g);
+            if (need_mask) va[0] = clear_missing(va[0]);
+        }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
-            acc[nt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[t], pb[nt], acc[nt][t], 0, 0, 0);
+            acc[nt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[STREAM ? 0 : t], pb[nt], acc[nt][t], 0, 0, 0);
+    }
 }
 
 // ---------------------------------------------------------------------------------------
 // prompt form
 // ---------------------------------------------------------------------------------------
+// The 4 waves of a workgroup need the same keys, so a 32-key block is fetched once per workgroup
+// into shared memory (the next block's loads are in flight while the current one is multiplied),
+// double-buffered, one barrier per block.
 template <int HS, int NT>
-__global__ __launch_bounds__(256) void attn_mfma_prompt_kernel(MfmaArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_mfma_prompt_kernel(MfmaArgs a) {
     constexpr int DC = HS / 32, DT = HS / 16;
+    constexpr int KS = HS + 8, VS = 32 + 8;               // padded row strides (elements)
+    constexpr int KV4 = 32 * HS / 8 / 256;                // uint4 loads per thread for K (and for V^T)
+    __shared__ __align__(16) bf16 k_s[2][32 * KS];
+    __shared__ __align__(16) bf16 v_s[2][HS * VS];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
     const int G = a.H / a.Hkv, GT = a.GT;
     const int n_head_tiles = (G + GT - 1) / GT;
     const int kvh = blockIdx.y / n_head_tiles, ht = blockIdx.y - kvh * n_head_tiles;
-    const int* tl = a.tiles + 4 * blockIdx.x;
+    const int* tl = a.tiles + 4 * (gridDim.x - 1 - blockIdx.x);     // later (longer) tiles start first
     const int seq = tl[0], tok0 = tl[1], n_tok = tl[2], pos0 = tl[3];
 
     bf16x8 q[NT][DC];
@@ -178,7 +217,7 @@ __global__ __launch_bounds__(256) void attn_mfma_prompt_kernel(MfmaArgs a) {
     int w_hi = -1, w_lo = 0x7fffffff, all_hi = 0x7fffffff, all_lo = 0;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        const int c = (wave * NT + nt) * 16 + n;            // column within the workgroup
+        const int c = (wave * NT + nt) * 16 + n;
         const int ti = c / GT, hg = ht * GT + (c - ti * GT);
         const bool ok = ti < n_tok && hg < G;
         head[nt] = kvh * G + hg;
@@ -193,7 +232,6 @@ __global__ __launch_bounds__(256) void attn_mfma_prompt_kernel(MfmaArgs a) {
         }
         if (ok) { w_hi = max(w_hi, qpos[nt]); w_lo = min(w_lo, lo[nt]); all_hi = min(all_hi, qpos[nt]); all_lo = max(all_lo, lo[nt]); }
     }
-    // the wave's key range and the range that every one of its columns sees
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
         w_hi = max(w_hi, __shfl_xor(w_hi, o, BN_WAVE));
@@ -201,7 +239,6 @@ __global__ __launch_bounds__(256) void attn_mfma_prompt_kernel(MfmaArgs a) {
         all_hi = min(all_hi, __shfl_xor(all_hi, o, BN_WAVE));
         all_lo = max(all_lo, __shfl_xor(all_lo, o, BN_WAVE));
     }
-    // columns that do not exist have q = 0 and are never written; they need no masking
     f32x4 acc[NT][DT];
     float m[NT], l[NT];
 #pragma unroll
@@ -211,16 +248,48 @@ __global__ __launch_bounds__(256) void attn_mfma_prompt_kernel(MfmaArgs a) {
         for (int t = 0; t < DT; ++t) acc[nt][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
     const float scale2 = a.scale * LOG2E;
-    if (w_hi >= 0) {
-        const size_t bt_row = (size_t)seq * a.bt_stride;
-        for (int kb = (w_lo / 32) * 32; kb <= w_hi; kb += 32) {
-            const int page = a.block_table[bt_row + kb / BN_PAGE];
-            const int koff = kb % BN_PAGE;
-            const bf16* kbase = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS;
-            const bf16* vbase = a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff;
-            const bool need_mask = (kb + 31 > all_hi) || (kb < all_lo);
-            attend_block<HS, NT>(kbase, vbase, kb, q, acc, m, l, qpos, lo, w_hi + 1, need_mask, scale2, lane);
+    // the workgroup's key range: every wave takes part in the staging of all of it
+    const int g_hi = pos0 + n_tok - 1;
+    const int g_lo = a.window > 0 ? max(0, pos0 + 1 - a.window) : 0;
+    const size_t bt_row = (size_t)seq * a.bt_stride;
+    uint4 kr[KV4], vr[KV4];
+    auto fetch = [&](int kb) {
+        const int page = a.block_table[bt_row + kb / BN_PAGE];
+        const int koff = kb % BN_PAGE;
+        const bf16* kg = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS;      // 32 rows of HS, contiguous
+        const bf16* vg = a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff;       // HS rows, 32 of 64 keys each
+#pragma unroll
+        for (int j = 0; j < KV4; ++j) {
+            const int idx = threadIdx.x + 256 * j;
+            kr[j] = *reinterpret_cast<const uint4*>(kg + (size_t)idx * 8);
+            const int vrow = idx >> 2, vcol = (idx & 3) * 8;
+            vr[j] = *reinterpret_cast<const uint4*>(vg + (size_t)vrow * BN_PAGE + vcol);
         }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < KV4; ++j) {
+            const int idx = threadIdx.x + 256 * j;
+            const int krow = (idx * 8) / HS, kchunk = ((idx * 8) % HS) / 8;
+            *reinterpret_cast<uint4*>(&k_s[buf][krow * KS + ((kchunk ^ ((krow >> 3) & 3)) * 8)]) = kr[j];
+            const int vrow = idx >> 2, vcol = (idx & 3) * 8;
+            *reinterpret_cast<uint4*>(&v_s[buf][vrow * VS + vcol]) = vr[j];
+        }
+    };
+    const int kb0 = (g_lo / 32) * 32;
+    fetch(kb0);
+    stash(0);
+    __syncthreads();
+    int buf = 0;
+    for (int kb = kb0; kb <= g_hi; kb += 32, buf ^= 1) {
+        const bool more = kb + 32 <= g_hi;
+        if (more) fetch(kb + 32);
+        if (w_hi >= 0 && kb <= w_hi && kb + 31 >= w_lo) {
+            const bool need_mask = (kb + 31 > all_hi) || (kb < all_lo);
+            attend_block<HS, NT, KS, VS, true>(k_s[buf], v_s[buf], kb, q, acc, m, l, qpos, lo, w_hi + 1, need_mask, scale2, lane);
+        }
+        if (more) stash(buf ^ 1);
+        __syncthreads();
     }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
