@@ -220,6 +220,9 @@ def _tiled(x, w, out_dtype):
     return y
 
 
+SKINNY_ROWS = 16      # bf16 products with more rows than this go to the library
+
+
 def skinny_supported(M: int, N: int, K: int, ldx: int, ldw: int) -> bool:
     return bool(_fn("skinny_gemm", "bn_skinny_gemm_supports")(M, N, K, ldx, ldw))
 
@@ -228,10 +231,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, *, allow_library: b
     """y[M, N] = x[M, K] . w[N, K]^T.
 
     float32: the tiled kernel (plain fmaf, a fixed order of summation).
-    bf16: up to 64 rows the matrix-core kernel that streams the weights once; above
-    that the library's matrix product (as the reference hands its batched prompt
-    products to a library, src/gpu_cuda.cu:11571); shapes neither takes go to the
-    tiled kernel."""
+    bf16: up to 16 rows (one MFMA tile of activations) the matrix-core kernel that streams
+    the weights once; above that the library's matrix product (as the reference hands its
+    batched products to a library, src/gpu_cuda.cu:11571), which from 32 rows on is about
+    twice as fast as the streaming kernel; float32 results from bf16 operands (logits) stay
+    with the streaming kernel, 64 rows at a time; shapes neither takes go to the tiled kernel."""
     require_gpu()
     _dev(x, "x", dims=2)
     _dev(w, "w", x.dtype, 2)
@@ -250,12 +254,13 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, *, allow_library: b
     if x.dtype != torch.bfloat16:
         raise KernelError(f"linear: unsupported dtype {x.dtype}")
     aligned = (x.data_ptr() % 16 == 0) and (w.data_ptr() % 16 == 0)
-    if M <= 64 and aligned and skinny_supported(M, N, K, ldx, ldw):
+    small = M <= SKINNY_ROWS or (M <= 64 and (out_dtype == torch.float32 or not allow_library))
+    if small and aligned and skinny_supported(M, N, K, ldx, ldw):
         y = torch.empty((M, N), dtype=out_dtype, device=x.device)
         _check(_fn("skinny_gemm", "bn_skinny_gemm")(_code(out_dtype), x.data_ptr(), w.data_ptr(), y.data_ptr(),
                                                     M, N, K, ldx, ldw, N, 0, 0, _stream()), "skinny_gemm")
         return y
-    if M > 64 and allow_library and out_dtype == torch.bfloat16:
+    if M > SKINNY_ROWS and allow_library and out_dtype == torch.bfloat16:
         return torch.matmul(x, w.t())
     if M > 64 and out_dtype == torch.float32 and aligned and skinny_supported(64, N, K, ldx, ldw):
         # float32 results from bf16 operands (logits at many positions): 64 rows at a time
@@ -279,7 +284,8 @@ def interleave_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor) -> torch.Tensor
     return torch.stack([w_gate.reshape(F // 8, 8, K), w_up.reshape(F // 8, 8, K)], dim=1).reshape(2 * F, K).contiguous()
 
 
-def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
+def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = False, *,
+                  allow_library: bool = True) -> torch.Tensor:
     """silu(x.Wg^T) * (x.Wu^T) for w_gate_up = [Wg; Wu] ([2F, K]), or the two interleaved in
     blocks of 8 rows (interleave_gate_up).  The decode-sized bf16 case is one kernel; every other
     case is the product followed by the SwiGLU kernel."""
@@ -295,14 +301,14 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = 
     if M == 0:
         return torch.empty((0, F), dtype=x.dtype, device=x.device)
     ldx, ldw = _rows(x, "x"), _rows(w_gate_up, "w_gate_up")
-    if (x.dtype == torch.bfloat16 and M <= 64 and x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0
-            and skinny_supported(M, F, K, ldx, ldw)):
+    if (x.dtype == torch.bfloat16 and (M <= SKINNY_ROWS or (M <= 64 and not allow_library))
+            and x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0 and skinny_supported(M, F, K, ldx, ldw)):
         y = torch.empty((M, F), dtype=x.dtype, device=x.device)
         _check(_fn("skinny_gemm", "bn_skinny_gemm")(_code(x.dtype), x.data_ptr(), w_gate_up.data_ptr(),
                                                     y.data_ptr(), M, F, K, ldx, ldw, F, 2 if interleaved else 1, F,
                                                     _stream()), "skinny_gemm(glu)")
         return y
-    return swiglu(linear(x, w_gate_up), interleaved)
+    return swiglu(linear(x, w_gate_up, allow_library=allow_library), interleaved)
 
 
 # --------------------------------------------------------------------------------------

@@ -254,3 +254,38 @@ def test_far_key_through_the_engine(model_folders, dtype, tmp_path):
         toks2 = list(toks)
         toks2[far] = 3
         assert rel_err(plain_logits(folder, toks2, dtype)[959:960], ref) > 20 * TOL[dtype], far
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_graph_replays_of_a_wide_batch(model_folders, dtype):
+    """24 sequences decode together: at this width the bf16 products are the library's, inside the
+    replayed graph.  Every replay is checked: against the same steps run without graphs (equal
+    bits are demanded: the same kernels run) and against the plain implementation, with eager
+    prompt steps of other sequences and synchronisations between the replays."""
+    from bitnet_c_amd import StepEntry
+    folder = model_folders("C", dtype)
+    rnd = random.Random(17)
+    engines = [make_engine(folder, dtype, max_tokens=64 * 40, use_graphs=g) for g in (True, False)]
+    vocab = engines[0].vocab_size
+    reqs = [[rnd.randrange(vocab) for _ in range(3 + i + 7)] for i in range(24)]
+    extra = [[rnd.randrange(vocab) for _ in range(20)] for _ in range(7)]
+    outs = []
+    for eng in engines:
+        slots = [eng.new_sequence() for _ in reqs]
+        got = [[] for _ in reqs]
+        out = eng.step([StepEntry(s, r[:-7], [len(r) - 8]) for s, r in zip(slots, reqs)])
+        for i in range(24):
+            got[i].append(out[i:i + 1])
+        for k in range(7):
+            other = eng.new_sequence()                              # eager work between the replays
+            eng.step([StepEntry(other, extra[k], [19])])
+            eng.release(other)
+            torch.cuda.synchronize()
+            out = eng.step([StepEntry(s, [r[len(r) - 7 + k]], [0]) for s, r in zip(slots, reqs)])
+            for i in range(24):
+                got[i].append(out[i:i + 1])
+        outs.append([torch.cat(g) for g in got])
+    for i, r in enumerate(reqs):
+        assert torch.equal(outs[0][i], outs[1][i]), i
+        ref = plain_logits(folder, r, dtype)[len(r) - 8:]
+        assert rel_err(outs[0][i], ref) < TOL[dtype], i

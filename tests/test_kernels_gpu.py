@@ -132,15 +132,16 @@ def test_skinny_gemm_bf16(M, N, K):
     ref = x.double() @ w.double().t()
     y32 = ops.linear(x.cuda(), w.cuda(), torch.float32)
     assert rel_err(y32, ref.float()) < 1e-5                       # bf16 products are exact in float32
-    y16 = ops.linear(x.cuda(), w.cuda())
-    assert y16.dtype == torch.bfloat16 and close(y16.float(), ref.float(), torch.bfloat16)
+    for lib in (True, False):                                     # above 16 rows: the library, or this kernel
+        y16 = ops.linear(x.cuda(), w.cuda(), allow_library=lib)
+        assert y16.dtype == torch.bfloat16 and close(y16.float(), ref.float(), torch.bfloat16)
 
 
 @pytest.mark.parametrize("M,F,K", [(1, 24, 64), (8, 172, 64), (20, 100, 264), (64, 1000, 512), (40, 14336, 256), (33, 8, 8), (17, 328, 120)])
 def test_skinny_gemm_dual_swiglu(M, F, K):
     ops = _ops()
     x, w = _rand((M, K), torch.bfloat16, 13), _rand((2 * F, K), torch.bfloat16, 14, 0.1)
-    y = ops.linear_swiglu(x.cuda(), w.cuda())
+    y = ops.linear_swiglu(x.cuda(), w.cuda(), allow_library=False)
     g = x.double() @ w[:F].double().t()
     u = x.double() @ w[F:].double().t()
     want = ((g / (1 + torch.exp(-g))) * u).float()
@@ -148,7 +149,7 @@ def test_skinny_gemm_dual_swiglu(M, F, K):
     if F % 8 == 0:          # gate and up rows interleaved in blocks of 8
         wi = ops.interleave_gate_up(w[:F].cuda(), w[F:].cuda())
         assert torch.equal(wi[:8].cpu(), w[:8]) and torch.equal(wi[8:16].cpu(), w[F:F + 8])
-        assert close(ops.linear_swiglu(x.cuda(), wi, True).float(), want, torch.bfloat16)
+        assert close(ops.linear_swiglu(x.cuda(), wi, True, allow_library=False).float(), want, torch.bfloat16)
         xl = _rand((100, K), torch.bfloat16, 15)                    # more than 64 rows: product, then the kernel
         yl = ops.linear(xl.cuda(), wi).float().cpu().reshape(100, F // 8, 2, 8)
         gl, ul = yl[:, :, 0].reshape(100, F), yl[:, :, 1].reshape(100, F)
