@@ -53,6 +53,47 @@ __global__ __launch_bounds__(SMP_THREADS) void argmax_kernel(const float* __rest
     if (threadIdx.x == 0) out[blockIdx.x] = r.i;
 }
 
+// Two stages for few rows of a large vocabulary (src/gpu_cuda.cu:9068, :9125 does the same): stage 1,
+// grid (rows, parts), the best of each contiguous part; stage 2, one wave per row, the best of the parts.
+// `better` prefers the lower index among equals at both stages, so the result is the first maximum.
+#define ARGMAX_PARTS 64
+__global__ __launch_bounds__(256) void argmax_part_kernel(const float* __restrict__ logits, int ld, int n,
+                                                          float* __restrict__ pv, int* __restrict__ pi) {
+    __shared__ ArgMax scratch[16];
+    const int part = blockIdx.y, per = (n + ARGMAX_PARTS - 1) / ARGMAX_PARTS;
+    const int lo = min(n, part * per), hi = min(n, lo + per);
+    const float* x = logits + (size_t)blockIdx.x * ld;
+    ArgMax best = {-INFINITY, 0x7fffffff};
+    for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+        ArgMax c = {x[i], i};
+        best = better(best, c);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        ArgMax c = {__shfl_xor(best.v, o, BN_WAVE), __shfl_xor(best.i, o, BN_WAVE)};
+        best = better(best, c);
+    }
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (lane == 0) scratch[w] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        ArgMax r = scratch[0];
+        for (int k = 1; k < (int)(blockDim.x >> 6); ++k) r = better(r, scratch[k]);
+        pv[blockIdx.x * ARGMAX_PARTS + part] = r.v;
+        pi[blockIdx.x * ARGMAX_PARTS + part] = r.i;
+    }
+}
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ pv, const int* __restrict__ pi,
+                                                          int* __restrict__ out) {
+    ArgMax best = {pv[blockIdx.x * ARGMAX_PARTS + threadIdx.x], pi[blockIdx.x * ARGMAX_PARTS + threadIdx.x]};
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        ArgMax c = {__shfl_xor(best.v, o, BN_WAVE), __shfl_xor(best.i, o, BN_WAVE)};
+        best = better(best, c);
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = best.i == 0x7fffffff ? 0 : best.i;
+}
+
 // recent: [rows, window] token ids, -1 = empty.  Each distinct token is penalised once.
 __global__ void repeat_penalty_kernel(float* __restrict__ logits, int ld, int n, const int* __restrict__ recent,
                                       int window, float penalty) {
@@ -234,8 +275,15 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(const float* __rest
     if (threadIdx.x == 0) out[blockIdx.x] = tok;
 }
 
-extern "C" int bn_argmax(const float* logits, int ld, int rows, int n, int* out, hipStream_t s) {
+// work: rows * 64 floats and rows * 64 ints for the two-stage form (may be null: one stage)
+extern "C" int bn_argmax(const float* logits, int ld, int rows, int n, int* out, float* work_v, int* work_i,
+                         hipStream_t s) {
     if (rows <= 0 || n <= 0 || ld < n) return BN_ERR_ARG;
+    if (work_v && work_i && rows <= 256 && n >= 16384 && rows <= 65535) {
+        hipLaunchKernelGGL(argmax_part_kernel, dim3(rows, ARGMAX_PARTS), dim3(256), 0, s, logits, ld, n, work_v, work_i);
+        hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(64), 0, s, work_v, work_i, out);
+        return bn_launch_status();
+    }
     hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(SMP_THREADS), 0, s, logits, ld, n, out);
     return bn_launch_status();
 }

@@ -58,7 +58,7 @@ _SIGNATURES = {
                            c_int, c_void_p],
     },
     "sampling": {
-        "bn_argmax": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p],
+        "bn_argmax": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
         "bn_repeat_penalty": [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_float, c_void_p],
         "bn_sample": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p],
     },
@@ -404,7 +404,9 @@ def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int):
     G = H // Hkv
     wgs = max(1, n_seqs * Hkv * ((G + GT - 1) // GT))
     pages = max(1, (max_len + PAGE - 1) // PAGE)
-    want = max(1, min(pages, 64, (1024 + wgs - 1) // wgs))
+    # about 512 workgroups, but no split shorter than 4 pages: below that the merging costs more
+    # than the parallelism gains (measured at batch 1, 8 and 64 of the 8B shape)
+    want = max(1, min(pages // 4, 64, (512 + wgs - 1) // wgs))
     chunk = ((pages + want - 1) // want) * PAGE
     n_splits = (pages * PAGE + chunk - 1) // chunk
     return n_splits, chunk
@@ -540,7 +542,13 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     B, V = logits.shape
     out = torch.empty((B,), dtype=torch.int32, device=logits.device)
     if B:
-        _check(_fn("sampling", "bn_argmax")(logits.data_ptr(), ld, B, V, out.data_ptr(), _stream()), "argmax")
+        wv = wi = None
+        if B <= 256 and V >= 16384:          # few rows of a large vocabulary: two stages
+            wv = torch.empty((B, 64), dtype=torch.float32, device=logits.device)
+            wi = torch.empty((B, 64), dtype=torch.int32, device=logits.device)
+        _check(_fn("sampling", "bn_argmax")(logits.data_ptr(), ld, B, V, out.data_ptr(),
+                                            wv.data_ptr() if wv is not None else None,
+                                            wi.data_ptr() if wi is not None else None, _stream()), "argmax")
     return out
 
 

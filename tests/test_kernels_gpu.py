@@ -387,6 +387,12 @@ def test_argmax_ties_and_odd_vocab():
     got = ops.argmax(x.cuda()).cpu().tolist()
     assert got == torch.argmax(x, dim=1).tolist() and got[1] == 17 and got[2] == 1008 and got[3] == 0
     assert ops.argmax(torch.tensor([[1.0, 3.0, 2.0, 0.5]]).cuda()).item() == 1        # test/test_safety.c:208-211
+    big = _rand((3, 128256), torch.float32, 401)                 # the two-stage form
+    big[0, 5] = big[0, 100000] = 9.0                             # a tie across parts: the lower index
+    big[1, 128255] = 9.0
+    big[2, 2004] = big[2, 2003] = 9.0                            # a tie at a part's edge (2004 per part)
+    assert ops.argmax(big.cuda()).cpu().tolist() == [5, 128255, 2003]
+    assert ops.argmax(torch.full((2, 20000), -float("inf")).cuda()).cpu().tolist() == [0, 0]
 
 
 @pytest.mark.parametrize("vocab", [4, 389, 128256])
