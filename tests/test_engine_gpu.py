@@ -289,3 +289,35 @@ def test_graph_replays_of_a_wide_batch(model_folders, dtype):
         assert torch.equal(outs[0][i], outs[1][i]), i
         ref = plain_logits(folder, r, dtype)[len(r) - 8:]
         assert rel_err(outs[0][i], ref) < TOL[dtype], i
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_more_sequences_than_a_graph_takes_and_a_long_context(model_folders, dtype):
+    """70 sequences decode in one step (more than the replayed graphs hold: the step runs eagerly),
+    and one sequence grows past 1,100 positions token by token, through several block-table widths."""
+    from bitnet_c_amd import StepEntry
+    folder = model_folders("A", dtype)
+    eng = make_engine(folder, dtype, max_tokens=64 * 110)
+    rnd = random.Random(18)
+    reqs = [[rnd.randrange(eng.vocab_size) for _ in range(2 + i % 5 + 3)] for i in range(70)]
+    slots = [eng.new_sequence() for _ in reqs]
+    eng.step([StepEntry(s, r[:-3], []) for s, r in zip(slots, reqs)])
+    got = [[] for _ in reqs]
+    for k in range(3):
+        out = eng.step([StepEntry(s, [r[len(r) - 3 + k]], [0]) for s, r in zip(slots, reqs)])
+        for i in range(70):
+            got[i].append(out[i:i + 1])
+    for i in (0, 1, 33, 68, 69):
+        assert rel_err(torch.cat(got[i]), plain_logits(folder, reqs[i], dtype)[-3:]) < TOL[dtype], i
+    for s in slots:
+        eng.release(s)
+    folder = model_folders("C", dtype)                 # its position limit is 2,048
+    eng = make_engine(folder, dtype, max_tokens=64 * 20)
+    long_req = [rnd.randrange(eng.vocab_size) for _ in range(1130)]
+    s = eng.new_sequence()
+    outs = [eng.step([StepEntry(s, long_req[:1000], [999])])]
+    for t in long_req[1000:]:
+        outs.append(eng.step([StepEntry(s, [t], [0])]))
+    eng.release(s)
+    assert rel_err(torch.cat(outs), plain_logits(folder, long_req, dtype)[999:]) < TOL[dtype]
+    eng.cache.check()

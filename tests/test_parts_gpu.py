@@ -326,3 +326,79 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
     assert s == slots[0]
     again = eng.step([StepEntry(s, reqs[1], list(range(7)))])
     assert rel_err(again, plain(reqs[1])) < TOL[torch.float32]
+
+
+def test_a_windowed_group_beside_a_full_one_through_the_engine(tmp_path):
+    """A toy architecture whose odd layers see only the last 70 positions: two cache groups with
+    storage of their own; the windowed one gives pages back while sequences grow, and the logits
+    match plain attention with the same window, for prompts and for decoding (with graphs)."""
+    from bitnet_c_amd import Engine, StepEntry
+    from bitnet_c_amd.config import Architecture, LlamaConfig, register_architecture
+    from bitnet_c_amd.config.base import _ARCHITECTURES
+    from bitnet_c_amd.config.llama_plan import build_llama_plan
+    from bitnet_c_amd.engine import LayerPlan
+    from bitnet_c_amd.parts import PartSpec
+    from bitnet_c_amd.weights import write_model_folder
+    from dataclasses import replace
+    W = 70
+
+    def build(c):
+        plan = build_llama_plan(c)
+        layers = []
+        for i, lp in enumerate(plan.layers):
+            if i % 2 == 1:
+                blk = dict(lp.block.params)
+                blk["mixer"] = PartSpec.of(blk["mixer"].kind, **dict(dict(blk["mixer"].params), window=W))
+                lp = LayerPlan(block=PartSpec.of(lp.block.kind, **blk), names=lp.names)
+            layers.append(lp)
+        return replace(plan, layers=layers)
+
+    class WinConfig(LlamaConfig):
+        def to_dict(self):
+            return dict(super().to_dict(), model_type="toy_window", architectures=["ToyWindow"])
+
+    if "toy_window" not in _ARCHITECTURES:
+        register_architecture(Architecture("toy_window", LlamaConfig, build))
+    from conftest import TINY_A
+    for dtype in (torch.float32, torch.bfloat16):
+        base = LlamaConfig.from_dict(dict(TINY_A, num_hidden_layers=4, head_dim=64, num_attention_heads=2,
+                                          num_key_value_heads=1, hidden_size=64))
+        cfg = WinConfig(**{f: getattr(base, f) for f in base.__dataclass_fields__})
+        folder = write_model_folder(str(tmp_path / f"win{dtype}"), cfg, 9, dtype)
+        eng = Engine.from_folder(folder, dtype=dtype, max_tokens=64 * 12)
+        assert len(eng.cache.groups) == 2 and sorted(g.need.window for g in eng.cache.groups) == [0, W]
+        c, Wt = pl.read_config(folder), pl.read_weights(folder)
+        rt = None if dtype == torch.float32 else torch.bfloat16
+        rnd = random.Random(3)
+        reqs = [[rnd.randrange(256) for _ in range(n)] for n in (300, 150)]
+
+        def plain(toks):
+            x = Wt["model.embed_tokens.weight"][toks]
+            pos = torch.arange(len(toks))
+            inv = pl.rope_inv_freq(c["head_dim"], c["theta"])
+            for l in range(4):
+                x = pl.decoder_layer(x, pos, Wt, l, c, inv, rt, W if l % 2 == 1 else None)
+            xn = pl._rt(pl.rmsnorm(x, Wt["model.norm.weight"], c["eps"]), rt)
+            return pl.linear(xn, Wt["lm_head.weight"])
+
+        slots = [eng.new_sequence() for _ in reqs]
+        fed = [len(r) - 40 for r in reqs]
+        out = eng.step([StepEntry(s, r[:f], list(range(f))) for s, r, f in zip(slots, reqs, fed)])
+        got, o = [[] for _ in reqs], 0
+        for i, f in enumerate(fed):
+            got[i].append(out[o:o + f])
+            o += f
+        for k in range(40):
+            out = eng.step([StepEntry(s, [r[f + k]], [0]) for s, r, f in zip(slots, reqs, fed)])
+            for i in range(2):
+                got[i].append(out[i:i + 1])
+            eng.cache.check()
+        full = [g for g in eng.cache.groups if g.need.window == 0][0]
+        win = [g for g in eng.cache.groups if g.need.window == W][0]
+        assert sum(p >= 0 for p in full.pages[slots[0]]) == 5 and sum(p >= 0 for p in win.pages[slots[0]]) == 2
+        for i, r in enumerate(reqs):
+            assert rel_err(torch.cat(got[i]), plain(r)) < TOL[dtype], (dtype, i)
+        for s in slots:
+            eng.release(s)
+        eng.cache.check()
+        assert win.pool.n_free == win.pool.n_pages
