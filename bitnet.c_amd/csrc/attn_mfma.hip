@@ -58,6 +58,22 @@ struct MfmaArgs {
 __device__ __forceinline__ bf16x8 ld16(const bf16* p) {
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
+// Combining a value with the ones 16 and 32 lanes away (the four lane groups of a column) without
+// going through shared memory: gfx950 swaps 16- and 32-lane halves between two registers.
+__device__ __forceinline__ float max_over_lane_groups(float x) {
+    const unsigned b = __float_as_uint(x);
+    auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    const unsigned c = __float_as_uint(fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1])));
+    auto t = __builtin_amdgcn_permlane32_swap(c, c, false, false);
+    return fmaxf(__uint_as_float(t[0]), __uint_as_float(t[1]));
+}
+__device__ __forceinline__ float sum_over_lane_groups(float x) {
+    const unsigned b = __float_as_uint(x);
+    auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    const unsigned c = __float_as_uint(__uint_as_float(r[0]) + __uint_as_float(r[1]));
+    auto t = __builtin_amdgcn_permlane32_swap(c, c, false, false);
+    return __uint_as_float(t[0]) + __uint_as_float(t[1]);
+}
 typedef __attribute__((ext_vector_type(8))) float f32x8;
 // eight floats to eight bf16, round to nearest even (gfx950 converts two a time in hardware)
 __device__ __forceinline__ bf16x8 pack8(const float (&s)[8]) {
@@ -75,12 +91,11 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
 // One 32-key block for NT column tiles.  kbase/vbase point at the block's first key inside its
 // page (row strides HS and BN_PAGE) or inside a staged copy in shared memory (KSTRIDE, VSTRIDE).  qpos/lo: per tile, this lane's column's position and first visible key (qpos < 0: no
 // such column).  key_hi: keys >= key_hi do not exist (decode: split end / length).
-template <int HS, int NT, int KSTRIDE = HS, int VSTRIDE = BN_PAGE, bool STREAM = false>
-__device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, const bf16* __restrict__ vbase,
-                                             int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
-                                             float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
-                                             const int (&lo)[NT], int key_hi, bool need_mask, float scale2,
-                                             int lane) {
+template <int HS, int NT, int KSTRIDE, int VSTRIDE, bool STREAM, bool need_mask>
+__device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, const bf16* __restrict__ vbase,
+                                               int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
+                                               float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
+                                               const int (&lo)[NT], int key_hi, float scale2, int lane) {
     // STREAM: the operands come from shared memory (short latency): fetch each one right before its
     // products instead of all of them up front, which keeps fewer registers live.
     constexpr int DC = HS / 32, DT = HS / 16;
@@ -103,9 +118,10 @@ __device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, con
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
         if (STREAM) {
-            // staged keys are stored with their 16-byte chunks swizzled by (row / 8): the four rows
-            // r, r+8, r+16, r+24 that one load touches would otherwise share their banks
-            const int chunk = ((c * 4 + g) ^ (i >> 2)) * 8;
+            // staged keys are stored with their 16-byte chunks swizzled (chunk ^ 4 for rows 8..15 and
+            // 24..31): the eight lanes that read together touch rows r..r+3 and r+8..r+11, which
+            // would otherwise share their banks
+            const int chunk = ((c * 4 + g) ^ ((i >> 2) & 1) * 4) * 8;
             ka[0][0] = ld16(kbase + (size_t)krow0 * KSTRIDE + chunk);
             ka[0][1] = ld16(kbase + (size_t)(krow0 + 4) * KSTRIDE + chunk);
         }
@@ -150,8 +166,7 @@ __device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, con
                 s[sb * 4 + r] = v;
             }
         float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
-        mx = fmaxf(mx, __shfl_xor(mx, 16, BN_WAVE));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, BN_WAVE));
+        mx = max_over_lane_groups(mx);
         mx *= scale2;                                  // scale2 > 0: the maximum of the scaled scores
         // The reference point of the exponents moves only when the maximum has grown by more than
         // 2^8: until then p = 2^(s - m) may exceed 1 (at most 256), which float32 sums and bf16
@@ -166,8 +181,7 @@ __device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, con
 #pragma unroll
             for (int e = 0; e < 8; ++e) { s[e] = __builtin_amdgcn_exp2f(fmaf(s[e], scale2, -m_new)); rs += s[e]; }
         }
-        rs += __shfl_xor(rs, 16, BN_WAVE);
-        rs += __shfl_xor(rs, 32, BN_WAVE);
+        rs = sum_over_lane_groups(rs);
         const bool moved = m_new != m[nt];
         if (__any(moved)) {
             const float alpha = (moved && m[nt] != -INFINITY) ? __builtin_amdgcn_exp2f(m[nt] - m_new) : (moved ? 0.f : 1.f);
@@ -189,6 +203,20 @@ __device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, con
         for (int nt = 0; nt < NT; ++nt)
             acc[nt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[STREAM ? 0 : t], pb[nt], acc[nt][t], 0, 0, 0);
     }
+}
+
+// The masked form (a block on the causal diagonal, at a window's edge or at the end of the keys) and
+// the plain one are separate instantiations: almost every block is plain, and it carries no mask code.
+template <int HS, int NT, int KSTRIDE = HS, int VSTRIDE = BN_PAGE, bool STREAM = false>
+__device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, const bf16* __restrict__ vbase,
+                                             int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
+                                             float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
+                                             const int (&lo)[NT], int key_hi, bool need_mask, float scale2,
+                                             int lane) {
+    if (need_mask)
+        attend_block_m<HS, NT, KSTRIDE, VSTRIDE, STREAM, true>(kbase, vbase, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
+    else
+        attend_block_m<HS, NT, KSTRIDE, VSTRIDE, STREAM, false>(kbase, vbase, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -271,7 +299,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int j = 0; j < KV4; ++j) {
             const int idx = threadIdx.x + 256 * j;
             const int krow = (idx * 8) / HS, kchunk = ((idx * 8) % HS) / 8;
-            *reinterpret_cast<uint4*>(&k_s[buf][krow * KS + ((kchunk ^ ((krow >> 3) & 3)) * 8)]) = kr[j];
+            *reinterpret_cast<uint4*>(&k_s[buf][krow * KS + ((kchunk ^ ((krow >> 3) & 1) * 4) * 8)]) = kr[j];
             const int vrow = idx >> 2, vcol = (idx & 3) * 8;
             *reinterpret_cast<uint4*>(&v_s[buf][vrow * VS + vcol]) = vr[j];
         }
