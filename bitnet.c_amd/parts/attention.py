@@ -46,8 +46,8 @@ class Attention(Part):
         t = {"wq": ParamSpec((self.q_dim, self.hidden)), "wk": ParamSpec((self.kv_dim, self.hidden)),
              "wv": ParamSpec((self.kv_dim, self.hidden)), "wo": ParamSpec((self.hidden, self.q_dim))}
         if self.has_bias:
-            t.update({"bq": ParamSpec((self.q_dim,), "zeros"), "bk": ParamSpec((self.kv_dim,), "zeros"),
-                      "bv": ParamSpec((self.kv_dim,), "zeros"), "bo": ParamSpec((self.hidden,), "zeros")})
+            t.update({"bq": ParamSpec((self.q_dim,), "normal"), "bk": ParamSpec((self.kv_dim,), "normal"),
+                      "bv": ParamSpec((self.kv_dim,), "normal"), "bo": ParamSpec((self.hidden,), "normal")})
         return t
 
     def load(self, tensors, device, dtype):

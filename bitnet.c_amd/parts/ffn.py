@@ -23,8 +23,8 @@ class SwiGLU(Part):
         t = {"w_gate": ParamSpec((self.F, self.hidden)), "w_up": ParamSpec((self.F, self.hidden)),
              "w_down": ParamSpec((self.hidden, self.F))}
         if self.has_bias:
-            t.update({"b_gate": ParamSpec((self.F,), "zeros"), "b_up": ParamSpec((self.F,), "zeros"),
-                      "b_down": ParamSpec((self.hidden,), "zeros")})
+            t.update({"b_gate": ParamSpec((self.F,), "normal"), "b_up": ParamSpec((self.F,), "normal"),
+                      "b_down": ParamSpec((self.hidden,), "normal")})
         return t
 
     def load(self, tensors, device, dtype):

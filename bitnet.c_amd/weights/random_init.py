@@ -52,6 +52,9 @@ def random_tensors(expected: Dict[str, TensorSpec], seed: int, dtype=torch.bfloa
 def write_model_folder(folder: str, config, seed: int, dtype=torch.bfloat16) -> str:
     """config: a typed configuration of a registered architecture."""
     from ..config.base import architecture_for
+    if isinstance(dtype, str):
+        dtype = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
+                 "fp32": torch.float32}[dtype]
     raw = config.to_dict()
     arch = architecture_for(raw)
     plan = arch.build_plan(config)

@@ -41,8 +41,14 @@ TINY_C = dict(
     vocab_size=131, hidden_size=72, intermediate_size=100, num_hidden_layers=1,
     num_attention_heads=6, num_key_value_heads=2, head_dim=32, max_position_embeddings=2048,
     rope_theta=20000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-SEEDS = {"A": 0, "B": 2, "C": 5}
+# a fourth one with the optional bias tensors on every projection, and head size 64 (matrix-core attention)
+TINY_D = dict(
+    model_type="llama", architectures=["LlamaForCausalLM"],
+    vocab_size=200, hidden_size=128, intermediate_size=264, num_hidden_layers=2,
+    num_attention_heads=4, num_key_value_heads=2, head_dim=64, max_position_embeddings=1024,
+    rope_theta=100000.0, rms_norm_eps=1e-5, tie_word_embeddings=False, attention_bias=True, mlp_bias=True)
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+SEEDS = {"A": 0, "B": 2, "C": 5, "D": 7}
 
 
 @pytest.fixture(scope="session")

@@ -159,18 +159,20 @@ def swiglu(g: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
     return silu(g) * u
 
 
-def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+def linear(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None = None) -> torch.Tensor:
     """out[row] = sum_col W[row, col] * x[col], W row-major [out, in]
-    (src/quant/f32_scalar.c:4-32, src/model.c:157-158)."""
-    return x.to(F32) @ w.to(F32).t()
+    (src/quant/f32_scalar.c:4-32, src/model.c:157-158); a bias, where the model has the
+    tensor, is added after the product (src/transformer/cpu.c:871-873)."""
+    y = x.to(F32) @ w.to(F32).t()
+    return y if b is None else y + b.to(F32)
 
 
-def feed_forward(xb: torch.Tensor, wg, wu, wd, round_to=None) -> torch.Tensor:
+def feed_forward(xb: torch.Tensor, wg, wu, wd, round_to=None, bg=None, bu=None, bd=None) -> torch.Tensor:
     """gate, up -> silu(gate)*up -> down (src/transformer/cpu.c:1270-1303)."""
-    g = _rt(linear(xb, wg), round_to)
-    u = _rt(linear(xb, wu), round_to)
+    g = _rt(linear(xb, wg, bg), round_to)
+    u = _rt(linear(xb, wu, bu), round_to)
     h = _rt(swiglu(g, u), round_to)
-    return _rt(linear(h, wd), round_to)
+    return _rt(linear(h, wd, bd), round_to)
 
 
 # ----------------------------------------------------------------------------------
@@ -184,17 +186,19 @@ def decoder_layer(x, positions, W, l, c, inv_freq, round_to=None, window=None):
     T = x.shape[0]
     H, Hkv, hs = c["heads"], c["kv_heads"], c["head_dim"]
     xb = _rt(rmsnorm(x, W[p + "input_layernorm.weight"], c["eps"]), round_to)
-    q = _rt(linear(xb, W[p + "self_attn.q_proj.weight"]), round_to).view(T, H, hs)
-    k = _rt(linear(xb, W[p + "self_attn.k_proj.weight"]), round_to).view(T, Hkv, hs)
-    v = _rt(linear(xb, W[p + "self_attn.v_proj.weight"]), round_to).view(T, Hkv, hs)
+    b = lambda name: W.get(p + name)              # optional bias tensors (Llama checkpoints have none)
+    q = _rt(linear(xb, W[p + "self_attn.q_proj.weight"], b("self_attn.q_proj.bias")), round_to).view(T, H, hs)
+    k = _rt(linear(xb, W[p + "self_attn.k_proj.weight"], b("self_attn.k_proj.bias")), round_to).view(T, Hkv, hs)
+    v = _rt(linear(xb, W[p + "self_attn.v_proj.weight"], b("self_attn.v_proj.bias")), round_to).view(T, Hkv, hs)
     q = _rt(apply_rope(q, positions, inv_freq), round_to)
     k = _rt(apply_rope(k, positions, inv_freq), round_to)     # the cache holds rotated keys
     scale = 1.0 / math.sqrt(hs)                               # src/model_arch.c:141-145
     o = _rt(attention(q, k, v, scale, window).reshape(T, H * hs), round_to)
-    x = x + _rt(linear(o, W[p + "self_attn.o_proj.weight"]), round_to)
+    x = x + _rt(linear(o, W[p + "self_attn.o_proj.weight"], b("self_attn.o_proj.bias")), round_to)
     xb = _rt(rmsnorm(x, W[p + "post_attention_layernorm.weight"], c["eps"]), round_to)
     x = x + feed_forward(xb, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"],
-                         W[p + "mlp.down_proj.weight"], round_to)
+                         W[p + "mlp.down_proj.weight"], round_to, b("mlp.gate_proj.bias"), b("mlp.up_proj.bias"),
+                         b("mlp.down_proj.bias"))
     return x
 
 
