@@ -14,6 +14,12 @@
 // gate rows 8t..8t+7, rows 16t+8..16t+15 the up rows of the same columns): every 16-row tile holds
 // both halves of 8 result columns, so the plain kernel does it with half the loads in flight.
 //
+// The activations: all workgroups read the same X, and a load in the operand layout (one row per
+// lane, 64 bytes of it per load) costs a full load instruction however few rows there are.  With
+// up to 16 rows (XS) a wave therefore fetches its K chunk of X with dense loads (32 lanes x 16 bytes
+// a row), parks it in a region of shared memory of its own (no workgroup barrier) and reads the
+// operand fragments from there; the vector memory pipe is left to the weights.
+//
 // Needs K % 8 == 0 and 16-byte aligned rows; other shapes go to the tiled kernel.
 #include "common.h"
 
@@ -24,7 +30,9 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
 
-template <int MT, bool DUAL, typename TO, bool GLU8 = false>
+#define SK_XROW 528           // bytes between rows of a wave's staged X chunk (512 + 16: conflict-free 16-byte reads)
+
+template <int MT, bool DUAL, typename TO, bool GLU8 = false, bool XS = false>
 __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                            TO* __restrict__ Y, int M, int N, int K, int ldx,
                                                            int ldw, int ldy, int up_off) {
@@ -41,10 +49,23 @@ __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_ke
     f32x4 acc[NA];
 #pragma unroll
     for (int a = 0; a < NA; ++a) acc[a] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    // XS: this wave's staging region, after the partial sums
+    unsigned char* xs = reinterpret_cast<unsigned char*>(red + (size_t)n_waves * NA * 256) + (size_t)wave * M * SK_XROW;
 
     for (int kc = wave * SK_CHUNK; kc < K; kc += n_waves * SK_CHUNK) {
         const int kb = kc + g * 8;                    // lane group g: 8 elements of every 32 (64 contiguous bytes per row and load)
         uint4 wv[8], uv[8];
+        uint4 xd[8];
+        if (XS) {                                     // issued before the weights: loads return in order
+            const int xk = kc + (lane & 31) * 8;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const int row = 2 * r + (lane >> 5);
+                if (2 * r < M)
+                    xd[r] = (row < M && xk < K) ? *reinterpret_cast<const uint4*>(X + (size_t)row * ldx + xk)
+                                                : make_uint4(0, 0, 0, 0);
+            }
+        }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int k = kb + j * 32;
@@ -56,10 +77,25 @@ __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_ke
             const int m = mt * 16 + i;
             const bf16* xrow = X + (size_t)m * ldx;
             uint4 xv[8];
+            if (XS) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int k = kb + j * 32;
-                xv[j] = (m < M && k < K) ? *reinterpret_cast<const uint4*>(xrow + k) : make_uint4(0, 0, 0, 0);
+                for (int r = 0; r < 8; ++r) {
+                    const int row = 2 * r + (lane >> 5);
+                    if (2 * r < M && row < M)
+                        *reinterpret_cast<uint4*>(xs + row * SK_XROW + (lane & 31) * 16) = xd[r];
+                }
+                __builtin_amdgcn_wave_barrier();      // one wave: its shared-memory operations run in order
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    xv[j] = (m < M) ? *reinterpret_cast<const uint4*>(xs + m * SK_XROW + j * 64 + g * 16)
+                                    : make_uint4(0, 0, 0, 0);
+                __builtin_amdgcn_wave_barrier();
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int k = kb + j * 32;
+                    xv[j] = (m < M && k < K) ? *reinterpret_cast<const uint4*>(xrow + k) : make_uint4(0, 0, 0, 0);
+                }
             }
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
@@ -102,8 +138,19 @@ template <int MT, bool DUAL, typename TO, bool GLU8 = false>
 static int launch(const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw, int ldy,
                   int up_off, int n_waves, hipStream_t s) {
     constexpr int NA = DUAL ? 2 * MT : MT;
-    const size_t smem = (size_t)n_waves * NA * 64 * 4 * sizeof(float);
-    hipLaunchKernelGGL((skinny_gemm_kernel<MT, DUAL, TO, GLU8>), dim3((N + 15) / 16), dim3(n_waves * 64), smem, s,
+    constexpr bool XS = MT == 1 && !DUAL;          // the two-block form has no registers to spare for it
+    const size_t smem = (size_t)n_waves * NA * 64 * 4 * sizeof(float) + (XS ? (size_t)n_waves * M * SK_XROW : 0);
+    auto kernel = skinny_gemm_kernel<MT, DUAL, TO, GLU8, XS>;
+    if (smem > 64 * 1024) {                           // beyond the default limit of dynamic shared memory
+        static bool raised = false;                   // per instantiation
+        if (!raised) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return (int)e;
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(n_waves * 64), smem, s,
                        (const bf16*)X, (const bf16*)W, (TO*)Y, M, N, K, ldx, ldw, ldy, up_off);
     return bn_launch_status();
 }
@@ -158,6 +205,7 @@ extern "C" int bn_skinny_gemm(int out_dtype, const void* X, const void* W, void*
     // the K chunks there are and by 48 KB of shared memory for the partial sums
     const int tiles = (N + 15) / 16;
     int n_waves = tiles >= 2048 ? 4 : (tiles >= 1024 ? 8 : 16);
+    if (MT == 1 && dual != 1) n_waves = 8;        // staged activations: measured best at every size (several workgroups per CU)
     if (g_force_waves > 0) n_waves = g_force_waves;
     const int k_chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
     while (n_waves > 1 && n_waves / 2 >= k_chunks) n_waves >>= 1;
