@@ -158,7 +158,7 @@ def main() -> int:
             print(f"[bench] decode b{b}: {s_b * 1e3:.3f} ms/step, {b / s_b:.1f} tok/s", file=sys.stderr, flush=True)
 
     rec = {
-        "metric": "decode tok/s @ batch 8 (Llama-3.1-8B shape, bf16)", "value": round(value, 1), "unit": "tok/s",
+        "metric": f"decode tok/s @ batch {args.batch} (Llama-3.1-8B shape, bf16)", "value": round(value, 1), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic: random N(0,0.02) weights, uniform random token ids, prompts of 128..2048 tokens",

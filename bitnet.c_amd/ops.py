@@ -234,8 +234,9 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, *, allow_library: b
     bf16: up to 16 rows (one MFMA tile of activations) the matrix-core kernel that streams
     the weights once; above that the library's matrix product (as the reference hands its
     batched products to a library, src/gpu_cuda.cu:11571), which from 32 rows on is about
-    twice as fast as the streaming kernel; float32 results from bf16 operands (logits) stay
-    with the streaming kernel, 64 rows at a time; shapes neither takes go to the tiled kernel."""
+    twice as fast as the streaming kernel, with a bf16 or a float32 result (logits); without the
+    library the streaming kernel takes 64 rows at a time; shapes neither takes go to the tiled
+    kernel."""
     require_gpu()
     _dev(x, "x", dims=2)
     _dev(w, "w", x.dtype, 2)
@@ -254,14 +255,17 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, *, allow_library: b
     if x.dtype != torch.bfloat16:
         raise KernelError(f"linear: unsupported dtype {x.dtype}")
     aligned = (x.data_ptr() % 16 == 0) and (w.data_ptr() % 16 == 0)
-    small = M <= SKINNY_ROWS or (M <= 64 and (out_dtype == torch.float32 or not allow_library))
+    small = M <= SKINNY_ROWS or (M <= 64 and not allow_library)
     if small and aligned and skinny_supported(M, N, K, ldx, ldw):
         y = torch.empty((M, N), dtype=out_dtype, device=x.device)
         _check(_fn("skinny_gemm", "bn_skinny_gemm")(_code(out_dtype), x.data_ptr(), w.data_ptr(), y.data_ptr(),
                                                     M, N, K, ldx, ldw, N, 0, 0, _stream()), "skinny_gemm")
         return y
-    if M > SKINNY_ROWS and allow_library and out_dtype == torch.bfloat16:
-        return torch.matmul(x, w.t())
+    if M > SKINNY_ROWS and allow_library:
+        if out_dtype == torch.bfloat16:
+            return torch.matmul(x, w.t())
+        if out_dtype == torch.float32:
+            return torch.mm(x, w.t(), out_dtype=torch.float32)
     if M > 64 and out_dtype == torch.float32 and aligned and skinny_supported(64, N, K, ldx, ldw):
         # float32 results from bf16 operands (logits at many positions): 64 rows at a time
         y = torch.empty((M, N), dtype=out_dtype, device=x.device)

@@ -130,9 +130,10 @@ def test_skinny_gemm_bf16(M, N, K):
     ops = _ops()
     x, w = _rand((M, K), torch.bfloat16, 11), _rand((N, K), torch.bfloat16, 12, 0.05)
     ref = x.double() @ w.double().t()
-    y32 = ops.linear(x.cuda(), w.cuda(), torch.float32)
-    assert rel_err(y32, ref.float()) < 1e-5                       # bf16 products are exact in float32
     for lib in (True, False):                                     # above 16 rows: the library, or this kernel
+        y32 = ops.linear(x.cuda(), w.cuda(), torch.float32, allow_library=lib)
+        assert y32.dtype == torch.float32
+        assert rel_err(y32, ref.float()) < 1e-5                   # bf16 products are exact in float32
         y16 = ops.linear(x.cuda(), w.cuda(), allow_library=lib)
         assert y16.dtype == torch.bfloat16 and close(y16.float(), ref.float(), torch.bfloat16)
 
