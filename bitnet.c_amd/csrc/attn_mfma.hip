@@ -351,6 +351,14 @@ __device__ __forceinline__ void rotate8(uint4& lo, uint4& hi, const float* __res
     }
 }
 
+// A read of p[idx] for an index that is the same in every lane, through the scalar unit (the
+// constant address space makes the compiler pick a scalar load).  Only for memory that no kernel
+// writes while this one runs (block tables, lengths).
+__device__ __forceinline__ int uniform_load(const int* p, size_t idx) {
+    typedef const int __attribute__((address_space(4))) * scalar_ptr;
+    return reinterpret_cast<scalar_ptr>(reinterpret_cast<uintptr_t>(p))[idx];
+}
+
 template <int HS>
 __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
     constexpr int DC = HS / 32, DT = HS / 16, HALF = HS / 2;
@@ -362,8 +370,11 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
     const int n = lane & 15, g = lane >> 4;
     const int G = a.H / a.Hkv, GT = a.GT;
     const int n_head_tiles = (G + GT - 1) / GT;
-    const int kvh = blockIdx.y / n_head_tiles, ht = blockIdx.y - kvh * n_head_tiles;
-    const int seq = blockIdx.x, split = blockIdx.z;
+    // kv heads run fastest in the grid: consecutive workgroups go to different XCDs, so every XCD gets
+    // a share of every sequence, however unequal their lengths (with the sequences fastest and a
+    // batch that is a multiple of 8, a sequence's heads all landed on one XCD)
+    const int kvh = blockIdx.x / n_head_tiles, ht = blockIdx.x - kvh * n_head_tiles;
+    const int seq = blockIdx.y, split = blockIdx.z;
     const int L = a.seq_lens[seq];
     const int hg = ht * GT + n;
     const bool ok = n < GT && hg < G && L > 0;
@@ -435,7 +446,9 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
     if (k_lo < k_hi) {
         const size_t bt_row = (size_t)seq * a.bt_stride;
         for (int kb = (k_lo / 32) * 32 + 32 * wave; kb < k_hi; kb += 128) {
-            const int page = a.block_table[bt_row + kb / BN_PAGE];
+            // the page index is the same for the whole wave: read through the scalar unit, so that it
+            // does not queue behind the vector loads
+            const int page = uniform_load(a.block_table, bt_row + __builtin_amdgcn_readfirstlane(kb / BN_PAGE));
             const int koff = kb % BN_PAGE;
             const bf16* kbase = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS;
             const bf16* vbase = a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff;
@@ -477,7 +490,7 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
     // the last workgroup of this (sequence, kv head, head tile) to arrive merges all splits, in split order
     __threadfence();
     __syncthreads();
-    int* counter = a.counters + ((size_t)seq * gridDim.y + blockIdx.y);
+    int* counter = a.counters + ((size_t)seq * gridDim.x + blockIdx.x);
     if (threadIdx.x == 0) ticket_s = atomicAdd(counter, 1);
     __syncthreads();
     if (ticket_s != a.n_splits - 1) return;
@@ -581,7 +594,8 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
         else hipLaunchKernelGGL((attn_mfma_prompt_kernel<128, 2>), grid, dim3(256), 0, s, a);
         return bn_launch_status();
     }
-    const dim3 grid(n_tiles, Hkv * n_head_tiles, n_splits);
+    if (n_tiles > 65535) return BN_ERR_ARG;                 // sequences are the grid's y
+    const dim3 grid(Hkv * n_head_tiles, n_tiles, n_splits);
     if (hs == 64) hipLaunchKernelGGL(attn_mfma_decode_kernel<64>, grid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL(attn_mfma_decode_kernel<128>, grid, dim3(256), 0, s, a);
     int rc = bn_launch_status();
