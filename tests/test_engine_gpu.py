@@ -14,7 +14,7 @@ from conftest import TOL, rel_err
 pytestmark = pytest.mark.gpu
 
 DTYPES = [torch.float32, torch.bfloat16]
-NAMES = ["A", "B", "C", "D"]
+NAMES = ["A", "B", "C", "D", "E"]
 
 
 def _requests(vocab, seed, lengths):
