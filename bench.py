@@ -2,7 +2,7 @@
 """Decode and prefill throughput of the Llama-3.1-8B shape with random bf16 weights on one
 MI355X.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--shape 8b|13b|70b]
 
 A step is one decode step of the whole batch: the step function, greedy sampling on the
 device and the read-back of the tokens, as generation does it.  `value` is decoded
@@ -24,13 +24,26 @@ sys.path.insert(0, ROOT)
 HBM_GBS = 8000.0
 PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "fp32": 157.3}
 
-# The Llama-3.1-8B shape (the benchmark configuration): context 4,096, prompts of 128..2048 tokens
-SHAPE = dict(model_type="llama", vocab_size=128256, hidden_size=4096, intermediate_size=14336,
-             num_hidden_layers=32, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
-             max_position_embeddings=131072, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
-             rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
-                               original_max_position_embeddings=8192))
-CONTEXT = 4096
+# The benchmark configuration is the Llama-3.1-8B shape: context 4,096, prompts of 128..2048 tokens.
+# The two other shapes are there for measurements at further sizes (--shape); they change nothing
+# in the default record.
+_LLAMA3_SCALING = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                       original_max_position_embeddings=8192)
+SHAPES = {
+    "8b": dict(name="llama-3.1-8b-shape", context=4096, prompt_lens=(128, 2048), config=dict(
+        model_type="llama", vocab_size=128256, hidden_size=4096, intermediate_size=14336,
+        num_hidden_layers=32, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+        max_position_embeddings=131072, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+        rope_scaling=_LLAMA3_SCALING)),
+    "13b": dict(name="llama-2-13b-shape", context=4096, prompt_lens=(64, 2048), config=dict(
+        model_type="llama", vocab_size=32000, hidden_size=5120, intermediate_size=13824,
+        num_hidden_layers=40, num_attention_heads=40, num_key_value_heads=40, head_dim=128,
+        max_position_embeddings=4096, rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)),
+    "70b": dict(name="llama-3-70b-shape", context=8192, prompt_lens=(512, 4096), config=dict(
+        model_type="llama", vocab_size=128256, hidden_size=8192, intermediate_size=28672,
+        num_hidden_layers=80, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
+        max_position_embeddings=8192, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)),
+}
 PREFILL_TOKENS = 2048
 
 
@@ -39,7 +52,9 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=SHAPE["num_hidden_layers"],
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="8b",
+                    help="8b is the benchmark configuration; the others are further sizes")
+    ap.add_argument("--layers", type=int, default=0,
                     help="fewer layers than the configuration has (named in the record)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points")
@@ -60,6 +75,9 @@ def main() -> int:
     from bitnet_c_amd.weights import random_tensors
 
     dev = "cuda:0"
+    shape = SHAPES[args.shape]
+    SHAPE, CONTEXT, (len_lo, len_hi) = shape["config"], shape["context"], shape["prompt_lens"]
+    args.layers = args.layers or SHAPE["num_hidden_layers"]
     raw = dict(SHAPE, num_hidden_layers=args.layers)
     cfg = bn.LlamaConfig.from_dict(raw)
     plan = architecture_for(raw).build_plan(cfg)
@@ -73,7 +91,7 @@ def main() -> int:
           file=sys.stderr, flush=True)
 
     max_batch = max(args.batch, 1 if args.no_points else 64)
-    per_seq = ((2048 + args.steps + args.warmup + 64 + 63) // 64) * 64
+    per_seq = ((len_hi + args.steps + args.warmup + 64 + 63) // 64) * 64
     engine = bn.Engine(model, max_tokens=max(max_batch * per_seq, 4096), max_seq_len=CONTEXT)
     L, H, Hkv, hs = cfg.num_hidden_layers, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
     kv_bytes_per_token = 2 * L * Hkv * hs * 2
@@ -112,7 +130,7 @@ def main() -> int:
 
     # ---- decode -----------------------------------------------------------------------
     def decode(batch, steps, warmup):
-        lens = [rnd.randint(128, 2048) for _ in range(batch)]
+        lens = [rnd.randint(len_lo, len_hi) for _ in range(batch)]
         slots = [engine.new_sequence() for _ in range(batch)]
         # the prompts, a few sequences a step to bound the activations
         last = [0] * batch
@@ -158,16 +176,16 @@ def main() -> int:
             print(f"[bench] decode b{b}: {s_b * 1e3:.3f} ms/step, {b / s_b:.1f} tok/s", file=sys.stderr, flush=True)
 
     rec = {
-        "metric": f"decode tok/s @ batch {args.batch} (Llama-3.1-8B shape, bf16)", "value": round(value, 1), "unit": "tok/s",
+        "metric": f"decode tok/s @ batch {args.batch} ({shape['name']}, bf16)", "value": round(value, 1), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic: random N(0,0.02) weights, uniform random token ids, prompts of 128..2048 tokens",
-        "config": {"model": "llama-3.1-8b-shape", "layers": cfg.num_hidden_layers,
+        "data": f"synthetic: random N(0,0.02) weights, uniform random token ids, prompts of {len_lo}..{len_hi} tokens",
+        "config": {"model": shape["name"], "layers": cfg.num_hidden_layers,
                    "layers_of_config": SHAPE["num_hidden_layers"], "hidden": cfg.hidden_size,
                    "heads": H, "kv_heads": Hkv, "head_dim": hs, "intermediate": cfg.intermediate_size,
-                   "vocab": cfg.vocab_size, "rope_theta": cfg.rope_theta, "rope_scaling": "llama3 f8 l1 h4 o8192",
+                   "vocab": cfg.vocab_size, "rope_theta": cfg.rope_theta, "rope_scaling": "llama3 f8 l1 h4 o8192" if cfg.rope_scaling else "none",
                    "rms_norm_eps": cfg.rms_norm_eps, "tied": cfg.tie_word_embeddings,
-                   "global_batch": args.batch, "seq_len": CONTEXT, "prompt_lens": "U[128,2048]",
+                   "global_batch": args.batch, "seq_len": CONTEXT, "prompt_lens": f"U[{len_lo},{len_hi}]",
                    "prefill_tokens": PREFILL_TOKENS, "parallelism": "none (1 GPU)"},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
