@@ -378,6 +378,54 @@ def test_attention_finds_a_far_key(dtype):
             assert rel_err(out.float(), want) < 1e-3, (far, n_splits)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,hs", [(8, 2, 128), (6, 3, 48)])
+def test_attention_over_a_long_context(dtype, H, Hkv, hs):
+    """20,000 cached positions: a decode row with the split plan the engine would pick, and a
+    prompt chunk of 70 tokens that continues at position 19,930.  The reference is the plain
+    formula for the wanted rows only (scores, softmax, weighted values in float64)."""
+    ops = _ops()
+    L, n_new = 20000, 70
+    k = _rand((L, Hkv, hs), dtype, 400)
+    v = _rand((L, Hkv, hs), dtype, 401)
+    q = _rand((n_new, H, hs), dtype, 402)
+    scale = 1.0 / math.sqrt(hs)
+    kp, vp, bt = _paged([k], [v], dtype, (L + 63) // 64 + 5, 403)
+    kp, vp, bt = kp.cuda(), vp.cuda(), bt.cuda()
+
+    def plain_rows(first_pos):
+        rows = []
+        for t in range(q.shape[0]):
+            n_kv = first_pos + t + 1
+            for h in range(H):
+                kh = h // (H // Hkv)
+                sc = (k[:n_kv, kh].double() @ q[t, h].double()) * scale
+                rows.append(pl.softmax(sc[None, :].float())[0].double() @ v[:n_kv, kh].double())
+        return torch.stack(rows).reshape(q.shape[0], H * hs).float()
+
+    def check(out, ref):
+        if ops.mfma_attention(dtype, hs):
+            assert mfma_close(out.float(), ref)
+        else:
+            assert close(out.float(), ref, dtype)
+
+    qkv = q.reshape(n_new, H * hs).contiguous().cuda()
+    # the chunk of a prompt: rows at positions L - n_new .. L - 1
+    _, _, qt = ops.attention_row_shape(H, Hkv, False, dtype, hs)
+    tiles = torch.tensor([(0, i, min(qt, n_new - i), L - n_new + i) for i in range(0, n_new, qt)], dtype=torch.int32).cuda()
+    out = torch.full((n_new, H * hs), float("nan"), dtype=dtype).cuda()
+    ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, scale, tiles=tiles, qt=qt)
+    ref = plain_rows(L - n_new)
+    check(out, ref)
+    # one decoded token at the last position, split as the engine splits it
+    n_splits, chunk = ops.decode_splits(1, H, Hkv, bt.shape[1] * 64)
+    assert n_splits > 1
+    out1 = torch.full((1, H * hs), float("nan"), dtype=dtype).cuda()
+    ops.attention(qkv[-1:].contiguous(), out1, kp, vp, bt, H, Hkv, hs, scale,
+                  seq_lens=torch.tensor([L], dtype=torch.int32).cuda(), n_splits=n_splits, chunk=chunk)
+    check(out1, ref[-1:])
+
+
 # ---------------------------------------------------------------------------------------
 def test_argmax_ties_and_odd_vocab():
     ops = _ops()
