@@ -22,6 +22,21 @@
 // the 4 waves take 32-key blocks in turn and merge through shared memory; long contexts are
 // also split over gridDim.z and merged by attn_mfma_combine_kernel in a fixed order.
 #include "common.h"
+
+#ifndef PROMPT_NG
+#define PROMPT_NG 0           // groups of 4 waves in a workgroup of the prompt form: 1, 2, or 0 = by the size of the launch
+#endif
+
+static int compute_units() {
+    static int n[64] = {0};                 // per device
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (n[dev] == 0) {
+        int v = 0;
+        n[dev] = (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) ? v : 256;
+    }
+    return n[dev];
+}
 #include <math.h>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -222,24 +237,30 @@ __device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, con
 // ---------------------------------------------------------------------------------------
 // prompt form
 // ---------------------------------------------------------------------------------------
-// The 4 waves of a workgroup need the same keys, so a 32-key block is fetched once per workgroup
-// into shared memory (the next block's loads are in flight while the current one is multiplied),
-// double-buffered, one barrier per block.
-template <int HS, int NT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_mfma_prompt_kernel(MfmaArgs a) {
+// The waves of a workgroup need the same keys, so a stage of keys is fetched once per workgroup
+// into shared memory (the next stage's loads are in flight while the current one is multiplied),
+// double-buffered, one barrier per stage.  A workgroup has NG groups of 4 waves; all groups hold the
+// same query rows and a stage is NG blocks of 32 keys, one for each group, so the chain of blocks
+// that a tile of late positions has to walk is NG times shorter; at the end the groups' partial
+// results (reference point, sum, accumulators) are merged through shared memory in group order.
+template <int HS, int NT, int NG>
+__global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_mfma_prompt_kernel(MfmaArgs a) {
     constexpr int DC = HS / 32, DT = HS / 16;
-    constexpr int KS = HS + 8, VS = 32 + 8;               // padded row strides (elements)
+    constexpr int KB = 32 * NG;                           // keys per stage
+    constexpr int KS = HS + 8, VS = KB + 8;               // padded row strides (elements)
     constexpr int KV4 = 32 * HS / 8 / 256;                // uint4 loads per thread for K (and for V^T)
-    __shared__ __align__(16) bf16 k_s[2][32 * KS];
-    __shared__ __align__(16) bf16 v_s[2][HS * VS];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int STAGE = (KB * KS + HS * VS) * 2;        // bytes of one buffer
+    constexpr int MERGE = NG > 1 ? 4 * 64 * (DT * 4 + 2) * 4 : 0;
+    __shared__ __align__(16) unsigned char smem[(2 * STAGE > MERGE) ? 2 * STAGE : MERGE];
+    auto k_s = [&](int b) { return reinterpret_cast<bf16*>(smem + b * STAGE); };
+    auto v_s = [&](int b) { return reinterpret_cast<bf16*>(smem + b * STAGE) + KB * KS; };
+    const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3, grp = threadIdx.x >> 8;
     const int n = lane & 15, g = lane >> 4;
     const int G = a.H / a.Hkv, GT = a.GT;
     const int n_head_tiles = (G + GT - 1) / GT;
     const int kvh = blockIdx.y / n_head_tiles, ht = blockIdx.y - kvh * n_head_tiles;
     // Later (longer) tiles start first; every other head walks the tiles the other way, so that the
-    // workgroups that share a CU while the whole launch is resident are a long one and a short one
-    // (measured: 4 to 6 % at 2,048 and 4,096 tokens, nothing lost at 8,192).
+    // workgroups that share a CU while the whole launch is resident are a long one and a short one.
     const bool ascending = blockIdx.y & 1;
     const int* tl = a.tiles + 4 * (ascending ? blockIdx.x : gridDim.x - 1 - blockIdx.x);
     const int seq = tl[0], tok0 = tl[1], n_tok = tl[2], pos0 = tl[3];
@@ -285,43 +306,82 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int g_lo = a.window > 0 ? max(0, pos0 + 1 - a.window) : 0;
     const size_t bt_row = (size_t)seq * a.bt_stride;
     uint4 kr[KV4], vr[KV4];
-    auto fetch = [&](int kb) {
+    auto fetch = [&](int kb) {                            // a stage never crosses a page: KB divides BN_PAGE
         const int page = a.block_table[bt_row + kb / BN_PAGE];
         const int koff = kb % BN_PAGE;
-        const bf16* kg = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS;      // 32 rows of HS, contiguous
-        const bf16* vg = a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff;       // HS rows, 32 of 64 keys each
+        const bf16* kg = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS;      // KB rows of HS, contiguous
+        const bf16* vg = a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff;       // HS rows, KB of 64 keys each
 #pragma unroll
         for (int j = 0; j < KV4; ++j) {
-            const int idx = threadIdx.x + 256 * j;
+            const int idx = threadIdx.x + 256 * NG * j;
             kr[j] = *reinterpret_cast<const uint4*>(kg + (size_t)idx * 8);
-            const int vrow = idx >> 2, vcol = (idx & 3) * 8;
+            const int vrow = idx / (KB / 8), vcol = (idx % (KB / 8)) * 8;
             vr[j] = *reinterpret_cast<const uint4*>(vg + (size_t)vrow * BN_PAGE + vcol);
         }
     };
     auto stash = [&](int buf) {
 #pragma unroll
         for (int j = 0; j < KV4; ++j) {
-            const int idx = threadIdx.x + 256 * j;
+            const int idx = threadIdx.x + 256 * NG * j;
             const int krow = (idx * 8) / HS, kchunk = ((idx * 8) % HS) / 8;
-            *reinterpret_cast<uint4*>(&k_s[buf][krow * KS + ((kchunk ^ ((krow >> 3) & 1) * 4) * 8)]) = kr[j];
-            const int vrow = idx >> 2, vcol = (idx & 3) * 8;
-            *reinterpret_cast<uint4*>(&v_s[buf][vrow * VS + vcol]) = vr[j];
+            *reinterpret_cast<uint4*>(k_s(buf) + krow * KS + ((kchunk ^ ((krow >> 3) & 1) * 4) * 8)) = kr[j];
+            const int vrow = idx / (KB / 8), vcol = (idx % (KB / 8)) * 8;
+            *reinterpret_cast<uint4*>(v_s(buf) + vrow * VS + vcol) = vr[j];
         }
     };
-    const int kb0 = (g_lo / 32) * 32;
+    const int kb0 = (g_lo / KB) * KB;
     fetch(kb0);
     stash(0);
     __syncthreads();
     int buf = 0;
-    for (int kb = kb0; kb <= g_hi; kb += 32, buf ^= 1) {
-        const bool more = kb + 32 <= g_hi;
-        if (more) fetch(kb + 32);
-        if (w_hi >= 0 && kb <= w_hi && kb + 31 >= w_lo) {
-            const bool need_mask = (kb + 31 > all_hi) || (kb < all_lo);
-            attend_block<HS, NT, KS, VS, true>(k_s[buf], v_s[buf], kb, q, acc, m, l, qpos, lo, w_hi + 1, need_mask, scale2, lane);
+    for (int kb = kb0; kb <= g_hi; kb += KB, buf ^= 1) {
+        const bool more = kb + KB <= g_hi;
+        if (more) fetch(kb + KB);
+        const int kbb = kb + 32 * grp;                    // this group's block of the stage
+        if (w_hi >= 0 && kbb <= w_hi && kbb + 31 >= w_lo) {
+            const bool need_mask = (kbb + 31 > all_hi) || (kbb < all_lo);
+            attend_block<HS, NT, KS, VS, true>(k_s(buf) + 32 * grp * KS, v_s(buf) + 32 * grp, kbb, q, acc, m, l, qpos, lo,
+                                               w_hi + 1, need_mask, scale2, lane);
         }
         if (more) stash(buf ^ 1);
         __syncthreads();
+    }
+    if (NG > 1) {
+        // the later groups hand their partial results to group 0, one column tile a time; the staging
+        // memory is free now (the loop ended with a barrier)
+        float* x_s = reinterpret_cast<float*>(smem);      // [wave][slot][lane]
+        constexpr int SLOTS = DT * 4 + 2;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            for (int src = 1; src < NG; ++src) {
+                float* mine = x_s + ((size_t)wave * SLOTS) * 64 + lane;
+                if (grp == src) {
+                    mine[0] = m[nt];
+                    mine[64] = l[nt];
+#pragma unroll
+                    for (int t = 0; t < DT; ++t)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) mine[(2 + t * 4 + r) * 64] = acc[nt][t][r];
+                }
+                __syncthreads();
+                if (grp == 0) {
+                    const float m1 = mine[0], l1 = mine[64];
+                    const float M = fmaxf(m[nt], m1);
+                    if (M != -INFINITY) {
+                        const float a0 = m[nt] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[nt] - M);
+                        const float a1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - M);
+                        l[nt] = l[nt] * a0 + l1 * a1;
+#pragma unroll
+                        for (int t = 0; t < DT; ++t)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) acc[nt][t][r] = acc[nt][t][r] * a0 + mine[(2 + t * 4 + r) * 64] * a1;
+                        m[nt] = M;
+                    }
+                }
+                __syncthreads();
+            }
+        }
+        if (grp != 0) return;
     }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -594,8 +654,15 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
     a.inv_freq = inv_freq; a.rotate = rotate; a.write_kv = write_kv; a.counters = counters;
     if (tiles) {
         const dim3 grid(n_tiles, Hkv * n_head_tiles);
-        if (hs == 64) hipLaunchKernelGGL((attn_mfma_prompt_kernel<64, 4>), grid, dim3(256), 0, s, a);
-        else hipLaunchKernelGGL((attn_mfma_prompt_kernel<128, 2>), grid, dim3(256), 0, s, a);
+        // Two wave groups halve the chain of key blocks of a workgroup but not the work of its CU:
+        // they pay (measured 19 % at 1,024 tokens of the 8B shape) only while there are no more
+        // workgroups than CUs, so that each has a CU to itself.
+        int ng = PROMPT_NG;
+        if (ng == 0) ng = ((long long)grid.x * grid.y <= compute_units()) ? 2 : 1;
+        if (hs == 64 && ng == 2) hipLaunchKernelGGL((attn_mfma_prompt_kernel<64, 4, 2>), grid, dim3(512), 0, s, a);
+        else if (hs == 64) hipLaunchKernelGGL((attn_mfma_prompt_kernel<64, 4, 1>), grid, dim3(256), 0, s, a);
+        else if (ng == 2) hipLaunchKernelGGL((attn_mfma_prompt_kernel<128, 2, 2>), grid, dim3(512), 0, s, a);
+        else hipLaunchKernelGGL((attn_mfma_prompt_kernel<128, 2, 1>), grid, dim3(256), 0, s, a);
         return bn_launch_status();
     }
     if (n_tiles > 65535) return BN_ERR_ARG;                 // sequences are the grid's y

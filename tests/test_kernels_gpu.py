@@ -319,6 +319,20 @@ def test_attention_prompt_form(dtype, H, Hkv, hs, window, force_vector):
     assert mfma_close(out.float(), ref) if ops.mfma_attention(dtype, hs) and not force_vector else close(out.float(), ref, dtype)
 
 
+@pytest.mark.parametrize("H,Hkv,hs,T", [(32, 8, 128, 1200), (32, 8, 64, 2200)])
+def test_attention_prompt_form_with_more_workgroups_than_cus(H, Hkv, hs, T):
+    """One long prompt: the launch has more workgroups than the chip has CUs, which is where the
+    matrix-core kernel runs its workgroups with one group of waves instead of two."""
+    dtype = torch.bfloat16
+    ops, qkv, kp, vp, bt, ref, scale = _attn_case(dtype, H, Hkv, hs, [0], [T], 0, 500)
+    _, _, qt = ops.attention_row_shape(H, Hkv, False, dtype, hs)
+    tiles = [(0, i, min(qt, T - i), i) for i in range(0, T, qt)]
+    assert len(tiles) * Hkv > 256
+    out = torch.full((T, H * hs), float("nan"), dtype=dtype).cuda()
+    ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, scale, tiles=torch.tensor(tiles, dtype=torch.int32).cuda(), qt=qt)
+    assert mfma_close(out.float(), ref)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,Hkv,hs,window", [(4, 2, 16, 0), (5, 5, 24, 0), (8, 2, 128, 0), (12, 4, 64, 0),
                                              (16, 1, 32, 0), (4, 2, 16, 50), (8, 8, 64, 129), (32, 8, 128, 0),
