@@ -68,6 +68,11 @@ struct MfmaArgs {
     const float* inv_freq;
     int rotate, write_kv;
     int* counters;
+    // by_length != null: the sequences ordered by length, longest first.  Workgroups are handed out
+    // in that order, every other run of `order_period` sequences backwards: when the launch puts
+    // two workgroups on every CU, the ones that share a CU are then a long and a short sequence.
+    const int* by_length;
+    int order_period;
 };
 
 __device__ __forceinline__ bf16x8 ld16(const bf16* p) {
@@ -438,7 +443,20 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
     // a share of every sequence, however unequal their lengths (with the sequences fastest and a
     // batch that is a multiple of 8, a sequence's heads all landed on one XCD)
     const int kvh = blockIdx.x / n_head_tiles, ht = blockIdx.x - kvh * n_head_tiles;
-    const int seq = blockIdx.y, split = blockIdx.z;
+    int seq = blockIdx.y;
+    const int split = blockIdx.z;
+    if (a.by_length) {
+        int r = seq;
+        if (a.order_period > 0) {
+            const int run = r / a.order_period;
+            if (run & 1) {
+                const int first = run * a.order_period, last = min(first + a.order_period, (int)gridDim.y) - 1;
+                r = first + (last - r);
+            }
+        }
+        seq = a.by_length[r];
+        if ((unsigned)seq >= gridDim.y) return;          // not a permutation: touch nothing
+    }
     const int L = a.seq_lens[seq];
     const int hg = ht * GT + n;
     const bool ok = n < GT && hg < G && L > 0;
@@ -632,7 +650,8 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
                             const void* vt_pages, const int* block_table, int bt_stride, const int* seq_lens,
                             const int* tiles, int n_tiles, int n_tokens, int H, int Hkv, int hs, int GT,
                             int window, float scale, int n_splits, int chunk, float* part_o, float* part_ml,
-                            const float* inv_freq, int rotate, int write_kv, int* counters, hipStream_t s) {
+                            const float* inv_freq, int rotate, int write_kv, int* counters, const int* by_length,
+                            hipStream_t s) {
     if (!bn_attn_mfma_supports(hs) || n_tiles <= 0 || n_tokens <= 0 || H <= 0 || Hkv <= 0 || H % Hkv) return BN_ERR_ARG;
     if (GT <= 0 || GT > 16 || (GT & (GT - 1)) || window < 0 || n_splits < 1 || n_splits > 64) return BN_ERR_ARG;
     if (n_splits > 1 && (chunk <= 0 || chunk % BN_PAGE || !part_o || !part_ml)) return BN_ERR_ARG;
@@ -652,6 +671,10 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
     a.H = H; a.Hkv = Hkv; a.GT = GT; a.window = window; a.scale = scale;
     a.n_splits = n_splits; a.chunk = n_splits > 1 ? chunk : 0x40000000;
     a.inv_freq = inv_freq; a.rotate = rotate; a.write_kv = write_kv; a.counters = counters;
+    // the order matters only when the launch holds more workgroups than CUs and no sequence is split
+    const int wgs_per_seq = Hkv * n_head_tiles;
+    a.by_length = (!tiles && n_splits == 1 && (long long)n_tiles * wgs_per_seq > compute_units()) ? by_length : nullptr;
+    a.order_period = compute_units() / wgs_per_seq;
     if (tiles) {
         const dim3 grid(n_tiles, Hkv * n_head_tiles);
         // Two wave groups halve the chain of key blocks of a workgroup but not the work of its CU:

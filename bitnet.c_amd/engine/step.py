@@ -40,8 +40,11 @@ class StepContext:
     """Device-side description of one step, shared by all parts."""
 
     def __init__(self, device, act_dtype, tokens, positions, seq_index, seq_lens, want_rows, slots_dev,
-                 is_decode, slots, n_new, pos0):
+                 is_decode, slots, n_new, pos0, by_length=None):
         self.device, self.act_dtype = device, act_dtype
+        # decode steps: the rows ordered by sequence length, longest first (a hint for kernels that
+        # balance their workgroups by it; None = no hint)
+        self.by_length = by_length
         self.tokens, self.positions, self.seq_index = tokens, positions, seq_index
         self.seq_lens, self.want_rows, self.slot_ids = seq_lens, want_rows, slots_dev
         self.is_decode = is_decode
@@ -73,6 +76,11 @@ class StepContext:
         return t
 
 
+def _by_length(lens) -> List[int]:
+    """The rows ordered by length, longest first (ties by row)."""
+    return sorted(range(len(lens)), key=lambda i: (-lens[i], i))
+
+
 def _bucket(n: int) -> int:
     b = 1
     while b < n:
@@ -88,7 +96,7 @@ class _DecodeGraph:
         self.rows, self.width = rows, width
         dev = engine.device
         n_groups = len(engine.cache.groups)
-        self.n_ints = 5 * rows + n_groups * rows * width
+        self.n_ints = 6 * rows + n_groups * rows * width
         self.host = torch.zeros(self.n_ints, dtype=torch.int32).pin_memory()
         self.dev = torch.zeros(self.n_ints, dtype=torch.int32, device=dev)
         self.copied = torch.cuda.Event()
@@ -102,11 +110,11 @@ class _DecodeGraph:
             return v
 
         self.tokens, self.positions, self.seq_index = take(rows), take(rows), take(rows)
-        self.seq_lens, self.want = take(rows), take(rows)
+        self.seq_lens, self.want, self.by_length = take(rows), take(rows), take(rows)
         self.tables = {g: take(rows * width).view(rows, width) for g in range(n_groups)}
         views = [engine.cache.view(i, self.tables, width * PAGE) for i in range(len(engine.model.plan.schedule))]
         self.ctx = StepContext(dev, engine.model.dtype, self.tokens, self.positions, self.seq_index, self.seq_lens,
-                               self.want, None, True, [-1] * rows, [1] * rows, [0] * rows)
+                               self.want, None, True, [-1] * rows, [1] * rows, [0] * rows, by_length=self.by_length)
         # padding rows everywhere: the warm-up and the capture run touch no sequence's pages
         self.fill([-1] * rows, [0] * rows, [0] * rows, engine)
         self.upload()
@@ -134,7 +142,8 @@ class _DecodeGraph:
         h[2 * rows:3 * rows] = torch.arange(rows, dtype=torch.int32)  # row b is sequence b
         h[3 * rows:3 * rows + n] = torch.tensor([max(l, 0) for l in lens_after], dtype=torch.int32)
         h[4 * rows:5 * rows] = torch.arange(rows, dtype=torch.int32)
-        o = 5 * rows
+        h[5 * rows:6 * rows] = torch.tensor(_by_length(list(lens_after) + [0] * (rows - n)), dtype=torch.int32)
+        o = 6 * rows
         for g in range(len(engine.cache.groups)):
             bt = engine.cache.block_table(g, list(slots) + [-1] * (rows - n), self.width)
             h[o:o + rows * self.width] = bt[:, :self.width].reshape(-1)
@@ -255,8 +264,9 @@ class Engine:
         lens_after = [p + n for p, n in zip(pos0, n_new)]
         tables = {g: self.cache.block_table(g, slots) for g in range(len(self.cache.groups))}
         # one upload for all integer inputs of the step
-        parts = [tokens, positions, seq_index, lens_after, want, slots] + [tables[g].reshape(-1).tolist()
-                                                                            for g in sorted(tables)]
+        order = _by_length(lens_after) if is_decode else []
+        parts = [tokens, positions, seq_index, lens_after, want, slots, order] + [tables[g].reshape(-1).tolist()
+                                                                                   for g in sorted(tables)]
         flat = torch.tensor([v for p in parts for v in p], dtype=torch.int32)
         devbuf = flat.to(dev)
         o = 0
@@ -268,9 +278,10 @@ class Engine:
             return v
 
         d_tokens, d_pos, d_seq, d_lens, d_want, d_slots = take(T), take(T), take(T), take(B), take(len(want)), take(B)
+        d_order = take(len(order)) if is_decode else None
         d_tables = {g: take(tables[g].numel()).view(tables[g].shape) for g in sorted(tables)}
         ctx = StepContext(dev, self.model.dtype, d_tokens, d_pos, d_seq, d_lens, d_want, d_slots, is_decode,
-                          slots, n_new, pos0)
+                          slots, n_new, pos0, by_length=d_order)
         max_len = max(lens_after)
         views = [self.cache.view(i, d_tables, max_len) for i in range(len(self.model.plan.schedule))]
         return self.model.forward(ctx, views)

@@ -46,7 +46,7 @@ _SIGNATURES = {
         "bn_attn_mfma_prompt_tokens": [c_int, c_int],
         "bn_attn_mfma": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p,
-                         c_void_p, c_int, c_int, c_void_p, c_void_p],
+                         c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p],
     },
     "gemm_tiled": {
         "bn_gemm_tiled": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
@@ -445,7 +445,7 @@ def can_fuse_decode(dtype, H: int, Hkv: int, hs: int) -> bool:
 def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
               block_table: torch.Tensor, H: int, Hkv: int, hs: int, scale: float, *, window: int = 0,
               tiles=None, qt: int = 0, seq_lens=None, n_splits: int = 1, chunk: int = 0,
-              force_vector: bool = False, fused_rotate=None, fused_write: bool = False) -> None:
+              force_vector: bool = False, fused_rotate=None, fused_write: bool = False, by_length=None) -> None:
     """Causal attention of the (rotated) Q heads in qkv over the paged cache.
 
     Prompt form: `tiles` [n, 4] int32 = (sequence, first token row, tokens (<= qt), position of
@@ -457,7 +457,10 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     attention_row_shape without dtype).
     Decode on the matrix cores can do the work of rope_kv_write itself (can_fuse_decode):
     fused_rotate = inv_freq [hs/2]: qkv arrives unrotated, Q and the new K are rotated inside;
-    fused_write: the new K, V of every row (from qkv) are stored at position seq_lens - 1 first."""
+    fused_write: the new K, V of every row (from qkv) are stored at position seq_lens - 1 first.
+    by_length (decode form, optional): [B] int32, a permutation of the rows, longest sequence
+    first; the matrix-core kernel hands out its workgroups in that order when a launch puts several
+    on every CU, so that long and short sequences share CUs.  It changes no result."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(out, "out", qkv.dtype, 2)
@@ -501,6 +504,10 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     pm = part_ml.data_ptr() if part_ml is not None else None
     sl = seq_lens.data_ptr() if decode else None
     tl = tiles.data_ptr() if not decode else None
+    if by_length is not None:
+        _dev(by_length, "by_length", torch.int32, 1)
+        if not decode or by_length.numel() != T or not by_length.is_contiguous():
+            raise KernelError("attention: by_length is one entry per row of the decode form")
     fused = fused_rotate is not None or fused_write
     if fused and not (use_mfma and decode and can_fuse_decode(qkv.dtype, H, Hkv, hs)):
         raise KernelError("attention: rotation / cache write inside the kernel needs the decode form on the "
@@ -521,7 +528,8 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
             block_table.data_ptr(), block_table.shape[1], sl, tl, n_tiles, T, H, Hkv, hs, GT, int(window),
             float(scale), int(n_splits), int(chunk), po, pm,
             fused_rotate.data_ptr() if fused_rotate is not None else None, int(fused_rotate is not None),
-            int(bool(fused_write)), counters.data_ptr() if counters is not None else None, _stream()),
+            int(bool(fused_write)), counters.data_ptr() if counters is not None else None,
+            by_length.data_ptr() if by_length is not None else None, _stream()),
             "attention(mfma)")
         return
     _check(_fn("attn_rows", "bn_attn_rows")(

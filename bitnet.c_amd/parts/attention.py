@@ -81,7 +81,7 @@ class Attention(Part):
                 n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
                           window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
-                          fused_rotate=inv_freq, fused_write=kv.writes)
+                          fused_rotate=inv_freq, fused_write=kv.writes, by_length=ctx.by_length)
             return self.o(out)
         self.position.encode_and_store(qkv, ctx, H, Hkv, hs, kv)
         if ctx.is_decode:
@@ -90,7 +90,8 @@ class Attention(Part):
             else:
                 n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
-                          window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk)
+                          window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
+                          by_length=ctx.by_length)
         else:
             _, _, qt = ops.attention_row_shape(H, Hkv, False, h.dtype, hs)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,

@@ -369,6 +369,28 @@ def test_attention_decode_form(dtype, H, Hkv, hs, window, force_splits, force_ve
     assert float(out[B:].float().abs().sum()) == 0.0
 
 
+def test_decode_attention_handed_out_by_length():
+    """70 sequences of unequal lengths, 8 kv heads: more workgroups than CUs, so the matrix-core
+    kernel hands them out by length when it is given the order.  The result is the plain one,
+    and bit for bit the one without the hint."""
+    dtype, H, Hkv, hs = torch.bfloat16, 8, 8, 128
+    rnd = random.Random(7)
+    lens_before = [rnd.randrange(0, 200) for _ in range(70)]
+    ops, qkv, kp, vp, bt, ref, scale = _attn_case(dtype, H, Hkv, hs, lens_before, [1] * 70, 0, 600)
+    lens = [p + 1 for p in lens_before]
+    d_lens = torch.tensor(lens, dtype=torch.int32).cuda()
+    order = sorted(range(70), key=lambda i: (-lens[i], i))
+    outs = []
+    for hint in (None, torch.tensor(order, dtype=torch.int32).cuda()):
+        out = torch.full((70, H * hs), float("nan"), dtype=dtype).cuda()
+        ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, scale, seq_lens=d_lens, by_length=hint)
+        outs.append(out.cpu())
+    assert mfma_close(outs[1].float(), ref)
+    assert torch.equal(outs[0], outs[1])
+    with pytest.raises(ops.KernelError):
+        ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, scale, seq_lens=d_lens, by_length=d_lens[:5].contiguous())
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_finds_a_far_key(dtype):
     """One key among 900 has a large score with the query: the output must be its value row,
