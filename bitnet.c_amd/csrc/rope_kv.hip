@@ -66,6 +66,95 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
     }
 }
 
+// bf16 with 8-element groups: the same work with 16-byte loads and stores (one thread rotates the 8
+// pairs of two 16-byte groups).  Needs hs, rope_dims / 2 and row_stride to be multiples of 8 and
+// 16-byte aligned buffers.
+__device__ __forceinline__ void rotate_groups(uint4& lo, uint4& hi, const float* __restrict__ c,
+                                              const float* __restrict__ sn) {
+    uint32_t* pl = reinterpret_cast<uint32_t*>(&lo);
+    uint32_t* ph = reinterpret_cast<uint32_t*>(&hi);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float a0 = bf16lo_to_f32(pl[k]), a1 = bf16hi_to_f32(pl[k]);
+        const float b0 = bf16lo_to_f32(ph[k]), b1 = bf16hi_to_f32(ph[k]);
+        const float c0 = c[2 * k], c1 = c[2 * k + 1], s0 = sn[2 * k], s1 = sn[2 * k + 1];
+        const bf16 l0 = __float2bfloat16(a0 * c0 - b0 * s0), l1 = __float2bfloat16(a1 * c1 - b1 * s1);
+        const bf16 h0 = __float2bfloat16(a0 * s0 + b0 * c0), h1 = __float2bfloat16(a1 * s1 + b1 * c1);
+        pl[k] = (uint32_t)__builtin_bit_cast(uint16_t, l0) | ((uint32_t)__builtin_bit_cast(uint16_t, l1) << 16);
+        ph[k] = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
+    }
+}
+
+__global__ __launch_bounds__(256) void rope_kv_write_bf16x8_kernel(bf16* __restrict__ qkv, int row_stride,
+                                                                   const int* __restrict__ positions,
+                                                                   const int* __restrict__ seq_index,
+                                                                   const int* __restrict__ block_table, int bt_stride,
+                                                                   bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
+                                                                   const float* __restrict__ inv_freq, int rope_dims,
+                                                                   int H, int Hkv, int hs, int v_transposed) {
+    extern __shared__ float cs[];            // cos[half], sin[half]
+    const int t = blockIdx.x;
+    const int pos = positions[t];
+    if (pos < 0) return;                     // a padding row
+    const int half = rope_dims / 2;
+    float* cos_s = cs;
+    float* sin_s = cs + half;
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        float s, c;
+        sincosf((float)pos * inv_freq[i], &s, &c);
+        cos_s[i] = c;
+        sin_s[i] = s;
+    }
+    __syncthreads();
+    bf16* row = qkv + (size_t)t * row_stride;
+    const int hg = half / 8;                 // 16-byte groups in half a rotated head
+    // Q in place
+    for (int idx = threadIdx.x; idx < H * hg; idx += blockDim.x) {
+        const int h = idx / hg, c = idx - h * hg;
+        uint4* lo = reinterpret_cast<uint4*>(row + h * hs + c * 8);
+        uint4* hi = reinterpret_cast<uint4*>(row + h * hs + half + c * 8);
+        uint4 a = *lo, b = *hi;
+        rotate_groups(a, b, cos_s + c * 8, sin_s + c * 8);
+        *lo = a;
+        *hi = b;
+    }
+    if (k_pages == nullptr) return;
+    const int page = block_table[(size_t)seq_index[t] * bt_stride + pos / BN_PAGE];
+    const int off = pos % BN_PAGE;
+    const bf16* krow = row + H * hs;
+    const bf16* vrow = krow + Hkv * hs;
+    // K: the rotated pairs, then what lies beyond rope_dims as it is
+    for (int idx = threadIdx.x; idx < Hkv * hg; idx += blockDim.x) {
+        const int kh = idx / hg, c = idx - kh * hg;
+        uint4 a = *reinterpret_cast<const uint4*>(krow + kh * hs + c * 8);
+        uint4 b = *reinterpret_cast<const uint4*>(krow + kh * hs + half + c * 8);
+        rotate_groups(a, b, cos_s + c * 8, sin_s + c * 8);
+        bf16* dst = k_pages + (((size_t)page * Hkv + kh) * BN_PAGE + off) * hs;
+        *reinterpret_cast<uint4*>(dst + c * 8) = a;
+        *reinterpret_cast<uint4*>(dst + half + c * 8) = b;
+    }
+    const int tail = (hs - rope_dims) / 8;
+    for (int idx = threadIdx.x; idx < Hkv * tail; idx += blockDim.x) {
+        const int kh = idx / tail, c = idx - kh * tail;
+        bf16* dst = k_pages + (((size_t)page * Hkv + kh) * BN_PAGE + off) * hs;
+        *reinterpret_cast<uint4*>(dst + rope_dims + c * 8) = *reinterpret_cast<const uint4*>(krow + kh * hs + rope_dims + c * 8);
+    }
+    // V
+    const int vg = hs / 8;
+    for (int idx = threadIdx.x; idx < Hkv * vg; idx += blockDim.x) {
+        const int kh = idx / vg, c = idx - kh * vg;
+        const uint4 v = *reinterpret_cast<const uint4*>(vrow + kh * hs + c * 8);
+        if (v_transposed) {                  // V pages [page, kv_head, head_dim, BN_PAGE]
+            const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
+            uint16_t* dst = reinterpret_cast<uint16_t*>(v_pages) + (((size_t)page * Hkv + kh) * hs + c * 8) * BN_PAGE + off;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) dst[(size_t)j * BN_PAGE] = e[j];
+        } else {
+            *reinterpret_cast<uint4*>(v_pages + (((size_t)page * Hkv + kh) * BN_PAGE + off) * hs + c * 8) = v;
+        }
+    }
+}
+
 // qkv: [n_tokens, row_stride] with Q heads first, then K heads, then V heads.
 // k_pages == null: rotate Q only (a layer that reads another layer's cache).
 // rope_dims == 0: no rotation, the write alone.
@@ -83,6 +172,11 @@ extern "C" int bn_rope_kv_write(int dtype, void* qkv, int row_stride, const int*
         hipLaunchKernelGGL(rope_kv_write_kernel<float>, dim3(n_tokens), dim3(256), smem, s,
                            (float*)qkv, row_stride, positions, seq_index, block_table, bt_stride,
                            (float*)k_pages, (float*)v_pages, inv_freq, rope_dims, H, Hkv, hs, v_transposed);
+    else if (dtype == BN_DT_BF16 && rope_dims > 0 && hs % 8 == 0 && rope_dims % 16 == 0 && row_stride % 8 == 0 &&
+             !(((uintptr_t)qkv | (uintptr_t)k_pages | (uintptr_t)v_pages) & 15))
+        hipLaunchKernelGGL(rope_kv_write_bf16x8_kernel, dim3(n_tokens), dim3(256), smem, s,
+                           (bf16*)qkv, row_stride, positions, seq_index, block_table, bt_stride,
+                           (bf16*)k_pages, (bf16*)v_pages, inv_freq, rope_dims, H, Hkv, hs, v_transposed);
     else if (dtype == BN_DT_BF16)
         hipLaunchKernelGGL(rope_kv_write_kernel<bf16>, dim3(n_tokens), dim3(256), smem, s,
                            (bf16*)qkv, row_stride, positions, seq_index, block_table, bt_stride,

@@ -201,7 +201,7 @@ def _paged(seqs_k, seqs_v, dtype, n_pages, seed):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,Hkv,hs,rope_dims", [(4, 2, 16, 16), (6, 3, 40, 24), (5, 5, 24, 24), (8, 1, 128, 128),
-                                                 (2, 2, 256, 64)])
+                                                 (2, 2, 256, 64), (8, 2, 64, 32)])
 def test_rope_kv_write(dtype, H, Hkv, hs, rope_dims):
     ops = _ops()
     lens_before, n_new = [0, 70, 130], [5, 1, 66]
