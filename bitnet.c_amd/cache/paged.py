@@ -87,6 +87,7 @@ class PagedCache:
         may hold together, each sequence's count rounded up to a multiple of PAGE."""
         if max_tokens < PAGE:
             raise CacheError(f"max_tokens {max_tokens} is below one page ({PAGE})")
+        self.tables_version = 0          # grows whenever any sequence's list of pages changes
         self.n_pages = max_tokens // PAGE
         self.max_slots = int(max_slots) if max_slots else self.n_pages
         self.dtype, self.device = dtype, device
@@ -134,6 +135,7 @@ class PagedCache:
             raise CacheFull(f"all {self.max_slots} sequence slots are in use")
         s = self._free_slots.pop()
         self._len[s] = 0
+        self.tables_version += 1
         for g in self.groups:
             g.pages[s] = []
         for t in self.states.values():
@@ -143,6 +145,7 @@ class PagedCache:
     def free_slot(self, slot: int) -> None:
         if slot not in self._len:
             raise CacheError(f"slot {slot} is freed but is not in use")
+        self.tables_version += 1
         for g in self.groups:
             g.pool.give_back([p for p in g.pages.pop(slot) if p >= 0])
         del self._len[slot]
@@ -182,6 +185,7 @@ class PagedCache:
         for g, s, need in plan:
             if need:
                 g.pages[s].extend(g.pool.take(need))
+                self.tables_version += 1
 
     def commit(self, slots: Sequence[int], n_new: Sequence[int]) -> None:
         """The step has run: lengths grow; groups that keep a window give back the pages that
@@ -196,6 +200,7 @@ class PagedCache:
                         if pl[i] >= 0 and PAGE * i + PAGE - 1 < first_visible:
                             g.pool.give_back([pl[i]])
                             pl[i] = -1
+                            self.tables_version += 1
 
     # ---- views ------------------------------------------------------------------
     def group_of(self, entry: int) -> Optional[int]:

@@ -98,6 +98,10 @@ class _DecodeGraph:
         n_groups = len(engine.cache.groups)
         self.n_ints = 6 * rows + n_groups * rows * width
         self.host = torch.zeros(self.n_ints, dtype=torch.int32).pin_memory()
+        self.host_np = self.host.numpy()                      # the same memory
+        self.host_np[2 * rows:3 * rows] = range(rows)         # row b is sequence b
+        self.host_np[4 * rows:5 * rows] = range(rows)         # wanted rows: all
+        self._tables_key = None
         self.dev = torch.zeros(self.n_ints, dtype=torch.int32, device=dev)
         self.copied = torch.cuda.Event()
         self.copied.record()
@@ -129,25 +133,26 @@ class _DecodeGraph:
             self.logits = engine.model.forward(self.ctx, views)
 
     def fill(self, slots, tokens, lens_after, engine):
-        rows, h = self.rows, self.host
+        """Writes the step's integers into the pinned buffer.  The block tables are rewritten only
+        when the slots or any sequence's pages have changed since the last fill."""
+        rows, h = self.rows, self.host_np
         self.copied.synchronize()
         n = len(slots)
-        h.zero_()
-        h[0:n] = torch.tensor(tokens, dtype=torch.int32)
-        h[rows:rows + n] = torch.tensor([l - 1 for l in lens_after], dtype=torch.int32)
-        h[rows + n:2 * rows] = -1                                     # padding rows: position -1
-        for i, s in enumerate(slots):
-            if s < 0:
-                h[rows + i] = -1
-        h[2 * rows:3 * rows] = torch.arange(rows, dtype=torch.int32)  # row b is sequence b
-        h[3 * rows:3 * rows + n] = torch.tensor([max(l, 0) for l in lens_after], dtype=torch.int32)
-        h[4 * rows:5 * rows] = torch.arange(rows, dtype=torch.int32)
-        h[5 * rows:6 * rows] = torch.tensor(_by_length(list(lens_after) + [0] * (rows - n)), dtype=torch.int32)
-        o = 6 * rows
-        for g in range(len(engine.cache.groups)):
-            bt = engine.cache.block_table(g, list(slots) + [-1] * (rows - n), self.width)
-            h[o:o + rows * self.width] = bt[:, :self.width].reshape(-1)
-            o += rows * self.width
+        h[0:rows] = 0
+        h[0:n] = tokens
+        h[rows:2 * rows] = -1                                         # padding rows: position -1
+        h[rows:rows + n] = [l - 1 if s >= 0 else -1 for s, l in zip(slots, lens_after)]
+        h[3 * rows:4 * rows] = 0
+        h[3 * rows:3 * rows + n] = [max(l, 0) for l in lens_after]
+        h[5 * rows:6 * rows] = _by_length(list(lens_after) + [0] * (rows - n))
+        key = (tuple(slots), engine.cache.tables_version)
+        if key != self._tables_key:
+            o = 6 * rows
+            for g in range(len(engine.cache.groups)):
+                bt = engine.cache.block_table(g, list(slots) + [-1] * (rows - n), self.width)
+                h[o:o + rows * self.width] = bt[:, :self.width].reshape(-1).numpy()
+                o += rows * self.width
+            self._tables_key = key
 
     def upload(self):
         self.dev.copy_(self.host, non_blocking=True)
