@@ -53,8 +53,14 @@ TINY_E = dict(
     vocab_size=300, hidden_size=192, intermediate_size=520, num_hidden_layers=2,
     num_attention_heads=8, num_key_value_heads=2, head_dim=128, max_position_embeddings=2048,
     rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=True)
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
-SEEDS = {"A": 0, "B": 2, "C": 5, "D": 7, "E": 11}
+# one layer with eight kv heads: a batch of 40 is more attention workgroups than the chip has CUs
+TINY_F = dict(
+    model_type="llama", architectures=["LlamaForCausalLM"],
+    vocab_size=150, hidden_size=80, intermediate_size=136, num_hidden_layers=1,
+    num_attention_heads=16, num_key_value_heads=8, head_dim=64, max_position_embeddings=512,
+    rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "F": TINY_F}
+SEEDS = {"A": 0, "B": 2, "C": 5, "D": 7, "E": 11, "F": 13}
 
 
 @pytest.fixture(scope="session")

@@ -321,3 +321,30 @@ def test_more_sequences_than_a_graph_takes_and_a_long_context(model_folders, dty
     eng.release(s)
     assert rel_err(torch.cat(outs), plain_logits(folder, long_req, dtype)[999:]) < TOL[dtype]
     eng.cache.check()
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+def test_forty_sequences_of_unequal_lengths_with_eight_kv_heads(model_folders, graphs):
+    """More attention workgroups than CUs in a decode step: the kernel then hands them out by
+    sequence length (the step context carries the order).  Every sequence's logits are the plain
+    ones; sequences end at different steps, so the order changes from step to step."""
+    from bitnet_c_amd import StepEntry
+    dtype = torch.bfloat16
+    folder = model_folders("F", dtype)
+    eng = make_engine(folder, dtype, max_tokens=64 * 100, use_graphs=graphs)
+    rnd = random.Random(21)
+    reqs = [[rnd.randrange(eng.vocab_size) for _ in range(rnd.randrange(3, 90) + 2 + i % 4)] for i in range(40)]
+    n_dec = [2 + i % 4 for i in range(40)]
+    slots = [eng.new_sequence() for _ in reqs]
+    eng.step([StepEntry(s, r[:-d], []) for s, r, d in zip(slots, reqs, n_dec)])
+    got = [[] for _ in reqs]
+    fed = [len(r) - d for r, d in zip(reqs, n_dec)]
+    live = list(range(40))
+    while live:
+        out = eng.step([StepEntry(slots[i], [reqs[i][fed[i]]], [0]) for i in live])
+        for r, i in enumerate(live):
+            got[i].append(out[r:r + 1])
+            fed[i] += 1
+        live = [i for i in live if fed[i] < len(reqs[i])]
+    for i in range(40):
+        assert rel_err(torch.cat(got[i]), plain_logits(folder, reqs[i], dtype)[-n_dec[i]:]) < TOL[dtype], i
