@@ -1,6 +1,7 @@
 """Each part alone against the plain implementation; the order of layers as data (a layer named
-twice, a layer that reads another layer's cache); and a toy mixer with a state of its own,
-defined here, registered, built and stepped without a change to the library's files."""
+twice, a layer that reads another layer's cache); and toy parts defined here, registered, built
+and stepped without a change to the library's files: a mixer with a state of its own, a
+feed-forward with routing, another position encoding."""
 import json
 import math
 import os
@@ -402,3 +403,153 @@ def test_a_windowed_group_beside_a_full_one_through_the_engine(tmp_path):
             eng.release(s)
         eng.cache.check()
         assert win.pool.n_free == win.pool.n_pages
+
+
+def _register_routed_toy():
+    """A feed-forward with routing (two experts, the better router logit wins) and another position
+    encoding (keys and queries at odd positions change their sign), both defined here."""
+    from bitnet_c_amd import ops
+    from bitnet_c_amd.config import Architecture, register_architecture
+    from bitnet_c_amd.config.base import _ARCHITECTURES
+    from bitnet_c_amd.engine import LayerPlan, ModelPlan, ScheduleEntry
+    from bitnet_c_amd.parts import BLOCKS, FEED_FORWARDS, POSITION_ENCODINGS, ParamSpec, Part, PartSpec
+    from bitnet_c_amd.parts.position import PositionEncoding
+
+    if "two_experts" not in FEED_FORWARDS:
+        @FEED_FORWARDS.register("two_experts")
+        class TwoExperts(Part):
+            def __init__(self, hidden, intermediate):
+                self.hidden = hidden
+                spec = PartSpec.of("swiglu", hidden=hidden, intermediate=intermediate)
+                self.experts = [FEED_FORWARDS.build(spec), FEED_FORWARDS.build(spec)]     # library parts inside
+
+            def tensors(self):
+                t = {"router": ParamSpec((2, self.hidden))}
+                for e, part in enumerate(self.experts):
+                    t.update({f"e{e}.{k}": v for k, v in part.tensors().items()})
+                return t
+
+            def load(self, tensors, device, dtype):
+                self.router = tensors["router"].float().to(device)                       # router logits in float32
+                for e, part in enumerate(self.experts):
+                    part.load({k[3:]: v for k, v in tensors.items() if k.startswith(f"e{e}.")}, device, dtype)
+
+            def forward(self, h, ctx):
+                logits = h.float() @ self.router.t()
+                first = (logits[:, 0] >= logits[:, 1])[:, None]
+                # a toy: both experts run on every row and the router picks (no shapes that depend on data,
+                # so that decode steps can be replayed from graphs)
+                return torch.where(first, self.experts[0].forward(h, ctx), self.experts[1].forward(h, ctx))
+
+    if "parity_sign" not in POSITION_ENCODINGS:
+        @POSITION_ENCODINGS.register("parity_sign")
+        class ParitySign(PositionEncoding):
+            def __init__(self, head_dim=0):
+                pass
+
+            def fusable(self, hs):
+                return False, None                                   # no kernel knows this encoding
+
+            def encode_and_store(self, qkv, ctx, H, Hkv, hs, kv):
+                sign = (1 - 2 * (ctx.positions & 1)).to(qkv.dtype)[:, None]
+                qkv[:, :(H + Hkv) * hs] *= sign
+                ops.rope_kv_write(qkv, ctx.positions, H, Hkv, hs, rope_dims=0,
+                                  seq_index=ctx.seq_index if kv.writes else None,
+                                  block_table=kv.block_table if kv.writes else None,
+                                  k_pages=kv.k_pages if kv.writes else None,
+                                  v_pages=kv.v_pages if kv.writes else None)
+
+    @dataclass(frozen=True)
+    class RoutedConfig:
+        vocab_size: int
+        hidden_size: int
+        n_layers: int
+        model_type: str = "toy_routed"
+
+        @staticmethod
+        def from_dict(raw):
+            return RoutedConfig(raw["vocab_size"], raw["hidden_size"], raw["n_layers"])
+
+        def to_dict(self):
+            return asdict(self)
+
+    def build(c):
+        norm = PartSpec.of("rmsnorm", dim=c.hidden_size, eps=1e-5)
+        ffn = PartSpec.of("two_experts", hidden=c.hidden_size, intermediate=40)
+        att = PartSpec.of("attention", hidden=c.hidden_size, n_heads=3, n_kv_heads=1, head_dim=16, scale=0.25,
+                          position=PartSpec.of("parity_sign"))
+        layers = []
+        for i in range(c.n_layers):
+            blk = PartSpec.of("prenorm", mixer=att, ffn=ffn, mixer_norm=norm, ffn_norm=norm)
+            names = {local: f"layers.{i}.{local}" for local in BLOCKS.build(blk).tensors()}
+            layers.append(LayerPlan(block=blk, names=names))
+        return ModelPlan(vocab_size=c.vocab_size, hidden_size=c.hidden_size, layers=layers,
+                         schedule=[ScheduleEntry(i) for i in range(c.n_layers)], final_norm=norm,
+                         embedding_name="embed.weight", final_norm_names={"weight": "norm.weight"},
+                         lm_head_name="head.weight")
+
+    if "toy_routed" not in _ARCHITECTURES:
+        register_architecture(Architecture("toy_routed", RoutedConfig, build))
+    return RoutedConfig
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_toy_feed_forward_with_routing_and_another_position_encoding(tmp_path, dtype):
+    from bitnet_c_amd import Engine, StepEntry
+    from bitnet_c_amd.weights import write_model_folder
+    RoutedConfig = _register_routed_toy()
+    cfg = RoutedConfig(vocab_size=50, hidden_size=48, n_layers=2)
+    folder = write_model_folder(str(tmp_path / "routed"), cfg, 17, dtype)
+    eng = Engine.from_folder(folder, dtype=dtype, max_tokens=512)
+    assert eng.use_graphs                                            # no state: decode steps are replayed
+    from safetensors.torch import load_file
+    W = {k: v.float() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    rt = None if dtype == torch.float32 else dtype
+    r_ = lambda x: x if rt is None else x.to(rt).float()
+
+    def plain(toks):
+        x = W["embed.weight"][toks]
+        n = len(toks)
+        sign = (1 - 2 * (torch.arange(n) % 2)).float()[:, None, None]
+        routes = []
+        for l in range(2):
+            p = f"layers.{l}."
+            xb = r_(pl.rmsnorm(x, W[p + "mixer_norm.weight"], 1e-5))
+            q = r_(r_(pl.linear(xb, W[p + "mixer.wq"])).view(n, 3, 16) * sign)
+            k = r_(r_(pl.linear(xb, W[p + "mixer.wk"])).view(n, 1, 16) * sign)
+            v = r_(pl.linear(xb, W[p + "mixer.wv"])).view(n, 1, 16)
+            x = x + r_(pl.linear(r_(pl.attention(q, k, v, 0.25).reshape(n, 48)), W[p + "mixer.wo"]))
+            xb = r_(pl.rmsnorm(x, W[p + "ffn_norm.weight"], 1e-5))
+            logits = xb @ W[p + "ffn.router"].t()
+            routes.append(logits[:, 0] - logits[:, 1])
+            ys = [pl.feed_forward(xb, W[p + f"ffn.e{e}.w_gate"], W[p + f"ffn.e{e}.w_up"], W[p + f"ffn.e{e}.w_down"], rt)
+                  for e in range(2)]
+            x = x + torch.where((logits[:, 0] >= logits[:, 1])[:, None], ys[0], ys[1])
+        return pl.linear(r_(pl.rmsnorm(x, W["norm.weight"], 1e-5)), W["head.weight"]), torch.stack(routes)
+
+    rnd = random.Random(19)
+    reqs = [[rnd.randrange(50) for _ in range(n)] for n in (21, 6, 34)]
+    slots = [eng.new_sequence() for _ in reqs]
+    fed = [len(r) - 5 for r in reqs]
+    out = eng.step([StepEntry(s, r[:f], list(range(f))) for s, r, f in zip(slots, reqs, fed)])
+    got, o = [[] for _ in reqs], 0
+    for i, f in enumerate(fed):
+        got[i].append(out[o:o + f])
+        o += f
+    for k in range(5):
+        out = eng.step([StepEntry(s, [r[f + k]], [0]) for s, r, f in zip(slots, reqs, fed)])
+        for i in range(3):
+            got[i].append(out[i:i + 1])
+    used = set()
+    for i, r in enumerate(reqs):
+        want, margin = plain(r)
+        used |= set((margin > 0).flatten().tolist())
+        g = torch.cat(got[i]).cpu()
+        # a router decision on a knife's edge may fall the other way in bfloat16: leave those rows out
+        sure = (margin.abs() > (1e-6 if dtype == torch.float32 else 2e-3)).all(dim=0)
+        first_unsure = int((~sure).float().argmax()) if not bool(sure.all()) else len(r)
+        if dtype == torch.float32:
+            assert first_unsure == len(r)
+        assert first_unsure >= 3                                       # enough rows are left to compare
+        assert rel_err(g[:first_unsure], want[:first_unsure]) < TOL[dtype], i
+    assert used == {True, False}                                       # both experts were chosen somewhere
