@@ -430,7 +430,7 @@ def _register_routed_toy():
                 return t
 
             def load(self, tensors, device, dtype):
-                self.router = tensors["router"].float().to(device)                       # router logits in float32
+                self.router = (64.0 * tensors["router"].float()).to(device)              # router logits in float32, decisive
                 for e, part in enumerate(self.experts):
                     part.load({k[3:]: v for k, v in tensors.items() if k.startswith(f"e{e}.")}, device, dtype)
 
@@ -520,14 +520,14 @@ def test_a_toy_feed_forward_with_routing_and_another_position_encoding(tmp_path,
             v = r_(pl.linear(xb, W[p + "mixer.wv"])).view(n, 1, 16)
             x = x + r_(pl.linear(r_(pl.attention(q, k, v, 0.25).reshape(n, 48)), W[p + "mixer.wo"]))
             xb = r_(pl.rmsnorm(x, W[p + "ffn_norm.weight"], 1e-5))
-            logits = xb @ W[p + "ffn.router"].t()
+            logits = xb @ (64.0 * W[p + "ffn.router"]).t()
             routes.append(logits[:, 0] - logits[:, 1])
             ys = [pl.feed_forward(xb, W[p + f"ffn.e{e}.w_gate"], W[p + f"ffn.e{e}.w_up"], W[p + f"ffn.e{e}.w_down"], rt)
                   for e in range(2)]
             x = x + torch.where((logits[:, 0] >= logits[:, 1])[:, None], ys[0], ys[1])
         return pl.linear(r_(pl.rmsnorm(x, W["norm.weight"], 1e-5)), W["head.weight"]), torch.stack(routes)
 
-    rnd = random.Random(19)
+    rnd = random.Random(20)      # with these requests no router decision is closer than 0.18 (typical margin: 6)
     reqs = [[rnd.randrange(50) for _ in range(n)] for n in (21, 6, 34)]
     slots = [eng.new_sequence() for _ in reqs]
     fed = [len(r) - 5 for r in reqs]
@@ -543,13 +543,7 @@ def test_a_toy_feed_forward_with_routing_and_another_position_encoding(tmp_path,
     used = set()
     for i, r in enumerate(reqs):
         want, margin = plain(r)
+        assert float(margin.abs().min()) > 0.05                        # no decision on a knife's edge
         used |= set((margin > 0).flatten().tolist())
-        g = torch.cat(got[i]).cpu()
-        # a router decision on a knife's edge may fall the other way in bfloat16: leave those rows out
-        sure = (margin.abs() > (1e-6 if dtype == torch.float32 else 2e-3)).all(dim=0)
-        first_unsure = int((~sure).float().argmax()) if not bool(sure.all()) else len(r)
-        if dtype == torch.float32:
-            assert first_unsure == len(r)
-        assert first_unsure >= 3                                       # enough rows are left to compare
-        assert rel_err(g[:first_unsure], want[:first_unsure]) < TOL[dtype], i
+        assert rel_err(torch.cat(got[i]), want) < TOL[dtype], i
     assert used == {True, False}                                       # both experts were chosen somewhere
