@@ -114,25 +114,56 @@ __global__ void repeat_penalty_kernel(float* __restrict__ logits, int ld, int n,
 
 __device__ __forceinline__ unsigned long long to_fixed(float p) { return (unsigned long long)((double)p * FIX_ONE); }
 
+#define SMP_WAVES (SMP_THREADS / 64)
+
+// Every wave owns a contiguous range of the row and walks it 64 consecutive elements a time (lane l
+// takes element l of each group): loads are coalesced, and (wave, group, lane) order is index order.
+__device__ __forceinline__ void wave_range(int n, int& lo, int& hi) {
+    const int per = ((n + SMP_WAVES - 1) / SMP_WAVES + 63) / 64 * 64;
+    lo = min(n, (int)(threadIdx.x >> 6) * per);
+    hi = min(n, lo + per);
+}
+
+__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned lo = __shfl_xor((unsigned)v, o, BN_WAVE), hi = __shfl_xor((unsigned)(v >> 32), o, BN_WAVE);
+        v += ((unsigned long long)hi << 32) | lo;
+    }
+    return v;
+}
+
 // Descending cumulative sum over {p_i >= cutoff}: finds the element at which the sum first
 // exceeds `bound` (fixed point).  Returns its index; *cum_out = the sum including it.  When the
 // sum never exceeds the bound the last (smallest) candidate and the whole sum are returned.
 __device__ int descend(const float* __restrict__ p, int n, float cutoff, unsigned long long bound,
                        unsigned long long* cum_out, unsigned long long* hist, int* ibuf) {
-    // ibuf: [SMP_THREADS + 8] ints of shared memory; hist: [256]
+    // ibuf: [SMP_THREADS + 8] ints of shared memory; hist: [258]
     uint32_t prefix = 0, mask = 0;
     unsigned long long above = 0;
-    const int chunk = (n + blockDim.x - 1) / blockDim.x;
-    const int i0 = min(n, (int)threadIdx.x * chunk), i1 = min(n, i0 + chunk);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int lo, hi;
+    wave_range(n, lo, hi);
     for (int level = 0; level < 4; ++level) {
         const int shift = 24 - 8 * level;
         for (int b = threadIdx.x; b < 256; b += blockDim.x) hist[b] = 0;
         __syncthreads();
-        for (int i = i0; i < i1; ++i) {
-            const float v = p[i];
+        for (int g0 = lo; g0 < hi; g0 += 64) {
+            const int i = g0 + lane;
+            const float v = i < hi ? p[i] : 0.f;
             const uint32_t bits = __float_as_uint(v);
-            if (v >= cutoff && (bits & mask) == prefix)
-                atomicAdd(&hist[(bits >> shift) & 255u], to_fixed(v));
+            const bool cand = i < hi && v >= cutoff && (bits & mask) == prefix;
+            const int bin = (bits >> shift) & 255u;
+            const unsigned long long any = __ballot(cand);
+            if (any == 0) continue;
+            // neighbours mostly fall into one bucket at the upper levels: then one add for the wave
+            const int first_bin = __shfl(bin, __ffsll((long long)any) - 1, BN_WAVE);
+            if (__all(!cand || bin == first_bin)) {
+                const unsigned long long sum = wave_sum_u64(cand ? to_fixed(v) : 0ull);
+                if (lane == 0) atomicAdd(&hist[first_bin], sum);
+            } else if (cand) {
+                atomicAdd(&hist[bin], to_fixed(v));
+            }
         }
         __syncthreads();
         if (threadIdx.x == 0) {
@@ -157,23 +188,27 @@ __device__ int descend(const float* __restrict__ p, int n, float cutoff, unsigne
         above = hist[256];
         __syncthreads();
     }
-    // the group of elements whose probability has exactly the bit pattern `prefix`
+    // the group of elements whose probability has exactly the bit pattern `prefix`, in index order
     const float v = __uint_as_float(prefix);
     const unsigned long long qv = to_fixed(v);
     int cnt = 0;
-    for (int i = i0; i < i1; ++i) cnt += (p[i] >= cutoff && __float_as_uint(p[i]) == prefix) ? 1 : 0;
-    ibuf[threadIdx.x] = cnt;
+    for (int g0 = lo; g0 < hi; g0 += 64) {
+        const int i = g0 + lane;
+        const bool hit = i < hi && p[i] >= cutoff && __float_as_uint(p[i]) == prefix;
+        cnt += __popcll(__ballot(hit));
+    }
+    if (lane == 0) ibuf[wave] = cnt;
     __syncthreads();
     if (threadIdx.x == 0) {
         int total = 0;
-        for (int t = 0; t < (int)blockDim.x; ++t) total += ibuf[t];
+        for (int t = 0; t < SMP_WAVES; ++t) total += ibuf[t];
         long long k = 1;
         if (qv > 0 && bound >= above) k = (long long)((bound - above) / qv) + 1;
         if (k > total) k = total;
         if (k < 1) k = 1;
-        // thread that holds the k-th element of the group
+        // wave that holds the k-th element of the group
         int seen = 0, owner = 0, rank = (int)k;
-        for (int t = 0; t < (int)blockDim.x; ++t) {
+        for (int t = 0; t < SMP_WAVES; ++t) {
             if (seen + ibuf[t] >= (int)k) { owner = t; rank = (int)k - seen; break; }
             seen += ibuf[t];
         }
@@ -184,14 +219,21 @@ __device__ int descend(const float* __restrict__ p, int n, float cutoff, unsigne
     }
     __syncthreads();
     const int owner = ibuf[SMP_THREADS + 1], rank = ibuf[SMP_THREADS + 2], total = ibuf[SMP_THREADS + 3];
-    if ((int)threadIdx.x == owner) {
-        int r = 0, found = n - 1;
-        for (int i = i0; i < i1; ++i) {
-            if (p[i] >= cutoff && __float_as_uint(p[i]) == prefix) {
-                if (++r == rank) { found = i; break; }
+    if (wave == owner) {
+        int seen = 0, found = n - 1;
+        for (int g0 = lo; g0 < hi; g0 += 64) {
+            const int i = g0 + lane;
+            const bool hit = i < hi && p[i] >= cutoff && __float_as_uint(p[i]) == prefix;
+            unsigned long long m = __ballot(hit);
+            const int c = __popcll(m);
+            if (seen + c >= rank) {
+                for (int skip = rank - seen - 1; skip > 0; --skip) m &= m - 1;       // drop the lower set bits
+                found = g0 + __ffsll((long long)m) - 1;
+                break;
             }
+            seen += c;
         }
-        ibuf[SMP_THREADS + 4] = total > 0 ? found : n - 1;
+        if (lane == 0) ibuf[SMP_THREADS + 4] = total > 0 ? found : n - 1;
     }
     __syncthreads();
     *cum_out = hist[257];
@@ -208,7 +250,7 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(const float* __rest
     __shared__ float fs[16];
     __shared__ unsigned long long hist[258];
     __shared__ int ibuf[SMP_THREADS + 8];
-    __shared__ float fbuf[SMP_THREADS];
+    __shared__ float wtot[SMP_WAVES];
     const float* x = logits + (size_t)blockIdx.x * ld;
     float* p = probs + (size_t)blockIdx.x * n;
     if (temperature == 0.0f) {
@@ -216,37 +258,39 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(const float* __rest
         if (threadIdx.x == 0) out[blockIdx.x] = a.i;
         return;
     }
-    // softmax(x / T): each thread owns a contiguous chunk, so sums have a fixed order
-    const int chunk = (n + blockDim.x - 1) / blockDim.x;
-    const int i0 = min(n, (int)threadIdx.x * chunk), i1 = min(n, i0 + chunk);
+    // softmax(x / T): the assignment of elements to lanes is fixed, so the sums have a fixed order
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int lo, hi;
+    wave_range(n, lo, hi);
     float mx = -INFINITY;
-    for (int i = i0; i < i1; ++i) mx = fmaxf(mx, x[i] / temperature);
+    for (int i = lo + lane; i < hi; i += 64) mx = fmaxf(mx, x[i] / temperature);
     mx = block_max(mx, fs);
     float part = 0.f;
-    for (int i = i0; i < i1; ++i) {
+    for (int i = lo + lane; i < hi; i += 64) {
         const float e = expf(x[i] / temperature - mx);
         p[i] = e;
         part += e;
     }
     const float total = block_sum(part, fs);
     part = 0.f;
-    for (int i = i0; i < i1; ++i) {
+    for (int i = lo + lane; i < hi; i += 64) {
         const float q = p[i] / total;
         p[i] = q;
         part += q;
     }
-    __syncthreads();
+    part = wave_sum(part);
+    if (lane == 0) wtot[wave] = part;
+    __syncthreads();                        // also: every lane's p[] is visible to the whole workgroup
     const float rr = r[blockIdx.x];
     if (n == 1) { if (threadIdx.x == 0) out[blockIdx.x] = 0; return; }
     if (top_p <= 0.0f || top_p >= 1.0f) {
-        // cdf walk: first i with rr < cdf_i (src/sampler.c:65-74); n-1 if none
-        fbuf[threadIdx.x] = part;
-        __syncthreads();
+        // cdf walk: first i with rr < cdf_i (src/sampler.c:65-74); n-1 if none.  First the wave whose
+        // range holds it, then that wave walks its range with a prefix sum over each 64 elements.
         if (threadIdx.x == 0) {
             float c = 0.f;
             int owner = -1;
-            for (int t = 0; t < (int)blockDim.x; ++t) {
-                const float s = fbuf[t];
+            for (int t = 0; t < SMP_WAVES; ++t) {
+                const float s = wtot[t];
                 if (owner < 0 && rr < c + s) { owner = t; fs[0] = c; }
                 c += s;
             }
@@ -255,14 +299,22 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(const float* __rest
         __syncthreads();
         const int owner = ibuf[0];
         if (owner < 0) { if (threadIdx.x == 0) out[blockIdx.x] = n - 1; return; }
-        if ((int)threadIdx.x == owner) {
+        if (wave == owner) {
             float c = fs[0];
-            int found = i1 - 1;
-            for (int i = i0; i < i1; ++i) {
-                c += p[i];
-                if (rr < c) { found = i; break; }
+            int found = hi - 1;
+            for (int g0 = lo; g0 < hi; g0 += 64) {
+                const int i = g0 + lane;
+                float sc = i < hi ? p[i] : 0.f;
+#pragma unroll
+                for (int o = 1; o < 64; o <<= 1) {
+                    const float t = __shfl_up(sc, o, BN_WAVE);
+                    if (lane >= o) sc += t;
+                }
+                const unsigned long long m = __ballot(i < hi && rr < c + sc);
+                if (m) { found = g0 + __ffsll((long long)m) - 1; break; }
+                c += __shfl(sc, 63, BN_WAVE);
             }
-            out[blockIdx.x] = found;
+            if (lane == 0) out[blockIdx.x] = found;
         }
         return;
     }

@@ -499,6 +499,30 @@ def test_sample_matches_the_plain_sampler(vocab, temperature, top_p):
     assert got == want
 
 
+def test_sample_among_equal_probabilities():
+    """All logits equal, or in a few equal groups: top-p orders equal probabilities by index, and the
+    walk has to find the k-th member of a group across the ranges that the waves own."""
+    ops = _ops()
+
+    class Fixed:
+        def __init__(self, r): self.r = r
+        def next_float(self): return self.r
+    rng = pl.XorShift64Star(7)
+    for vocab in (1000, 70000):
+        for kind in ("flat", "steps"):
+            lg = torch.zeros(8, vocab) if kind == "flat" else (torch.arange(vocab) % 5).float().repeat(8, 1) * 0.5
+            rs = [rng.next_float() for _ in range(8)]
+            for top_p in (0.9, 0.3, 1.0):
+                got = ops.sample(lg.cuda(), 1.0, top_p, torch.tensor(rs, dtype=torch.float32).cuda()).cpu().tolist()
+                want = [pl.sample(lg[i], 1.0, top_p, Fixed(rs[i])) for i in range(8)]
+                # The plain sampler adds float32 probabilities one by one, the kernel adds them exactly (in
+                # fixed point): among thousands of equal probabilities the two walks may stop one member of
+                # the group apart (the next index with that probability), never further.
+                step = 1 if kind == "flat" else 5
+                assert all(abs(g - w) in (0, step) for g, w in zip(got, want)), (vocab, kind, top_p, got, want)
+                assert all(float(lg[i, g]) == float(lg[i, w]) for i, (g, w) in enumerate(zip(got, want)))
+
+
 def test_sample_reference_cases_on_device():
     ops = _ops()
     # top-p 0.5 with a dominant logit: always token 0 (test/test_safety.c:256-272)
