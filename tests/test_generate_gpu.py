@@ -99,3 +99,31 @@ def test_command_line(model_folders):
         assert "tok/s" in p.stderr
     p = subprocess.run(base[:3] + ["--prompt-token-ids", "1,999"], capture_output=True, text=True, timeout=300)
     assert p.returncode != 0 and "999" in p.stderr
+
+
+def test_command_line_with_a_text_prompt(model_folders, tmp_path):
+    """-p needs the folder's tokenizer.json: a word-level one is made here for a copy of the tiny
+    model; the prompt is encoded with it and the generated ids are printed as its words."""
+    import shutil
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    src = model_folders("A", torch.float32)
+    folder = str(tmp_path / "with_tokenizer")
+    shutil.copytree(src, folder)
+    words = {f"w{i}": i for i in range(256)}
+    tok = Tokenizer(models.WordLevel(vocab=words, unk_token="w0"))
+    tok.pre_tokenizer = pre_tokenizers.Whitespace()
+    tok.save(os.path.join(folder, "tokenizer.json"))
+    c, W = pl.read_config(folder), pl.read_weights(folder)
+    prompt = [3, 1, 4, 1, 5]
+    want = pl.generate(c, W, prompt, 5)
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "bitnet"), folder, "-p", " ".join(f"w{t}" for t in prompt),
+                        "-n", "5", "--repeat-penalty", "1.0", "--fp32", "--token-ids", "--no-bos"],
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-1500:]
+    ids = [l for l in p.stderr.splitlines() if l and l[0].isdigit()][0]
+    assert [int(x) for x in ids.split(",")] == want
+    assert p.stdout.split() == [f"w{t}" for t in want] or p.stdout.replace(" ", "").strip() == "".join(f"w{t}" for t in want)
+    # without the tokenizer a text prompt is refused with a message that says what to do
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "bitnet"), src, "-p", "w1 w2", "-n", "2", "--fp32"],
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode != 0 and "tokenizer.json" in p.stderr + p.stdout
