@@ -59,6 +59,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
         }
         const size_t dst = (((size_t)page * Hkv + kh) * BN_PAGE + off) * hs + d;
         k_pages[dst] = from_f32<T>(o);
+        if (v_transposed == 2) continue;        // the page-tile kernel below stores V
         if (v_transposed)       // V pages [page, kv_head, head_dim, BN_PAGE]
             v_pages[(((size_t)page * Hkv + kh) * hs + d) * BN_PAGE + off] = vrow[idx];
         else
@@ -139,9 +140,9 @@ __global__ __launch_bounds__(256) void rope_kv_write_bf16x8_kernel(bf16* __restr
         bf16* dst = k_pages + (((size_t)page * Hkv + kh) * BN_PAGE + off) * hs;
         *reinterpret_cast<uint4*>(dst + rope_dims + c * 8) = *reinterpret_cast<const uint4*>(krow + kh * hs + rope_dims + c * 8);
     }
-    // V
+    // V (v_transposed == 2: the page-tile kernel below stores it)
     const int vg = hs / 8;
-    for (int idx = threadIdx.x; idx < Hkv * vg; idx += blockDim.x) {
+    for (int idx = threadIdx.x; v_transposed != 2 && idx < Hkv * vg; idx += blockDim.x) {
         const int kh = idx / vg, c = idx - kh * vg;
         const uint4 v = *reinterpret_cast<const uint4*>(vrow + kh * hs + c * 8);
         if (v_transposed) {                  // V pages [page, kv_head, head_dim, BN_PAGE]
@@ -155,9 +156,71 @@ __global__ __launch_bounds__(256) void rope_kv_write_bf16x8_kernel(bf16* __restr
     }
 }
 
+// V into transposed pages for the tokens of a prompt: a workgroup takes the rows of one sequence
+// that fall into one page (tile = sequence, first row, rows, position of the first) and one kv
+// head, turns the [rows, hs] block through shared memory and stores runs of 8 positions with
+// 16 bytes, instead of 2 bytes a position and dimension.
+#define VT_PAD 2
+__global__ __launch_bounds__(256) void v_transposed_write_kernel(const bf16* __restrict__ qkv, int row_stride,
+                                                                 const int* __restrict__ tiles,
+                                                                 const int* __restrict__ block_table, int bt_stride,
+                                                                 bf16* __restrict__ v_pages, int H, int Hkv, int hs) {
+    extern __shared__ uint16_t vt_s[];       // [hs][BN_PAGE + VT_PAD], column = position inside the page
+    const int* tl = tiles + 4 * blockIdx.x;
+    const int seq = tl[0], row0 = tl[1], n = tl[2], pos0 = tl[3];
+    const int kh = blockIdx.y;
+    const int off = pos0 % BN_PAGE;
+    if (n <= 0 || off + n > BN_PAGE) return;
+    const int page = block_table[(size_t)seq * bt_stride + pos0 / BN_PAGE];
+    const int ld = BN_PAGE + VT_PAD;
+    const int groups = hs / 8;
+    for (int idx = threadIdx.x; idx < n * groups; idx += blockDim.x) {
+        const int r = idx / groups, c = idx - r * groups;
+        const uint4 v = *reinterpret_cast<const uint4*>(qkv + (size_t)(row0 + r) * row_stride + (size_t)(H + Hkv + kh) * hs + c * 8);
+        const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) vt_s[(c * 8 + j) * ld + off + r] = e[j];
+    }
+    __syncthreads();
+    uint16_t* dst = reinterpret_cast<uint16_t*>(v_pages) + ((size_t)page * Hkv + kh) * hs * BN_PAGE;
+    for (int idx = threadIdx.x; idx < hs * (BN_PAGE / 8); idx += blockDim.x) {
+        const int d = idx / (BN_PAGE / 8), p8 = (idx - d * (BN_PAGE / 8)) * 8;     // positions p8 .. p8+7 of the page
+        if (p8 + 8 <= off || p8 >= off + n) continue;
+        const uint16_t* src = vt_s + d * ld + p8;
+        if (p8 >= off && p8 + 8 <= off + n) {
+            uint4 w;
+            w.x = src[0] | ((uint32_t)src[1] << 16);
+            w.y = src[2] | ((uint32_t)src[3] << 16);
+            w.z = src[4] | ((uint32_t)src[5] << 16);
+            w.w = src[6] | ((uint32_t)src[7] << 16);
+            *reinterpret_cast<uint4*>(dst + (size_t)d * BN_PAGE + p8) = w;
+        } else {
+            for (int j = 0; j < 8; ++j)
+                if (p8 + j >= off && p8 + j < off + n) dst[(size_t)d * BN_PAGE + p8 + j] = src[j];
+        }
+    }
+}
+
+// tiles: [n_tiles, 4] int32 as above; every tile lies inside one page.  V heads are read from qkv.
+extern "C" int bn_v_transposed_write(const void* qkv, int row_stride, const int* tiles, int n_tiles,
+                                     const int* block_table, int bt_stride, void* v_pages, int H, int Hkv, int hs,
+                                     hipStream_t s) {
+    if (n_tiles <= 0 || H <= 0 || Hkv <= 0 || hs <= 0 || hs % 8 || row_stride % 8 || row_stride < (H + 2 * Hkv) * hs ||
+        !tiles || !block_table || !v_pages || n_tiles > 0x7fffffff / 4 || Hkv > 65535)
+        return BN_ERR_ARG;
+    if (((uintptr_t)qkv | (uintptr_t)v_pages) & 15) return BN_ERR_ARG;
+    const size_t smem = (size_t)hs * (BN_PAGE + VT_PAD) * sizeof(uint16_t);
+    if (smem > 64 * 1024) return BN_ERR_ARG;
+    hipLaunchKernelGGL(v_transposed_write_kernel, dim3(n_tiles, Hkv), dim3(256), smem, s, (const bf16*)qkv, row_stride,
+                       tiles, block_table, bt_stride, (bf16*)v_pages, H, Hkv, hs);
+    return bn_launch_status();
+}
+
 // qkv: [n_tokens, row_stride] with Q heads first, then K heads, then V heads.
 // k_pages == null: rotate Q only (a layer that reads another layer's cache).
 // rope_dims == 0: no rotation, the write alone.
+// v_transposed: 0 = V pages like K pages, 1 = transposed pages, 2 = transposed pages that
+// bn_v_transposed_write fills (V is left alone here).
 extern "C" int bn_rope_kv_write(int dtype, void* qkv, int row_stride, const int* positions,
                                 const int* seq_index, const int* block_table, int bt_stride,
                                 void* k_pages, void* v_pages, const float* inv_freq, int rope_dims,

@@ -52,6 +52,7 @@ class StepContext:
         self.n_rows = int(tokens.numel())
         self.n_seqs = len(self.slots)
         self._tiles: Dict[int, torch.Tensor] = {}
+        self._page_tiles = None
 
     def row_ranges(self):
         """(first row, rows) of every sequence in the flattened batch."""
@@ -60,6 +61,14 @@ class StepContext:
             out.append((r, n))
             r += n
         return out
+
+    def page_tiles(self) -> torch.Tensor:
+        """[n, 4] int32: the new tokens cut at page boundaries (sequence, first row, rows, position of
+        the first), for kernels that store a page's positions together."""
+        if self._page_tiles is None:
+            self._page_tiles = torch.tensor(_page_tiles(self.n_new, self.pos0),
+                                            dtype=torch.int32).reshape(-1, 4).to(self.device)
+        return self._page_tiles
 
     def tiles(self, qt: int) -> torch.Tensor:
         """[n, 4] int32: (sequence, first row, rows <= qt, position of the first) covering all new
@@ -74,6 +83,20 @@ class StepContext:
             t = torch.tensor(rows, dtype=torch.int32).reshape(-1, 4).to(self.device)
             self._tiles[qt] = t
         return t
+
+
+def _page_tiles(n_new, pos0) -> List[tuple]:
+    """(sequence, first row, rows, position of the first) for every run of a sequence's new tokens
+    inside one page."""
+    rows, r = [], 0
+    for s, (n, p0) in enumerate(zip(n_new, pos0)):
+        i = 0
+        while i < n:
+            m = min(n - i, PAGE - (p0 + i) % PAGE)
+            rows.append((s, r + i, m, p0 + i))
+            i += m
+        r += n
+    return rows
 
 
 def _by_length(lens) -> List[int]:

@@ -32,6 +32,8 @@ _SIGNATURES = {
         "bn_bias_add": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
     },
     "rope_kv": {
+        "bn_v_transposed_write": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
+                                  c_void_p],
         "bn_rope_kv_write": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                              c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
@@ -339,10 +341,13 @@ def _check_pages(k_pages, v_pages, Hkv, hs, dtype):
 
 def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, hs: int, *,
                   inv_freq=None, rope_dims: int = 0, seq_index=None, block_table=None,
-                  k_pages=None, v_pages=None) -> None:
+                  k_pages=None, v_pages=None, page_tiles=None) -> None:
     """Rotate the Q heads of qkv ([T, (H+2Hkv)*hs]) in place, rotate the K heads and store
     them and the V heads at each token's position of its sequence's pages.
-    k_pages None: rotate Q only.  rope_dims 0: no rotation.  positions < 0: padding rows."""
+    k_pages None: rotate Q only.  rope_dims 0: no rotation.  positions < 0: padding rows.
+    page_tiles (optional, [n, 4] int32 = sequence, first row, rows, position of the first; each
+    tile inside one page, all rows covered): transposed V pages are then filled by a kernel
+    that stores runs of positions instead of single elements."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(positions, "positions", torch.int32, 1)
@@ -367,13 +372,24 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
         bt_stride = block_table.shape[1]
     if T == 0:
         return
+    tiled_v = (page_tiles is not None and k_pages is not None and vt and hs % 8 == 0 and stride % 8 == 0
+               and qkv.data_ptr() % 16 == 0 and hs * (PAGE + 2) * 2 <= 65536 and Hkv <= 65535)
+    if tiled_v:
+        _dev(page_tiles, "page_tiles", torch.int32, 2)
+        if page_tiles.shape[1] != 4 or not page_tiles.is_contiguous() or page_tiles.shape[0] == 0:
+            raise KernelError("rope_kv_write: page_tiles must be a contiguous [n, 4] tensor")
     _check(_fn("rope_kv", "bn_rope_kv_write")(
         _code(qkv.dtype), qkv.data_ptr(), stride, positions.data_ptr(),
         seq_index.data_ptr() if k_pages is not None else None,
         block_table.data_ptr() if k_pages is not None else None, bt_stride,
         k_pages.data_ptr() if k_pages is not None else None,
         v_pages.data_ptr() if k_pages is not None else None,
-        inv_freq.data_ptr() if rope_dims else None, rope_dims, T, H, Hkv, hs, int(vt), _stream()), "rope_kv_write")
+        inv_freq.data_ptr() if rope_dims else None, rope_dims, T, H, Hkv, hs, 2 if tiled_v else int(vt), _stream()),
+        "rope_kv_write")
+    if tiled_v:
+        _check(_fn("rope_kv", "bn_v_transposed_write")(
+            qkv.data_ptr(), stride, page_tiles.data_ptr(), page_tiles.shape[0], block_table.data_ptr(), bt_stride,
+            v_pages.data_ptr(), H, Hkv, hs, _stream()), "v_transposed_write")
 
 
 def _pow2_at_least(n: int) -> int:

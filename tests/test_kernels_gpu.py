@@ -250,6 +250,20 @@ def test_rope_kv_write(dtype, H, Hkv, hs, rope_dims):
     g3 = q_in.clone().cuda()
     ops.rope_kv_write(g3, pos.cuda(), H, Hkv, hs, inv_freq=inv_freq.cuda(), rope_dims=rope_dims)
     assert torch.equal(g3.cpu(), g.cpu())
+    # with the tokens cut at page boundaries, transposed V pages are written in runs of positions: the
+    # same bytes (the sequences start at 0, 70, 130: unaligned runs, whole pages and a page's tail)
+    from bitnet_c_amd.engine.step import _page_tiles
+    tiles = _page_tiles(n_new, lens_before)
+    assert sum(t[2] for t in tiles) == T and all(t[3] // 64 == (t[3] + t[2] - 1) // 64 for t in tiles)
+    g4 = q_in.clone().cuda()
+    kp4 = torch.zeros((n_pages, Hkv, 64, hs), dtype=dtype).cuda()
+    vp4 = torch.zeros((n_pages, Hkv, hs, 64) if vt else (n_pages, Hkv, 64, hs), dtype=dtype).cuda()
+    ops.rope_kv_write(g4, pos.cuda(), H, Hkv, hs, inv_freq=inv_freq.cuda(), rope_dims=rope_dims,
+                      seq_index=torch.tensor(seq_index, dtype=torch.int32).cuda(), block_table=bt.cuda(),
+                      k_pages=kp4, v_pages=vp4, page_tiles=torch.tensor(tiles, dtype=torch.int32).cuda())
+    vp_first = vp.transpose(2, 3) if vt else vp
+    assert torch.equal(g4.cpu(), g.cpu()) and torch.equal(kp4.cpu().float(), kp)
+    assert torch.equal(vp4.cpu().float(), vp_first.contiguous())
 
 
 def test_rope_reference_vector_on_device():
