@@ -596,6 +596,8 @@ def repeat_penalty_(logits: torch.Tensor, recent: torch.Tensor, penalty: float) 
 def sample(logits: torch.Tensor, temperature: float, top_p: float, uniforms=None) -> torch.Tensor:
     """One token id per row.  temperature 0: argmax.  uniforms: float32 [B] in [0, 1)."""
     require_gpu()
+    if temperature == 0.0:
+        return argmax(logits)                 # the same first maximum, in two stages for a large vocabulary
     ld = _logits_ok(logits)
     B, V = logits.shape
     out = torch.empty((B,), dtype=torch.int32, device=logits.device)
