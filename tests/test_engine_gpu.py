@@ -348,3 +348,66 @@ def test_forty_sequences_of_unequal_lengths_with_eight_kv_heads(model_folders, g
         live = [i for i in live if fed[i] < len(reqs[i])]
     for i in range(40):
         assert rel_err(torch.cat(got[i]), plain_logits(folder, reqs[i], dtype)[-n_dec[i]:]) < TOL[dtype], i
+
+
+def test_cuts_and_batches_agree_at_the_benchmark_layer_sizes():
+    """Two layers of the Llama-3.1-8B shape (bfloat16, random weights made on the device): the
+    kernels at their real sizes, where a prompt's products go to the library and a decoded token's
+    to the streaming kernel.  There is no plain run at this size; the same request whole, with its
+    last 32 tokens one by one, and inside a batch of unequal partners must agree within the
+    bfloat16 tolerance, and all of them with a float32 engine on the same (bfloat16) weights."""
+    import bitnet_c_amd as bn
+    from bitnet_c_amd.config import architecture_for
+    from bitnet_c_amd.engine import DecoderModel
+    from bitnet_c_amd.weights import random_tensors
+    raw = dict(model_type="llama", vocab_size=128256, hidden_size=4096, intermediate_size=14336,
+               num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+               max_position_embeddings=131072, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+               rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                 original_max_position_embeddings=8192))
+    cfg = bn.LlamaConfig.from_dict(raw)
+    plan = architecture_for(raw).build_plan(cfg)
+    tensors = random_tensors(plan.expected_tensors(), 3, torch.bfloat16, device="cuda:0")
+    engines = {}
+    for dtype in (torch.bfloat16, torch.float32):
+        model = DecoderModel(plan, dtype, "cuda:0")
+        model.load(tensors)
+        engines[dtype] = bn.Engine(model, max_tokens=4096)
+    del tensors
+    rnd = random.Random(31)
+    toks, p1, p2 = ([rnd.randrange(cfg.vocab_size) for _ in range(n)] for n in (300, 70, 513))
+    last = list(range(268, 300))
+
+    def run(eng):
+        s = eng.new_sequence()
+        whole = eng.step([bn.StepEntry(s, toks, last)])
+        eng.release(s)
+        s = eng.new_sequence()
+        eng.step([bn.StepEntry(s, toks[:268], [])])
+        one_by_one = torch.cat([eng.step([bn.StepEntry(s, [t], [0])]) for t in toks[268:]])
+        eng.release(s)
+        a, b, c = eng.new_sequence(), eng.new_sequence(), eng.new_sequence()
+        out = eng.step([bn.StepEntry(a, p1, []), bn.StepEntry(b, toks[:268], []), bn.StepEntry(c, p2, [512])])
+        rows = []
+        for t in toks[268:]:                       # the partners go on too, with tokens of their own
+            o = eng.step([bn.StepEntry(a, [5], []), bn.StepEntry(b, [t], [0]), bn.StepEntry(c, [7], [0])])
+            rows.append(o[:1])
+        for x in (a, b, c):
+            eng.release(x)
+        eng.cache.check()
+        return whole, one_by_one, torch.cat(rows)
+
+    ref = run(engines[torch.float32])
+    assert rel_err(ref[1], ref[0]) < TOL[torch.float32] and rel_err(ref[2], ref[0]) < TOL[torch.float32]
+    got = run(engines[torch.bfloat16])
+    # 32 x 128,256 logits: the largest of four million differences is no measure (rounding noise of
+    # standard deviation s has its largest value near 5.5 s there).  What rounding looks like at this
+    # width: a difference of about 1.4 % of the logits' root mean square, the same in every row, with
+    # no value far outside it.  A fault (a wrong key, a lost column) breaks one of the three.
+    rms = float(ref[0].double().pow(2).mean().sqrt())
+    for g in got:
+        d = (g - ref[0]).double()
+        per_row = d.pow(2).mean(dim=1).sqrt() / rms
+        assert float(per_row.max()) < 0.025, per_row
+        assert float(per_row.max() / per_row.min()) < 2.0, per_row
+        assert float(d.abs().max() / d.pow(2).mean().sqrt()) < 7.0
