@@ -108,12 +108,38 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
     return (ua >> 16) | (ub & 0xffff0000u);
 }
 
+// Shared memory serves 16 lanes of a 16-byte read at once, from 64 banks of 4 bytes.  The lanes
+// that read a staged key block together hold rows 8a + b (+4 for the second tile), a, b in 0..3, and
+// all want the same 16-byte chunk: rows are stored without padding and chunk c of row r lives at
+// c ^ f(r), with f distinct for those 16 rows over the 256 bytes that the banks span (head size
+// 128: a row is 256 bytes, f = 4a + b; head size 64: two rows share 256 bytes, the row's parity is
+// one bit already and f = 2a + b/2 supplies the other three).
+template <int HS>
+__device__ __forceinline__ int k_swizzle(int row) {
+    const int a = (row >> 3) & 3, b = row & 3;
+    return HS == 128 ? (a << 2 | b) : (a << 1 | b >> 1);
+}
+
+// A 16-byte read serves the lanes in four turns of 16: quads of lanes {0, 3, 5, 6}, {1, 2, 4, 7} and
+// the same of the upper 32 lanes (measured with a probe kernel and the bank-conflict counter).  In
+// the operand layout lane = i + 16 g, so a turn holds two values of g (0 and 1, or 2 and 3) and, for
+// the even one, i/4 in {0, 3}, for the odd one i/4 in {1, 2} (the other turn: the other way round).
+// The staged V^T block (rows = dimensions, 16-byte chunks of 8 keys) is stored without padding with
+// chunk c of row r at c ^ v_swizzle(r): h(i/4) = (-(i/4)) & 3 makes g ^ h distinct over a turn for
+// rows that share their position inside 256 bytes; with 64 keys a row (two rows in 256 bytes, the
+// row's lowest bit separates them) bit 1 of the row goes into bit 2 of the chunk as well.
+template <int KEYS>
+__device__ __forceinline__ int v_swizzle(int row) {
+    const int h = (-(row >> 2)) & 3;
+    return KEYS == 64 ? (h | ((row >> 1) & 1) << 2) : h;
+}
+
 // One 32-key block for NT column tiles.  kbase/vbase point at the block's first key inside its
 // page (row strides HS and BN_PAGE) or inside a staged copy in shared memory (KSTRIDE, VSTRIDE).  qpos/lo: per tile, this lane's column's position and first visible key (qpos < 0: no
 // such column).  key_hi: keys >= key_hi do not exist (decode: split end / length).
 template <int HS, int NT, int KSTRIDE, int VSTRIDE, bool STREAM, bool need_mask>
 __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, const bf16* __restrict__ vbase,
-                                               int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
+                                               int vchunk0, int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
                                                float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
                                                const int (&lo)[NT], int key_hi, float scale2, int lane) {
     // STREAM: the operands come from shared memory (short latency): fetch each one right before its
@@ -138,10 +164,9 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
         if (STREAM) {
-            // staged keys are stored with their 16-byte chunks swizzled (chunk ^ 4 for rows 8..15 and
-            // 24..31): the eight lanes that read together touch rows r..r+3 and r+8..r+11, which
-            // would otherwise share their banks
-            const int chunk = ((c * 4 + g) ^ ((i >> 2) & 1) * 4) * 8;
+            // staged keys are stored with their 16-byte chunks swizzled (k_swizzle): the 16 lanes that read
+            // together want the same chunk of 16 different rows
+            const int chunk = ((c * 4 + g) ^ k_swizzle<HS>(krow0)) * 8;
             ka[0][0] = ld16(kbase + (size_t)krow0 * KSTRIDE + chunk);
             ka[0][1] = ld16(kbase + (size_t)(krow0 + 4) * KSTRIDE + chunk);
         }
@@ -216,7 +241,8 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
         if (STREAM) {
-            va[0] = ld16(vbase + (size_t)(t * 16 + i) * VSTRIDE + 8 * g);
+            // staged: VSTRIDE keys a row, this group's keys start at chunk vchunk0
+            va[0] = ld16(vbase + (size_t)(t * 16 + i) * VSTRIDE + ((vchunk0 + g) ^ v_swizzle<VSTRIDE>(i)) * 8);
             if (need_mask) va[0] = clear_missing(va[0]);
         }
 #pragma unroll
@@ -229,14 +255,14 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
 // the plain one are separate instantiations: almost every block is plain, and it carries no mask code.
 template <int HS, int NT, int KSTRIDE = HS, int VSTRIDE = BN_PAGE, bool STREAM = false>
 __device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, const bf16* __restrict__ vbase,
-                                             int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
+                                             int vchunk0, int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
                                              float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
                                              const int (&lo)[NT], int key_hi, bool need_mask, float scale2,
                                              int lane) {
     if (need_mask)
-        attend_block_m<HS, NT, KSTRIDE, VSTRIDE, STREAM, true>(kbase, vbase, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
+        attend_block_m<HS, NT, KSTRIDE, VSTRIDE, STREAM, true>(kbase, vbase, vchunk0, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
     else
-        attend_block_m<HS, NT, KSTRIDE, VSTRIDE, STREAM, false>(kbase, vbase, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
+        attend_block_m<HS, NT, KSTRIDE, VSTRIDE, STREAM, false>(kbase, vbase, vchunk0, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -252,7 +278,7 @@ template <int HS, int NT, int NG>
 __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_mfma_prompt_kernel(MfmaArgs a) {
     constexpr int DC = HS / 32, DT = HS / 16;
     constexpr int KB = 32 * NG;                           // keys per stage
-    constexpr int KS = HS + 8, VS = KB + 8;               // padded row strides (elements)
+    constexpr int KS = HS, VS = KB;                       // row strides (elements); both blocks swizzled, no padding
     constexpr int KV4 = 32 * HS / 8 / 256;                // uint4 loads per thread for K (and for V^T)
     constexpr int STAGE = (KB * KS + HS * VS) * 2;        // bytes of one buffer
     constexpr int MERGE = NG > 1 ? 4 * 64 * (DT * 4 + 2) * 4 : 0;
@@ -329,9 +355,9 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
         for (int j = 0; j < KV4; ++j) {
             const int idx = threadIdx.x + 256 * NG * j;
             const int krow = (idx * 8) / HS, kchunk = ((idx * 8) % HS) / 8;
-            *reinterpret_cast<uint4*>(k_s(buf) + krow * KS + ((kchunk ^ ((krow >> 3) & 1) * 4) * 8)) = kr[j];
+            *reinterpret_cast<uint4*>(k_s(buf) + krow * KS + ((kchunk ^ k_swizzle<HS>(krow)) * 8)) = kr[j];
             const int vrow = idx / (KB / 8), vcol = (idx % (KB / 8)) * 8;
-            *reinterpret_cast<uint4*>(v_s(buf) + vrow * VS + vcol) = vr[j];
+            *reinterpret_cast<uint4*>(v_s(buf) + vrow * VS + (((vcol >> 3) ^ v_swizzle<KB>(vrow & 15)) * 8)) = vr[j];
         }
     };
     const int kb0 = (g_lo / KB) * KB;
@@ -345,7 +371,7 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
         const int kbb = kb + 32 * grp;                    // this group's block of the stage
         if (w_hi >= 0 && kbb <= w_hi && kbb + 31 >= w_lo) {
             const bool need_mask = (kbb + 31 > all_hi) || (kbb < all_lo);
-            attend_block<HS, NT, KS, VS, true>(k_s(buf) + 32 * grp * KS, v_s(buf) + 32 * grp, kbb, q, acc, m, l, qpos, lo,
+            attend_block<HS, NT, KS, VS, true>(k_s(buf) + 32 * grp * KS, v_s(buf), 4 * grp, kbb, q, acc, m, l, qpos, lo,
                                                w_hi + 1, need_mask, scale2, lane);
         }
         if (more) stash(buf ^ 1);
@@ -535,7 +561,7 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
             const bf16* kbase = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS;
             const bf16* vbase = a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff;
             const bool need_mask = (kb + 32 > k_hi) || (kb < k_lo);
-            attend_block<HS, 1>(kbase, vbase, kb, q, acc, m, l, qpos, lo, k_hi, need_mask, scale2, lane);
+            attend_block<HS, 1>(kbase, vbase, 0, kb, q, acc, m, l, qpos, lo, k_hi, need_mask, scale2, lane);
         }
     }
     // merge the four waves: every wave's (m, l, O^T) through shared memory, in wave order
