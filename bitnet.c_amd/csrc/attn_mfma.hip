@@ -87,13 +87,6 @@ __device__ __forceinline__ float max_over_lane_groups(float x) {
     auto t = __builtin_amdgcn_permlane32_swap(c, c, false, false);
     return fmaxf(__uint_as_float(t[0]), __uint_as_float(t[1]));
 }
-__device__ __forceinline__ float sum_over_lane_groups(float x) {
-    const unsigned b = __float_as_uint(x);
-    auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
-    const unsigned c = __float_as_uint(__uint_as_float(r[0]) + __uint_as_float(r[1]));
-    auto t = __builtin_amdgcn_permlane32_swap(c, c, false, false);
-    return __uint_as_float(t[0]) + __uint_as_float(t[1]);
-}
 typedef __attribute__((ext_vector_type(8))) float f32x8;
 // eight floats to eight bf16, round to nearest even (gfx950 converts two a time in hardware)
 __device__ __forceinline__ bf16x8 pack8(const float (&s)[8]) {
@@ -218,15 +211,13 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
         // weights hold as well, and the accumulators need no rescaling.  The result is the same.
         float m_new = m[nt];
         if (mx > m[nt] + 8.0f || m[nt] == -INFINITY) m_new = mx;
-        float rs = 0.f;
         if (m_new == -INFINITY) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) s[e] = 0.f;
         } else {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) { s[e] = __builtin_amdgcn_exp2f(fmaf(s[e], scale2, -m_new)); rs += s[e]; }
+            for (int e = 0; e < 8; ++e) s[e] = __builtin_amdgcn_exp2f(fmaf(s[e], scale2, -m_new));
         }
-        rs = sum_over_lane_groups(rs);
         const bool moved = m_new != m[nt];
         if (__any(moved)) {
             const float alpha = (moved && m[nt] != -INFINITY) ? __builtin_amdgcn_exp2f(m[nt] - m_new) : (moved ? 0.f : 1.f);
@@ -234,9 +225,18 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
 #pragma unroll
             for (int t = 0; t < DT; ++t) acc[nt][t] *= alpha;
         }
-        l[nt] += rs;
         m[nt] = m_new;
         pb[nt] = pack8(s);
+    }
+    // The sums of the weights come from the matrix cores too: a tile of ones times P gives every lane
+    // the sum over the 32 keys for its column (the same bf16 weights that multiply V, so numerator
+    // and denominator agree), instead of eight additions and two exchanges between lane groups.
+    f32x4 lsum[NT];
+    {
+        const bf16x8 ones = __builtin_bit_cast(bf16x8, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+            lsum[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[nt], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
     }
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
@@ -249,6 +249,8 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
         for (int nt = 0; nt < NT; ++nt)
             acc[nt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[STREAM ? 0 : t], pb[nt], acc[nt][t], 0, 0, 0);
     }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) l[nt] += lsum[nt][0];
 }
 
 // The masked form (a block on the causal diagonal, at a window's edge or at the end of the keys) and
