@@ -101,6 +101,14 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
     return (ua >> 16) | (ub & 0xffff0000u);
 }
 
+// A read of p[idx] for an index that is the same in every lane, through the scalar unit (the
+// constant address space makes the compiler pick a scalar load).  Only for memory that no kernel
+// writes while this one runs (block tables, lengths).
+__device__ __forceinline__ int uniform_load(const int* p, size_t idx) {
+    typedef const int __attribute__((address_space(4))) * scalar_ptr;
+    return reinterpret_cast<scalar_ptr>(reinterpret_cast<uintptr_t>(p))[idx];
+}
+
 // Shared memory serves 16 lanes of a 16-byte read at once, from 64 banks of 4 bytes.  The lanes
 // that read a staged key block together hold rows 8a + b (+4 for the second tile), a, b in 0..3, and
 // all want the same 16-byte chunk: rows are stored without padding and chunk c of row r lives at
@@ -338,29 +346,32 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int g_hi = pos0 + n_tok - 1;
     const int g_lo = a.window > 0 ? max(0, pos0 + 1 - a.window) : 0;
     const size_t bt_row = (size_t)seq * a.bt_stride;
-    uint4 kr[KV4], vr[KV4];
+    // the stage in flight: one or two 16-byte pieces of K and of V^T per thread, in named registers (arrays
+    // indexed in a loop end up in memory when they have to live across the products)
+    static_assert(KV4 == 1 || KV4 == 2, "a thread stages one or two pieces of K and of V^T");
+    uint4 kr0 = make_uint4(0, 0, 0, 0), kr1 = kr0, vr0 = kr0, vr1 = kr0;
     auto fetch = [&](int kb) {                            // a stage never crosses a page: KB divides BN_PAGE
-        const int page = a.block_table[bt_row + kb / BN_PAGE];
+        const int page = uniform_load(a.block_table, bt_row + kb / BN_PAGE);
         const int koff = kb % BN_PAGE;
         const bf16* kg = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS;      // KB rows of HS, contiguous
         const bf16* vg = a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff;       // HS rows, KB of 64 keys each
-#pragma unroll
-        for (int j = 0; j < KV4; ++j) {
-            const int idx = threadIdx.x + 256 * NG * j;
-            kr[j] = *reinterpret_cast<const uint4*>(kg + (size_t)idx * 8);
-            const int vrow = idx / (KB / 8), vcol = (idx % (KB / 8)) * 8;
-            vr[j] = *reinterpret_cast<const uint4*>(vg + (size_t)vrow * BN_PAGE + vcol);
+        const int i0 = threadIdx.x, i1 = threadIdx.x + 256 * NG;
+        kr0 = *reinterpret_cast<const uint4*>(kg + (size_t)i0 * 8);
+        vr0 = *reinterpret_cast<const uint4*>(vg + (size_t)(i0 / (KB / 8)) * BN_PAGE + (i0 % (KB / 8)) * 8);
+        if (KV4 > 1) {
+            kr1 = *reinterpret_cast<const uint4*>(kg + (size_t)i1 * 8);
+            vr1 = *reinterpret_cast<const uint4*>(vg + (size_t)(i1 / (KB / 8)) * BN_PAGE + (i1 % (KB / 8)) * 8);
         }
     };
-    auto stash = [&](int buf) {
-#pragma unroll
-        for (int j = 0; j < KV4; ++j) {
-            const int idx = threadIdx.x + 256 * NG * j;
-            const int krow = (idx * 8) / HS, kchunk = ((idx * 8) % HS) / 8;
-            *reinterpret_cast<uint4*>(k_s(buf) + krow * KS + ((kchunk ^ k_swizzle<HS>(krow)) * 8)) = kr[j];
-            const int vrow = idx / (KB / 8), vcol = (idx % (KB / 8)) * 8;
-            *reinterpret_cast<uint4*>(v_s(buf) + vrow * VS + (((vcol >> 3) ^ v_swizzle<KB>(vrow & 15)) * 8)) = vr[j];
-        }
+    auto stash_one = [&](int buf, int idx, const uint4& kv, const uint4& vv) {
+        const int krow = (idx * 8) / HS, kchunk = ((idx * 8) % HS) / 8;
+        *reinterpret_cast<uint4*>(k_s(buf) + krow * KS + ((kchunk ^ k_swizzle<HS>(krow)) * 8)) = kv;
+        const int vrow = idx / (KB / 8), vchunk = idx % (KB / 8);
+        *reinterpret_cast<uint4*>(v_s(buf) + vrow * VS + ((vchunk ^ v_swizzle<KB>(vrow & 15)) * 8)) = vv;
+    };
+    auto stash = [&](int buf, int zero = 0) {             // zero: 0, in a form the compiler cannot see through
+        stash_one(buf, threadIdx.x + zero, kr0, vr0);
+        if (KV4 > 1) stash_one(buf, threadIdx.x + 256 * NG + zero, kr1, vr1);
     };
     const int kb0 = (g_lo / KB) * KB;
     fetch(kb0);
@@ -376,7 +387,13 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
             attend_block<HS, NT, KS, VS, true>(k_s(buf) + 32 * grp * KS, v_s(buf), 4 * grp, kbb, q, acc, m, l, qpos, lo,
                                                w_hi + 1, need_mask, scale2, lane);
         }
-        if (more) stash(buf ^ 1);
+        // The stores of the next stage must stay behind the products: next to their loads (where the
+        // compiler puts them otherwise, both being under the same condition) they would wait out the
+        // whole memory latency before the block is multiplied, instead of hiding it behind the block.
+        // An empty asm makes the store offset look as if it came out of the last product.
+        int after_products = 0;
+        asm volatile("" : "+v"(after_products) : "v"(acc[NT - 1][DT - 1][3]));
+        if (more) stash(buf ^ 1, after_products);
         __syncthreads();
     }
     if (NG > 1) {
@@ -446,14 +463,6 @@ __device__ __forceinline__ void rotate8(uint4& lo, uint4& hi, const float* __res
         pl[k] = pack2(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
         ph[k] = pack2(a0 * s0 + b0 * c0, a1 * s1 + b1 * c1);
     }
-}
-
-// A read of p[idx] for an index that is the same in every lane, through the scalar unit (the
-// constant address space makes the compiler pick a scalar load).  Only for memory that no kernel
-// writes while this one runs (block tables, lengths).
-__device__ __forceinline__ int uniform_load(const int* p, size_t idx) {
-    typedef const int __attribute__((address_space(4))) * scalar_ptr;
-    return reinterpret_cast<scalar_ptr>(reinterpret_cast<uintptr_t>(p))[idx];
 }
 
 template <int HS>
