@@ -195,6 +195,17 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
 #pragma unroll
         for (int t = 0; t < DT; ++t) va[t] = clear_missing(va[t]);
     }
+    // staged values: the first tiles of V^T are asked for now, so that they arrive while the weights are
+    // computed; every later tile is asked for when an earlier one has been used
+    constexpr int PF = DT < 4 ? DT : 4;
+    bf16x8 vpre[PF];
+    auto staged_v = [&](int t) {
+        return ld16(vbase + (size_t)(t * 16 + i) * VSTRIDE + ((vchunk0 + g) ^ v_swizzle<VSTRIDE>(i)) * 8);
+    };
+    if (STREAM) {
+#pragma unroll
+        for (int t = 0; t < PF; ++t) vpre[t] = staged_v(t);
+    }
     bf16x8 pb[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -211,27 +222,29 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
                 }
                 s[sb * 4 + r] = v;
             }
+        // The reference point m of the exponents moves only when some score of the column exceeds it
+        // by more than 2^8: until then p = 2^(s - m) may exceed 1 (at most 256), which float32 sums
+        // and bf16 weights hold as well, and nothing has to be rescaled.  So the common block only
+        // asks whether any lane of the wave sees such a score; the exchange between the four lane
+        // groups of a column, the new reference point and the rescaling happen when one does.
         float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
-        mx = max_over_lane_groups(mx);
         mx *= scale2;                                  // scale2 > 0: the maximum of the scaled scores
-        // The reference point of the exponents moves only when the maximum has grown by more than
-        // 2^8: until then p = 2^(s - m) may exceed 1 (at most 256), which float32 sums and bf16
-        // weights hold as well, and the accumulators need no rescaling.  The result is the same.
         float m_new = m[nt];
-        if (mx > m[nt] + 8.0f || m[nt] == -INFINITY) m_new = mx;
-        if (m_new == -INFINITY) {
+        if (__any(mx > m[nt] + 8.0f)) {                // also true for a column's first visible key (m = -inf)
+            mx = max_over_lane_groups(mx);
+            if (mx > m[nt] + 8.0f) m_new = mx;
+            const bool moved = m_new != m[nt];
+            const float alpha = (moved && m[nt] != -INFINITY) ? __builtin_amdgcn_exp2f(m[nt] - m_new) : (moved ? 0.f : 1.f);
+            l[nt] *= alpha;
+#pragma unroll
+            for (int t = 0; t < DT; ++t) acc[nt][t] *= alpha;
+        }
+        if (need_mask && m_new == -INFINITY) {         // a column that has seen no key yet (only behind a mask)
 #pragma unroll
             for (int e = 0; e < 8; ++e) s[e] = 0.f;
         } else {
 #pragma unroll
             for (int e = 0; e < 8; ++e) s[e] = __builtin_amdgcn_exp2f(fmaf(s[e], scale2, -m_new));
-        }
-        const bool moved = m_new != m[nt];
-        if (__any(moved)) {
-            const float alpha = (moved && m[nt] != -INFINITY) ? __builtin_amdgcn_exp2f(m[nt] - m_new) : (moved ? 0.f : 1.f);
-            l[nt] *= alpha;
-#pragma unroll
-            for (int t = 0; t < DT; ++t) acc[nt][t] *= alpha;
         }
         m[nt] = m_new;
         pb[nt] = pack8(s);
@@ -249,8 +262,8 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
         if (STREAM) {
-            // staged: VSTRIDE keys a row, this group's keys start at chunk vchunk0
-            va[0] = ld16(vbase + (size_t)(t * 16 + i) * VSTRIDE + ((vchunk0 + g) ^ v_swizzle<VSTRIDE>(i)) * 8);
+            va[0] = vpre[t % PF];
+            if (t + PF < DT) vpre[t % PF] = staged_v(t + PF);
             if (need_mask) va[0] = clear_missing(va[0]);
         }
 #pragma unroll
@@ -346,21 +359,21 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int g_hi = pos0 + n_tok - 1;
     const int g_lo = a.window > 0 ? max(0, pos0 + 1 - a.window) : 0;
     const size_t bt_row = (size_t)seq * a.bt_stride;
-    // the stage in flight: one or two 16-byte pieces of K and of V^T per thread, in named registers (arrays
-    // indexed in a loop end up in memory when they have to live across the products)
+    // Two stages are in flight: one or two 16-byte pieces of K and of V^T per thread and stage, in named
+    // registers (arrays indexed in a loop end up in memory when they have to live across the products).
     static_assert(KV4 == 1 || KV4 == 2, "a thread stages one or two pieces of K and of V^T");
-    uint4 kr0 = make_uint4(0, 0, 0, 0), kr1 = kr0, vr0 = kr0, vr1 = kr0;
-    auto fetch = [&](int kb) {                            // a stage never crosses a page: KB divides BN_PAGE
+    struct Stage { uint4 k0, k1, v0, v1; };
+    auto fetch = [&](int kb, Stage& st) {                 // a stage never crosses a page: KB divides BN_PAGE
         const int page = uniform_load(a.block_table, bt_row + kb / BN_PAGE);
         const int koff = kb % BN_PAGE;
         const bf16* kg = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS;      // KB rows of HS, contiguous
         const bf16* vg = a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff;       // HS rows, KB of 64 keys each
         const int i0 = threadIdx.x, i1 = threadIdx.x + 256 * NG;
-        kr0 = *reinterpret_cast<const uint4*>(kg + (size_t)i0 * 8);
-        vr0 = *reinterpret_cast<const uint4*>(vg + (size_t)(i0 / (KB / 8)) * BN_PAGE + (i0 % (KB / 8)) * 8);
+        st.k0 = *reinterpret_cast<const uint4*>(kg + (size_t)i0 * 8);
+        st.v0 = *reinterpret_cast<const uint4*>(vg + (size_t)(i0 / (KB / 8)) * BN_PAGE + (i0 % (KB / 8)) * 8);
         if (KV4 > 1) {
-            kr1 = *reinterpret_cast<const uint4*>(kg + (size_t)i1 * 8);
-            vr1 = *reinterpret_cast<const uint4*>(vg + (size_t)(i1 / (KB / 8)) * BN_PAGE + (i1 % (KB / 8)) * 8);
+            st.k1 = *reinterpret_cast<const uint4*>(kg + (size_t)i1 * 8);
+            st.v1 = *reinterpret_cast<const uint4*>(vg + (size_t)(i1 / (KB / 8)) * BN_PAGE + (i1 % (KB / 8)) * 8);
         }
     };
     auto stash_one = [&](int buf, int idx, const uint4& kv, const uint4& vv) {
@@ -369,18 +382,14 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
         const int vrow = idx / (KB / 8), vchunk = idx % (KB / 8);
         *reinterpret_cast<uint4*>(v_s(buf) + vrow * VS + ((vchunk ^ v_swizzle<KB>(vrow & 15)) * 8)) = vv;
     };
-    auto stash = [&](int buf, int zero = 0) {             // zero: 0, in a form the compiler cannot see through
-        stash_one(buf, threadIdx.x + zero, kr0, vr0);
-        if (KV4 > 1) stash_one(buf, threadIdx.x + 256 * NG + zero, kr1, vr1);
+    auto stash = [&](int buf, const Stage& st, int zero = 0) {    // zero: 0, in a form the compiler cannot see through
+        stash_one(buf, threadIdx.x + zero, st.k0, st.v0);
+        if (KV4 > 1) stash_one(buf, threadIdx.x + 256 * NG + zero, st.k1, st.v1);
     };
-    const int kb0 = (g_lo / KB) * KB;
-    fetch(kb0);
-    stash(0);
-    __syncthreads();
-    int buf = 0;
-    for (int kb = kb0; kb <= g_hi; kb += KB, buf ^= 1) {
-        const bool more = kb + KB <= g_hi;
-        if (more) fetch(kb + KB);
+    // One stage of the walk: the loads of the stage after next go out, the current one (in shared memory
+    // `buf`) is multiplied, the next one (`have`, loaded a stage ago) is stored into the other buffer.
+    auto step = [&](int kb, int buf, Stage& want, const Stage& have) {
+        if (kb + 2 * KB <= g_hi) fetch(kb + 2 * KB, want);
         const int kbb = kb + 32 * grp;                    // this group's block of the stage
         if (w_hi >= 0 && kbb <= w_hi && kbb + 31 >= w_lo) {
             const bool need_mask = (kbb + 31 > all_hi) || (kbb < all_lo);
@@ -388,13 +397,24 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
                                                w_hi + 1, need_mask, scale2, lane);
         }
         // The stores of the next stage must stay behind the products: next to their loads (where the
-        // compiler puts them otherwise, both being under the same condition) they would wait out the
-        // whole memory latency before the block is multiplied, instead of hiding it behind the block.
-        // An empty asm makes the store offset look as if it came out of the last product.
+        // compiler puts them otherwise) they would wait out the memory latency before the block is
+        // multiplied, instead of hiding it behind the block.  An empty asm makes the store offset look
+        // as if it came out of the last product.
         int after_products = 0;
         asm volatile("" : "+v"(after_products) : "v"(acc[NT - 1][DT - 1][3]));
-        if (more) stash(buf ^ 1, after_products);
+        if (kb + KB <= g_hi) stash(buf ^ 1, have, after_products);
         __syncthreads();
+    };
+    Stage sa = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)}, sb = sa;
+    const int kb0 = (g_lo / KB) * KB;
+    fetch(kb0, sa);
+    stash(0, sa);
+    if (kb0 + KB <= g_hi) fetch(kb0 + KB, sa);
+    __syncthreads();
+    for (int kb = kb0; kb <= g_hi; kb += 2 * KB) {
+        step(kb, 0, sb, sa);
+        if (kb + KB > g_hi) break;
+        step(kb + KB, 1, sa, sb);
     }
     if (NG > 1) {
         // the later groups hand their partial results to group 0, one column tile a time; the staging
