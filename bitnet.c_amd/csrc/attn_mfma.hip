@@ -138,6 +138,132 @@ __device__ __forceinline__ int v_swizzle(int row) {
 // One 32-key block for NT column tiles.  kbase/vbase point at the block's first key inside its
 // page (row strides HS and BN_PAGE) or inside a staged copy in shared memory (KSTRIDE, VSTRIDE).  qpos/lo: per tile, this lane's column's position and first visible key (qpos < 0: no
 // such column).  key_hi: keys >= key_hi do not exist (decode: split end / length).
+// The same block for operands that come straight from the pages (the decode form: STREAM is false
+// here).  It is a copy of its own on purpose: the decode kernel is sensitive to how the compiler lays
+// this code out, and changes made for the staged form below must not move it.
+template <int HS, int NT, int KSTRIDE, int VSTRIDE, bool STREAM, bool need_mask>
+__device__ __forceinline__ void attend_block_direct_m(const bf16* __restrict__ kbase, const bf16* __restrict__ vbase,
+                                               int vchunk0, int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
+                                               float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
+                                               const int (&lo)[NT], int key_hi, float scale2, int lane) {
+    // STREAM: the operands come from shared memory (short latency): fetch each one right before its
+    // products instead of all of them up front, which keeps fewer registers live.
+    constexpr int DC = HS / 32, DT = HS / 16;
+    const int i = lane & 15, g = lane >> 4;
+    const int krow0 = 8 * (i >> 2) + (i & 3);        // key row of tile 0; tile 1 is 4 further
+    f32x4 st[NT][2];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) { st[nt][0] = (f32x4){0.f, 0.f, 0.f, 0.f}; st[nt][1] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
+    bf16x8 ka[STREAM ? 1 : DC][2];
+    bf16x8 va[STREAM ? 1 : DT];
+    if (!STREAM) {
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+            ka[c][0] = ld16(kbase + (size_t)krow0 * KSTRIDE + c * 32 + g * 8);
+            ka[c][1] = ld16(kbase + (size_t)(krow0 + 4) * KSTRIDE + c * 32 + g * 8);
+        }
+#pragma unroll
+        for (int t = 0; t < DT; ++t) va[t] = ld16(vbase + (size_t)(t * 16 + i) * VSTRIDE + 8 * g);
+    }
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+        if (STREAM) {
+            // staged keys are stored with their 16-byte chunks swizzled (k_swizzle): the 16 lanes that read
+            // together want the same chunk of 16 different rows
+            const int chunk = ((c * 4 + g) ^ k_swizzle<HS>(krow0)) * 8;
+            ka[0][0] = ld16(kbase + (size_t)krow0 * KSTRIDE + chunk);
+            ka[0][1] = ld16(kbase + (size_t)(krow0 + 4) * KSTRIDE + chunk);
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            st[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[STREAM ? 0 : c][0], q[nt][c], st[nt][0], 0, 0, 0);
+            st[nt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[STREAM ? 0 : c][1], q[nt][c], st[nt][1], 0, 0, 0);
+        }
+    }
+    // keys that do not exist may hold anything, NaN included: they are cleared in V^T (0 * NaN is NaN)
+    const int first = kb + 8 * g;                     // this lane's 8 keys are first .. first+7
+    auto clear_missing = [&](bf16x8 x) {
+        uint4 v = __builtin_bit_cast(uint4, x);
+        if (first + 0 >= key_hi) v.x &= 0xffff0000u;
+        if (first + 1 >= key_hi) v.x &= 0x0000ffffu;
+        if (first + 2 >= key_hi) v.y &= 0xffff0000u;
+        if (first + 3 >= key_hi) v.y &= 0x0000ffffu;
+        if (first + 4 >= key_hi) v.z &= 0xffff0000u;
+        if (first + 5 >= key_hi) v.z &= 0x0000ffffu;
+        if (first + 6 >= key_hi) v.w &= 0xffff0000u;
+        if (first + 7 >= key_hi) v.w &= 0x0000ffffu;
+        return __builtin_bit_cast(bf16x8, v);
+    };
+    if (!STREAM && need_mask) {
+#pragma unroll
+        for (int t = 0; t < DT; ++t) va[t] = clear_missing(va[t]);
+    }
+    bf16x8 pb[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        // raw scores; the scale (with log2 e folded in) is applied inside the exponent's fma
+        float s[8];
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float v = st[nt][sb][r];
+                if (need_mask) {
+                    const int key = kb + 8 * g + 4 * sb + r;
+                    if (key > qpos[nt] || key < lo[nt] || key >= key_hi) v = -INFINITY;
+                }
+                s[sb * 4 + r] = v;
+            }
+        float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+        mx = max_over_lane_groups(mx);
+        mx *= scale2;                                  // scale2 > 0: the maximum of the scaled scores
+        // The reference point of the exponents moves only when the maximum has grown by more than
+        // 2^8: until then p = 2^(s - m) may exceed 1 (at most 256), which float32 sums and bf16
+        // weights hold as well, and the accumulators need no rescaling.  The result is the same.
+        float m_new = m[nt];
+        if (mx > m[nt] + 8.0f || m[nt] == -INFINITY) m_new = mx;
+        if (m_new == -INFINITY) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s[e] = 0.f;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s[e] = __builtin_amdgcn_exp2f(fmaf(s[e], scale2, -m_new));
+        }
+        const bool moved = m_new != m[nt];
+        if (__any(moved)) {
+            const float alpha = (moved && m[nt] != -INFINITY) ? __builtin_amdgcn_exp2f(m[nt] - m_new) : (moved ? 0.f : 1.f);
+            l[nt] *= alpha;
+#pragma unroll
+            for (int t = 0; t < DT; ++t) acc[nt][t] *= alpha;
+        }
+        m[nt] = m_new;
+        pb[nt] = pack8(s);
+    }
+    // The sums of the weights come from the matrix cores too: a tile of ones times P gives every lane
+    // the sum over the 32 keys for its column (the same bf16 weights that multiply V, so numerator
+    // and denominator agree), instead of eight additions and two exchanges between lane groups.
+    f32x4 lsum[NT];
+    {
+        const bf16x8 ones = __builtin_bit_cast(bf16x8, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+            lsum[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[nt], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+        if (STREAM) {
+            // staged: VSTRIDE keys a row, this group's keys start at chunk vchunk0
+            va[0] = ld16(vbase + (size_t)(t * 16 + i) * VSTRIDE + ((vchunk0 + g) ^ v_swizzle<VSTRIDE>(i)) * 8);
+            if (need_mask) va[0] = clear_missing(va[0]);
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+            acc[nt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[STREAM ? 0 : t], pb[nt], acc[nt][t], 0, 0, 0);
+    }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) l[nt] += lsum[nt][0];
+}
+
 template <int HS, int NT, int KSTRIDE, int VSTRIDE, bool STREAM, bool need_mask>
 __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, const bf16* __restrict__ vbase,
                                                int vchunk0, int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
@@ -228,16 +354,18 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
         // asks whether any lane of the wave sees such a score; the exchange between the four lane
         // groups of a column, the new reference point and the rescaling happen when one does.
         float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
-        mx *= scale2;                                  // scale2 > 0: the maximum of the scaled scores
         float m_new = m[nt];
+        mx *= scale2;                                  // scale2 > 0: the maximum of the scaled scores
         if (__any(mx > m[nt] + 8.0f)) {                // also true for a column's first visible key (m = -inf)
             mx = max_over_lane_groups(mx);
             if (mx > m[nt] + 8.0f) m_new = mx;
             const bool moved = m_new != m[nt];
-            const float alpha = (moved && m[nt] != -INFINITY) ? __builtin_amdgcn_exp2f(m[nt] - m_new) : (moved ? 0.f : 1.f);
-            l[nt] *= alpha;
+            if (__any(moved)) {
+                const float alpha = (moved && m[nt] != -INFINITY) ? __builtin_amdgcn_exp2f(m[nt] - m_new) : (moved ? 0.f : 1.f);
+                l[nt] *= alpha;
 #pragma unroll
-            for (int t = 0; t < DT; ++t) acc[nt][t] *= alpha;
+                for (int t = 0; t < DT; ++t) acc[nt][t] *= alpha;
+            }
         }
         if (need_mask && m_new == -INFINITY) {         // a column that has seen no key yet (only behind a mask)
 #pragma unroll
@@ -282,7 +410,12 @@ __device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, con
                                              float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
                                              const int (&lo)[NT], int key_hi, bool need_mask, float scale2,
                                              int lane) {
-    if (need_mask)
+    if (!STREAM) {
+        if (need_mask)
+            attend_block_direct_m<HS, NT, KSTRIDE, VSTRIDE, false, true>(kbase, vbase, vchunk0, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
+        else
+            attend_block_direct_m<HS, NT, KSTRIDE, VSTRIDE, false, false>(kbase, vbase, vchunk0, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
+    } else if (need_mask)
         attend_block_m<HS, NT, KSTRIDE, VSTRIDE, STREAM, true>(kbase, vbase, vchunk0, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
     else
         attend_block_m<HS, NT, KSTRIDE, VSTRIDE, STREAM, false>(kbase, vbase, vchunk0, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
