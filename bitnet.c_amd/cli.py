@@ -1,7 +1,8 @@
 """Command line in the manner of the reference's `bitnet <model> [options]`
 (src/main.c:110-168, 224-431): the same option names with the same meaning and the same
 defaults where this library has the feature (-p, --prompt-token-ids, -n, --temp, --topp,
---seed, --maxseq, --repeat-penalty, --no-prefill, --quiet, --token-ids, --bos/--no-bos).
+--seed, --maxseq, --repeat-penalty, --no-prefill, --quiet, --token-ids, --bos/--no-bos,
+--top-logits, --benchmark-runs, --benchmark-warmup-runs, --bench-warmup-tokens).
 The model is a folder (config.json + model.safetensors) instead of a GGUF file.  Text
 prompts need the folder's tokenizer.json; token ids in, token ids out always works.
 """
@@ -29,7 +30,14 @@ def _parser() -> argparse.ArgumentParser:
     ap.add_argument("--token-ids", action="store_true", help="print generated token ids to stderr")
     ap.add_argument("--bos", dest="bos", action="store_true", default=True, help="prepend BOS to a text prompt")
     ap.add_argument("--no-bos", dest="bos", action="store_false")
+    ap.add_argument("--top-logits", type=int, default=0, help="print the K largest logits before every sampling (at most 32)")
+    ap.add_argument("--benchmark-runs", type=int, default=0, help="measured runs of the same request on one loaded model")
+    ap.add_argument("--benchmark-warmup-runs", type=int, default=0, help="unreported runs before the measured ones")
+    ap.add_argument("--bench-warmup-tokens", type=int, default=0,
+                    help="tokens generated after the prompt before the clock of tok/s starts")
     ap.add_argument("--fp32", action="store_true", help="run the whole model in float32")
+    ap.add_argument("--random", default=None, metavar="CONFIG_JSON",
+                    help="first write MODEL as a new folder: this configuration with random weights from --seed")
     ap.add_argument("--batch-file", default=None, help="file with one comma-separated prompt (token ids) a line")
     ap.add_argument("--batch", type=int, default=8, help="sequences per batch with --batch-file (default 8)")
     return ap
@@ -49,13 +57,58 @@ def _ids(text: str, vocab: int):
     return out
 
 
+MAX_TOP_LOGITS = 32      # src/generate.c:64
+
+
+def _with_top_logits(sample_fn, k: int):
+    """A sampler that first prints the k largest logits of every row, in the lines of
+    src/generate.c:83-86 (one block per row; `step` counts the samplings)."""
+    import torch
+    k = min(k, MAX_TOP_LOGITS)
+    step = [0]
+
+    def fn(logits, samplers):
+        kk = min(k, logits.shape[1])
+        vals, idx = torch.topk(logits.float(), kk, dim=1)
+        for row, (v, i) in enumerate(zip(vals.tolist(), idx.tolist())):
+            label = "generate" if logits.shape[0] == 1 else f"generate[{row}]"
+            print(f"top_logits {label} step={step[0]} k={kk}", file=sys.stderr)
+            for r, (x, t) in enumerate(zip(v, i)):
+                print(f"top_logit step={step[0]} rank={r + 1} token={t} logit={x:.9g}", file=sys.stderr)
+        step[0] += 1
+        return sample_fn(logits, samplers)
+    return fn
+
+
+def _check_benchmark_args(args) -> None:
+    # src/main.c:921-931
+    if args.benchmark_runs < 0 or args.benchmark_warmup_runs < 0 or args.bench_warmup_tokens < 0:
+        raise SystemExit("--benchmark-runs, --benchmark-warmup-runs and --bench-warmup-tokens must not be negative")
+    if args.benchmark_warmup_runs > 0 and args.benchmark_runs == 0:
+        raise SystemExit("--benchmark-warmup-runs requires --benchmark-runs")
+    if (args.benchmark_runs > 0 or args.bench_warmup_tokens > 0) and args.batch_file:
+        raise SystemExit("--benchmark-runs and --bench-warmup-tokens take one prompt, not --batch-file")
+
+
 def main(argv=None) -> int:
     args = _parser().parse_args(argv)
+    _check_benchmark_args(args)
     import torch
     from . import api
     from .engine import Request, StepEntry, generate
     from .sampling import SamplingParams, sample_batch
 
+    if args.random:
+        import json
+        from .config import architecture_for
+        from .weights import write_model_folder
+        if os.path.exists(os.path.join(args.model, "model.safetensors")):
+            raise SystemExit(f"--random: {args.model} already holds a model")
+        with open(args.random) as f:
+            raw = json.load(f)
+        write_model_folder(args.model, architecture_for(raw).config_cls.from_dict(raw), args.seed,
+                           "float32" if args.fp32 else "bfloat16")
+        print(f"[bitnet] wrote {args.model} (random weights, seed {args.seed})", file=sys.stderr)
     tok = None
     tok_path = os.path.join(args.model, "tokenizer.json")
     if os.path.isfile(tok_path):
@@ -89,37 +142,63 @@ def main(argv=None) -> int:
     params = SamplingParams(temperature=args.temp, top_p=args.topp, seed=args.seed,
                             repeat_penalty=args.repeat_penalty)
     stop = tuple(eng.model.plan.stop_ids)
-    reqs = [Request(p, args.n_tokens, params, stop) for p in prompts]
+    warm = args.bench_warmup_tokens
+    reqs = [Request(p, args.n_tokens + warm, params, stop) for p in prompts]
+    repeated = args.benchmark_runs > 0
+    sampler = _with_top_logits(sample_batch, args.top_logits) if args.top_logits > 0 else sample_batch
+    stamps = []                                       # when each token of the (single) request came
 
     def emit(i, t):
-        if not args.quiet and len(prompts) == 1:
+        stamps.append(time.time())
+        if len(stamps) <= warm:
+            return False
+        if not args.quiet and not repeated and len(prompts) == 1:
             sys.stdout.write(tok.decode([t]) if tok is not None else f"{t} ")
             sys.stdout.flush()
         return False
 
-    torch.cuda.synchronize()
-    t1 = time.time()
-    if args.no_prefill and len(prompts) == 1:
-        # the prompt one token at a time (src/generate.c:405-416), then the usual loop
-        class OneByOne:
-            def __init__(self, e):
-                self.e = e
-                self.cache, self.max_seq_len = e.cache, e.max_seq_len
-            def new_sequence(self): return self.e.new_sequence()
-            def release(self, s): self.e.release(s)
-            def step(self, entries):
-                ent = entries[0]
-                if len(ent.tokens) == 1:
-                    return self.e.step(entries)
-                for t in ent.tokens[:-1]:
-                    self.e.step([StepEntry(ent.slot, [t], [])])
-                return self.e.step([StepEntry(ent.slot, [ent.tokens[-1]], [0])])
-        results = generate(OneByOne(eng), reqs, sample_batch, batch_size=1, on_token=emit)
-    else:
-        results = generate(eng, reqs, sample_batch, batch_size=args.batch, on_token=emit)
-    torch.cuda.synchronize()
-    dt = time.time() - t1
-    if not args.quiet and len(prompts) == 1:
+    # the prompt one token at a time (src/generate.c:405-416), then the usual loop
+    class OneByOne:
+        def __init__(self, e):
+            self.e = e
+            self.cache, self.max_seq_len = e.cache, e.max_seq_len
+        def new_sequence(self): return self.e.new_sequence()
+        def release(self, s): self.e.release(s)
+        def step(self, entries):
+            ent = entries[0]
+            if len(ent.tokens) == 1:
+                return self.e.step(entries)
+            for t in ent.tokens[:-1]:
+                self.e.step([StepEntry(ent.slot, [t], [])])
+            return self.e.step([StepEntry(ent.slot, [ent.tokens[-1]], [0])])
+
+    # Repetitions start from fresh request state (a new slot, a new generator) and keep the loaded
+    # model (src/main.c:1607-1616).
+    total_runs = args.benchmark_warmup_runs + args.benchmark_runs if repeated else 1
+    for run in range(total_runs):
+        del stamps[:]
+        torch.cuda.synchronize()
+        t1 = time.time()
+        if args.no_prefill and len(prompts) == 1:
+            results = generate(OneByOne(eng), reqs, sampler, batch_size=1, on_token=emit)
+        else:
+            results = generate(eng, reqs, sampler, batch_size=args.batch, on_token=emit)
+        torch.cuda.synchronize()
+        t2 = time.time()
+        if len(prompts) == 1:
+            # the clock of tok/s starts after the prompt and the warm-up tokens (src/main.c:1651-1668)
+            timed = max(0, len(stamps) - warm)
+            # the first token is sampled from the prompt's logits: the prompt phase ends there
+            prompt_end = stamps[0] if stamps else t2
+            gen_start = stamps[warm] if warm and len(stamps) > warm else prompt_end
+            for r in results:
+                r.tokens = r.tokens[warm:]
+            speed = timed / (t2 - gen_start) if timed and t2 > gen_start else 0.0
+            if repeated and run >= args.benchmark_warmup_runs:
+                print(f"Benchmark sample run={run - args.benchmark_warmup_runs + 1} tokens={timed} "
+                      f"tok/s={speed:.2f} prompt_ms={(prompt_end - t1) * 1e3:.1f}", file=sys.stderr)
+    dt = t2 - t1
+    if not args.quiet and not repeated and len(prompts) == 1:
         sys.stdout.write("\n")
     n_gen = sum(len(r.tokens) for r in results)
     for i, r in enumerate(results):
@@ -127,8 +206,12 @@ def main(argv=None) -> int:
             print(f"[bitnet] request {i}: {r.finish}", file=sys.stderr)
         if args.token_ids or len(prompts) > 1:
             print(("" if len(prompts) == 1 else f"{i}: ") + ",".join(str(t) for t in r.tokens), file=sys.stderr)
-    print(f"tokens: {n_gen}  tok/s: {n_gen / dt if dt > 0 else 0.0:.2f}  total_ms: {dt * 1e3:.1f}  "
-          f"load_ms: {load_s * 1e3:.0f}", file=sys.stderr)
+    if len(prompts) == 1:
+        print(f"tokens: {n_gen}  tok/s: {speed:.2f}  prompt_ms: {(prompt_end - t1) * 1e3:.1f}  "
+              f"total_ms: {dt * 1e3:.1f}  load_ms: {load_s * 1e3:.0f}", file=sys.stderr)
+    else:
+        print(f"tokens: {n_gen}  tok/s: {n_gen / dt if dt > 0 else 0.0:.2f}  total_ms: {dt * 1e3:.1f}  "
+              f"load_ms: {load_s * 1e3:.0f}", file=sys.stderr)
     return 0
 
 

@@ -127,3 +127,48 @@ def test_command_line_with_a_text_prompt(model_folders, tmp_path):
     p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "bitnet"), src, "-p", "w1 w2", "-n", "2", "--fp32"],
                        capture_output=True, text=True, timeout=300)
     assert p.returncode != 0 and "tokenizer.json" in p.stderr + p.stdout
+
+
+def test_command_line_benchmark_runs_top_logits_and_a_random_folder(tmp_path):
+    """--random writes the folder from a configuration and --seed; --benchmark-runs repeats the
+    request on the loaded model (every run from fresh request state: the same tokens); the
+    --bench-warmup-tokens are generated but neither printed nor counted; --top-logits prints the
+    largest logits before every sampling, the first of which is the token greedy decoding takes."""
+    import json
+    from conftest import TINY_B
+    cfg_path = str(tmp_path / "cfg.json")
+    with open(cfg_path, "w") as f:
+        json.dump(TINY_B, f)
+    folder = str(tmp_path / "made")
+    prompt = [7, 2, 9, 4]
+    exe = [sys.executable, os.path.join(ROOT, "bin", "bitnet")]
+    common = ["--prompt-token-ids", ",".join(map(str, prompt)), "--repeat-penalty", "1.0", "--fp32", "--token-ids", "--quiet"]
+    p = subprocess.run(exe + [folder, "--random", cfg_path, "--seed", "5", "-n", "7", "--top-logits", "3"] + common,
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-1500:]
+    assert os.path.isfile(os.path.join(folder, "model.safetensors")) and os.path.isfile(os.path.join(folder, "config.json"))
+    c, W = pl.read_config(folder), pl.read_weights(folder)
+    want = pl.generate(c, W, prompt, 7)
+    ids = [l for l in p.stderr.splitlines() if l and l[0].isdigit()][0]
+    assert [int(x) for x in ids.split(",")] == want
+    heads = [l for l in p.stderr.splitlines() if l.startswith("top_logits generate step=")]
+    assert len(heads) == 7 and heads[0].endswith("k=3")
+    firsts = [int(l.split("token=")[1].split()[0]) for l in p.stderr.splitlines() if l.startswith("top_logit ") and "rank=1 " in l]
+    assert firsts == want
+    lg = pl.forward(c, W, prompt)[-1]
+    first_line = [l for l in p.stderr.splitlines() if l.startswith("top_logit step=0 rank=1 ")][0]
+    assert abs(float(first_line.split("logit=")[1]) - float(lg.max())) <= 1e-4 * float(lg.pow(2).mean().sqrt())
+    # the folder exists now: --random refuses to overwrite it
+    p = subprocess.run(exe + [folder, "--random", cfg_path, "-n", "1"] + common, capture_output=True, text=True, timeout=300)
+    assert p.returncode != 0 and "already holds a model" in p.stderr + p.stdout
+    # repeated runs: 1 unreported + 2 reported, 2 warm-up tokens each
+    p = subprocess.run(exe + [folder, "-n", "5", "--benchmark-runs", "2", "--benchmark-warmup-runs", "1",
+                              "--bench-warmup-tokens", "2"] + common, capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-1500:]
+    samples = [l for l in p.stderr.splitlines() if l.startswith("Benchmark sample run=")]
+    assert [l.split()[2] for l in samples] == ["run=1", "run=2"]
+    assert all("tokens=5" in l and "tok/s=" in l and "prompt_ms=" in l for l in samples)
+    ids = [l for l in p.stderr.splitlines() if l and l[0].isdigit()][0]
+    assert [int(x) for x in ids.split(",")] == want[2:]
+    p = subprocess.run(exe + [folder, "-n", "1", "--benchmark-warmup-runs", "1"] + common, capture_output=True, text=True, timeout=300)
+    assert p.returncode != 0 and "--benchmark-runs" in p.stderr + p.stdout
