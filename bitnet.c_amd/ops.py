@@ -9,6 +9,7 @@ step can be captured into a HIP graph.
 from __future__ import annotations
 
 import ctypes
+import os
 from ctypes import c_float, c_int, c_longlong, c_void_p
 
 import torch
@@ -53,6 +54,10 @@ _SIGNATURES = {
     "gemm_tiled": {
         "bn_gemm_tiled": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                           c_void_p],
+    },
+    "gemm_mfma": {
+        "bn_gemm_mfma_supports": [c_int, c_int, c_int, c_int, c_int],
+        "bn_gemm_mfma": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "skinny_gemm": {
         "bn_skinny_gemm_supports": [c_int, c_int, c_int, c_int, c_int],
@@ -222,6 +227,30 @@ def _tiled(x, w, out_dtype):
     return y
 
 
+def gemm_mfma(x: torch.Tensor, w: torch.Tensor, out_dtype=None, glu8: bool = False) -> torch.Tensor:
+    """The library-free bf16 product for many rows: y[M, N] = x[M, K] . w[N, K]^T on the matrix cores,
+    or with glu8 silu(gate) * up for w = gate and up rows interleaved in blocks of 8 ([2N, K])."""
+    require_gpu()
+    _dev(x, "x", torch.bfloat16, 2)
+    _dev(w, "w", torch.bfloat16, 2)
+    M, K = x.shape
+    rows = w.shape[0]
+    if w.shape[1] != K or (glu8 and rows % 16):
+        raise KernelError(f"gemm_mfma: x {tuple(x.shape)} and w {tuple(w.shape)} do not agree")
+    N = rows // 2 if glu8 else rows
+    out_dtype = out_dtype or torch.bfloat16
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    if M == 0:
+        return y
+    _check(_fn("gemm_mfma", "bn_gemm_mfma")(_code(out_dtype), x.data_ptr(), w.data_ptr(), y.data_ptr(), M, N, K,
+                                            _rows(x, "x"), _rows(w, "w"), N, int(glu8), _stream()), "gemm_mfma")
+    return y
+
+
+def gemm_mfma_supported(M: int, N: int, K: int, ldx: int, ldw: int) -> bool:
+    return bool(_fn("gemm_mfma", "bn_gemm_mfma_supports")(M, N, K, ldx, ldw))
+
+
 SKINNY_ROWS = 16      # bf16 products with more rows than this go to the library
 
 
@@ -229,16 +258,22 @@ def skinny_supported(M: int, N: int, K: int, ldx: int, ldw: int) -> bool:
     return bool(_fn("skinny_gemm", "bn_skinny_gemm_supports")(M, N, K, ldx, ldw))
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, *, allow_library: bool = True) -> torch.Tensor:
+# bf16 products with many rows: the library's matrix product (as the reference hands its batched
+# products to a library, src/gpu_cuda.cu:11571) unless this is False or BITNET_NO_LIBRARY is set;
+# then this library's own matrix-core kernel (gemm_mfma) does them.
+LIBRARY_PRODUCTS = os.environ.get("BITNET_NO_LIBRARY", "") in ("", "0")
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, *, allow_library: Optional[bool] = None) -> torch.Tensor:
     """y[M, N] = x[M, K] . w[N, K]^T.
 
     float32: the tiled kernel (plain fmaf, a fixed order of summation).
     bf16: up to 16 rows (one MFMA tile of activations) the matrix-core kernel that streams
-    the weights once; above that the library's matrix product (as the reference hands its
-    batched products to a library, src/gpu_cuda.cu:11571), which from 32 rows on is about
-    twice as fast as the streaming kernel, with a bf16 or a float32 result (logits); without the
-    library the streaming kernel takes 64 rows at a time; shapes neither takes go to the tiled
-    kernel."""
+    the weights once; above that the library's matrix product, which from 32 rows on is about
+    twice as fast as the streaming kernel, with a bf16 or a float32 result (logits).  Without the
+    library (allow_library False; None follows LIBRARY_PRODUCTS) the streaming kernel takes up to 64
+    rows and the tiled matrix-core kernel (gemm_mfma) everything above; shapes that none of them
+    takes (rows that are not 16-byte aligned) go to the plain tiled kernel."""
     require_gpu()
     _dev(x, "x", dims=2)
     _dev(w, "w", x.dtype, 2)
@@ -247,6 +282,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, *, allow_library: b
     if w.shape[1] != K:
         raise KernelError(f"linear: x {tuple(x.shape)} and w {tuple(w.shape)} do not agree")
     out_dtype = out_dtype or x.dtype
+    if allow_library is None:
+        allow_library = LIBRARY_PRODUCTS
     if M == 0:
         return torch.empty((0, N), dtype=out_dtype, device=x.device)
     ldx, ldw = _rows(x, "x"), _rows(w, "w")
@@ -268,15 +305,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, *, allow_library: b
             return torch.matmul(x, w.t())
         if out_dtype == torch.float32:
             return torch.mm(x, w.t(), out_dtype=torch.float32)
-    if M > 64 and out_dtype == torch.float32 and aligned and skinny_supported(64, N, K, ldx, ldw):
-        # float32 results from bf16 operands (logits at many positions): 64 rows at a time
-        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
-        f = _fn("skinny_gemm", "bn_skinny_gemm")
-        for m0 in range(0, M, 64):
-            m = min(64, M - m0)
-            _check(f(_code(out_dtype), x[m0:].data_ptr(), w.data_ptr(), y[m0:].data_ptr(), m, N, K, ldx, ldw,
-                     N, 0, 0, _stream()), "skinny_gemm")
-        return y
+    if aligned and gemm_mfma_supported(M, N, K, ldx, ldw):
+        return gemm_mfma(x, w, out_dtype)
     return _tiled(x, w, out_dtype)
 
 
@@ -291,10 +321,11 @@ def interleave_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor) -> torch.Tensor
 
 
 def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = False, *,
-                  allow_library: bool = True) -> torch.Tensor:
+                  allow_library: Optional[bool] = None) -> torch.Tensor:
     """silu(x.Wg^T) * (x.Wu^T) for w_gate_up = [Wg; Wu] ([2F, K]), or the two interleaved in
-    blocks of 8 rows (interleave_gate_up).  The decode-sized bf16 case is one kernel; every other
-    case is the product followed by the SwiGLU kernel."""
+    blocks of 8 rows (interleave_gate_up).  The decode-sized bf16 case is one kernel, and so is the
+    interleaved case without the library; every other case is the product followed by the SwiGLU
+    kernel."""
     require_gpu()
     _dev(x, "x", dims=2)
     _dev(w_gate_up, "w_gate_up", x.dtype, 2)
@@ -304,16 +335,22 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = 
     F = w_gate_up.shape[0] // 2
     if interleaved and F % 8:
         raise KernelError("linear_swiglu: the interleaved layout needs F to be a multiple of 8")
+    if allow_library is None:
+        allow_library = LIBRARY_PRODUCTS
     if M == 0:
         return torch.empty((0, F), dtype=x.dtype, device=x.device)
     ldx, ldw = _rows(x, "x"), _rows(w_gate_up, "w_gate_up")
+    aligned = x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0
     if (x.dtype == torch.bfloat16 and (M <= SKINNY_ROWS or (M <= 64 and not allow_library))
-            and x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0 and skinny_supported(M, F, K, ldx, ldw)):
+            and aligned and skinny_supported(M, F, K, ldx, ldw)):
         y = torch.empty((M, F), dtype=x.dtype, device=x.device)
         _check(_fn("skinny_gemm", "bn_skinny_gemm")(_code(x.dtype), x.data_ptr(), w_gate_up.data_ptr(),
                                                     y.data_ptr(), M, F, K, ldx, ldw, F, 2 if interleaved else 1, F,
                                                     _stream()), "skinny_gemm(glu)")
         return y
+    if (x.dtype == torch.bfloat16 and interleaved and not allow_library and aligned
+            and gemm_mfma_supported(M, 2 * F, K, ldx, ldw)):
+        return gemm_mfma(x, w_gate_up, x.dtype, glu8=True)
     return swiglu(linear(x, w_gate_up, allow_library=allow_library), interleaved)
 
 

@@ -54,6 +54,27 @@ def test_whole_requests_alone(model_folders, name, dtype):
     eng.cache.check()
 
 
+@pytest.mark.parametrize("name", NAMES)
+def test_whole_requests_without_the_library(model_folders, name, monkeypatch):
+    """bf16 with the library's matrix product switched off: prompts of more than 64 tokens then go
+    through this library's own matrix-core kernel (with the SwiGLU epilogue where the feed-forward
+    keeps gate and up interleaved); batches of 17 to 64 rows through the streaming kernel."""
+    from bitnet_c_amd import StepEntry, ops
+    folder = model_folders(name, torch.bfloat16)
+    monkeypatch.setattr(ops, "LIBRARY_PRODUCTS", False)
+    called = []
+    real = ops.gemm_mfma
+    monkeypatch.setattr(ops, "gemm_mfma", lambda *a, **k: (called.append(1), real(*a, **k))[1])
+    eng = make_engine(folder, torch.bfloat16)
+    for toks in _requests(eng.vocab_size, 11, [33, 65, 150, 300]):
+        s = eng.new_sequence()
+        got = eng.step([StepEntry(s, toks, list(range(len(toks))))])
+        eng.release(s)
+        assert rel_err(got, plain_logits(folder, toks, torch.bfloat16)) < TOL[torch.bfloat16], len(toks)
+    assert called
+    eng.cache.check()
+
+
 @pytest.mark.parametrize("graphs", [True, False])
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", NAMES)

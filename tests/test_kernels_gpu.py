@@ -138,6 +138,71 @@ def test_skinny_gemm_bf16(M, N, K):
         assert y16.dtype == torch.bfloat16 and close(y16.float(), ref.float(), torch.bfloat16)
 
 
+@pytest.mark.parametrize("width", [0, 256, 192, 128])
+@pytest.mark.parametrize("M,N,K", [(65, 16, 8), (100, 200, 328), (256, 256, 64), (300, 520, 192), (777, 1000, 136),
+                                   (513, 4104, 1032), (1, 31, 264)])
+def test_gemm_mfma(M, N, K, width):
+    """The tiled matrix-core product, every tile width, at sizes that fill no tile: float32 results are
+    the exact sums up to their order, bf16 results one rounding of them."""
+    ops = _ops()
+    from bitnet_c_amd.csrc import build
+    x, w = _rand((M, K), torch.bfloat16, 21), _rand((N, K), torch.bfloat16, 22, 0.05)
+    ref = (x.double() @ w.double().t()).float()
+    lib = build.load("gemm_mfma")
+    lib.bn_gemm_mfma_force_width(width)
+    try:
+        y32 = ops.gemm_mfma(x.cuda(), w.cuda(), torch.float32)
+        y16 = ops.gemm_mfma(x.cuda(), w.cuda())
+        # rows of a larger buffer (a row stride above K), as the stacked projections pass them
+        xw = torch.zeros(M, K + 24, dtype=torch.bfloat16)
+        xw[:, :K] = x
+        y_strided = ops.gemm_mfma(xw.cuda()[:, :K], w.cuda(), torch.float32)
+    finally:
+        lib.bn_gemm_mfma_force_width(0)
+    assert y32.dtype == torch.float32 and rel_err(y32, ref) < 1e-5
+    assert y16.dtype == torch.bfloat16 and close(y16.float(), ref, torch.bfloat16)
+    assert torch.equal(y_strided, y32)
+    # through the dispatcher: without the library, more than 64 rows take this kernel
+    if M > 64:
+        assert torch.equal(ops.linear(x.cuda(), w.cuda(), torch.float32, allow_library=False), y32)
+
+
+@pytest.mark.parametrize("width", [0, 256, 192, 128])
+@pytest.mark.parametrize("M,F,K", [(65, 8, 8), (100, 328, 120), (300, 1000, 512), (260, 2056, 264)])
+def test_gemm_mfma_swiglu(M, F, K, width):
+    """The same kernel with gate and up rows interleaved in blocks of 8 and the SwiGLU epilogue."""
+    ops = _ops()
+    from bitnet_c_amd.csrc import build
+    x, w = _rand((M, K), torch.bfloat16, 23), _rand((2 * F, K), torch.bfloat16, 24, 0.1)
+    g = x.double() @ w[:F].double().t()
+    u = x.double() @ w[F:].double().t()
+    want = ((g / (1 + torch.exp(-g))) * u).float()
+    wi = ops.interleave_gate_up(w[:F].cuda(), w[F:].cuda())
+    lib = build.load("gemm_mfma")
+    lib.bn_gemm_mfma_force_width(width)
+    try:
+        y32 = ops.gemm_mfma(x.cuda(), wi, torch.float32, glu8=True)
+        y16 = ops.gemm_mfma(x.cuda(), wi, glu8=True)
+        via = ops.linear_swiglu(x.cuda(), wi, True, allow_library=False)
+    finally:
+        lib.bn_gemm_mfma_force_width(0)
+    assert y32.shape == (M, F) and close(y32, want, torch.float32)
+    assert close(y16.float(), want, torch.bfloat16)
+    assert torch.equal(via, y16)
+
+
+def test_gemm_mfma_refuses_what_it_cannot_take():
+    ops = _ops()
+    x, w = _rand((70, 36), torch.bfloat16, 25).cuda(), _rand((16, 36), torch.bfloat16, 26).cuda()
+    with pytest.raises(ops.KernelError):
+        ops.gemm_mfma(x, w)                               # K is not a multiple of 8
+    with pytest.raises(ops.KernelError):
+        ops.gemm_mfma(x.float(), w.float())               # bf16 only
+    # the dispatcher sends such a shape to the plain tiled kernel instead
+    y = ops.linear(x, w, allow_library=False)
+    assert close(y.float(), (x.double().cpu() @ w.double().cpu().t()).float(), torch.bfloat16)
+
+
 @pytest.mark.parametrize("M,F,K", [(1, 24, 64), (8, 172, 64), (20, 100, 264), (64, 1000, 512), (40, 14336, 256), (33, 8, 8), (17, 328, 120)])
 def test_skinny_gemm_dual_swiglu(M, F, K):
     ops = _ops()
