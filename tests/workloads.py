@@ -4,6 +4,7 @@
     python3 tests/workloads.py skinny            # the decode products at 8 rows, cold weights
     python3 tests/workloads.py attention_prompt  # prompt attention over 2,048 and 8,192 tokens
     python3 tests/workloads.py attention_decode  # decode attention, batch 8 and 64, unequal lengths
+    python3 tests/workloads.py gemm              # the prompt products at 2,048 rows, this library's own kernel
 
 No test: nothing is checked here; the numerics of these kernels are in test_kernels_gpu.py.
 """
@@ -33,6 +34,18 @@ def skinny(rows=8, copies=3):
                 ops.linear(x, w, torch.float32 if name == "output" else None)
         torch.cuda.synchronize()
         del ws
+
+
+def gemm(rows=2048, reps=3):
+    shapes = [("qkv", 6144, 4096, False), ("o", 4096, 4096, False), ("gate_up", 14336, 4096, True),
+              ("down", 4096, 14336, False)]
+    for name, n, k, glu in shapes:
+        w = torch.randn((2 * n if glu else n), k, device=DEV, dtype=torch.bfloat16) * 0.02
+        x = torch.randn(rows, k, device=DEV, dtype=torch.bfloat16)
+        for _ in range(reps):
+            ops.gemm_mfma(x, w, None, glu)
+        torch.cuda.synchronize()
+        del w
 
 
 def _cache(lengths):
@@ -78,6 +91,6 @@ def attention_decode():
 
 if __name__ == "__main__":
     which = sys.argv[1] if len(sys.argv) > 1 else ""
-    if which not in ("skinny", "attention_prompt", "attention_decode"):
+    if which not in ("skinny", "attention_prompt", "attention_decode", "gemm"):
         sys.exit(__doc__)
-    {"skinny": skinny, "attention_prompt": attention_prompt, "attention_decode": attention_decode}[which]()
+    {"skinny": skinny, "attention_prompt": attention_prompt, "attention_decode": attention_decode, "gemm": gemm}[which]()
