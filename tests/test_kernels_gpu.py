@@ -494,6 +494,45 @@ def test_attention_finds_a_far_key(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,hs,window", [(4, 2, 32, 70), (8, 2, 128, 64), (6, 6, 64, 129)])
+def test_attention_at_the_window_s_edge(dtype, H, Hkv, hs, window):
+    """A key with a large score just inside the window is the whole answer, and the same key one
+    position further back (just outside) must not be seen at all: the decode form for the last
+    position, the prompt form for a chunk of rows whose windows begin at different keys."""
+    ops = _ops()
+    L, n_new = 300, 40
+    scale = 1 / math.sqrt(hs)
+    for back in (window - 1, window):                       # the last key inside, the first one outside
+        k = _rand((L, Hkv, hs), dtype, 310, 0.1)
+        v = _rand((L, Hkv, hs), dtype, 311)
+        q = _rand((L, H, hs), dtype, 312, 0.1)
+        t = L - 1
+        far = t - back
+        k[far] = 0
+        k[far, :, 0] = 16.0
+        q[:, :, 0] = 16.0
+        kp, vp, bt = _paged([k], [v], dtype, 8, far)
+        ref = pl.attention(q.float(), k.float(), v.float(), scale, window).reshape(L, H * hs)
+        if back == window - 1:                              # inside: the answer is that key's value row
+            assert rel_err(ref[t:t + 1], v[far].float().repeat_interleave(H // Hkv, dim=0).reshape(1, H * hs)) < 1e-3
+        else:                                               # outside: the plain answer without it is something else
+            assert rel_err(ref[t:t + 1], v[far].float().repeat_interleave(H // Hkv, dim=0).reshape(1, H * hs)) > 0.5
+        check = (lambda o, r: mfma_close(o, r)) if ops.mfma_attention(dtype, hs) else (lambda o, r: close(o, r, dtype))
+        # decode form: the row at position t
+        out = torch.empty((1, H * hs), dtype=dtype).cuda()
+        ops.attention(q[t:t + 1].reshape(1, H * hs).contiguous().cuda(), out, kp.cuda(), vp.cuda(), bt.cuda(), H, Hkv, hs,
+                      scale, window=window, seq_lens=torch.tensor([L], dtype=torch.int32).cuda())
+        assert check(out.float(), ref[t:t + 1]), ("decode", back)
+        # prompt form: the last n_new rows; the key leaves the window of each row at a different place
+        _, _, qt = ops.attention_row_shape(H, Hkv, False, dtype, hs)
+        tiles = torch.tensor([(0, i, min(qt, n_new - i), L - n_new + i) for i in range(0, n_new, qt)], dtype=torch.int32).cuda()
+        outp = torch.empty((n_new, H * hs), dtype=dtype).cuda()
+        ops.attention(q[L - n_new:].reshape(n_new, H * hs).contiguous().cuda(), outp, kp.cuda(), vp.cuda(), bt.cuda(), H, Hkv,
+                      hs, scale, window=window, tiles=tiles, qt=qt)
+        assert check(outp.float(), ref[L - n_new:]), ("prompt", back)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,Hkv,hs", [(8, 2, 128), (6, 3, 48)])
 def test_attention_over_a_long_context(dtype, H, Hkv, hs):
     """20,000 cached positions: a decode row with the split plan the engine would pick, and a
