@@ -134,6 +134,182 @@ __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_ke
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// The same product for up to 16 rows with the neighbouring norm folded in, so that a decode layer
+// needs no kernel for its two norms:
+//   RES: the product is a part's output.  The epilogue adds it to the float32 residual stream in
+//        place (its 16 columns), writes a bf16 copy of the new stream multiplied by the next norm's
+//        weights, and the sum of the squares of its 16 columns of every row into a slot of its own.
+//   PRE: the activations are such a copy.  1/sqrt(mean(x^2) + eps) (src/transformer/rmsnorm_scalar.c:4-13)
+//        multiplies a whole row of the result, so it is applied in the epilogue: every wave fetches the
+//        slots of two rows before its K loop and adds them up behind it (lane-strided sums, a tree over
+//        the lanes: a fixed order); the staged activations need no work at all.
+// GLU8 as above.  bf16 result (RES: no result of its own).
+#define SK_SLOT_LOADS 8       // slots per row and lane: at most 512 column tiles (a stream of 8,192 columns)
+
+struct SkinnyFused {
+    const float* slots_in;    // [M, n_slots] sums of squares, PRE
+    int n_slots;
+    float inv_width, eps;     // 1 / columns of the stream, the norm's eps, PRE
+    float* resid;             // [M, ld_resid] float32 stream, RES
+    bf16* resid_bf16;         // [M, ld_rb] its bf16 copy times next_weight, RES
+    const float* next_weight; // [N] weights of the norm that reads the copy, RES
+    float* slots_out;         // [M, gridDim.x], RES
+    int ld_resid, ld_rb;
+};
+
+template <bool GLU8, bool PRE, bool RES, int SL>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, bf16* __restrict__ Y, int M, int N,
+                              int K, int ldx, int ldw, int ldy, SkinnyFused f) {
+    constexpr int NW = 8;                              // always eight waves: wave w owns rows w and w + 8 of the norm
+    extern __shared__ __align__(16) float red[];       // [NW][64][4], then 16 row scales, then the staging
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int n = min(n0 + i, N - 1);
+    const bf16* wrow = W + (size_t)n * ldw;
+    float* scale_s = red + NW * 256;
+    unsigned char* xs = reinterpret_cast<unsigned char*>(red + NW * 256 + 16) + (size_t)wave * M * SK_XROW;
+
+    f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+    auto step = [&](int kc) {
+        const int kb = kc + g * 8;
+        const int xk = kc + (lane & 31) * 8;
+        uint4 wv[8], xd[8], xv[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const int row = 2 * r + (lane >> 5);
+            if (2 * r < M)
+                xd[r] = (row < M && xk < K) ? *reinterpret_cast<const uint4*>(X + (size_t)row * ldx + xk) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int k = kb + j * 32;
+            wv[j] = (k < K) ? *reinterpret_cast<const uint4*>(wrow + k) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const int row = 2 * r + (lane >> 5);
+            if (2 * r < M && row < M) *reinterpret_cast<uint4*>(xs + row * SK_XROW + (lane & 31) * 16) = xd[r];
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            xv[j] = (i < M) ? *reinterpret_cast<const uint4*>(xs + i * SK_XROW + j * 64 + g * 16) : make_uint4(0, 0, 0, 0);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xv[j]), as_bf16x8(wv[j]), acc, 0, 0, 0);
+    };
+    // all chunks of this wave but its last; the slots of the norm are asked for before the last one, so that they
+    // arrive while it waits for its weights and occupy registers only there
+    int kc = wave * SK_CHUNK;
+    for (; kc + NW * SK_CHUNK < K; kc += NW * SK_CHUNK) step(kc);
+    float sv[2][SL];                                   // PRE: this lane's slots of rows wave and wave + 8
+    if (PRE) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int m = wave + NW * h;
+#pragma unroll
+            for (int j = 0; j < SL; ++j) {
+                const int t = lane + 64 * j;
+                sv[h][j] = (m < M && t < f.n_slots) ? f.slots_in[(size_t)m * f.n_slots + t] : 0.f;
+            }
+        }
+    }
+    if (kc < K) step(kc);
+    if (PRE) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            float v = 0.f;
+#pragma unroll
+            for (int j = 0; j < SL; ++j) v += sv[h][j];
+            v = wave_sum(v);
+            if (lane == 0 && wave + NW * h < 16) scale_s[wave + NW * h] = 1.0f / sqrtf(v * f.inv_width + f.eps);
+        }
+    }
+    *reinterpret_cast<f32x4*>(red + ((size_t)wave * 64 + lane) * 4) = acc;
+    __syncthreads();
+    // waves 0..3: thread (l, r = wave): C row 4*(l/16)+r, column l%16; sums over waves in wave order
+    if (wave < 4) {
+        const int l = lane, r = wave;
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) v += red[((size_t)w * 64 + l) * 4 + r];
+        const int m = 4 * (l >> 4) + r;
+        const int nn = n0 + (l & 15);
+        if (PRE) v *= scale_s[m];
+        if (GLU8) {
+            const float up = __shfl_xor(v, 8, BN_WAVE);
+            if ((l & 8) == 0 && m < M && nn < N)
+                Y[(size_t)m * ldy + (n0 >> 1) + (l & 7)] = __float2bfloat16((v / (1.0f + expf(-v))) * up);
+        } else if (RES) {
+            float xn = 0.f;
+            if (m < M && nn < N) {
+                xn = f.resid[(size_t)m * f.ld_resid + nn] + v;
+                f.resid[(size_t)m * f.ld_resid + nn] = xn;
+                f.resid_bf16[(size_t)m * f.ld_rb + nn] = __float2bfloat16(xn * f.next_weight[nn]);
+            }
+            float sq = xn * xn;                                   // the 16 columns of row m: lanes 16 (l / 16) + 0..15
+#pragma unroll
+            for (int o = 1; o < 16; o <<= 1) sq += __shfl_xor(sq, o, BN_WAVE);
+            if ((l & 15) == 0 && m < M) f.slots_out[(size_t)m * gridDim.x + blockIdx.x] = sq;
+        } else if (m < M && nn < N) {
+            Y[(size_t)m * ldy + nn] = __float2bfloat16(v);
+        }
+    }
+}
+
+extern "C" int bn_skinny_gemm_supports(int M, int N, int K, int ldx, int ldw);
+
+// X, W, Y as bn_skinny_gemm with a bf16 result and M <= 16; glu8 as dual == 2 there.
+// slots_in != null (PRE): X is a stream's bf16 copy as a RES call leaves it, slots_in [M, n_slots] its rows'
+// sums of squares in parts, stream_width its number of columns; the result's rows are scaled by
+// 1/sqrt(sum / stream_width + eps).
+// resid != null (RES): the product is added to resid [M, N] in place; resid_bf16 [M, N] becomes the new stream
+// times next_weight [N], slots_out [M, (N + 15) / 16] the sums of squares of its groups of 16 columns (glu8 == 0, no Y).
+extern "C" int bn_skinny_gemm_fused(const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw, int ldy,
+                                    int glu8, const float* slots_in, int n_slots, int stream_width, float eps,
+                                    float* resid, int ld_resid, void* resid_bf16, int ld_rb, const float* next_weight,
+                                    float* slots_out, hipStream_t s) {
+    if (!bn_skinny_gemm_supports(M, N, K, ldx, ldw) || M > 16) return BN_ERR_ARG;
+    if (((uintptr_t)X | (uintptr_t)W) & 15) return BN_ERR_ARG;
+    const bool pre = slots_in != nullptr, res = resid != nullptr;
+    if (!pre && !res) return BN_ERR_ARG;
+    if (pre && (n_slots < 1 || n_slots > 64 * SK_SLOT_LOADS || stream_width < 1)) return BN_ERR_ARG;
+    if (res && (glu8 || !resid_bf16 || !next_weight || !slots_out || ld_resid < N || ld_rb < N)) return BN_ERR_ARG;
+    if (!res && (!Y || ldy < N)) return BN_ERR_ARG;
+    if (glu8) {
+        if (N % 8) return BN_ERR_ARG;
+        N *= 2;
+    }
+    SkinnyFused f;
+    f.slots_in = slots_in; f.n_slots = n_slots; f.inv_width = pre ? 1.0f / (float)stream_width : 0.f; f.eps = eps;
+    f.resid = resid; f.resid_bf16 = (bf16*)resid_bf16; f.next_weight = next_weight; f.slots_out = slots_out;
+    f.ld_resid = ld_resid; f.ld_rb = ld_rb;
+    const size_t smem = (size_t)(8 * 256 + 16) * sizeof(float) + (size_t)8 * M * SK_XROW;
+    const dim3 grid((N + 15) / 16), block(8 * 64);
+    auto go = [&](auto kernel) {
+        if (smem > 64 * 1024) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return (int)e;
+        }
+        hipLaunchKernelGGL(kernel, grid, block, smem, s, (const bf16*)X, (const bf16*)W, (bf16*)Y, M, N, K, ldx, ldw, ldy, f);
+        return bn_launch_status();
+    };
+    const bool few = n_slots <= 256;                  // four slot loads per row and lane are enough
+    if (glu8) {
+        if (!pre) return BN_ERR_ARG;
+        return few ? go(skinny_gemm_fused_kernel<true, true, false, 4>) : go(skinny_gemm_fused_kernel<true, true, false, 8>);
+    }
+    if (pre && res)
+        return few ? go(skinny_gemm_fused_kernel<false, true, true, 4>) : go(skinny_gemm_fused_kernel<false, true, true, 8>);
+    if (pre) return few ? go(skinny_gemm_fused_kernel<false, true, false, 4>) : go(skinny_gemm_fused_kernel<false, true, false, 8>);
+    return go(skinny_gemm_fused_kernel<false, false, true, 4>);
+}
+
 template <int MT, bool DUAL, typename TO, bool GLU8 = false>
 static int launch(const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw, int ldy,
                   int up_off, int n_waves, hipStream_t s) {

@@ -11,6 +11,8 @@ from __future__ import annotations
 import ctypes
 import os
 from ctypes import c_float, c_int, c_longlong, c_void_p
+from dataclasses import dataclass
+from typing import Optional
 
 import torch
 
@@ -63,6 +65,9 @@ _SIGNATURES = {
         "bn_skinny_gemm_supports": [c_int, c_int, c_int, c_int, c_int],
         "bn_skinny_gemm": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                            c_int, c_void_p],
+        "bn_skinny_gemm_fused": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                 c_void_p, c_int, c_int, c_float, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
+                                 c_void_p],
     },
     "sampling": {
         "bn_argmax": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
@@ -352,6 +357,127 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = 
             and gemm_mfma_supported(M, 2 * F, K, ldx, ldw)):
         return gemm_mfma(x, w_gate_up, x.dtype, glu8=True)
     return swiglu(linear(x, w_gate_up, allow_library=allow_library), interleaved)
+
+
+# --------------------------------------------------------------------------------------
+# decode products with the neighbouring RMSNorm folded in
+# --------------------------------------------------------------------------------------
+# Set False (or BITNET_NO_FUSED_NORM=1) to keep every norm a kernel of its own.
+FUSE_NORMS = os.environ.get("BITNET_NO_FUSED_NORM", "") in ("", "0")
+FUSED_ROWS = 16           # rows the fused products take (one MFMA tile of activations)
+FUSED_SLOTS = 512         # column tiles of 16 whose sums of squares a consumer adds up: streams up to 8,192 wide
+
+
+@dataclass
+class DeferredNorm:
+    """An RMSNorm that has not been applied yet.  `scaled` is the bf16 copy of the stream already
+    multiplied by the norm's weights, `slots` [M, n] the sums of squares of the stream's rows in
+    parts; a product that consumes it (linear_prenorm, linear_swiglu_prenorm) multiplies its
+    result's rows by 1/sqrt(mean + eps).  `stream`, `weight`, `eps` are what the plain kernel needs
+    when the consumer cannot take it (materialize)."""
+    scaled: torch.Tensor
+    slots: torch.Tensor
+    stream: torch.Tensor
+    weight: torch.Tensor
+    eps: float
+
+    @property
+    def shape(self):
+        return self.scaled.shape
+
+    @property
+    def dtype(self):
+        return self.scaled.dtype
+
+    @property
+    def device(self):
+        return self.scaled.device
+
+    def materialize(self, out_dtype=None, rows=None) -> torch.Tensor:
+        return add_rmsnorm(self.stream, None, self.weight, self.eps, out_dtype or self.scaled.dtype, rows)
+
+
+def can_fuse_norm(M: int, N: int, K: int, dtype) -> bool:
+    """Whether a product of these sizes can take a norm into its kernel (either side of it)."""
+    return (dtype == torch.bfloat16 and 1 <= M <= FUSED_ROWS and K % 8 == 0 and N >= 1
+            and torch.cuda.is_available() and skinny_supported(M, N, K, K, K))
+
+
+def _fused_call(x, w, y, M, N, K, glu8, pre: Optional[DeferredNorm], resid, resid_bf16, next_weight, slots_out):
+    _check(_fn("skinny_gemm", "bn_skinny_gemm_fused")(
+        x.data_ptr(), w.data_ptr(), y.data_ptr() if y is not None else None, M, N, K, _rows(x, "x"), _rows(w, "w"),
+        N if y is not None else 0, int(glu8),
+        pre.slots.data_ptr() if pre is not None else None, pre.slots.shape[1] if pre is not None else 0,
+        pre.stream.shape[1] if pre is not None else 0, float(pre.eps) if pre is not None else 0.0,
+        resid.data_ptr() if resid is not None else None, _rows(resid, "resid") if resid is not None else 0,
+        resid_bf16.data_ptr() if resid_bf16 is not None else None, N if resid_bf16 is not None else 0,
+        next_weight.data_ptr() if next_weight is not None else None,
+        slots_out.data_ptr() if slots_out is not None else None, _stream()), "skinny_gemm(fused)")
+
+
+def _check_deferred(pre: DeferredNorm, K: int) -> int:
+    _dev(pre.scaled, "deferred norm: scaled", torch.bfloat16, 2)
+    _dev(pre.slots, "deferred norm: slots", torch.float32, 2)
+    M = pre.scaled.shape[0]
+    if (pre.scaled.shape[1] != K or pre.stream.shape[1] != K or pre.slots.shape[0] != M
+            or not pre.slots.is_contiguous() or pre.slots.shape[1] > FUSED_SLOTS or pre.scaled.data_ptr() % 16):
+        raise KernelError(f"deferred norm: copy {tuple(pre.scaled.shape)}, slots {tuple(pre.slots.shape)} do not fit "
+                          f"an input width of {K}")
+    return M
+
+
+def linear_prenorm(pre: DeferredNorm, w: torch.Tensor) -> torch.Tensor:
+    """linear(rmsnorm(stream), w) for a deferred norm, in one kernel (bf16, up to 16 rows)."""
+    require_gpu()
+    _dev(w, "w", torch.bfloat16, 2)
+    N, K = w.shape
+    M = _check_deferred(pre, K)
+    if not can_fuse_norm(M, N, K, torch.bfloat16) or w.data_ptr() % 16:
+        raise KernelError(f"linear_prenorm: {M} rows, w {tuple(w.shape)} cannot be fused")
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+    _fused_call(pre.scaled, w, y, M, N, K, False, pre, None, None, None, None)
+    return y
+
+
+def linear_swiglu_prenorm(pre: DeferredNorm, w_gate_up: torch.Tensor) -> torch.Tensor:
+    """linear_swiglu(rmsnorm(stream), w) for gate and up interleaved in blocks of 8, in one kernel."""
+    require_gpu()
+    _dev(w_gate_up, "w_gate_up", torch.bfloat16, 2)
+    F, K = w_gate_up.shape[0] // 2, w_gate_up.shape[1]
+    M = _check_deferred(pre, K)
+    if w_gate_up.shape[0] % 16 or not can_fuse_norm(M, F, K, torch.bfloat16) or w_gate_up.data_ptr() % 16:
+        raise KernelError(f"linear_swiglu_prenorm: {M} rows, w {tuple(w_gate_up.shape)} cannot be fused")
+    y = torch.empty((M, F), dtype=torch.bfloat16, device=w_gate_up.device)
+    _fused_call(pre.scaled, w_gate_up, y, M, F, K, True, pre, None, None, None, None)
+    return y
+
+
+def can_defer_norm(M: int, N: int, K: int, dtype) -> bool:
+    """Whether linear_into_stream takes a product of these sizes (N is the stream's width)."""
+    return FUSE_NORMS and can_fuse_norm(M, N, K, dtype) and (N + 15) // 16 <= FUSED_SLOTS
+
+
+def linear_into_stream(x: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, weight: torch.Tensor,
+                       eps: float) -> DeferredNorm:
+    """stream += linear(x, w) (float32 stream [M, N], in place), and what the next norm (weights
+    `weight`, `eps`) needs: the bf16 copy of the new stream times the weights and the rows' sums of
+    squares in parts.  Returns that norm, deferred."""
+    require_gpu()
+    _dev(x, "x", torch.bfloat16, 2)
+    _dev(w, "w", torch.bfloat16, 2)
+    _dev(stream, "stream", torch.float32, 2)
+    _dev(weight, "weight", torch.float32, 1)
+    M, K = x.shape
+    N = w.shape[0]
+    if w.shape[1] != K or tuple(stream.shape) != (M, N) or weight.numel() != N or not weight.is_contiguous():
+        raise KernelError(f"linear_into_stream: x {tuple(x.shape)}, w {tuple(w.shape)}, stream {tuple(stream.shape)}, "
+                          f"weight {tuple(weight.shape)} do not agree")
+    if not can_defer_norm(M, N, K, torch.bfloat16) or x.data_ptr() % 16 or w.data_ptr() % 16:
+        raise KernelError(f"linear_into_stream: {M} rows, w {tuple(w.shape)} cannot be fused")
+    scaled = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    slots = torch.empty((M, (N + 15) // 16), dtype=torch.float32, device=x.device)
+    _fused_call(x, w, None, M, N, K, False, None, stream, scaled, weight, slots)
+    return DeferredNorm(scaled, slots, stream, weight, float(eps))
 
 
 # --------------------------------------------------------------------------------------

@@ -22,6 +22,9 @@ from .linear import Linear
 
 @MIXERS.register("attention")
 class Attention(Part):
+    takes_deferred_norm = True      # forward accepts an ops.DeferredNorm for h
+    gives_lazy_delta = True         # forward(..., lazy_ok=True) may return a LazyDelta
+
     def __init__(self, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
                  position: PartSpec, window: int = 0, bias: bool = False):
         if n_heads % n_kv_heads:
@@ -62,8 +65,9 @@ class Attention(Part):
     def cache_need(self) -> CacheNeed:
         return CacheNeed(kv=KVNeed(self.Hkv, self.hs, self.window))
 
-    def forward(self, h, ctx, kv):
+    def forward(self, h, ctx, kv, lazy_ok: bool = False):
         H, Hkv, hs = self.H, self.Hkv, self.hs
+        last = self.o.lazy if lazy_ok else self.o
         if kv.writes:
             qkv = self.qkv(h)                                   # [T, (H + 2 Hkv) hs]
         else:
@@ -82,7 +86,7 @@ class Attention(Part):
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
                           window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
                           fused_rotate=inv_freq, fused_write=kv.writes, by_length=ctx.by_length)
-            return self.o(out)
+            return last(out)
         self.position.encode_and_store(qkv, ctx, H, Hkv, hs, kv)
         if ctx.is_decode:
             if self.window:                   # a window is short; its keys are not split
@@ -96,4 +100,4 @@ class Attention(Part):
             _, _, qt = ops.attention_row_shape(H, Hkv, False, h.dtype, hs)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
                           window=self.window, tiles=ctx.tiles(qt), qt=qt)
-        return self.o(out)
+        return last(out)

@@ -133,29 +133,57 @@ class KVView:
     max_len: int = 0                            # bound of the key count in this step (sizes the splits)
 
 
+class LazyDelta:
+    """A part's output that is still a product to be done: activations and the Linear that ends the
+    part.  The stream either lets the product add itself to the stream and leave the next norm
+    deferred (one kernel, ops.linear_into_stream), or computes it the plain way."""
+
+    def __init__(self, act: torch.Tensor, linear):
+        self.act, self.linear = act, linear
+
+    def compute(self) -> torch.Tensor:
+        return self.linear(self.act)
+
+
 class ResidualStream:
     """The float32 residual stream of a step.  A part's output is held back as `pending` and
     is added by the kernel of the next norm, so the sum is formed once, in float32, without a
-    pass of its own."""
+    pass of its own.  At decode sizes a part may hand in its last product undone (LazyDelta) and a
+    consumer may take the norm undone (ops.DeferredNorm): the product then adds itself to the stream
+    and the consumer's first product applies the norm, and neither the sum nor the norm is a kernel."""
 
     def __init__(self, x: torch.Tensor):
         self.x = x
-        self.pending: Optional[torch.Tensor] = None
+        self.pending = None                      # a tensor, a LazyDelta or None
 
-    def add(self, delta: torch.Tensor) -> None:
+    def add(self, delta) -> None:
         if self.pending is not None:
             self.flush()
         self.pending = delta
 
+    def _pending_tensor(self):
+        if isinstance(self.pending, LazyDelta):
+            self.pending = self.pending.compute()
+        return self.pending
+
     def flush(self) -> torch.Tensor:
         if self.pending is not None:
             from .. import ops
-            ops.residual_add(self.x, self.pending)
+            ops.residual_add(self.x, self._pending_tensor())
             self.pending = None
         return self.x
 
-    def normed(self, norm, out_dtype, rows=None) -> torch.Tensor:
-        h = norm.apply(self.x, self.pending, out_dtype, rows)
+    def normed(self, norm, out_dtype, rows=None, consumer=None):
+        """The normed stream for the next part.  `consumer`: the part that will read it; when it
+        declares `takes_deferred_norm` and the pending output is a LazyDelta that the norm can be
+        folded around, the result is an ops.DeferredNorm instead of a tensor."""
+        if (rows is None and isinstance(self.pending, LazyDelta) and getattr(consumer, "takes_deferred_norm", False)
+                and getattr(norm, "deferrable", False)):
+            deferred = self.pending.linear.into_stream(self.pending.act, self.x, norm.weight, norm.eps)
+            if deferred is not None:
+                self.pending = None
+                return deferred
+        h = norm.apply(self.x, self._pending_tensor(), out_dtype, rows)
         if rows is None:
             self.pending = None
         return h

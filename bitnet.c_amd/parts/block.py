@@ -29,7 +29,15 @@ class PreNormBlock(Part):
         return self.mixer.cache_need()
 
     def forward(self, stream, ctx, kv):
-        h = stream.normed(self.mixer_norm, ctx.act_dtype)
-        stream.add(self.mixer.forward(h, ctx, kv))
-        h = stream.normed(self.ffn_norm, ctx.act_dtype)
-        stream.add(self.ffn.forward(h, ctx))
+        # A part that says so may get its norm undone (it applies it inside its first product) and may hand
+        # its last product in undone (it then adds itself to the stream): see ResidualStream.
+        h = stream.normed(self.mixer_norm, ctx.act_dtype, consumer=self.mixer)
+        if getattr(self.mixer, "gives_lazy_delta", False):
+            stream.add(self.mixer.forward(h, ctx, kv, lazy_ok=True))
+        else:
+            stream.add(self.mixer.forward(h, ctx, kv))
+        h = stream.normed(self.ffn_norm, ctx.act_dtype, consumer=self.ffn)
+        if getattr(self.ffn, "gives_lazy_delta", False):
+            stream.add(self.ffn.forward(h, ctx, lazy_ok=True))
+        else:
+            stream.add(self.ffn.forward(h, ctx))

@@ -15,6 +15,9 @@ from .linear import Linear
 
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(Part):
+    takes_deferred_norm = True      # forward accepts an ops.DeferredNorm for h
+    gives_lazy_delta = True         # forward(..., lazy_ok=True) may return a LazyDelta
+
     def __init__(self, hidden: int, intermediate: int, bias: bool = False):
         self.hidden, self.F, self.has_bias = int(hidden), int(intermediate), bool(bias)
         self.gate_up, self.down = Linear(), Linear()
@@ -41,9 +44,16 @@ class SwiGLU(Part):
         self.gate_up.load(w, b, device, dtype)
         self.down.load(tensors["w_down"], tensors.get("b_down") if self.has_bias else None, device, dtype)
 
-    def forward(self, h, ctx):
+    def forward(self, h, ctx, lazy_ok: bool = False):
+        if isinstance(h, ops.DeferredNorm):
+            w = self.gate_up.weight
+            if (not self.has_bias and self.interleaved and w.dtype == torch.bfloat16
+                    and ops.can_fuse_norm(h.shape[0], self.F, self.hidden, w.dtype)):
+                act = ops.linear_swiglu_prenorm(h, w)
+                return self.down.lazy(act) if lazy_ok else self.down(act)
+            h = h.materialize()
         if self.has_bias:
             act = ops.swiglu(self.gate_up(h), self.interleaved)
         else:
             act = ops.linear_swiglu(h, self.gate_up.weight, self.interleaved)
-        return self.down(act)
+        return self.down.lazy(act) if lazy_ok else self.down(act)

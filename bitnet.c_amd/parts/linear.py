@@ -16,9 +16,32 @@ class Linear:
         self.weight = weight.to(dtype).to(device).contiguous()
         self.bias = bias.to(torch.float32).to(device).contiguous() if bias is not None else None
 
-    def __call__(self, x: torch.Tensor, out_dtype=None, rows: slice | None = None) -> torch.Tensor:
+    def __call__(self, x, out_dtype=None, rows: slice | None = None) -> torch.Tensor:
+        """x: activations, or an ops.DeferredNorm whose norm this product applies itself when it can."""
         w = self.weight if rows is None else self.weight[rows]
+        if isinstance(x, ops.DeferredNorm):
+            M, (N, K) = x.shape[0], w.shape
+            if (self.bias is None and out_dtype in (None, torch.bfloat16) and w.dtype == torch.bfloat16
+                    and ops.can_fuse_norm(M, N, K, w.dtype) and w.data_ptr() % 16 == 0):
+                return ops.linear_prenorm(x, w)
+            x = x.materialize()
         y = ops.linear(x, w, out_dtype)
         if self.bias is not None:
             ops.bias_add(y, self.bias if rows is None else self.bias[rows].contiguous())
         return y
+
+    def lazy(self, x: torch.Tensor):
+        """The product as a LazyDelta when it could add itself to a residual stream (decode sizes, bf16, no
+        bias), else its result."""
+        from .base import LazyDelta
+        M, (N, K) = x.shape[0], self.weight.shape
+        if (self.bias is None and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16
+                and ops.can_defer_norm(M, N, K, x.dtype) and x.data_ptr() % 16 == 0):
+            return LazyDelta(x, self)
+        return self(x)
+
+    def into_stream(self, x: torch.Tensor, stream: torch.Tensor, norm_weight: torch.Tensor, eps: float):
+        """stream += self(x) in one kernel that leaves the next norm deferred; None if the stream does not fit."""
+        if tuple(stream.shape) != (x.shape[0], self.weight.shape[0]) or not stream.is_contiguous():
+            return None
+        return ops.linear_into_stream(x, self.weight, stream, norm_weight, eps)

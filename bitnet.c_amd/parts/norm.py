@@ -11,6 +11,8 @@ from .base import NORMS, ParamSpec, Part
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Part):
+    deferrable = True        # a product may fold this norm around itself (weight and eps are all it needs)
+
     def __init__(self, dim: int, eps: float):
         self.dim, self.eps = int(dim), float(eps)
         self.weight = None

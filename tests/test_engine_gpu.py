@@ -54,6 +54,60 @@ def test_whole_requests_alone(model_folders, name, dtype):
     eng.cache.check()
 
 
+@pytest.mark.parametrize("graphs", [True, False])
+@pytest.mark.parametrize("name", ["A", "B", "E"])
+def test_decode_steps_fold_their_norms_into_the_products(model_folders, name, graphs, monkeypatch):
+    """bf16 decode steps of up to 16 rows: a part's last product adds itself to the stream and the next
+    part's first product applies the norm, so that no norm kernel runs between them.  The logits agree
+    with the plain implementation, and with the same steps run with every norm as a kernel of its own,
+    within rounding."""
+    from bitnet_c_amd import StepEntry, ops
+    folder = model_folders(name, torch.bfloat16)
+    reqs = _requests(pl.read_config(folder)["vocab"], 21, [70, 19, 33])
+    n_dec = 12
+
+    def run(fuse):
+        monkeypatch.setattr(ops, "FUSE_NORMS", fuse)
+        calls = {"into": 0, "pre": 0, "norm": 0}
+        real = {n: getattr(ops, n) for n in ("linear_into_stream", "linear_prenorm", "linear_swiglu_prenorm", "add_rmsnorm")}
+        monkeypatch.setattr(ops, "linear_into_stream", lambda *a, **k: (calls.__setitem__("into", calls["into"] + 1), real["linear_into_stream"](*a, **k))[1])
+        monkeypatch.setattr(ops, "linear_prenorm", lambda *a, **k: (calls.__setitem__("pre", calls["pre"] + 1), real["linear_prenorm"](*a, **k))[1])
+        monkeypatch.setattr(ops, "linear_swiglu_prenorm", lambda *a, **k: (calls.__setitem__("pre", calls["pre"] + 1), real["linear_swiglu_prenorm"](*a, **k))[1])
+        monkeypatch.setattr(ops, "add_rmsnorm", lambda *a, **k: (calls.__setitem__("norm", calls["norm"] + 1), real["add_rmsnorm"](*a, **k))[1])
+        eng = make_engine(folder, torch.bfloat16, use_graphs=graphs)
+        slots = [eng.new_sequence() for _ in reqs]
+        eng.step([StepEntry(s, r[:-n_dec], []) for s, r in zip(slots, reqs)])
+        before = dict(calls)
+        outs = []
+        for t in range(n_dec):
+            outs.append(eng.step([StepEntry(s, [r[len(r) - n_dec + t]], [0]) for s, r in zip(slots, reqs)]).clone())
+        for s in slots:
+            eng.release(s)
+        for n in real:
+            monkeypatch.setattr(ops, n, real[n])
+        return torch.stack(outs, dim=1), {k: calls[k] - before[k] for k in calls}    # [request, step, vocab]
+
+    fused, n_fused = run(True)
+    plain_k, n_plain = run(False)
+    cfg = pl.read_config(folder)
+    L = cfg["layers"]
+    assert n_plain["into"] == 0 and n_plain["pre"] == 0 and n_fused["into"] > 0
+    # Counted on the eager run (a graph's first run launches every kernel again for its warm-up and capture) and
+    # where the feed-forward's width is a multiple of 8 (configuration A's is not: its feed-forward asks for the
+    # plain norm and computes its last product the plain way, only the attention's output product folds).
+    assert n_fused["pre"] > 0 or cfg["ffn"] % 8
+    if not graphs and cfg["ffn"] % 8 == 0:
+        assert n_fused["into"] == 2 * L * n_dec - n_dec          # every product that ends a part but the last layer's
+        assert n_fused["pre"] == 2 * L * n_dec - n_dec           # every product that begins a part but the first layer's
+        assert n_fused["norm"] == 2 * n_dec                      # the first layer's norm and the final norm
+        assert n_plain["norm"] == (2 * L + 1) * n_dec
+    for i, r in enumerate(reqs):
+        want = plain_logits(folder, r, torch.bfloat16)[len(r) - n_dec:]
+        assert rel_err(fused[i], want) < TOL[torch.bfloat16]
+        assert rel_err(plain_k[i], want) < TOL[torch.bfloat16]
+        assert rel_err(fused[i], plain_k[i]) < TOL[torch.bfloat16]
+
+
 @pytest.mark.parametrize("name", NAMES)
 def test_whole_requests_without_the_library(model_folders, name, monkeypatch):
     """bf16 with the library's matrix product switched off: prompts of more than 64 tokens then go

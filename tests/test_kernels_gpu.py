@@ -138,6 +138,65 @@ def test_skinny_gemm_bf16(M, N, K):
         assert y16.dtype == torch.bfloat16 and close(y16.float(), ref.float(), torch.bfloat16)
 
 
+@pytest.mark.parametrize("M", [1, 2, 5, 8, 9, 16])
+@pytest.mark.parametrize("D,F", [(64, 40), (4096, 1024), (200, 328), (136, 16), (8192, 64)])
+def test_products_with_the_norm_folded_in(M, D, F):
+    """A part's last product adds itself to the stream and leaves the next norm deferred (the stream's
+    bf16 copy times the norm's weights, sums of squares in parts); the next part's first product, plain
+    or with the SwiGLU epilogue, applies it.  Against the plain formulas: the stream exactly (float32),
+    the products within the rounding of their bf16 inputs and output."""
+    ops = _ops()
+    eps = 1e-5
+    stream = _rand((M, D), torch.float32, 31, 2.0)
+    act = _rand((M, F), torch.bfloat16, 32)
+    w_out = _rand((D, F), torch.bfloat16, 33, 0.1)                   # the part's last product: F -> D
+    norm_w = (_rand((D,), torch.float32, 34) * 0.2 + 1.0)
+    w_in = _rand((2 * F, D), torch.bfloat16, 35, 0.05)               # the next part's first product: D -> F (gate, up)
+    assert ops.can_defer_norm(M, D, F, torch.bfloat16)
+    x = stream.clone().cuda()
+    pre = ops.linear_into_stream(act.cuda(), w_out.cuda(), x, norm_w.cuda(), eps)
+    want_x = stream.double() + act.double() @ w_out.double().t()
+    assert rel_err(x, want_x.float()) < 1e-5                         # the stream itself: float32
+    assert pre.scaled.dtype == torch.bfloat16 and close(pre.scaled.float(), (want_x * norm_w.double()).float(), torch.bfloat16)
+    assert rel_err(pre.slots.sum(dim=1), want_x.pow(2).sum(dim=1).float()) < 1e-5
+    # the plain path from the same stream: norm kernel, then the product
+    h = ops.add_rmsnorm(x, None, norm_w.cuda(), eps, torch.bfloat16)
+    assert torch.equal(pre.materialize(), h)
+    exact_h = pl.rmsnorm(want_x.float(), norm_w, eps).double()
+    exact = exact_h @ w_in[:F].double().t()
+    got = ops.linear_prenorm(pre, w_in[:F].cuda().contiguous())
+    classic = ops.linear(h, w_in[:F].cuda().contiguous())
+    # both round the activations to bf16 once (at different places) and the result once: the fused product is
+    # not further from the exact result than twice the plain one, plus one rounding of the result
+    e_got, e_classic = rel_err(got.float(), exact.float()), rel_err(classic.float(), exact.float())
+    assert e_got <= 2.0 * e_classic + 2.0 ** -7, (e_got, e_classic)
+    if F % 8 == 0:
+        wi = ops.interleave_gate_up(w_in[:F].cuda(), w_in[F:].cuda())
+        g, u = exact_h @ w_in[:F].double().t(), exact_h @ w_in[F:].double().t()
+        exact_glu = ((g / (1 + torch.exp(-g))) * u).float()
+        got = ops.linear_swiglu_prenorm(pre, wi)
+        classic = ops.linear_swiglu(h, wi, True)
+        e_got, e_classic = rel_err(got.float(), exact_glu), rel_err(classic.float(), exact_glu)
+        assert e_got <= 2.0 * e_classic + 2.0 ** -7, (e_got, e_classic)
+    # a second product into the same stream (the next part's last one) keeps adding
+    act2 = _rand((M, F), torch.bfloat16, 36)
+    pre2 = ops.linear_into_stream(act2.cuda(), w_out.cuda(), x, norm_w.cuda(), eps)
+    want_x2 = want_x + act2.double() @ w_out.double().t()
+    assert rel_err(x, want_x2.float()) < 1e-5
+    assert rel_err(pre2.slots.sum(dim=1), want_x2.pow(2).sum(dim=1).float()) < 1e-5
+
+
+def test_products_with_the_norm_folded_in_refuse_what_they_cannot_take():
+    ops = _ops()
+    assert not ops.can_defer_norm(17, 64, 64, torch.bfloat16)              # more than one tile of rows
+    assert not ops.can_defer_norm(8, 64, 64, torch.float32)
+    assert not ops.can_defer_norm(8, 16 * 513, 64, torch.bfloat16)         # more column tiles than a consumer adds up
+    x = torch.zeros(17, 64, device="cuda")
+    with pytest.raises(ops.KernelError):
+        ops.linear_into_stream(torch.zeros(17, 64, dtype=torch.bfloat16, device="cuda"),
+                               torch.zeros(64, 64, dtype=torch.bfloat16, device="cuda"), x, torch.ones(64, device="cuda"), 1e-5)
+
+
 @pytest.mark.parametrize("width", [0, 256, 192, 128])
 @pytest.mark.parametrize("M,N,K", [(65, 16, 8), (100, 200, 328), (256, 256, 64), (300, 520, 192), (777, 1000, 136),
                                    (513, 4104, 1032), (1, 31, 264)])
