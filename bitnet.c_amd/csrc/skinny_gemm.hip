@@ -143,7 +143,8 @@ __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_ke
 //   PRE: the activations are such a copy.  1/sqrt(mean(x^2) + eps) (src/transformer/rmsnorm_scalar.c:4-13)
 //        multiplies a whole row of the result, so it is applied in the epilogue: every wave fetches the
 //        slots of two rows before its K loop and adds them up behind it (lane-strided sums, a tree over
-//        the lanes: a fixed order); the staged activations need no work at all.
+//        the lanes: a fixed order); the staged activations need no work at all.  (Asked for later, before
+//        the wave's last chunk, the same loads cost three times as much.)
 // GLU8 as above.  bf16 result (RES: no result of its own).
 #define SK_SLOT_LOADS 8       // slots per row and lane: at most 512 column tiles (a stream of 8,192 columns)
 
@@ -202,10 +203,7 @@ void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict
         for (int j = 0; j < 8; ++j)
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xv[j]), as_bf16x8(wv[j]), acc, 0, 0, 0);
     };
-    // all chunks of this wave but its last; the slots of the norm are asked for before the last one, so that they
-    // arrive while it waits for its weights and occupy registers only there
-    int kc = wave * SK_CHUNK;
-    for (; kc + NW * SK_CHUNK < K; kc += NW * SK_CHUNK) step(kc);
+    // the slots of the norm are asked for first: they arrive while the wave waits for its first weights
     float sv[2][SL];                                   // PRE: this lane's slots of rows wave and wave + 8
     if (PRE) {
 #pragma unroll
@@ -218,7 +216,7 @@ void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict
             }
         }
     }
-    if (kc < K) step(kc);
+    for (int kc = wave * SK_CHUNK; kc < K; kc += NW * SK_CHUNK) step(kc);
     if (PRE) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
