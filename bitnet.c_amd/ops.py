@@ -253,7 +253,9 @@ def gemm_mfma(x: torch.Tensor, w: torch.Tensor, out_dtype=None, glu8: bool = Fal
 
 
 def gemm_mfma_supported(M: int, N: int, K: int, ldx: int, ldw: int) -> bool:
-    return bool(_fn("gemm_mfma", "bn_gemm_mfma_supports")(M, N, K, ldx, ldw))
+    """The conditions of bn_gemm_mfma_supports, checked here so that asking does not load (and at
+    first use compile) a kernel that a model may never need."""
+    return M >= 1 and N >= 1 and K >= 8 and K % 8 == 0 and ldx % 8 == 0 and ldw % 8 == 0 and ldx >= K and ldw >= K
 
 
 SKINNY_ROWS = 16      # bf16 products with more rows than this go to the library

@@ -257,6 +257,12 @@ def test_gemm_mfma_refuses_what_it_cannot_take():
         ops.gemm_mfma(x, w)                               # K is not a multiple of 8
     with pytest.raises(ops.KernelError):
         ops.gemm_mfma(x.float(), w.float())               # bf16 only
+    # the check that the dispatcher makes without loading the kernel is the kernel's own
+    from bitnet_c_amd.csrc import build
+    supports = build.load("gemm_mfma").bn_gemm_mfma_supports
+    for M, N, K, ldx, ldw in [(70, 16, 36, 36, 36), (70, 16, 40, 40, 40), (1, 1, 8, 8, 8), (5, 5, 4, 8, 8), (5, 5, 16, 12, 16),
+                              (5, 5, 16, 8, 16), (0, 5, 16, 16, 16), (5, 0, 16, 16, 16), (3000, 4104, 4096, 4104, 4096)]:
+        assert ops.gemm_mfma_supported(M, N, K, ldx, ldw) == bool(supports(M, N, K, ldx, ldw)), (M, N, K, ldx, ldw)
     # the dispatcher sends such a shape to the plain tiled kernel instead
     y = ops.linear(x, w, allow_library=False)
     assert close(y.float(), (x.double().cpu() @ w.double().cpu().t()).float(), torch.bfloat16)
