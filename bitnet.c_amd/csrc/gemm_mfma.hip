@@ -8,8 +8,12 @@
 // waits for shared memory) owns a tile of 256 rows of X by BN (256, 192 or 128) rows of W and
 // walks K in steps of 64.  Both operands are K-contiguous, so a lane's MFMA operand is 16
 // contiguous bytes of one row.  A step's two tiles are fetched with 16-byte loads (eight threads
-// cover the 128 bytes of a row) into registers while the previous step is multiplied, then parked
-// in the other half of shared memory: one barrier a step.  Rows are stored without padding and
+// cover the 128 bytes of a row) into registers while earlier steps are multiplied, then parked
+// in the other half of shared memory: one barrier a step.  The narrower tiles have registers for
+// a second set of loads and fetch two steps ahead.  The loop's body has no branch (rows past the
+// end are clamped, a K tail is peeled off), and scheduling barriers keep the loads ahead of the
+// products and the stores behind them: left alone, the compiler moves the loads down to their
+// stores and every step waits out the memory latency.  Rows are stored without padding and
 // their 16-byte chunks swizzled (chunk c of row r at c ^ swizzle(r)) so that the sixteen lanes
 // which shared memory serves together never meet in a bank.
 //
@@ -77,44 +81,45 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_mfma_kernel(const bf16* __res
 #pragma unroll
         for (int b = 0; b < MT; ++b) acc[a][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    uint4 xd[XL], wd[WL];
-    auto fetch = [&](int k0) {
-        const int k = k0 + schunk * 8;
+    struct Regs { uint4 x[XL]; uint4 w[WL]; };
+    // rows past the end are clamped (their results are dropped), so that a full step's loads carry no predicate
+    const bf16* xbase = X + (size_t)min(m0 + srow, M - 1) * ldx + schunk * 8;
+    const bf16* wbase = W + (size_t)min(n0 + srow, N - 1) * ldw + schunk * 8;
+    const int xrows_left = M - 1 - (m0 + srow), wrows_left = N - 1 - (n0 + srow);
+    auto fetch_full = [&](Regs& r, int k0) {
 #pragma unroll
-        for (int j = 0; j < XL; ++j) {
-            const int m = m0 + srow + PASS * j;
-            xd[j] = (m < M && k < K) ? *reinterpret_cast<const uint4*>(X + (size_t)m * ldx + k) : make_uint4(0, 0, 0, 0);
-        }
+        for (int j = 0; j < XL; ++j)
+            r.x[j] = *reinterpret_cast<const uint4*>(xbase + (size_t)max(0, min(PASS * j, xrows_left)) * ldx + k0);
 #pragma unroll
-        for (int j = 0; j < WL; ++j) {
-            const int n = n0 + srow + PASS * j;
-            wd[j] = (n < N && k < K) ? *reinterpret_cast<const uint4*>(W + (size_t)n * ldw + k) : make_uint4(0, 0, 0, 0);
-        }
+        for (int j = 0; j < WL; ++j)
+            r.w[j] = *reinterpret_cast<const uint4*>(wbase + (size_t)max(0, min(PASS * j, wrows_left)) * ldw + k0);
     };
-    auto park = [&](int buf) {
+    auto fetch_tail = [&](Regs& r, int k0) {
+        const bool in = k0 + schunk * 8 < K;
+#pragma unroll
+        for (int j = 0; j < XL; ++j)
+            r.x[j] = in ? *reinterpret_cast<const uint4*>(xbase + (size_t)max(0, min(PASS * j, xrows_left)) * ldx + k0) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < WL; ++j)
+            r.w[j] = in ? *reinterpret_cast<const uint4*>(wbase + (size_t)max(0, min(PASS * j, wrows_left)) * ldw + k0) : make_uint4(0, 0, 0, 0);
+    };
+    auto park = [&](const Regs& r, int buf) {
         unsigned char* xs = smem + (size_t)buf * STAGE;
         unsigned char* ws = xs + GM_BM * 128;
 #pragma unroll
         for (int j = 0; j < XL; ++j) {
-            const int r = srow + PASS * j;
-            *reinterpret_cast<uint4*>(xs + r * 128 + ((schunk ^ gm_swizzle(r & 15)) << 4)) = xd[j];
+            const int row = srow + PASS * j;
+            *reinterpret_cast<uint4*>(xs + row * 128 + ((schunk ^ gm_swizzle(row & 15)) << 4)) = r.x[j];
         }
 #pragma unroll
         for (int j = 0; j < WL; ++j) {
-            const int r = srow + PASS * j;
-            *reinterpret_cast<uint4*>(ws + r * 128 + ((schunk ^ gm_swizzle(r & 15)) << 4)) = wd[j];
+            const int row = srow + PASS * j;
+            *reinterpret_cast<uint4*>(ws + row * 128 + ((schunk ^ gm_swizzle(row & 15)) << 4)) = r.w[j];
         }
     };
-
-    const int n_steps = (K + GM_BK - 1) / GM_BK;
-    fetch(0);
-    park(0);
-    __syncthreads();
     const int swz = gm_swizzle(i);
-    for (int s = 0; s < n_steps; ++s) {
-        const bool more = s + 1 < n_steps;
-        if (more) fetch((s + 1) * GM_BK);
-        const unsigned char* xs = smem + (size_t)(s & 1) * STAGE;
+    auto multiply = [&](int buf) {
+        const unsigned char* xs = smem + (size_t)buf * STAGE;
         const unsigned char* ws = xs + GM_BM * 128;
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
@@ -130,8 +135,66 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_mfma_kernel(const bf16* __res
                 for (int b = 0; b < MT; ++b)
                     acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gm_as_bf16x8(wf[a]), gm_as_bf16x8(xf[b]), acc[a][b], 0, 0, 0);
         }
-        if (more) park((s + 1) & 1);
+    };
+
+    const int n_steps = (K + GM_BK - 1) / GM_BK;
+    const int full = K / GM_BK;                       // steps that need no K guard
+    constexpr bool TWO = BN < 256;                    // a second set of staging registers: loads two steps ahead
+    Regs r0, r1;
+    int s = 0;
+    if (TWO) {
+        fetch_tail(r0, 0);
+        if (n_steps > 1) fetch_tail(r1, GM_BK);
+        park(r0, 0);
         __syncthreads();
+        // even s: buffer 0 holds step s, r1 step s + 1 (on its way), r0 is free
+        for (; s + 3 < full; s += 2) {
+            fetch_full(r0, (s + 2) * GM_BK);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(0);
+            __builtin_amdgcn_sched_barrier(0);
+            park(r1, 1);
+            __syncthreads();
+            fetch_full(r1, (s + 3) * GM_BK);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(1);
+            __builtin_amdgcn_sched_barrier(0);
+            park(r0, 0);
+            __syncthreads();
+        }
+        // the rest one step ahead: the step on its way is parked first, then r0 alone carries on
+        if (s < n_steps) {
+            multiply(0);
+            if (s + 1 < n_steps) park(r1, 1);
+            __syncthreads();
+            ++s;
+        }
+        for (; s < n_steps; ++s) {
+            const bool more = s + 1 < n_steps;
+            if (more) fetch_tail(r0, (s + 1) * GM_BK);
+            multiply(s & 1);
+            if (more) park(r0, (s + 1) & 1);
+            __syncthreads();
+        }
+    } else {
+        if (full > 0) fetch_full(r0, 0); else fetch_tail(r0, 0);
+        park(r0, 0);
+        __syncthreads();
+        for (; s + 1 < full; ++s) {                   // the next step is a full one: no branch in the body
+            fetch_full(r0, (s + 1) * GM_BK);
+            __builtin_amdgcn_sched_barrier(0);        // the loads stay ahead of the products ...
+            multiply(s & 1);
+            __builtin_amdgcn_sched_barrier(0);        // ... and the stores of their data behind them
+            park(r0, (s + 1) & 1);
+            __syncthreads();
+        }
+        for (; s < n_steps; ++s) {
+            const bool more = s + 1 < n_steps;
+            if (more) fetch_tail(r0, (s + 1) * GM_BK);
+            multiply(s & 1);
+            if (more) park(r0, (s + 1) & 1);
+            __syncthreads();
+        }
     }
 
     // acc[a][b]: lane (i, g) holds columns n = 4g..4g+3 of row m = i of the result tile (a, b); vec: rows of Y
