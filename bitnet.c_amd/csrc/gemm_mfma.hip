@@ -233,7 +233,10 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_mfma_kernel(const bf16* __res
                 if (g < 2 && m < M) {
                     const int f = ((n0 + wn + a * 16) >> 1) + 4 * g;      // result column of v[0]
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) v[r] = (v[r] / (1.0f + expf(-v[r]))) * up[r];
+                    // silu(g) * u with the hardware's exp2 and reciprocal (an ulp each, far below the result's
+                    // rounding): expf and a division cost 25 vector instructions a value, a tenth of this kernel's time
+                    for (int r = 0; r < 4; ++r)
+                        v[r] = v[r] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504f * v[r])) * up[r];
                     store4(Y + (size_t)m * ldy + f, v, (N >> 1) - f);
                 }
             } else if (m < M) {
