@@ -1,11 +1,11 @@
 """The Python entry point: load a model folder, generate."""
 from __future__ import annotations
 
-from typing import Callable, List, Optional, Sequence
+from typing import Callable, Optional, Sequence
 
 import torch
 
-from .engine import Engine, Request, Result, generate
+from .engine import Engine, Request, generate
 from .sampling import SamplingParams, sample_batch
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,

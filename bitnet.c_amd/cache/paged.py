@@ -24,7 +24,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-from ..parts.base import CacheNeed, KVNeed, KVView, StateNeed
+from ..parts.base import CacheNeed, KVNeed, KVView
 
 PAGE = 64
 

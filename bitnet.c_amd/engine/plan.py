@@ -10,7 +10,7 @@ holds the same decisions in per-layer plan structs that it recomputes on every c
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, List, Optional
 
 from ..parts.base import PartSpec

@@ -13,8 +13,8 @@ all new keys and values are in the cache before any new token attends
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Sequence
+from dataclasses import dataclass
+from typing import Dict, List, Sequence
 
 import torch
 

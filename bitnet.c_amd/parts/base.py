@@ -32,7 +32,7 @@ here the decision is made once, when the model is built.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, Optional, Tuple
 
 import torch

@@ -3,7 +3,6 @@ twice, a layer that reads another layer's cache); and toy parts defined here, re
 and stepped without a change to the library's files: a mixer with a state of its own, a
 feed-forward with routing, another position encoding."""
 import json
-import math
 import os
 import random
 from dataclasses import asdict, dataclass
