@@ -486,3 +486,46 @@ def test_cuts_and_batches_agree_at_the_benchmark_layer_sizes():
         assert float(per_row.max()) < 0.025, per_row
         assert float(per_row.max() / per_row.min()) < 2.0, per_row
         assert float(d.abs().max() / d.pow(2).mean().sqrt()) < 7.0
+
+
+@pytest.mark.parametrize("n_seqs", [20, 50])
+def test_graph_replays_of_a_wide_batch_at_the_benchmark_layer_sizes(n_seqs):
+    """20 or 50 sequences decode together at the Llama-3.1-8B layer sizes (two layers, bfloat16): 32 or 64
+    rows a step, whose products are the library's, replayed from a HIP graph.  A library kernel may clear a
+    work buffer inside the graph, and such a node has to give the right result on every replay, not
+    only on the first: every replay is compared with the same step run without graphs, with eager
+    prompt steps of other sequences and synchronisations between the replays."""
+    import bitnet_c_amd as bn
+    from bitnet_c_amd.config import architecture_for
+    from bitnet_c_amd.engine import DecoderModel
+    from bitnet_c_amd.weights import random_tensors
+    raw = dict(model_type="llama", vocab_size=32000, hidden_size=4096, intermediate_size=14336,
+               num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+               max_position_embeddings=8192, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+    cfg = bn.LlamaConfig.from_dict(raw)
+    plan = architecture_for(raw).build_plan(cfg)
+    model = DecoderModel(plan, torch.bfloat16, "cuda:0")
+    model.load(random_tensors(plan.expected_tensors(), 5, torch.bfloat16, device="cuda:0"))
+    engines = [bn.Engine(model, max_tokens=64 * 160, use_graphs=g) for g in (True, False)]
+    rnd = random.Random(41)
+    reqs = [[rnd.randrange(cfg.vocab_size) for _ in range(10 + 3 * i)] for i in range(n_seqs)]
+    extra = [[rnd.randrange(cfg.vocab_size) for _ in range(40)] for _ in range(6)]
+    outs = []
+    for eng in engines:
+        slots = [eng.new_sequence() for _ in reqs]
+        eng.step([bn.StepEntry(s, r[:-6], []) for s, r in zip(slots, reqs)])
+        got = []
+        for k in range(6):
+            other = eng.new_sequence()                              # eager work between the replays
+            eng.step([bn.StepEntry(other, extra[k], [39])])
+            eng.release(other)
+            torch.cuda.synchronize()
+            got.append(eng.step([bn.StepEntry(s, [r[len(r) - 6 + k]], [0]) for s, r in zip(slots, reqs)]).clone())
+        for s in slots:
+            eng.release(s)
+        eng.cache.check()
+        outs.append(torch.stack(got))                               # [replay, sequence, vocab]
+    assert engines[0]._graphs, "the decode steps were meant to be replayed from a graph"
+    for k in range(6):
+        # the same kernels run on both sides; a library product may sum in an order of its own from run to run
+        assert rel_err(outs[0][k], outs[1][k]) < 1e-2, k
