@@ -526,6 +526,13 @@ def test_graph_replays_of_a_wide_batch_at_the_benchmark_layer_sizes(n_seqs):
         eng.cache.check()
         outs.append(torch.stack(got))                               # [replay, sequence, vocab]
     assert engines[0]._graphs, "the decode steps were meant to be replayed from a graph"
+    # The graph pads the batch to 32 or 64 rows and the library may pick another kernel for that many rows than for
+    # 20 or 50, so the two sides differ by bfloat16 rounding: about 1 % of the logits' root mean square in every
+    # row of every replay, with no value far outside it.  A buffer that was not cleared on a replay is not noise.
+    rms = float(outs[1].double().pow(2).mean().sqrt())
     for k in range(6):
-        # the same kernels run on both sides; a library product may sum in an order of its own from run to run
-        assert rel_err(outs[0][k], outs[1][k]) < 1e-2, k
+        d = (outs[0][k] - outs[1][k]).double()
+        per_row = d.pow(2).mean(dim=1).sqrt() / rms
+        assert float(per_row.max()) < 0.025, (k, per_row)
+        sd = float(d.pow(2).mean().sqrt())                           # 0: the same kernels ran on both sides
+        assert sd == 0.0 or float(d.abs().max()) / sd < 8.0, k
