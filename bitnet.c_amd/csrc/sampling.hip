@@ -327,6 +327,365 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(const float* __rest
     if (threadIdx.x == 0) out[blockIdx.x] = tok;
 }
 
+// ---------------------------------------------------------------------------------------
+// The same sampling with a row spread over many workgroups, for large vocabularies: one workgroup
+// walks a row of 128k logits 17 times (half a millisecond); here every pass is a launch of
+// rows x WIDE_PARTS workgroups that read a part each, and what one workgroup decided alone
+// (the maximum, the sum, each level's bucket of the radix descent) is recomputed by every
+// workgroup from small per-row tables in a work buffer: per-part maxima and sums, the 2 x 4
+// histograms of the two descents (added up with 64-bit atomics in fixed point, so the order cannot
+// matter), per-part counts of the final bit pattern.  Probabilities are never stored: every pass
+// computes q_i = expf(x_i / T - max) / sum again, the same value each time.
+// ---------------------------------------------------------------------------------------
+#define WIDE_PARTS 32
+#define WIDE_THREADS 256
+#define WIDE_HIST (2 * 4 * 256)                      // 64-bit words of histograms per row
+#define WIDE_ROW_WORDS (WIDE_HIST + 3 * WIDE_PARTS)  // + maxima, sums, cdf sums (floats) and counts (2 x parts ints)
+
+struct WideArgs {
+    const float* logits;
+    int ld, n, part_len;
+    unsigned long long* ws;      // [rows][WIDE_ROW_WORDS], zero when the first kernel starts
+    const float* r;
+    float temperature, top_p;
+    int* out;
+};
+
+struct WideRow {
+    unsigned long long* hist;    // [2][4][256]
+    float *pmax, *psum, *pcdf;   // [WIDE_PARTS] each
+    int* cnt;                    // [2][WIDE_PARTS]
+};
+
+__device__ __forceinline__ WideRow wide_row(const WideArgs& a, int row) {
+    WideRow w;
+    w.hist = a.ws + (size_t)row * WIDE_ROW_WORDS;
+    w.pmax = reinterpret_cast<float*>(w.hist + WIDE_HIST);
+    w.psum = w.pmax + WIDE_PARTS;
+    w.pcdf = w.psum + WIDE_PARTS;
+    w.cnt = reinterpret_cast<int*>(w.pcdf + WIDE_PARTS);
+    return w;
+}
+
+// The row's maximum and sum from the per-part tables, in part order (every thread computes them: 64 loads).
+__device__ __forceinline__ void wide_stats(const WideRow& w, float& mx, float& total) {
+    mx = -INFINITY;
+    for (int p = 0; p < WIDE_PARTS; ++p) mx = fmaxf(mx, w.pmax[p]);
+    total = 0.f;
+    for (int p = 0; p < WIDE_PARTS; ++p) total += w.psum[p];
+}
+
+// One level of the descent, decided by a whole wave from the level's 256 sums (lane l holds the bins
+// 4l .. 4l+3): the highest bin b with a non-zero sum for which above + sum(bins >= b) exceeds the bound,
+// else the lowest non-zero bin (bin 0 when all are empty); `above` becomes the sum over the bins above it.
+// The same choice as the loop over the bins from 255 down in descend().
+__device__ __forceinline__ int wide_choose(const unsigned long long h[4], unsigned long long& above,
+                                           unsigned long long bound, int lane) {
+    unsigned long long own = h[0] + h[1] + h[2] + h[3];
+    unsigned long long suf = own;                      // inclusive suffix sum over the lanes (lane 63 first)
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const unsigned lo32 = __shfl_down((unsigned)suf, o, BN_WAVE), hi32 = __shfl_down((unsigned)(suf >> 32), o, BN_WAVE);
+        if (lane + o < 64) suf += ((unsigned long long)hi32 << 32) | lo32;
+    }
+    const unsigned long long higher = above + suf - own;       // above + sum over the bins of higher lanes
+    int best = -1, lowest = -1;
+    unsigned long long acc_best = 0, acc_low = 0, acc = higher;
+#pragma unroll
+    for (int j = 3; j >= 0; --j) {
+        if (h[j] != 0) {
+            lowest = 4 * lane + j; acc_low = acc;
+            if (best < 0 && acc + h[j] > bound) { best = 4 * lane + j; acc_best = acc; }
+        }
+        acc += h[j];
+    }
+    // the highest lane that found one wins
+    const unsigned long long found = __ballot(best >= 0);
+    if (found) {
+        const int src = 63 - __clzll((long long)found);
+        above = ((unsigned long long)__shfl((unsigned)(acc_best >> 32), src, BN_WAVE) << 32) | __shfl((unsigned)acc_best, src, BN_WAVE);
+        return __shfl(best, src, BN_WAVE);
+    }
+    const unsigned long long any = __ballot(lowest >= 0);
+    if (any) {
+        const int src = __ffsll((long long)any) - 1;   // the lowest lane that has a non-zero bin
+        above = ((unsigned long long)__shfl((unsigned)(acc_low >> 32), src, BN_WAVE) << 32) | __shfl((unsigned)acc_low, src, BN_WAVE);
+        return __shfl(lowest, src, BN_WAVE);
+    }
+    return 0;                                          // nothing there: bin 0, `above` as it was
+}
+
+struct WideState {            // what a descent has decided so far
+    uint32_t prefix, mask;
+    unsigned long long above;
+};
+
+// Wave 0 replays `levels` levels of descent d from the stored histograms.
+__device__ __forceinline__ WideState wide_replay(const WideRow& w, int d, int levels, unsigned long long bound, int lane) {
+    WideState st = {0u, 0u, 0ull};
+    unsigned long long h[4][4];
+#pragma unroll
+    for (int l = 0; l < 4; ++l)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) h[l][j] = l < levels ? w.hist[(d * 4 + l) * 256 + 4 * lane + j] : 0ull;
+#pragma unroll
+    for (int l = 0; l < 4; ++l) {
+        if (l < levels) {
+            const int shift = 24 - 8 * l;
+            const int chosen = wide_choose(h[l], st.above, bound, lane);
+            st.prefix |= ((uint32_t)chosen) << shift;
+            st.mask |= 255u << shift;
+        }
+    }
+    return st;
+}
+
+// The end of a descent: how many elements of the final bit pattern are taken (k) and the sum including them.
+__device__ __forceinline__ long long wide_take(const WideState& st, unsigned long long bound, int total,
+                                               unsigned long long& cum) {
+    const unsigned long long qv = to_fixed(__uint_as_float(st.prefix));
+    long long k = 1;
+    if (qv > 0 && bound >= st.above) k = (long long)((bound - st.above) / qv) + 1;
+    if (k > total) k = total;
+    if (k < 1) k = 1;
+    cum = st.above + (unsigned long long)k * qv;
+    return k;
+}
+
+__device__ __forceinline__ int wide_total(const WideRow& w, int d) {
+    int t = 0;
+    for (int p = 0; p < WIDE_PARTS; ++p) t += w.cnt[d * WIDE_PARTS + p];
+    return t;
+}
+
+// The bound of descent d: top_p itself for the first, r times the first descent's sum for the second.
+__device__ __forceinline__ unsigned long long wide_bound(const WideArgs& a, const WideRow& w, int d, int row, int lane) {
+    const unsigned long long b0 = to_fixed(a.top_p);
+    if (d == 0) return b0;
+    const WideState s0 = wide_replay(w, 0, 4, b0, lane);
+    unsigned long long cum0 = 0;
+    (void)wide_take(s0, b0, wide_total(w, 0), cum0);
+    return (unsigned long long)((double)a.r[row] * (double)cum0);
+}
+
+// The probability of one element; every kernel computes it with this one function, so that an element has the
+// same bit pattern in every pass.
+__device__ __forceinline__ float wide_q(float x, float temperature, float mx, float total) {
+    return expf(x / temperature - mx) / total;
+}
+
+__device__ __forceinline__ void wide_part(const WideArgs& a, int& lo, int& hi) {
+    lo = min(a.n, (int)blockIdx.x * a.part_len);
+    hi = min(a.n, lo + a.part_len);
+}
+
+__global__ __launch_bounds__(WIDE_THREADS) void wide_max_kernel(WideArgs a) {
+    __shared__ float fs[16];
+    const int row = blockIdx.y;
+    const float* x = a.logits + (size_t)row * a.ld;
+    int lo, hi;
+    wide_part(a, lo, hi);
+    float mx = -INFINITY;
+    for (int i = lo + threadIdx.x; i < hi; i += WIDE_THREADS) mx = fmaxf(mx, x[i] / a.temperature);
+    mx = block_max(mx, fs);
+    if (threadIdx.x == 0) wide_row(a, row).pmax[blockIdx.x] = mx;
+}
+
+// CDF != 0: the part's sum of the probabilities (for the plain cdf walk) instead of the exponentials
+template <bool CDF>
+__global__ __launch_bounds__(WIDE_THREADS) void wide_sum_kernel(WideArgs a) {
+    __shared__ float fs[16];
+    const int row = blockIdx.y;
+    const WideRow w = wide_row(a, row);
+    const float* x = a.logits + (size_t)row * a.ld;
+    int lo, hi;
+    wide_part(a, lo, hi);
+    float mx, total = 1.f;
+    if (CDF) {
+        wide_stats(w, mx, total);
+    } else {
+        mx = -INFINITY;
+        for (int p = 0; p < WIDE_PARTS; ++p) mx = fmaxf(mx, w.pmax[p]);
+    }
+    float part = 0.f;
+    for (int i = lo + threadIdx.x; i < hi; i += WIDE_THREADS) {
+        part += CDF ? wide_q(x[i], a.temperature, mx, total) : expf(x[i] / a.temperature - mx);
+    }
+    part = block_sum(part, fs);
+    if (threadIdx.x == 0) (CDF ? w.pcdf : w.psum)[blockIdx.x] = part;
+}
+
+// The plain cdf walk: first i with r < cdf_i (src/sampler.c:65-74), n - 1 if none.  The part that holds it is
+// found from the parts' sums; one wave of that part's workgroup walks it with a prefix sum over each 64 elements.
+__global__ __launch_bounds__(64) void wide_walk_kernel(WideArgs a) {
+    const int row = blockIdx.y, lane = threadIdx.x;
+    const WideRow w = wide_row(a, row);
+    const float rr = a.r[row];
+    float c = 0.f, c0 = 0.f;
+    int owner = -1;
+    for (int p = 0; p < WIDE_PARTS; ++p) {
+        const float s = w.pcdf[p];
+        if (owner < 0 && rr < c + s) { owner = p; c0 = c; }
+        c += s;
+    }
+    if (owner < 0) { if (blockIdx.x == 0 && lane == 0) a.out[row] = a.n - 1; return; }
+    if ((int)blockIdx.x != owner) return;
+    float mx, total;
+    wide_stats(w, mx, total);
+    const float* x = a.logits + (size_t)row * a.ld;
+    int lo, hi;
+    wide_part(a, lo, hi);
+    c = c0;
+    int found = hi - 1;
+    for (int g0 = lo; g0 < hi; g0 += 64) {
+        const int i = g0 + lane;
+        float sc = i < hi ? wide_q(x[i], a.temperature, mx, total) : 0.f;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const float t = __shfl_up(sc, o, BN_WAVE);
+            if (lane >= o) sc += t;
+        }
+        const unsigned long long m = __ballot(i < hi && rr < c + sc);
+        if (m) { found = g0 + __ffsll((long long)m) - 1; break; }
+        c += __shfl(sc, 63, BN_WAVE);
+    }
+    if (lane == 0) a.out[row] = found;
+}
+
+// One level of a descent: the sums of the candidates' probabilities by the next 8 bits of their bit pattern.
+__global__ __launch_bounds__(WIDE_THREADS) void wide_hist_kernel(WideArgs a, int d, int level) {
+    __shared__ unsigned long long hist[256];
+    __shared__ uint32_t st_s[2];
+    const int row = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const WideRow w = wide_row(a, row);
+    hist[threadIdx.x] = 0;                              // 256 threads, 256 bins
+    if (wave == 0) {
+        const unsigned long long bound = wide_bound(a, w, d, row, lane);
+        const WideState st = wide_replay(w, d, level, bound, lane);
+        if (lane == 0) { st_s[0] = st.prefix; st_s[1] = st.mask; }
+    }
+    __syncthreads();
+    const uint32_t prefix = st_s[0], mask = st_s[1];
+    float mx, total;
+    wide_stats(w, mx, total);
+    const float cutoff = (1.0f - a.top_p) / (float)(a.n - 1);
+    const int shift = 24 - 8 * level;
+    const float* x = a.logits + (size_t)row * a.ld;
+    int lo, hi;
+    wide_part(a, lo, hi);
+    for (int i = lo + threadIdx.x; i < hi; i += WIDE_THREADS) {
+        const float v = wide_q(x[i], a.temperature, mx, total);
+        const uint32_t bits = __float_as_uint(v);
+        if (v >= cutoff && (bits & mask) == prefix) atomicAdd(&hist[(bits >> shift) & 255u], to_fixed(v));
+    }
+    __syncthreads();
+    const unsigned long long mine = hist[threadIdx.x];
+    if (mine) atomicAdd(&w.hist[(d * 4 + level) * 256 + threadIdx.x], mine);
+}
+
+// After the four levels the bit pattern is complete: how many elements of this part have it.
+__global__ __launch_bounds__(WIDE_THREADS) void wide_count_kernel(WideArgs a, int d) {
+    __shared__ uint32_t st_s[1];
+    __shared__ int cs[WIDE_THREADS / 64];
+    const int row = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const WideRow w = wide_row(a, row);
+    if (wave == 0) {
+        const unsigned long long bound = wide_bound(a, w, d, row, lane);
+        const WideState st = wide_replay(w, d, 4, bound, lane);
+        if (lane == 0) st_s[0] = st.prefix;
+    }
+    __syncthreads();
+    const uint32_t prefix = st_s[0];
+    float mx, total;
+    wide_stats(w, mx, total);
+    const float cutoff = (1.0f - a.top_p) / (float)(a.n - 1);
+    const float* x = a.logits + (size_t)row * a.ld;
+    int lo, hi;
+    wide_part(a, lo, hi);
+    int c = 0;
+    for (int i = lo + threadIdx.x; i < hi; i += WIDE_THREADS) {
+        const float v = wide_q(x[i], a.temperature, mx, total);
+        c += (v >= cutoff && __float_as_uint(v) == prefix) ? 1 : 0;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, BN_WAVE);
+    if (lane == 0) cs[wave] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int t = 0;
+        for (int k = 0; k < WIDE_THREADS / 64; ++k) t += cs[k];
+        w.cnt[d * WIDE_PARTS + blockIdx.x] = t;
+    }
+}
+
+// The token: the k-th element, in index order, of those with the second descent's bit pattern.
+__global__ __launch_bounds__(64) void wide_pick_kernel(WideArgs a) {
+    const int row = blockIdx.y, lane = threadIdx.x;
+    const WideRow w = wide_row(a, row);
+    const unsigned long long bound = wide_bound(a, w, 1, row, lane);
+    const WideState st = wide_replay(w, 1, 4, bound, lane);
+    const int total_hits = wide_total(w, 1);
+    unsigned long long cum = 0;
+    const long long k = wide_take(st, bound, total_hits, cum);
+    if (total_hits <= 0) { if (blockIdx.x == 0 && lane == 0) a.out[row] = a.n - 1; return; }
+    int seen = 0, owner = WIDE_PARTS - 1, rank = 1;
+    for (int p = 0; p < WIDE_PARTS; ++p) {
+        const int c = w.cnt[WIDE_PARTS + p];
+        if (seen + c >= (int)k) { owner = p; rank = (int)k - seen; break; }
+        seen += c;
+    }
+    if ((int)blockIdx.x != owner) return;
+    float mx, total;
+    wide_stats(w, mx, total);
+    const float cutoff = (1.0f - a.top_p) / (float)(a.n - 1);
+    const float* x = a.logits + (size_t)row * a.ld;
+    int lo, hi;
+    wide_part(a, lo, hi);
+    int found = a.n - 1;
+    seen = 0;
+    for (int g0 = lo; g0 < hi; g0 += 64) {
+        const int i = g0 + lane;
+        const float v = i < hi ? wide_q(x[i], a.temperature, mx, total) : 0.f;
+        unsigned long long m = __ballot(i < hi && v >= cutoff && __float_as_uint(v) == st.prefix);
+        const int c = __popcll(m);
+        if (seen + c >= rank) {
+            for (int skip = rank - seen - 1; skip > 0; --skip) m &= m - 1;       // drop the lower set bits
+            found = g0 + __ffsll((long long)m) - 1;
+            break;
+        }
+        seen += c;
+    }
+    if (lane == 0) a.out[row] = found;
+}
+
+// 64-bit words of zeroed work memory that bn_sample_wide needs for `rows` rows.
+extern "C" long long bn_sample_wide_words(int rows) { return (long long)rows * WIDE_ROW_WORDS; }
+
+// As bn_sample for temperature > 0, a row spread over WIDE_PARTS workgroups.  ws: bn_sample_wide_words(rows)
+// 64-bit words, all zero.
+extern "C" int bn_sample_wide(const float* logits, int ld, int rows, int n, unsigned long long* ws, const float* r,
+                              float temperature, float top_p, int* out, hipStream_t s) {
+    if (rows <= 0 || rows > 65535 || n < 2 || ld < n || !(temperature > 0.f) || !ws || !r || !out) return BN_ERR_ARG;
+    WideArgs a;
+    a.logits = logits; a.ld = ld; a.n = n; a.ws = ws; a.r = r; a.temperature = temperature; a.top_p = top_p; a.out = out;
+    a.part_len = ((n + WIDE_PARTS - 1) / WIDE_PARTS + 63) / 64 * 64;
+    const dim3 grid(WIDE_PARTS, rows);
+    hipLaunchKernelGGL(wide_max_kernel, grid, dim3(WIDE_THREADS), 0, s, a);
+    hipLaunchKernelGGL(wide_sum_kernel<false>, grid, dim3(WIDE_THREADS), 0, s, a);
+    if (top_p <= 0.0f || top_p >= 1.0f) {
+        hipLaunchKernelGGL(wide_sum_kernel<true>, grid, dim3(WIDE_THREADS), 0, s, a);
+        hipLaunchKernelGGL(wide_walk_kernel, grid, dim3(64), 0, s, a);
+        return bn_launch_status();
+    }
+    for (int d = 0; d < 2; ++d) {
+        for (int level = 0; level < 4; ++level)
+            hipLaunchKernelGGL(wide_hist_kernel, grid, dim3(WIDE_THREADS), 0, s, a, d, level);
+        hipLaunchKernelGGL(wide_count_kernel, grid, dim3(WIDE_THREADS), 0, s, a, d);
+    }
+    hipLaunchKernelGGL(wide_pick_kernel, grid, dim3(64), 0, s, a);
+    return bn_launch_status();
+}
+
 // work: rows * 64 floats and rows * 64 ints for the two-stage form (may be null: one stage)
 extern "C" int bn_argmax(const float* logits, int ld, int rows, int n, int* out, float* work_v, int* work_i,
                          hipStream_t s) {

@@ -72,6 +72,7 @@ _SIGNATURES = {
         "bn_argmax": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
         "bn_repeat_penalty": [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_float, c_void_p],
         "bn_sample": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p],
+        "bn_sample_wide": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p],
     },
 }
 _fns = {}
@@ -757,7 +758,12 @@ def repeat_penalty_(logits: torch.Tensor, recent: torch.Tensor, penalty: float) 
                                                     _stream()), "repeat_penalty")
 
 
-def sample(logits: torch.Tensor, temperature: float, top_p: float, uniforms=None) -> torch.Tensor:
+WIDE_SAMPLE_VOCAB = 16384                 # from this many logits a row on, sampling spreads a row over 32 workgroups
+_WIDE_ROW_WORDS = 2 * 4 * 256 + 3 * 32    # WIDE_ROW_WORDS of csrc/sampling.hip
+
+
+def sample(logits: torch.Tensor, temperature: float, top_p: float, uniforms=None, *,
+           force_one_workgroup: bool = False) -> torch.Tensor:
     """One token id per row.  temperature 0: argmax.  uniforms: float32 [B] in [0, 1)."""
     require_gpu()
     if temperature == 0.0:
@@ -767,6 +773,20 @@ def sample(logits: torch.Tensor, temperature: float, top_p: float, uniforms=None
     out = torch.empty((B,), dtype=torch.int32, device=logits.device)
     if B == 0:
         return out
+    _dev(uniforms, "uniforms", torch.float32, 1)
+    if uniforms.numel() != B or not uniforms.is_contiguous():
+        raise KernelError("sample: one uniform number per row")
+    if V >= WIDE_SAMPLE_VOCAB and B <= 65535 and not force_one_workgroup:
+        # a large vocabulary: every pass over a row is spread over 32 workgroups
+        ws = torch.zeros((B, _WIDE_ROW_WORDS), dtype=torch.int64, device=logits.device)
+        _check(_fn("sampling", "bn_sample_wide")(logits.data_ptr(), ld, B, V, ws.data_ptr(), uniforms.data_ptr(),
+                                                 float(temperature), float(top_p), out.data_ptr(), _stream()),
+               "sample(wide)")
+        return out
+    probs = torch.empty((B, V), dtype=torch.float32, device=logits.device)
+    _check(_fn("sampling", "bn_sample")(logits.data_ptr(), ld, B, V, probs.data_ptr(), uniforms.data_ptr(),
+                                        float(temperature), float(top_p), out.data_ptr(), _stream()), "sample")
+    return out
     probs = None
     if temperature != 0.0:
         _dev(uniforms, "uniforms", torch.float32, 1)

@@ -682,6 +682,37 @@ def test_sample_matches_the_plain_sampler(vocab, temperature, top_p):
     assert got == want
 
 
+@pytest.mark.parametrize("vocab", [16384, 70001, 128256])
+def test_sample_with_a_row_spread_over_many_workgroups(vocab):
+    """From 16,384 logits a row on, every pass of the sampler is a launch of 32 workgroups a row.  It has to
+    draw what the one-workgroup form and the plain sampler draw: peaked and flat rows, plain cdf walk and
+    top-p, a batch of rows with different uniform numbers."""
+    ops = _ops()
+    B = 12
+    g = torch.Generator().manual_seed(vocab)
+    rows = [torch.randn(vocab, generator=g) * s for s in (0.5, 3.0, 8.0)] * 4                 # flat ... peaked
+    logits = torch.stack(rows)
+    rng = pl.XorShift64Star(5)
+    rs = [rng.next_float() for _ in range(B)]
+    r = torch.tensor(rs, dtype=torch.float32).cuda()
+
+    class Fixed:
+        def __init__(self, r): self.r = r
+        def next_float(self): return self.r
+    for temperature, top_p in ((1.0, 0.9), (0.7, 0.5), (1.3, 1.0), (1.0, 0.999), (0.05, 0.9)):
+        wide = ops.sample(logits.cuda(), temperature, top_p, r).cpu().tolist()
+        one = ops.sample(logits.cuda(), temperature, top_p, r, force_one_workgroup=True).cpu().tolist()
+        want = [pl.sample(logits[i], temperature, top_p, Fixed(rs[i])) for i in range(B)]
+        # the three add the probabilities in different orders; a draw changes only where r falls within
+        # rounding of a boundary, which 12 draws do not hit
+        assert wide == want, (temperature, top_p, wide, want)
+        assert one == want, (temperature, top_p, one, want)
+    # a dominant logit far from the start of the row, top-p below its probability: always that token
+    lg = torch.zeros(3, vocab)
+    lg[:, vocab - 7] = 30.0
+    assert ops.sample(lg.cuda(), 1.0, 0.5, r[:3].contiguous()).cpu().tolist() == [vocab - 7] * 3
+
+
 def test_sample_among_equal_probabilities():
     """All logits equal, or in a few equal groups: top-p orders equal probabilities by index, and the
     walk has to find the k-th member of a group across the ranges that the waves own."""
