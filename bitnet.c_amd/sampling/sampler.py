@@ -84,11 +84,9 @@ def sample_batch(logits: torch.Tensor, samplers: Sequence[SequenceSampler]) -> L
     for (temp, top_p, penalty, window), rows in groups.items():
         sub = logits if whole else logits[rows].contiguous()
         if penalty != 1.0 and any(samplers[i].recent for i in rows):
-            rec = torch.full((len(rows), window), -1, dtype=torch.int32)
-            for r, i in enumerate(rows):
-                rc = samplers[i].recent
-                if rc:
-                    rec[r, :len(rc)] = torch.tensor(rc, dtype=torch.int32)
+            # one host tensor for all rows (-1 = empty place), one upload
+            rec = torch.tensor([list(samplers[i].recent)[:window] + [-1] * (window - min(window, len(samplers[i].recent)))
+                                for i in rows], dtype=torch.int32)
             ops.repeat_penalty_(sub, rec.to(sub.device), penalty)
         uniforms = None
         if temp != 0.0:
