@@ -162,12 +162,15 @@ struct SkinnyFused {
 template <bool GLU8, bool PRE, bool RES, int SL>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, bf16* __restrict__ Y, int M, int N,
-                              int K, int ldx, int ldw, int ldy, SkinnyFused f) {
+                              int K, int ldx, int ldw, int ldy, int tile_cols, SkinnyFused f) {
     constexpr int NW = 8;                              // always eight waves: wave w owns rows w and w + 8 of the norm
     extern __shared__ __align__(16) float red[];       // [NW][64][4], then 16 row scales, then the staging
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * 16;
+    // A workgroup owns tile_cols <= 16 columns (the rest of its MFMA tile is not loaded and not stored): the
+    // host picks the width that spreads the column tiles evenly over the CUs.
+    const int n0 = blockIdx.x * tile_cols;
+    const bool col = i < tile_cols;
     const int n = min(n0 + i, N - 1);
     const bf16* wrow = W + (size_t)n * ldw;
     float* scale_s = red + NW * 256;
@@ -187,7 +190,7 @@ void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int k = kb + j * 32;
-            wv[j] = (k < K) ? *reinterpret_cast<const uint4*>(wrow + k) : make_uint4(0, 0, 0, 0);
+            wv[j] = (col && k < K) ? *reinterpret_cast<const uint4*>(wrow + k) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
@@ -237,23 +240,24 @@ void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict
         for (int w = 0; w < NW; ++w) v += red[((size_t)w * 64 + l) * 4 + r];
         const int m = 4 * (l >> 4) + r;
         const int nn = n0 + (l & 15);
+        const bool mine = (l & 15) < tile_cols && nn < N;                 // a column this workgroup owns
         if (PRE) v *= scale_s[m];
         if (GLU8) {
             const float up = __shfl_xor(v, 8, BN_WAVE);
-            if ((l & 8) == 0 && m < M && nn < N)
+            if ((l & 8) == 0 && m < M && nn < N)                          // GLU8: tile_cols is 16
                 Y[(size_t)m * ldy + (n0 >> 1) + (l & 7)] = __float2bfloat16((v / (1.0f + expf(-v))) * up);
         } else if (RES) {
             float xn = 0.f;
-            if (m < M && nn < N) {
+            if (m < M && mine) {
                 xn = f.resid[(size_t)m * f.ld_resid + nn] + v;
                 f.resid[(size_t)m * f.ld_resid + nn] = xn;
                 f.resid_bf16[(size_t)m * f.ld_rb + nn] = __float2bfloat16(xn * f.next_weight[nn]);
             }
-            float sq = xn * xn;                                   // the 16 columns of row m: lanes 16 (l / 16) + 0..15
+            float sq = xn * xn;                                   // the tile's columns of row m: lanes 16 (l / 16) + 0..15
 #pragma unroll
             for (int o = 1; o < 16; o <<= 1) sq += __shfl_xor(sq, o, BN_WAVE);
             if ((l & 15) == 0 && m < M) f.slots_out[(size_t)m * gridDim.x + blockIdx.x] = sq;
-        } else if (m < M && nn < N) {
+        } else if (m < M && mine) {
             Y[(size_t)m * ldy + nn] = __float2bfloat16(v);
         }
     }
@@ -261,12 +265,49 @@ void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict
 
 extern "C" int bn_skinny_gemm_supports(int M, int N, int K, int ldx, int ldw);
 
+static int sk_compute_units() {
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
+        else cus = 256;
+    }
+    return cus;
+}
+
+// Columns per workgroup of the fused kernel for a product of N columns (not GLU8): 16, or fewer when that spreads
+// the column tiles so much more evenly over the CUs that the busiest CU has at least 15 % fewer columns
+// (6,144 columns: 384 tiles of 16 are one and a half rounds over 256 CUs, 512 tiles of 12 are two even ones).
+// A CU pulls its bytes no faster when others idle, so the busiest CU's columns are the kernel's time.
+static int sk_fused_tile_cols(int N) {
+    const int cus = sk_compute_units();
+    auto busiest = [&](int tc) { const int tiles = (N + tc - 1) / tc; return (long long)((tiles + cus - 1) / cus) * tc; };
+    int pick = 16;
+    long long best = busiest(16);
+    for (int tc = 14; tc >= 8; tc -= 2) {
+        const int tiles = (N + tc - 1) / tc;
+        if (tiles > 64 * SK_SLOT_LOADS) continue;                 // a consumer adds up at most that many slots
+        const long long c = busiest(tc);
+        if (c * 100 <= best * 85 && c < busiest(pick)) pick = tc;
+    }
+    return pick;
+}
+
+// Column tiles (= slots per row that a RES call writes) of the fused kernel for N columns.
+extern "C" int bn_skinny_gemm_fused_tiles(int N) {
+    if (N < 1) return 0;
+    const int tc = sk_fused_tile_cols(N);
+    return (N + tc - 1) / tc;
+}
+
 // X, W, Y as bn_skinny_gemm with a bf16 result and M <= 16; glu8 as dual == 2 there.
 // slots_in != null (PRE): X is a stream's bf16 copy as a RES call leaves it, slots_in [M, n_slots] its rows'
 // sums of squares in parts, stream_width its number of columns; the result's rows are scaled by
 // 1/sqrt(sum / stream_width + eps).
 // resid != null (RES): the product is added to resid [M, N] in place; resid_bf16 [M, N] becomes the new stream
-// times next_weight [N], slots_out [M, (N + 15) / 16] the sums of squares of its groups of 16 columns (glu8 == 0, no Y).
+// times next_weight [N], slots_out [M, bn_skinny_gemm_fused_tiles(N)] the sums of squares of its column tiles
+// (glu8 == 0, no Y).
 extern "C" int bn_skinny_gemm_fused(const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw, int ldy,
                                     int glu8, const float* slots_in, int n_slots, int stream_width, float eps,
                                     float* resid, int ld_resid, void* resid_bf16, int ld_rb, const float* next_weight,
@@ -287,14 +328,16 @@ extern "C" int bn_skinny_gemm_fused(const void* X, const void* W, void* Y, int M
     f.resid = resid; f.resid_bf16 = (bf16*)resid_bf16; f.next_weight = next_weight; f.slots_out = slots_out;
     f.ld_resid = ld_resid; f.ld_rb = ld_rb;
     const size_t smem = (size_t)(8 * 256 + 16) * sizeof(float) + (size_t)8 * M * SK_XROW;
-    const dim3 grid((N + 15) / 16), block(8 * 64);
+    const int tile_cols = glu8 ? 16 : sk_fused_tile_cols(N);
+    const dim3 grid((N + tile_cols - 1) / tile_cols), block(8 * 64);
     auto go = [&](auto kernel) {
         if (smem > 64 * 1024) {
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e != hipSuccess) return (int)e;
         }
-        hipLaunchKernelGGL(kernel, grid, block, smem, s, (const bf16*)X, (const bf16*)W, (bf16*)Y, M, N, K, ldx, ldw, ldy, f);
+        hipLaunchKernelGGL(kernel, grid, block, smem, s, (const bf16*)X, (const bf16*)W, (bf16*)Y, M, N, K, ldx, ldw, ldy,
+                           tile_cols, f);
         return bn_launch_status();
     };
     const bool few = n_slots <= 256;                  // four slot loads per row and lane are enough

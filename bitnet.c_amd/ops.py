@@ -64,6 +64,7 @@ _SIGNATURES = {
         "bn_skinny_gemm_supports": [c_int, c_int, c_int, c_int, c_int],
         "bn_skinny_gemm": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                            c_int, c_void_p],
+        "bn_skinny_gemm_fused_tiles": [c_int],
         "bn_skinny_gemm_fused": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                  c_void_p, c_int, c_int, c_float, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                  c_void_p],
@@ -454,9 +455,14 @@ def linear_swiglu_prenorm(pre: DeferredNorm, w_gate_up: torch.Tensor) -> torch.T
     return y
 
 
+def _fused_tiles(N: int) -> int:
+    """Column tiles of the fused product kernel for N columns: one partial sum of squares per row and tile."""
+    return int(_fn("skinny_gemm", "bn_skinny_gemm_fused_tiles")(int(N)))
+
+
 def can_defer_norm(M: int, N: int, K: int, dtype) -> bool:
     """Whether linear_into_stream takes a product of these sizes (N is the stream's width)."""
-    return FUSE_NORMS and can_fuse_norm(M, N, K, dtype) and (N + 15) // 16 <= FUSED_SLOTS
+    return FUSE_NORMS and can_fuse_norm(M, N, K, dtype) and _fused_tiles(N) <= FUSED_SLOTS
 
 
 def linear_into_stream(x: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, weight: torch.Tensor,
@@ -477,7 +483,7 @@ def linear_into_stream(x: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, w
     if not can_defer_norm(M, N, K, torch.bfloat16) or x.data_ptr() % 16 or w.data_ptr() % 16:
         raise KernelError(f"linear_into_stream: {M} rows, w {tuple(w.shape)} cannot be fused")
     scaled = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-    slots = torch.empty((M, (N + 15) // 16), dtype=torch.float32, device=x.device)
+    slots = torch.empty((M, _fused_tiles(N)), dtype=torch.float32, device=x.device)
     _fused_call(x, w, None, M, N, K, False, None, stream, scaled, weight, slots)
     return DeferredNorm(scaled, slots, stream, weight, float(eps))
 
