@@ -3,6 +3,7 @@
 MI355X.  One JSON line on stdout.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--shape 8b|13b|70b]
+                    [--context C] [--prompt-lens LO,HI] [--prefill-tokens T]      (further lengths; not the default record)
 
 A step is one decode step of the whole batch: the step function, greedy sampling on the
 device and the read-back of the tokens, as generation does it.  `value` is decoded
@@ -61,6 +62,9 @@ def main() -> int:
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="for profiling: run one phase alone (the record then lacks the other)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--context", type=int, default=0, help="longest sequence (default: the shape's)")
+    ap.add_argument("--prompt-lens", default=None, metavar="LO,HI", help="prompt lengths of the decode batches")
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS, help="tokens of the measured prompt step")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -77,6 +81,10 @@ def main() -> int:
     dev = "cuda:0"
     shape = SHAPES[args.shape]
     SHAPE, CONTEXT, (len_lo, len_hi) = shape["config"], shape["context"], shape["prompt_lens"]
+    if args.prompt_lens:
+        len_lo, len_hi = (int(v) for v in args.prompt_lens.split(","))
+    CONTEXT = args.context or max(CONTEXT, len_hi + args.steps + args.warmup + 1, args.prefill_tokens)
+    PREFILL = args.prefill_tokens
     args.layers = args.layers or SHAPE["num_hidden_layers"]
     raw = dict(SHAPE, num_hidden_layers=args.layers)
     cfg = bn.LlamaConfig.from_dict(raw)
@@ -92,7 +100,7 @@ def main() -> int:
 
     max_batch = max(args.batch, 1 if args.no_points else 64)
     per_seq = ((len_hi + args.steps + args.warmup + 64 + 63) // 64) * 64
-    engine = bn.Engine(model, max_tokens=max(max_batch * per_seq, 4096), max_seq_len=CONTEXT)
+    engine = bn.Engine(model, max_tokens=max(max_batch * per_seq, 4096, PREFILL + 64), max_seq_len=CONTEXT)
     L, H, Hkv, hs = cfg.num_hidden_layers, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
     kv_bytes_per_token = 2 * L * Hkv * hs * 2
     weight_bytes = model.weight_bytes() - (0 if cfg.tie_word_embeddings else model.embedding.numel() * 2)
@@ -117,10 +125,10 @@ def main() -> int:
     if args.only == "decode":
         p_ms = float("nan")
     else:
-        prefill_once(PREFILL_TOKENS)
-        prefill_once(PREFILL_TOKENS)
-        p_ms = sorted(prefill_once(PREFILL_TOKENS) for _ in range(5))[2] * 1e3
-    T = PREFILL_TOKENS
+        prefill_once(PREFILL)
+        prefill_once(PREFILL)
+        p_ms = sorted(prefill_once(PREFILL) for _ in range(5))[2] * 1e3
+    T = PREFILL
     lin_params = L * (cfg.hidden_size * (cfg.q_dim + 2 * cfg.kv_dim) + cfg.q_dim * cfg.hidden_size
                       + 3 * cfg.hidden_size * cfg.intermediate_size)
     flops = 2.0 * T * lin_params + 4.0 * T * T * hs * H * L / 2 + 2.0 * cfg.vocab_size * cfg.hidden_size
@@ -186,7 +194,7 @@ def main() -> int:
                    "vocab": cfg.vocab_size, "rope_theta": cfg.rope_theta, "rope_scaling": "llama3 f8 l1 h4 o8192" if cfg.rope_scaling else "none",
                    "rms_norm_eps": cfg.rms_norm_eps, "tied": cfg.tie_word_embeddings,
                    "global_batch": args.batch, "seq_len": CONTEXT, "prompt_lens": f"U[{len_lo},{len_hi}]",
-                   "prefill_tokens": PREFILL_TOKENS, "parallelism": "none (1 GPU)"},
+                   "prefill_tokens": PREFILL, "parallelism": "none (1 GPU)"},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBS, 4)},

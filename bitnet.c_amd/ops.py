@@ -90,13 +90,27 @@ def _fn(lib: str, name: str):
     return f
 
 
+_gpu_seen = False
+
+
 def require_gpu() -> None:
+    global _gpu_seen
+    if _gpu_seen:                      # asked before every launch: a GPU that was there stays
+        return
     if not torch.cuda.is_available():
         raise KernelError("no GPU: the kernels of this library are HIP code for gfx950 and there is "
                           "no CPU implementation behind them")
+    _gpu_seen = True
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _stream() -> int:
+    """The current HIP stream's handle (it changes under a graph capture, so it is asked for at every launch; the
+    raw query costs a fraction of building a torch.cuda.Stream object)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
