@@ -24,7 +24,7 @@ ARCH = "gfx950"
 # -packed-fp32-ops off: hipcc otherwise forms packed float32 instructions by itself
 FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
-SOURCES = ("elementwise", "rope_kv", "attn_rows", "attn_mfma", "gemm_tiled", "gemm_mfma", "skinny_gemm", "sampling")
+SOURCES = ("elementwise", "rope_kv", "attn_rows", "attn_mfma", "gemm_tiled", "gemm_mfma", "skinny_gemm", "splitk_gemm", "sampling")
 HEADERS = ("common.h",)
 
 _libs = {}

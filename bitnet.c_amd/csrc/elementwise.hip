@@ -25,20 +25,23 @@ __global__ void embed_gather_kernel(float* __restrict__ x, const T* __restrict__
 //   out[r] = s * rsqrt(mean(s^2) + eps) * w     (src/transformer/rmsnorm_scalar.c:4-13;
 //   the fused add is the reference's residual_rmsnorm, src/gpu_cuda.cu:5077)
 // The sum of squares is float32: per thread in index order, then a fixed tree.
-template <typename T>
-__global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta,
+// delta may come as n_parts slabs (part_stride elements apart) that are added in slab order: the partial sums of
+// a product whose K was split over workgroups (splitk_gemm.hip); TD is the slabs' type.
+template <typename T, typename TD>
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta, int n_parts, size_t part_stride,
                                    const float* __restrict__ w, T* __restrict__ out,
                                    const int* __restrict__ rows, int dim, float eps) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const int src = rows ? rows[r] : r;
     float* xr = x + (size_t)src * dim;
-    const T* dr = delta ? delta + (size_t)src * dim : nullptr;
+    const TD* dr = delta ? delta + (size_t)src * dim : nullptr;
     const bool write_back = (dr != nullptr) && (rows == nullptr);
     float ss = 0.f;
     for (int i = threadIdx.x; i < dim; i += blockDim.x) {
         float v = xr[i];
-        if (dr) v += to_f32(dr[i]);
+        if (dr)
+            for (int p = 0; p < n_parts; ++p) v += to_f32(dr[p * part_stride + i]);
         if (write_back) xr[i] = v;
         ss += v * v;
     }
@@ -47,7 +50,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ 
     T* o = out + (size_t)r * dim;
     for (int i = threadIdx.x; i < dim; i += blockDim.x) {
         float v = xr[i];
-        if (dr && !write_back) v += to_f32(dr[i]);
+        if (dr && !write_back)
+            for (int p = 0; p < n_parts; ++p) v += to_f32(dr[p * part_stride + i]);
         o[i] = from_f32<T>(v * scale * w[i]);
     }
 }
@@ -55,15 +59,16 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ 
 // The same for rows of up to 256*4*NV elements (a multiple of 4): every load of the row is
 // issued before anything waits, the row stays in registers, one block reduction, one store.
 // Each thread's partial sum runs over its elements in index order; the tree is the same as above.
-template <typename T, int NV>
-__global__ __launch_bounds__(256) void add_rmsnorm_row_kernel(float* __restrict__ x, const T* __restrict__ delta,
+template <typename T, typename TD, int NV>
+__global__ __launch_bounds__(256) void add_rmsnorm_row_kernel(float* __restrict__ x, const TD* __restrict__ delta,
+                                                              int n_parts, size_t part_stride,
                                                               const float* __restrict__ w, T* __restrict__ out,
                                                               const int* __restrict__ rows, int dim, float eps) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const int src = rows ? rows[r] : r;
     float* xr = x + (size_t)src * dim;
-    const T* dr = delta ? delta + (size_t)src * dim : nullptr;
+    const TD* dr = delta ? delta + (size_t)src * dim : nullptr;
     const bool write_back = (dr != nullptr) && (rows == nullptr);
     float4 v[NV], wv[NV];
 #pragma unroll
@@ -77,19 +82,22 @@ __global__ __launch_bounds__(256) void add_rmsnorm_row_kernel(float* __restrict_
         }
     }
     if (dr) {
+#pragma unroll 4
+        for (int p = 0; p < n_parts; ++p, dr += part_stride) {       // several slabs' loads in flight at once
 #pragma unroll
-        for (int k = 0; k < NV; ++k) {
-            const int i = (k * 256 + threadIdx.x) * 4;
-            if (i < dim) {
-                float d[4];
-                if (sizeof(T) == 2) {
-                    const uint2 t = *reinterpret_cast<const uint2*>(dr + i);
-                    d[0] = bf16lo_to_f32(t.x); d[1] = bf16hi_to_f32(t.x); d[2] = bf16lo_to_f32(t.y); d[3] = bf16hi_to_f32(t.y);
-                } else {
-                    const float4 t = *reinterpret_cast<const float4*>(dr + i);
-                    d[0] = t.x; d[1] = t.y; d[2] = t.z; d[3] = t.w;
+            for (int k = 0; k < NV; ++k) {
+                const int i = (k * 256 + threadIdx.x) * 4;
+                if (i < dim) {
+                    float d[4];
+                    if (sizeof(TD) == 2) {
+                        const uint2 t = *reinterpret_cast<const uint2*>(dr + i);
+                        d[0] = bf16lo_to_f32(t.x); d[1] = bf16hi_to_f32(t.x); d[2] = bf16lo_to_f32(t.y); d[3] = bf16hi_to_f32(t.y);
+                    } else {
+                        const float4 t = *reinterpret_cast<const float4*>(dr + i);
+                        d[0] = t.x; d[1] = t.y; d[2] = t.z; d[3] = t.w;
+                    }
+                    v[k].x += d[0]; v[k].y += d[1]; v[k].z += d[2]; v[k].w += d[3];
                 }
-                v[k].x += d[0]; v[k].y += d[1]; v[k].z += d[2]; v[k].w += d[3];
             }
         }
     }
@@ -121,11 +129,69 @@ __global__ __launch_bounds__(256) void add_rmsnorm_row_kernel(float* __restrict_
     }
 }
 
+// The same sum and norm for many slabs in two launches that use the whole chip (one workgroup a row, as above, has a
+// CU pull all slabs of its row alone): first x += the slabs in slab order, 1,024 columns of a row per workgroup, and
+// the sum of squares of each such piece to ssq[row][piece]; then the norm from those sums (pieces added in order).
+#define SP_PIECE 1024
+__global__ __launch_bounds__(256) void sum_parts_kernel(float* __restrict__ x, const float* __restrict__ parts, int n_parts,
+                                                        size_t part_stride, float* __restrict__ ssq, int dim) {
+    __shared__ float scratch[16];
+    const int row = blockIdx.y, i = blockIdx.x * SP_PIECE + threadIdx.x * 4;
+    const bool in = i < dim;                                  // dim is a multiple of 4
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (in) {
+        float* xr = x + (size_t)row * dim + i;
+        const float* pr = parts + (size_t)row * dim + i;
+        v = *reinterpret_cast<const float4*>(xr);
+#pragma unroll 8
+        for (int p = 0; p < n_parts; ++p) {
+            const float4 d = *reinterpret_cast<const float4*>(pr + (size_t)p * part_stride);
+            v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+        }
+        *reinterpret_cast<float4*>(xr) = v;
+    }
+    float ss = 0.f;
+    ss += v.x * v.x; ss += v.y * v.y; ss += v.z * v.z; ss += v.w * v.w;
+    ss = block_sum(ss, scratch);
+    if (threadIdx.x == 0) ssq[(size_t)row * gridDim.x + blockIdx.x] = ss;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_ssq_kernel(const float* __restrict__ x, const float* __restrict__ ssq,
+                                                          int n_pieces, const float* __restrict__ w, T* __restrict__ out,
+                                                          int dim, float eps) {
+    const int row = blockIdx.x;
+    float ss = 0.f;
+    for (int p = 0; p < n_pieces; ++p) ss += ssq[(size_t)row * n_pieces + p];
+    const float scale = 1.0f / sqrtf(ss / (float)dim + eps);
+    const float* xr = x + (size_t)row * dim;
+    T* o = out + (size_t)row * dim;
+    for (int i = threadIdx.x * 4; i < dim; i += 1024) {
+        const float4 v = *reinterpret_cast<const float4*>(xr + i), wv = *reinterpret_cast<const float4*>(w + i);
+        const float a = v.x * scale * wv.x, b = v.y * scale * wv.y, c = v.z * scale * wv.z, d = v.w * scale * wv.w;
+        if (sizeof(T) == 2) {
+            bf16 t[4] = {from_f32<bf16>(a), from_f32<bf16>(b), from_f32<bf16>(c), from_f32<bf16>(d)};
+            *reinterpret_cast<uint2*>(o + i) = *reinterpret_cast<const uint2*>(t);
+        } else {
+            *reinterpret_cast<float4*>(o + i) = make_float4(a, b, c, d);
+        }
+    }
+}
+
 // x[t, :] += delta[t, :]   (src/transformer/cpu_backend.c:252-256)
 template <typename T>
 __global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__ delta, size_t n) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) x[i] += to_f32(delta[i]);
+}
+
+// x += the n_parts float32 slabs of n elements each, in slab order
+__global__ void residual_add_parts_kernel(float* __restrict__ x, const float* __restrict__ parts, int n_parts, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float v = x[i];
+    for (int p = 0; p < n_parts; ++p) v += parts[(size_t)p * n + i];
+    x[i] = v;
 }
 
 // out[t, f] = silu(gu[t, f]) * gu[t, F + f], silu(g) = g / (1 + exp(-g))
@@ -188,13 +254,14 @@ extern "C" int bn_embed_gather(int dtype, void* x, const void* table, const int*
     return BN_ERR_DTYPE;
 }
 
-template <typename T>
+template <typename T, typename TD = T>
 static void launch_add_rmsnorm(float* x, const void* delta, const float* w, void* out, const int* rows, int n_rows,
-                               int dim, float eps, hipStream_t s) {
-    const bool aligned = dim % 4 == 0 && !(((uintptr_t)x | (uintptr_t)w | (uintptr_t)out | (uintptr_t)delta) & 15);
+                               int dim, float eps, hipStream_t s, int n_parts = 1, size_t part_stride = 0) {
+    const bool aligned = dim % 4 == 0 && part_stride % 4 == 0 &&
+                         !(((uintptr_t)x | (uintptr_t)w | (uintptr_t)out | (uintptr_t)delta) & 15);
     const int nv = (dim + 1023) / 1024;
     if (aligned && nv <= 8) {
-#define ROW_CASE(NV) hipLaunchKernelGGL((add_rmsnorm_row_kernel<T, NV>), dim3(n_rows), dim3(256), 0, s, x, (const T*)delta, w, (T*)out, rows, dim, eps)
+#define ROW_CASE(NV) hipLaunchKernelGGL((add_rmsnorm_row_kernel<T, TD, NV>), dim3(n_rows), dim3(256), 0, s, x, (const TD*)delta, n_parts, part_stride, w, (T*)out, rows, dim, eps)
         switch (nv) {
             case 1: ROW_CASE(1); break;
             case 2: ROW_CASE(2); break;
@@ -205,8 +272,8 @@ static void launch_add_rmsnorm(float* x, const void* delta, const float* w, void
         return;
     }
     const int threads = dim >= 2048 ? 512 : 256;
-    hipLaunchKernelGGL(add_rmsnorm_kernel<T>, dim3(n_rows), dim3(threads), 0, s, x, (const T*)delta, w, (T*)out, rows,
-                       dim, eps);
+    hipLaunchKernelGGL((add_rmsnorm_kernel<T, TD>), dim3(n_rows), dim3(threads), 0, s, x, (const TD*)delta, n_parts, part_stride,
+                       w, (T*)out, rows, dim, eps);
 }
 
 extern "C" int bn_add_rmsnorm(int dtype, void* x, const void* delta, const float* w, void* out,
@@ -215,6 +282,45 @@ extern "C" int bn_add_rmsnorm(int dtype, void* x, const void* delta, const float
     if (dtype == BN_DT_F32) launch_add_rmsnorm<float>((float*)x, delta, w, out, rows, n_rows, dim, eps, s);
     else if (dtype == BN_DT_BF16) launch_add_rmsnorm<bf16>((float*)x, delta, w, out, rows, n_rows, dim, eps, s);
     else return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+// The same with delta given as n_parts float32 slabs [n_parts][total_rows][dim] that are added in slab order
+// (total_rows: the rows of x, which the slabs match).
+extern "C" int bn_add_rmsnorm_parts(int dtype, void* x, const float* parts, int n_parts, int total_rows, const float* w,
+                                    void* out, const int* rows, int n_rows, int dim, float eps, hipStream_t s) {
+    if (n_rows <= 0 || dim <= 0 || n_parts < 1 || total_rows < 1 || !parts) return BN_ERR_ARG;
+    const size_t stride = (size_t)total_rows * dim;
+    if (dtype == BN_DT_F32) launch_add_rmsnorm<float, float>((float*)x, parts, w, out, rows, n_rows, dim, eps, s, n_parts, stride);
+    else if (dtype == BN_DT_BF16) launch_add_rmsnorm<bf16, float>((float*)x, parts, w, out, rows, n_rows, dim, eps, s, n_parts, stride);
+    else return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+// Pieces of a row (= floats of ssq per row) that bn_add_rmsnorm_parts_wide wants for rows of dim elements
+extern "C" int bn_add_rmsnorm_parts_pieces(int dim) { return dim > 0 ? (dim + SP_PIECE - 1) / SP_PIECE : 0; }
+
+// x[total_rows, dim] += the n_parts slabs, all rows normed into out (no row selection); ssq: total_rows x pieces floats of
+// work space.  dim a multiple of 4, everything 16-byte aligned.
+extern "C" int bn_add_rmsnorm_parts_wide(int dtype, void* x, const float* parts, int n_parts, int total_rows, const float* w,
+                                         void* out, float* ssq, int dim, float eps, hipStream_t s) {
+    if (dim <= 0 || dim % 4 || n_parts < 1 || total_rows < 1 || total_rows > 65535 || !parts || !ssq) return BN_ERR_ARG;
+    if (((uintptr_t)x | (uintptr_t)parts | (uintptr_t)w | (uintptr_t)out) & 15) return BN_ERR_ARG;
+    if (dtype != BN_DT_F32 && dtype != BN_DT_BF16) return BN_ERR_DTYPE;
+    const int pieces = bn_add_rmsnorm_parts_pieces(dim);
+    hipLaunchKernelGGL(sum_parts_kernel, dim3(pieces, total_rows), dim3(256), 0, s, (float*)x, parts, n_parts,
+                       (size_t)total_rows * dim, ssq, dim);
+    if (dtype == BN_DT_F32)
+        hipLaunchKernelGGL(rmsnorm_ssq_kernel<float>, dim3(total_rows), dim3(256), 0, s, (const float*)x, ssq, pieces, w, (float*)out, dim, eps);
+    else
+        hipLaunchKernelGGL(rmsnorm_ssq_kernel<bf16>, dim3(total_rows), dim3(256), 0, s, (const float*)x, ssq, pieces, w, (bf16*)out, dim, eps);
+    return bn_launch_status();
+}
+
+extern "C" int bn_residual_add_parts(void* x, const float* parts, int n_parts, long long n, hipStream_t s) {
+    if (n <= 0 || n_parts < 1 || !parts) return BN_ERR_ARG;
+    hipLaunchKernelGGL(residual_add_parts_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (float*)x, parts, n_parts,
+                       (size_t)n);
     return bn_launch_status();
 }
 

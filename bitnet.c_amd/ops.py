@@ -30,6 +30,12 @@ _SIGNATURES = {
         "bn_embed_gather": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "bn_add_rmsnorm": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p],
         "bn_residual_add": [c_int, c_void_p, c_void_p, c_longlong, c_void_p],
+        "bn_add_rmsnorm_parts": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                 c_float, c_void_p],
+        "bn_residual_add_parts": [c_void_p, c_void_p, c_int, c_longlong, c_void_p],
+        "bn_add_rmsnorm_parts_pieces": [c_int],
+        "bn_add_rmsnorm_parts_wide": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_float,
+                                      c_void_p],
         "bn_swiglu": [c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "bn_bias_add": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
     },
@@ -68,6 +74,11 @@ _SIGNATURES = {
         "bn_skinny_gemm_fused": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                  c_void_p, c_int, c_int, c_float, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                  c_void_p],
+    },
+    "splitk_gemm": {
+        "bn_splitk_gemm_supports": [c_int, c_int, c_int, c_int, c_int],
+        "bn_splitk_gemm_splits": [c_int, c_int],
+        "bn_splitk_gemm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "sampling": {
         "bn_argmax": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
@@ -176,7 +187,11 @@ def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor, eps: float, out_dt
     T, D = x.shape
     if not x.is_contiguous() or weight.numel() != D or not weight.is_contiguous():
         raise KernelError(f"add_rmsnorm: x {tuple(x.shape)} must be contiguous and weight have {D} elements")
-    if delta is not None:
+    parts = delta if isinstance(delta, PartialSums) else None
+    if parts is not None:
+        if parts.shape != x.shape:
+            raise KernelError(f"add_rmsnorm: partial sums {tuple(parts.shape)} do not match x {tuple(x.shape)}")
+    elif delta is not None:
         _dev(delta, "delta", out_dtype, 2)
         if delta.shape != x.shape or not delta.is_contiguous():
             raise KernelError(f"add_rmsnorm: delta {tuple(delta.shape)} does not match x {tuple(x.shape)}")
@@ -189,6 +204,19 @@ def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor, eps: float, out_dt
     out = torch.empty((n, D), dtype=out_dtype, device=x.device)
     if n == 0:
         return out
+    if parts is not None and rows is None and D % 4 == 0 and parts.slabs.shape[0] > 2 and T <= 65535:
+        # many slabs: the sum over the whole chip first, then the norm (one workgroup a row would pull all of its slabs alone)
+        ssq = torch.empty((T, _fn("elementwise", "bn_add_rmsnorm_parts_pieces")(D)), dtype=torch.float32, device=x.device)
+        _check(_fn("elementwise", "bn_add_rmsnorm_parts_wide")(_code(out_dtype), x.data_ptr(), parts.slabs.data_ptr(),
+                                                               parts.slabs.shape[0], T, weight.data_ptr(), out.data_ptr(),
+                                                               ssq.data_ptr(), D, float(eps), _stream()), "add_rmsnorm")
+        return out
+    if parts is not None:
+        _check(_fn("elementwise", "bn_add_rmsnorm_parts")(_code(out_dtype), x.data_ptr(), parts.slabs.data_ptr(),
+                                                          parts.slabs.shape[0], T, weight.data_ptr(), out.data_ptr(),
+                                                          rows.data_ptr() if rows is not None else None,
+                                                          n, D, float(eps), _stream()), "add_rmsnorm")
+        return out
     _check(_fn("elementwise", "bn_add_rmsnorm")(_code(out_dtype), x.data_ptr(),
                                                 delta.data_ptr() if delta is not None else None,
                                                 weight.data_ptr(), out.data_ptr(),
@@ -197,9 +225,16 @@ def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor, eps: float, out_dt
     return out
 
 
-def residual_add(x: torch.Tensor, delta: torch.Tensor) -> None:
+def residual_add(x: torch.Tensor, delta) -> None:
+    """x (float32) += delta (a tensor of x's shape, or PartialSums)."""
     require_gpu()
     _dev(x, "x", torch.float32)
+    if isinstance(delta, PartialSums):
+        if tuple(delta.shape) != tuple(x.shape) or not x.is_contiguous():
+            raise KernelError("residual_add: partial sums do not match x, or x is not contiguous")
+        _check(_fn("elementwise", "bn_residual_add_parts")(x.data_ptr(), delta.slabs.data_ptr(), delta.slabs.shape[0],
+                                                           x.numel(), _stream()), "residual_add")
+        return
     _dev(delta, "delta")
     if x.shape != delta.shape or not x.is_contiguous() or not delta.is_contiguous():
         raise KernelError("residual_add: shapes differ or tensors are not contiguous")
@@ -380,6 +415,51 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = 
 # decode products with the neighbouring RMSNorm folded in
 # --------------------------------------------------------------------------------------
 # Set False (or BITNET_NO_FUSED_NORM=1) to keep every norm a kernel of its own.
+SPLIT_SUMS = os.environ.get("BITNET_NO_SPLIT_SUMS", "") in ("", "0")
+SPLIT_SUM_ROWS = (17, 128)      # rows for which a product that ends a part is left as partial sums
+
+
+@dataclass
+class PartialSums:
+    """A product that is still a sum to be formed: `slabs` [S, M, N] float32, the products over S ranges of K
+    (splitk_gemm).  add_rmsnorm and residual_add take it in place of a delta and add the slabs in order."""
+    slabs: torch.Tensor
+
+    @property
+    def shape(self):
+        return self.slabs.shape[1:]
+
+    @property
+    def device(self):
+        return self.slabs.device
+
+
+def can_split_sums(M: int, N: int, K: int, dtype) -> bool:
+    """Whether a product of these sizes whose result goes to the residual stream is done as partial sums."""
+    return (SPLIT_SUMS and dtype == torch.bfloat16 and SPLIT_SUM_ROWS[0] <= M <= SPLIT_SUM_ROWS[1] and K % 8 == 0
+            and K >= 8 and N >= 1)
+
+
+def linear_partial_sums(x: torch.Tensor, w: torch.Tensor) -> PartialSums:
+    """x [M, K] . w[N, K]^T as float32 partial sums over ranges of K (bf16 operands, 1 to 128 rows)."""
+    require_gpu()
+    _dev(x, "x", torch.bfloat16, 2)
+    _dev(w, "w", torch.bfloat16, 2)
+    ldx, ldw = _rows(x, "x"), _rows(w, "w")
+    M, K = x.shape
+    N = w.shape[0]
+    if w.shape[1] != K:
+        raise KernelError(f"linear_partial_sums: x {tuple(x.shape)} and w {tuple(w.shape)} do not fit")
+    if not _fn("splitk_gemm", "bn_splitk_gemm_supports")(M, N, K, ldx, ldw) or (x.data_ptr() | w.data_ptr()) % 16:
+        raise KernelError(f"linear_partial_sums: the kernel takes 1 to 128 rows, K a multiple of 8 and 16-byte aligned "
+                          f"operands, not x {tuple(x.shape)} (row stride {ldx}), w {tuple(w.shape)} (row stride {ldw})")
+    S = _fn("splitk_gemm", "bn_splitk_gemm_splits")(N, K)
+    slabs = torch.empty((S, M, N), dtype=torch.float32, device=x.device)
+    _check(_fn("splitk_gemm", "bn_splitk_gemm")(x.data_ptr(), w.data_ptr(), slabs.data_ptr(), M, N, K, ldx, ldw, S,
+                                                _stream()), "splitk_gemm")
+    return PartialSums(slabs)
+
+
 FUSE_NORMS = os.environ.get("BITNET_NO_FUSED_NORM", "") in ("", "0")
 FUSED_ROWS = 16           # rows the fused products take (one MFMA tile of activations)
 FUSED_SLOTS = 512         # column tiles of 16 whose sums of squares a consumer adds up: streams up to 8,192 wide

@@ -154,7 +154,7 @@ class ResidualStream:
 
     def __init__(self, x: torch.Tensor):
         self.x = x
-        self.pending = None                      # a tensor, a LazyDelta or None
+        self.pending = None                      # a tensor, a LazyDelta, ops.PartialSums or None
 
     def add(self, delta) -> None:
         if self.pending is not None:
@@ -183,7 +183,11 @@ class ResidualStream:
             if deferred is not None:
                 self.pending = None
                 return deferred
-        h = norm.apply(self.x, self._pending_tensor(), out_dtype, rows)
+        delta = self._pending_tensor()
+        if delta is not None and not isinstance(delta, torch.Tensor) and not getattr(norm, "takes_partial_sums", False):
+            self.flush()                         # partial sums, and a norm that only knows tensors: add them up first
+            delta = None
+        h = norm.apply(self.x, delta, out_dtype, rows)
         if rows is None:
             self.pending = None
         return h

@@ -31,13 +31,17 @@ class Linear:
         return y
 
     def lazy(self, x: torch.Tensor):
-        """The product as a LazyDelta when it could add itself to a residual stream (decode sizes, bf16, no
-        bias), else its result."""
+        """The product in the form in which it reaches a residual stream cheapest (bf16, no bias): a LazyDelta at
+        decode sizes, where it can add itself to the stream; partial sums over ranges of K (ops.PartialSums) at up
+        to 128 rows, which the kernel of the next norm adds up; else its result."""
         from .base import LazyDelta
         M, (N, K) = x.shape[0], self.weight.shape
-        if (self.bias is None and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16
-                and ops.can_defer_norm(M, N, K, x.dtype) and x.data_ptr() % 16 == 0):
+        plain = (self.bias is None and x.dim() == 2 and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16
+                 and x.data_ptr() % 16 == 0 and self.weight.data_ptr() % 16 == 0)
+        if plain and ops.can_defer_norm(M, N, K, x.dtype):
             return LazyDelta(x, self)
+        if plain and ops.can_split_sums(M, N, K, x.dtype) and x.stride(1) == 1 and x.stride(0) % 8 == 0:
+            return ops.linear_partial_sums(x, self.weight)
         return self(x)
 
     def into_stream(self, x: torch.Tensor, stream: torch.Tensor, norm_weight: torch.Tensor, eps: float):

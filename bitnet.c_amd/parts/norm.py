@@ -12,6 +12,7 @@ from .base import NORMS, ParamSpec, Part
 @NORMS.register("rmsnorm")
 class RMSNorm(Part):
     deferrable = True        # a product may fold this norm around itself (weight and eps are all it needs)
+    takes_partial_sums = True    # apply() accepts ops.PartialSums as the delta
 
     def __init__(self, dim: int, eps: float):
         self.dim, self.eps = int(dim), float(eps)

@@ -197,6 +197,61 @@ def test_products_with_the_norm_folded_in_refuse_what_they_cannot_take():
                                torch.zeros(64, 64, dtype=torch.bfloat16, device="cuda"), x, torch.ones(64, device="cuda"), 1e-5)
 
 
+@pytest.mark.parametrize("M", [1, 17, 33, 64, 100, 128])
+@pytest.mark.parametrize("N,K", [(4096, 4096), (200, 328), (72, 1000), (136, 16), (264, 3592)])
+def test_products_left_as_partial_sums(M, N, K):
+    """A product that ends a part at 17 to 128 rows: float32 partial sums over ranges of K, which the kernel of the
+    next norm (or the plain add) adds to the stream in slab order.  The sums are exact up to their order; the norm
+    is the plain formula on the sum."""
+    ops = _ops()
+    eps = 1e-6
+    x, w = _rand((M, K), torch.bfloat16, 41), _rand((N, K), torch.bfloat16, 42, 0.05)
+    stream = _rand((M, N), torch.float32, 43, 2.0)
+    norm_w = _rand((N,), torch.float32, 44) * 0.2 + 1.0
+    ref = x.double() @ w.double().t()
+    assert ops.can_split_sums(M, N, K, torch.bfloat16) == (17 <= M <= 128)
+    parts = ops.linear_partial_sums(x.cuda(), w.cuda())
+    assert parts.slabs.dtype == torch.float32 and tuple(parts.shape) == (M, N)
+    assert rel_err(parts.slabs.sum(dim=0), ref.float()) < 1e-5
+    # rows of a larger buffer (a row stride above K), as a part's activations may come
+    xw = torch.zeros(M, K + 24, dtype=torch.bfloat16)
+    xw[:, :K] = x
+    assert torch.equal(ops.linear_partial_sums(xw.cuda()[:, :K], w.cuda()).slabs, parts.slabs)
+    want_x = stream.double() + ref
+    for out_dtype in (torch.bfloat16, torch.float32):
+        xs = stream.clone().cuda()
+        h = ops.add_rmsnorm(xs, parts, norm_w.cuda(), eps, out_dtype)
+        assert rel_err(xs, want_x.float()) < 1e-5                                  # the stream took the sum
+        assert h.dtype == out_dtype and close(h.float(), pl.rmsnorm(want_x.float(), norm_w, eps), out_dtype)
+    # only some rows normed: the stream stays as it is
+    rows = torch.tensor([M - 1, 0, M // 2], dtype=torch.int32)
+    xs = stream.clone().cuda()
+    h = ops.add_rmsnorm(xs, parts, norm_w.cuda(), eps, torch.float32, rows.cuda())
+    assert torch.equal(xs.cpu(), stream)
+    assert close(h, pl.rmsnorm(want_x.float(), norm_w, eps)[rows.long()], torch.float32)
+    xs = stream.clone().cuda()
+    ops.residual_add(xs, parts)
+    assert rel_err(xs, want_x.float()) < 1e-5
+
+
+def test_partial_sums_refuse_what_they_cannot_take():
+    ops = _ops()
+    assert not ops.can_split_sums(16, 64, 64, torch.bfloat16) and not ops.can_split_sums(129, 64, 64, torch.bfloat16)
+    assert not ops.can_split_sums(64, 64, 172, torch.bfloat16) and not ops.can_split_sums(64, 64, 64, torch.float32)
+    z = lambda *shape: torch.zeros(*shape, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ops.KernelError):
+        ops.linear_partial_sums(z(129, 64), z(64, 64))                 # more rows than the staged block holds
+    with pytest.raises(ops.KernelError):
+        ops.linear_partial_sums(z(32, 172), z(64, 172))                # K no multiple of 8
+    with pytest.raises(ops.KernelError):
+        ops.linear_partial_sums(z(32, 64), z(64, 72))                  # K of x and w differ
+    parts = ops.linear_partial_sums(z(32, 64), z(48, 64))
+    with pytest.raises(ops.KernelError):
+        ops.add_rmsnorm(torch.zeros(32, 64, device="cuda"), parts, torch.ones(64, device="cuda"), 1e-5, torch.bfloat16)
+    with pytest.raises(ops.KernelError):
+        ops.residual_add(torch.zeros(31, 48, device="cuda"), parts)
+
+
 @pytest.mark.parametrize("width", [0, 256, 192, 128])
 @pytest.mark.parametrize("M,N,K", [(65, 16, 8), (100, 200, 328), (256, 256, 64), (300, 520, 192), (777, 1000, 136),
                                    (513, 4104, 1032), (1, 31, 264)])

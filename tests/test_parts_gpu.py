@@ -74,6 +74,50 @@ def test_norm_and_feed_forward_parts(dtype):
     assert part_close(fb.forward(h.to(DEV), None).float(), want, dtype, exact)
 
 
+@pytest.mark.parametrize("T", [8, 40, 128, 200])
+def test_a_feed_forward_s_last_product_reaches_the_stream_in_every_form(T):
+    """bfloat16: at 8 rows the last product adds itself to the stream and leaves the norm deferred, at 40 and 128
+    rows it comes as partial sums over ranges of K that the kernels of the next norm add up, at 200 rows as a
+    tensor.  The stream and the normed rows are the plain formulas' in every form; a norm that knows only tensors
+    (defined here) gets the sum formed for it."""
+    from bitnet_c_amd import ops
+    from bitnet_c_amd.parts import FEED_FORWARDS, NORMS, LazyDelta, PartSpec, ResidualStream
+    dtype, D, F = torch.bfloat16, 1024, 2048                     # K = 2,048 columns of the last product: four ranges
+    ffn = FEED_FORWARDS.build(PartSpec.of("swiglu", hidden=D, intermediate=F))
+    t = {"w_gate": _rand((F, D), 3, 0.05).to(dtype), "w_up": _rand((F, D), 4, 0.05).to(dtype),
+         "w_down": _rand((D, F), 5, 0.05).to(dtype)}
+    ffn.load(t, DEV, dtype)
+    norm = NORMS.build(PartSpec.of("rmsnorm", dim=D, eps=1e-5))
+    nw = _rand((D,), 6) * 0.2 + 1.0
+    norm.load({"weight": nw}, DEV, dtype)
+    h, x0 = _rand((T, D), 7).to(dtype), _rand((T, D), 8, 2.0)
+    delta = ffn.forward(h.to(DEV), None, lazy_ok=True)
+    kind = LazyDelta if T <= 16 else ops.PartialSums if T <= 128 else torch.Tensor
+    assert isinstance(delta, kind), type(delta)
+    if kind is ops.PartialSums:
+        assert delta.slabs.shape[0] == 4
+    act = pl.swiglu(pl.linear(h.float(), t["w_gate"].float()).to(dtype).float(), pl.linear(h.float(), t["w_up"].float()).to(dtype).float())
+    exact_x = x0.double() + pl.linear(act.to(dtype).float(), t["w_down"].float()).double()
+
+    class TensorsOnlyNorm:
+        weight, eps = norm.weight, norm.eps
+
+        def apply(self, x, d, out_dtype, rows=None):
+            assert d is None or isinstance(d, torch.Tensor)
+            return ops.add_rmsnorm(x, d, self.weight, self.eps, out_dtype, rows)
+
+    for n in (norm, TensorsOnlyNorm()):
+        stream = ResidualStream(x0.clone().to(DEV))
+        stream.add(ffn.forward(h.to(DEV), None, lazy_ok=True))
+        got = stream.normed(n, dtype, consumer=None)
+        assert stream.pending is None
+        # the activations of the last product differ from the plain ones by one bf16 step here and there, and the plain
+        # path at 200 rows rounds the product to bf16 before it is added
+        assert rel_err(stream.x, exact_x.float()) < 2e-2
+        assert part_close(got.float(), pl.rmsnorm(exact_x.float(), nw, 1e-5).to(dtype).float(), dtype,
+                          pl.rmsnorm(exact_x.float(), nw, 1e-5))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,Hkv,hs,window,pos_kind", [(6, 2, 32, 0, "rope"), (4, 4, 16, 40, "rope"), (3, 1, 24, 0, "none")])
 def test_attention_part_alone(dtype, H, Hkv, hs, window, pos_kind):
