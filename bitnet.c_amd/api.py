@@ -20,6 +20,17 @@ class LLM:
     def config(self):
         return getattr(self.engine, "config", None)
 
+    # the step function under the loop, for callers that bring their own: logits [wanted, vocab] (float32) at the
+    # places that the entries (engine.StepEntry(slot, tokens, want)) ask for
+    def new_sequence(self) -> int:
+        return self.engine.new_sequence()
+
+    def step(self, entries) -> torch.Tensor:
+        return self.engine.step(entries)
+
+    def release(self, slot: int) -> None:
+        self.engine.release(slot)
+
     def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 256, temperature: float = 0.0,
                  top_p: float = 0.9, seed: int = 42, repeat_penalty: float = 1.0, stop_ids: Optional[Sequence[int]] = None,
                  batch_size: int = 8, on_token: Optional[Callable[[int, int], bool]] = None,

@@ -34,6 +34,12 @@ def test_greedy_generation_float32(model_folders, name, lengths, n_new):
     assert [llm.generate([p], max_new_tokens=n_new, stop_ids=())[0] for p in prompts] == want
     llm.engine.cache.check()
     assert not llm.engine.cache.live_slots()
+    # the step function through the entry object: the logits at a prompt's end pick the first generated token
+    slot = llm.new_sequence()
+    logits = llm.step([bn.StepEntry(slot, prompts[0], [len(prompts[0]) - 1])])
+    assert logits.shape == (1, c["vocab"]) and int(logits[0].argmax()) == want[0][0]
+    llm.release(slot)
+    assert not llm.engine.cache.live_slots()
 
 
 def test_stop_tokens_and_budgets(model_folders):
