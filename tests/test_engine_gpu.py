@@ -536,3 +536,57 @@ def test_graph_replays_of_a_wide_batch_at_the_benchmark_layer_sizes(n_seqs):
         assert float(per_row.max()) < 0.025, (k, per_row)
         sd = float(d.pow(2).mean().sqrt())                           # 0: the same kernels ran on both sides
         assert sd == 0.0 or float(d.abs().max()) / sd < 8.0, k
+
+
+# Further sizes than the tiny configurations': head sizes in steps of 16 up to 256, one to 64 heads in groups of 1 to 16,
+# widths and vocabularies that are no power of two (some no multiple of 8), one to three layers, both rope forms, tied and
+# untied, with and without biases; (head size, heads, kv heads, hidden, intermediate, vocab, layers, tied, biases, llama3
+# scaling, prompt lengths)
+FURTHER_SIZES = [
+    (112, 16, 4, 264, 264, 256, 1, False, False, False, [7, 33, 33, 33, 70]),
+    (112, 16, 1, 120, 520, 389, 2, True, False, False, [7, 70, 7, 70, 7, 19, 19, 19, 130, 7, 2, 2, 100, 1, 130, 7, 70, 70, 33, 100]),
+    (256, 3, 3, 72, 172, 1000, 3, False, False, True, [1, 2, 130]),
+    (96, 10, 2, 120, 1000, 389, 3, True, True, True, [19, 33, 100, 7, 100, 100, 130, 19, 19, 130, 1, 33, 33, 130, 130, 70, 2, 2, 19, 130]),
+    (80, 64, 8, 64, 328, 97, 3, True, False, False, [2, 1, 70, 7, 33, 19, 7, 7, 1, 130, 1, 19, 100, 7, 130, 2, 2, 33, 100, 19]),
+    (160, 4, 4, 72, 264, 2053, 3, True, False, True, [100]),
+    (16, 4, 4, 136, 1000, 256, 1, False, False, True, [33, 33, 7, 33, 2, 2, 130, 19, 2, 130, 2, 130, 7, 2, 70, 100, 19, 2, 130, 19]),
+    (48, 16, 8, 100, 173, 131, 2, False, False, False, [1, 40, 17]),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", range(len(FURTHER_SIZES)))
+def test_further_sizes(tmp_path, case, dtype):
+    """Unequal prompts in one step (logits at every place), then four tokens each, at sizes that the other tests
+    do not have; against the plain implementation."""
+    import bitnet_c_amd as bn
+    hs, H, Hkv, hidden, F, V, L, tied, biases, scaling, lens = FURTHER_SIZES[case]
+    raw = dict(model_type="llama", vocab_size=V, hidden_size=hidden, intermediate_size=F, num_hidden_layers=L,
+               num_attention_heads=H, num_key_value_heads=Hkv, head_dim=hs, max_position_embeddings=1024,
+               rope_theta=500000.0 if scaling else 10000.0, rms_norm_eps=1e-6 if tied else 1e-5,
+               tie_word_embeddings=tied, attention_bias=False, mlp_bias=biases)
+    if scaling:
+        raw["rope_scaling"] = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                   original_max_position_embeddings=64)
+    folder = bn.write_model_folder(str(tmp_path / "m"), bn.LlamaConfig.from_dict(raw), 100 + case, dtype)
+    c, W = pl.read_config(folder), pl.read_weights(folder)
+    eng = bn.Engine.from_folder(folder, dtype=dtype, max_tokens=max(2048, 64 * 4 * len(lens)))
+    n_dec = 4
+    reqs = _requests(V, 200 + case, [n + n_dec for n in lens])
+    slots = [eng.new_sequence() for _ in reqs]
+    got = [[] for _ in reqs]
+    lg = eng.step([bn.StepEntry(s, r[:-n_dec], list(range(len(r) - n_dec))) for s, r in zip(slots, reqs)])
+    at = 0
+    for i, r in enumerate(reqs):
+        got[i].append(lg[at:at + len(r) - n_dec])
+        at += len(r) - n_dec
+    for t in range(n_dec):
+        lg = eng.step([bn.StepEntry(s, [r[len(r) - n_dec + t]], [0]) for s, r in zip(slots, reqs)])
+        for i in range(len(reqs)):
+            got[i].append(lg[i:i + 1].clone())
+    for s in slots:
+        eng.release(s)
+    eng.cache.check()
+    for i, r in enumerate(reqs):
+        want = pl.forward(c, W, r, torch.bfloat16 if dtype == torch.bfloat16 else None)
+        assert rel_err(torch.cat(got[i]), want) < TOL[dtype], (i, len(r))
