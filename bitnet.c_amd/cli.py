@@ -38,6 +38,11 @@ def _parser() -> argparse.ArgumentParser:
     ap.add_argument("--fp32", action="store_true", help="run the whole model in float32")
     ap.add_argument("--random", default=None, metavar="CONFIG_JSON",
                     help="first write MODEL as a new folder: this configuration with random weights from --seed")
+    # switches of the reference's runtime that select what is always so here, or what this library does not have: taken so
+    # that a command line written for the reference runs, and answered with one line each (src/main.c:120-167, 268-275)
+    ap.add_argument("-t", dest="threads", type=int, default=None, help="CPU threads of the reference: no effect (one GPU)")
+    ap.add_argument("--flash", action="store_true", help="online-softmax attention: always on here")
+    ap.add_argument("--kv16", action="store_true", help="16-bit cache: always so in bfloat16; refused with --fp32")
     ap.add_argument("--batch-file", default=None, help="file with one comma-separated prompt (token ids) a line")
     ap.add_argument("--batch", type=int, default=8, help="sequences per batch with --batch-file (default 8)")
     return ap
@@ -90,9 +95,21 @@ def _check_benchmark_args(args) -> None:
         raise SystemExit("--benchmark-runs and --bench-warmup-tokens take one prompt, not --batch-file")
 
 
+def _note_reference_switches(args) -> None:
+    if args.threads is not None:
+        print("[bitnet] -t: no CPU threads to set, the model runs on one GPU", file=sys.stderr)
+    if args.flash:
+        print("[bitnet] --flash: attention is always computed with the online softmax here", file=sys.stderr)
+    if args.kv16:
+        if args.fp32:
+            raise SystemExit("--kv16 with --fp32: the float32 path keeps a float32 cache (run without --fp32 for a 16-bit one)")
+        print("[bitnet] --kv16: the bfloat16 path keeps its cache in 16 bits already", file=sys.stderr)
+
+
 def main(argv=None) -> int:
     args = _parser().parse_args(argv)
     _check_benchmark_args(args)
+    _note_reference_switches(args)
     import torch
     from . import api
     from .engine import Request, StepEntry, generate

@@ -97,12 +97,16 @@ def test_command_line(model_folders):
     want = pl.generate(c, W, prompt, 6)
     base = [sys.executable, os.path.join(ROOT, "bin", "bitnet"), folder, "--prompt-token-ids",
             ",".join(map(str, prompt)), "-n", "6", "--repeat-penalty", "1.0", "--fp32", "--token-ids", "--quiet"]
-    for extra in ([], ["--no-prefill"], ["--maxseq", "64"]):
+    # the last one: switches of the reference's runtime that are always so here are taken and answered with a line
+    for extra in ([], ["--no-prefill"], ["--maxseq", "64"], ["-t", "4", "--flash"]):
         p = subprocess.run(base + extra, capture_output=True, text=True, timeout=300)
         assert p.returncode == 0, p.stderr[-1500:]
         ids = [l for l in p.stderr.splitlines() if l and l[0].isdigit()][0]
         assert [int(x) for x in ids.split(",")] == want, extra
         assert "tok/s" in p.stderr
+        assert ("--flash" in p.stderr) == ("--flash" in extra)
+    p = subprocess.run(base + ["--kv16"], capture_output=True, text=True, timeout=300)
+    assert p.returncode != 0 and "--kv16" in p.stderr                 # a 16-bit cache and the float32 path exclude each other
     p = subprocess.run(base[:3] + ["--prompt-token-ids", "1,999"], capture_output=True, text=True, timeout=300)
     assert p.returncode != 0 and "999" in p.stderr
 
