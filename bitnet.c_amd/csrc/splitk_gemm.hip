@@ -10,29 +10,35 @@
 // through shared memory (double-buffered, one barrier a step) and read by all 8 waves.  K is split over
 // workgroups so that columns/128 x splits is about the number of CUs: a CU pulls its bytes no faster when
 // others idle, and a long chain of steps in few workgroups leaves most of the chip waiting.
+//
+// The same loop with four waves (64 columns a workgroup), K unsplit and a SwiGLU epilogue is the gate/up product of a
+// feed-forward at these row counts: W holds gate and up rows interleaved in blocks of 8, a wave's 16 columns are 8 gate
+// and 8 up columns of the same 8 outputs, out = silu(gate) * up in bf16 (src/transformer/cpu.c:1164-1304).
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
 
-#define SG_WAVES 8
-#define SG_COLS (SG_WAVES * 16)       // columns of W per workgroup
+#define SG_WAVES 8                    // waves per workgroup of the partial-sum form
+#define SG_COLS (SG_WAVES * 16)       // its columns of W per workgroup
+#define SG_GLU_WAVES 4                // waves per workgroup of the SwiGLU form
 #define SG_STEP 256                   // K per step
 #define SG_XROW 528                   // bytes of a staged row of X: 512 + 16, so that the 16 rows a read touches spread over the banks
 #define SG_MAX_ROWS 128
 
-template <int MT>
-__global__ __launch_bounds__(SG_WAVES * 64) void splitk_gemm_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
-                                                                    float* __restrict__ P, int M, int N, int K, int ldx,
-                                                                    int ldw, int k_per_split) {
+// GLU: P is unused and Y [M, N / 2] (row stride ldy) takes silu(gate) * up; else Y is unused and P takes the partial sums.
+template <int MT, int NWV, bool GLU>
+__global__ __launch_bounds__(NWV * 64) void splitk_gemm_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
+                                                               float* __restrict__ P, bf16* __restrict__ Y, int M, int N, int K,
+                                                               int ldx, int ldw, int ldy, int k_per_split) {
     extern __shared__ __align__(16) unsigned char xs[];       // [2][MT * 16][SG_XROW]
     constexpr int ROWS = MT * 16;
-    constexpr int RP = SG_WAVES * 2;                          // rows staged per pass of the workgroup (32 threads a row)
+    constexpr int RP = NWV * 2;                               // rows staged per pass of the workgroup (32 threads a row)
     constexpr int XL = (ROWS + RP - 1) / RP;                  // staging loads per thread and step
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int i = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * SG_COLS + wave * 16;
+    const int n0 = blockIdx.x * (NWV * 16) + wave * 16;
     const bf16* wrow = W + (size_t)min(n0 + i, N - 1) * ldw;
     const int k_begin = blockIdx.y * k_per_split;
     const int k_end = min(K, k_begin + k_per_split);
@@ -95,6 +101,20 @@ __global__ __launch_bounds__(SG_WAVES * 64) void splitk_gemm_kernel(const bf16* 
         __syncthreads();
     }
     // result layout: lane (i, g) holds rows 4g..4g+3 of every 16-row tile at column n0 + i
+    if (GLU) {
+        // columns n0..n0+7 are gate, n0+8..n0+15 up of outputs n0/2..n0/2+7: lane i < 8 gets its up value from lane i + 8
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float v = acc[mt][r];
+                const float up = __shfl_xor(v, 8, BN_WAVE);
+                const int m = mt * 16 + 4 * g + r;
+                if ((i & 8) == 0 && m < M && n0 + i < N)
+                    Y[(size_t)m * ldy + (n0 >> 1) + i] = __float2bfloat16((v / (1.0f + expf(-v))) * up);
+            }
+        return;
+    }
     float* out = P + (size_t)blockIdx.y * M * N;
     if (n0 + i < N) {
 #pragma unroll
@@ -157,18 +177,53 @@ extern "C" int bn_splitk_gemm(const void* X, const void* W, float* P, int M, int
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
             if (e != hipSuccess) return (int)e;
         }
-        hipLaunchKernelGGL(kernel, grid, block, smem, s, (const bf16*)X, (const bf16*)W, P, M, N, K, ldx, ldw, kps);
+        hipLaunchKernelGGL(kernel, grid, block, smem, s, (const bf16*)X, (const bf16*)W, P, (bf16*)nullptr, M, N, K, ldx, ldw, 0,
+                           kps);
         return bn_launch_status();
     };
     switch (MT) {
-        case 1: return go(splitk_gemm_kernel<1>);
-        case 2: return go(splitk_gemm_kernel<2>);
-        case 3: return go(splitk_gemm_kernel<3>);
-        case 4: return go(splitk_gemm_kernel<4>);
-        case 5: return go(splitk_gemm_kernel<5>);
-        case 6: return go(splitk_gemm_kernel<6>);
-        case 7: return go(splitk_gemm_kernel<7>);
-        case 8: return go(splitk_gemm_kernel<8>);
+        case 1: return go(splitk_gemm_kernel<1, SG_WAVES, false>);
+        case 2: return go(splitk_gemm_kernel<2, SG_WAVES, false>);
+        case 3: return go(splitk_gemm_kernel<3, SG_WAVES, false>);
+        case 4: return go(splitk_gemm_kernel<4, SG_WAVES, false>);
+        case 5: return go(splitk_gemm_kernel<5, SG_WAVES, false>);
+        case 6: return go(splitk_gemm_kernel<6, SG_WAVES, false>);
+        case 7: return go(splitk_gemm_kernel<7, SG_WAVES, false>);
+        case 8: return go(splitk_gemm_kernel<8, SG_WAVES, false>);
+    }
+    return BN_ERR_ARG;
+}
+
+// Y[M, F] (bf16, row stride ldy) = silu(X . Wg^T) * (X . Wu^T) for W [2F, K] with gate and up rows interleaved in blocks
+// of 8 (F a multiple of 8); X, W as above.
+extern "C" int bn_splitk_gemm_swiglu(const void* X, const void* W, void* Y, int M, int F, int K, int ldx, int ldw, int ldy,
+                                     hipStream_t s) {
+    if (F < 8 || F % 8 || F > (1 << 29) || !bn_splitk_gemm_supports(M, 2 * F, K, ldx, ldw) || !X || !W || !Y || ldy < F)
+        return BN_ERR_ARG;
+    if (((uintptr_t)X | (uintptr_t)W) & 15) return BN_ERR_ARG;
+    const int N = 2 * F, MT = (M + 15) / 16;
+    const int kps = (K + SG_STEP - 1) / SG_STEP * SG_STEP;
+    const dim3 grid((N + SG_GLU_WAVES * 16 - 1) / (SG_GLU_WAVES * 16), 1), block(SG_GLU_WAVES * 64);
+    const size_t smem = (size_t)2 * MT * 16 * SG_XROW;
+    auto go = [&](auto kernel) {
+        if (smem > 64 * 1024) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e != hipSuccess) return (int)e;
+        }
+        hipLaunchKernelGGL(kernel, grid, block, smem, s, (const bf16*)X, (const bf16*)W, (float*)nullptr, (bf16*)Y, M, N, K, ldx,
+                           ldw, ldy, kps);
+        return bn_launch_status();
+    };
+    switch (MT) {
+        case 1: return go(splitk_gemm_kernel<1, SG_GLU_WAVES, true>);
+        case 2: return go(splitk_gemm_kernel<2, SG_GLU_WAVES, true>);
+        case 3: return go(splitk_gemm_kernel<3, SG_GLU_WAVES, true>);
+        case 4: return go(splitk_gemm_kernel<4, SG_GLU_WAVES, true>);
+        case 5: return go(splitk_gemm_kernel<5, SG_GLU_WAVES, true>);
+        case 6: return go(splitk_gemm_kernel<6, SG_GLU_WAVES, true>);
+        case 7: return go(splitk_gemm_kernel<7, SG_GLU_WAVES, true>);
+        case 8: return go(splitk_gemm_kernel<8, SG_GLU_WAVES, true>);
     }
     return BN_ERR_ARG;
 }
