@@ -379,10 +379,10 @@ def interleave_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor) -> torch.Tensor
 
 
 # Rows at which the interleaved gate/up product with its SwiGLU epilogue is the kernel that stages the activations once
-# per 64 columns (splitk_gemm.hip): measured on the 8B shape faster than the library's product and the SwiGLU kernel after
-# it up to about 48 rows (54 us against 58 + 5 at 24 rows, 53 against 54 + 6 at 32), equal at 64.  Without the library it
-# takes every row count of the kernel.
-SWIGLU_STAGED_ROWS = (17, 48)
+# per 64 columns (splitk_gemm.hip): measured on the 8B shape against the library's product and the SwiGLU kernel after it
+# 50 us against 55 at 17 and 24 rows, 52 against 54.5 at 32, 54 against 53 at 40, 58 against 54 at 64.  Without the library
+# it takes every row count of the kernel.
+SWIGLU_STAGED_ROWS = (17, 32)
 
 
 def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = False, *,
