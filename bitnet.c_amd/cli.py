@@ -43,6 +43,13 @@ def _parser() -> argparse.ArgumentParser:
     ap.add_argument("-t", dest="threads", type=int, default=None, help="CPU threads of the reference: no effect (one GPU)")
     ap.add_argument("--flash", action="store_true", help="online-softmax attention: always on here")
     ap.add_argument("--kv16", action="store_true", help="16-bit cache: always so in bfloat16; refused with --fp32")
+    # diagnostics of the reference (src/main.c:144-147, 333-340; the text dump is its BN_DUMP_LAYER_INP)
+    ap.add_argument("--dump-binary", default=None, metavar="PATH", help="write a selected state of the residual stream as float32")
+    ap.add_argument("--dump-tag", default=None, help="which state: bitnet_inp (a layer's input), bitnet_ffn_inp, bitnet_lout")
+    ap.add_argument("--dump-layer", type=int, default=None, help="select the layer of the dumps")
+    ap.add_argument("--dump-pos", type=int, default=None, help="select the token position of the dumps")
+    ap.add_argument("--dump-stats", default=os.environ.get("BN_DUMP_LAYER_INP"), metavar="PATH",
+                    help="append a line of statistics per dumped state (default: $BN_DUMP_LAYER_INP)")
     ap.add_argument("--batch-file", default=None, help="file with one comma-separated prompt (token ids) a line")
     ap.add_argument("--batch", type=int, default=8, help="sequences per batch with --batch-file (default 8)")
     return ap
@@ -83,6 +90,45 @@ def _with_top_logits(sample_fn, k: int):
         step[0] += 1
         return sample_fn(logits, samplers)
     return fn
+
+
+DUMP_POINTS = {"layer_in": "bitnet_inp", "ffn_in": "bitnet_ffn_inp", "layer_out": "bitnet_lout"}   # src/transformer/cpu.c:401, :951, :981
+
+
+def _dump_tap(args):
+    """The engine's diagnostic tap for --dump-binary / --dump-stats: the residual stream of the selected layer
+    and position at the reference's dump points, as the float32 vector (the file is rewritten at every
+    match, as in src/transformer/cpu.c:221-229) and as the reference's line of statistics (:231-251)."""
+    if not args.dump_binary and not args.dump_stats:
+        return None
+    if args.dump_binary and not args.dump_tag:
+        raise SystemExit("--dump-binary needs --dump-tag (bitnet_inp, bitnet_ffn_inp or bitnet_lout)")
+    if args.dump_tag and args.dump_tag not in DUMP_POINTS.values():
+        raise SystemExit(f"--dump-tag: one of {', '.join(DUMP_POINTS.values())}")
+
+    def tap(point, entry, stream, ctx):
+        tag = DUMP_POINTS[point]
+        if args.dump_layer is not None and entry != args.dump_layer:
+            return
+        if not args.dump_stats and tag != args.dump_tag:
+            return
+        x = stream.flush()                              # the sum itself: a part's output is held back until the next norm
+        row = 0
+        for p0, n in zip(ctx.pos0, ctx.n_new):
+            for pos in range(p0, p0 + n):
+                if args.dump_pos is None or pos == args.dump_pos:
+                    v = x[row].float().cpu()
+                    if args.dump_binary and tag == args.dump_tag:
+                        with open(args.dump_binary, "wb") as f:
+                            f.write(v.numpy().astype("<f4").tobytes())
+                    if args.dump_stats:
+                        first = ",".join(f"{t:.9g}" for t in v[:16].tolist())
+                        with open(args.dump_stats, "a") as f:
+                            f.write(f"{tag} pos={pos} layer={entry} dim={v.numel()} sum={float(v.sum()):.9g} "
+                                    f"ss={float((v * v).sum()):.9g} min={float(v.min()):.9g} max={float(v.max()):.9g} "
+                                    f"first={first}\n")
+                row += 1
+    return tap
 
 
 def _check_benchmark_args(args) -> None:
@@ -140,6 +186,7 @@ def main(argv=None) -> int:
                    max_tokens=max(64, (max_seq or 4096) * (args.batch if args.batch_file else 1)),
                    max_seq_len=max_seq)
     eng = llm.engine
+    eng.tap = _dump_tap(args)
     vocab = eng.vocab_size
     cfg = llm.config
     if args.batch_file:

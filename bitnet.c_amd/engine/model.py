@@ -74,6 +74,7 @@ class DecoderModel:
         x = ops.embed_gather(self.embedding, ctx.tokens)          # src/model_embed.c:6-28
         stream = ResidualStream(x)
         for i, e in enumerate(self.plan.schedule):
+            ctx.entry = i
             self.blocks[e.layer].forward(stream, ctx, views[i])
         # final norm on the wanted rows only, then the output matrix (src/transformer/logits.c:249-314)
         h = stream.normed(self.final_norm, self.dtype, rows=ctx.want_rows)

@@ -51,6 +51,11 @@ class StepContext:
         self.slots, self.n_new, self.pos0 = list(slots), list(n_new), list(pos0)   # host copies
         self.n_rows = int(tokens.numel())
         self.n_seqs = len(self.slots)
+        # diagnostics: a callable (point, schedule entry, ResidualStream, ctx) that blocks call at "layer_in",
+        # "ffn_in" and "layer_out" (the reference's bitnet_inp / bitnet_ffn_inp / bitnet_lout dumps,
+        # src/transformer/cpu.c:401, :951, :981); `entry` is the schedule entry that is running
+        self.tap = None
+        self.entry = -1
         self._tiles: Dict[int, torch.Tensor] = {}
         self._page_tiles = None
 
@@ -205,6 +210,7 @@ class Engine:
         # a mixer that keeps a state addresses it by the host's slot list, which a replayed graph
         # cannot see: such models run their decode steps eagerly
         self.use_graphs = use_graphs and all(n.state is None for n in needs)
+        self.tap = None                     # see StepContext.tap; while it is set, steps run without graphs
         self._graphs: Dict[tuple, _DecodeGraph] = {}
         self.steps_run = 0
 
@@ -270,7 +276,7 @@ class Engine:
         except CacheFull as err:
             raise StepError(str(err)) from None
         is_decode = all(n == 1 for n in n_new)
-        if is_decode and self.use_graphs and len(entries) <= 64:
+        if is_decode and self.use_graphs and self.tap is None and len(entries) <= 64:
             logits = self._step_graph(entries, slots, pos0)
         else:
             logits = self._step_eager(entries, slots, n_new, pos0, is_decode)
@@ -310,6 +316,7 @@ class Engine:
         d_tables = {g: take(tables[g].numel()).view(tables[g].shape) for g in sorted(tables)}
         ctx = StepContext(dev, self.model.dtype, d_tokens, d_pos, d_seq, d_lens, d_want, d_slots, is_decode,
                           slots, n_new, pos0, by_length=d_order)
+        ctx.tap = self.tap
         max_len = max(lens_after)
         views = [self.cache.view(i, d_tables, max_len) for i in range(len(self.model.plan.schedule))]
         return self.model.forward(ctx, views)

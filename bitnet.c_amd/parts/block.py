@@ -31,13 +31,20 @@ class PreNormBlock(Part):
     def forward(self, stream, ctx, kv):
         # A part that says so may get its norm undone (it applies it inside its first product) and may hand
         # its last product in undone (it then adds itself to the stream): see ResidualStream.
+        tap = getattr(ctx, "tap", None)        # diagnostics (StepContext.tap): the stream at the reference's three dump points
+        if tap is not None:
+            tap("layer_in", ctx.entry, stream, ctx)
         h = stream.normed(self.mixer_norm, ctx.act_dtype, consumer=self.mixer)
         if getattr(self.mixer, "gives_lazy_delta", False):
             stream.add(self.mixer.forward(h, ctx, kv, lazy_ok=True))
         else:
             stream.add(self.mixer.forward(h, ctx, kv))
+        if tap is not None:
+            tap("ffn_in", ctx.entry, stream, ctx)
         h = stream.normed(self.ffn_norm, ctx.act_dtype, consumer=self.ffn)
         if getattr(self.ffn, "gives_lazy_delta", False):
             stream.add(self.ffn.forward(h, ctx, lazy_ok=True))
         else:
             stream.add(self.ffn.forward(h, ctx))
+        if tap is not None:
+            tap("layer_out", ctx.entry, stream, ctx)

@@ -9,7 +9,7 @@ import pytest
 import torch
 
 import plain_llama as pl
-from conftest import ROOT
+from conftest import ROOT, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -182,3 +182,60 @@ def test_command_line_benchmark_runs_top_logits_and_a_random_folder(tmp_path):
     assert [int(x) for x in ids.split(",")] == want[2:]
     p = subprocess.run(exe + [folder, "-n", "1", "--benchmark-warmup-runs", "1"] + common, capture_output=True, text=True, timeout=300)
     assert p.returncode != 0 and "--benchmark-runs" in p.stderr + p.stdout
+
+
+@pytest.mark.parametrize("fp32", [True, False])
+def test_command_line_dumps_of_the_residual_stream(model_folders, tmp_path, fp32):
+    """--dump-binary / --dump-tag / --dump-layer / --dump-pos and the statistics lines (the reference's
+    diagnostics, src/main.c:144-147, src/transformer/cpu.c:213-251): the stream at a layer's input, before its
+    feed-forward and at its output, against the plain implementation's layers; and the tokens are the same
+    with the dumps as without."""
+    import numpy as np
+    dtype = torch.float32 if fp32 else torch.bfloat16
+    folder = model_folders("B", dtype)
+    c, W = pl.read_config(folder), pl.read_weights(folder)
+    prompt = [3, 1, 4, 1, 5, 9, 2, 6, 5, 3]
+    rt = None if fp32 else torch.bfloat16
+    toks = torch.tensor(prompt)
+    inv_freq = pl.rope_inv_freq(c["head_dim"], c["theta"], c["rope_scaling"])
+    xs = [W["model.embed_tokens.weight"][toks].float()]                 # the stream at every layer's input
+    for l in range(c["layers"]):
+        xs.append(pl.decoder_layer(xs[-1], torch.arange(len(prompt)), W, l, c, inv_freq, rt))
+    base = [sys.executable, os.path.join(ROOT, "bin", "bitnet"), folder, "--prompt-token-ids", ",".join(map(str, prompt)),
+            "-n", "4", "--repeat-penalty", "1.0", "--token-ids", "--quiet"] + (["--fp32"] if fp32 else [])
+    plain_run = subprocess.run(base, capture_output=True, text=True, timeout=300)
+    assert plain_run.returncode == 0, plain_run.stderr[-1500:]
+    ids = lambda p: [l for l in p.stderr.splitlines() if l and l[0].isdigit()][0]
+    tol = 1e-4 if fp32 else 3e-2
+    stats = tmp_path / "stats.txt"
+    for tag, layer, pos, want in (("bitnet_inp", 1, 7, xs[1][7]), ("bitnet_lout", 2, 9, xs[3][9]), ("bitnet_inp", 0, 0, xs[0][0])):
+        out = tmp_path / f"{tag}_{layer}_{pos}.f32"
+        p = subprocess.run(base + ["--dump-binary", str(out), "--dump-tag", tag, "--dump-layer", str(layer), "--dump-pos", str(pos),
+                                   "--dump-stats", str(stats)], capture_output=True, text=True, timeout=300)
+        assert p.returncode == 0, p.stderr[-1500:]
+        assert ids(p) == ids(plain_run)
+        got = torch.from_numpy(np.fromfile(out, dtype="<f4").copy())
+        assert got.shape == want.shape and rel_err(got, want) < tol, (tag, layer, pos)
+    # the lines of statistics: every tag of the selected layer and position, the numbers those of the vector
+    lines = [l for l in stats.read_text().splitlines() if l.startswith("bitnet_lout pos=9 layer=2 ")]
+    assert len(lines) == 1
+    fields = dict(f.split("=", 1) for f in lines[0].split()[1:])
+    assert int(fields["dim"]) == c["dim"]
+    assert abs(float(fields["sum"]) - float(xs[3][9].sum())) < tol * float(xs[3][9].abs().sum())
+    first = [float(v) for v in fields["first"].split(",")]
+    assert len(first) == 16 and rel_err(torch.tensor(first), xs[3][9][:16]) < tol
+    # the state before the feed-forward lies between the layer's input and its output: lout - ffn_inp is the feed-forward's output
+    out = tmp_path / "ffn_inp.f32"
+    p = subprocess.run(base + ["--dump-binary", str(out), "--dump-tag", "bitnet_ffn_inp", "--dump-layer", "1", "--dump-pos", "4"],
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-1500:]
+    x_mid = torch.from_numpy(np.fromfile(out, dtype="<f4").copy())
+    pfx = "model.layers.1."
+    xb = pl.rmsnorm(x_mid[None, :], W[pfx + "post_attention_layernorm.weight"], c["eps"])
+    if rt is not None:
+        xb = xb.to(rt).float()
+    ffn = pl.feed_forward(xb, W[pfx + "mlp.gate_proj.weight"].float(), W[pfx + "mlp.up_proj.weight"].float(),
+                          W[pfx + "mlp.down_proj.weight"].float(), rt)[0]
+    assert rel_err(x_mid + ffn, xs[2][4]) < tol
+    bad = subprocess.run(base + ["--dump-binary", str(out)], capture_output=True, text=True, timeout=300)
+    assert bad.returncode != 0 and "--dump-tag" in bad.stderr
