@@ -172,10 +172,12 @@ extern "C" int bn_splitk_gemm(const void* X, const void* W, float* P, int M, int
     const dim3 grid((N + SG_COLS - 1) / SG_COLS, splits), block(SG_WAVES * 64);
     const size_t smem = (size_t)2 * MT * 16 * SG_XROW;
     auto go = [&](auto kernel) {
-        if (smem > 64 * 1024) {                   // more than the default limit of dynamic shared memory
+        static bool raised = false;               // per instantiation of this lambda, that is per kernel
+        if (smem > 64 * 1024 && !raised) {        // more than the default limit of dynamic shared memory
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e != hipSuccess) return (int)e;
+            raised = true;
         }
         hipLaunchKernelGGL(kernel, grid, block, smem, s, (const bf16*)X, (const bf16*)W, P, (bf16*)nullptr, M, N, K, ldx, ldw, 0,
                            kps);
@@ -206,10 +208,12 @@ extern "C" int bn_splitk_gemm_swiglu(const void* X, const void* W, void* Y, int 
     const dim3 grid((N + SG_GLU_WAVES * 16 - 1) / (SG_GLU_WAVES * 16), 1), block(SG_GLU_WAVES * 64);
     const size_t smem = (size_t)2 * MT * 16 * SG_XROW;
     auto go = [&](auto kernel) {
-        if (smem > 64 * 1024) {
+        static bool raised = false;               // per instantiation of this lambda, that is per kernel
+        if (smem > 64 * 1024 && !raised) {        
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e != hipSuccess) return (int)e;
+            raised = true;
         }
         hipLaunchKernelGGL(kernel, grid, block, smem, s, (const bf16*)X, (const bf16*)W, (float*)nullptr, (bf16*)Y, M, N, K, ldx,
                            ldw, ldy, kps);
