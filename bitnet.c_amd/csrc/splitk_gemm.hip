@@ -1,5 +1,5 @@
-// Products of 17 to 128 activation rows whose result is added to the residual stream (the output
-// projection of a mixer, the last product of a feed-forward): P[s, M, N] = X[M, k-range s] . W[N, k-range s]^T,
+// Products of up to 128 activation rows whose result is added to the residual stream (the last product of a
+// feed-forward, the output projection of a mixer): P[s, M, N] = X[M, k-range s] . W[N, k-range s]^T,
 // float32 partial sums, one slab per k-range; the kernel of the next norm adds the slabs to the stream in
 // slab order (elementwise.hip), so no pass of its own forms the sum and the product is never rounded to bf16.
 // Same formula as every matrix product here (src/transformer/cpu.c:933-939, :1301-1303).

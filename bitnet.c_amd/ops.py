@@ -378,19 +378,19 @@ def interleave_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor) -> torch.Tensor
     return torch.stack([w_gate.reshape(F // 8, 8, K), w_up.reshape(F // 8, 8, K)], dim=1).reshape(2 * F, K).contiguous()
 
 
-# Rows at which the interleaved gate/up product with its SwiGLU epilogue is the kernel that stages the activations once
-# per 64 columns (splitk_gemm.hip): measured on the 8B shape against the library's product and the SwiGLU kernel after it
-# 50 us against 55 at 17 and 24 rows, 52 against 54.5 at 32, 54 against 53 at 40, 58 against 54 at 64.  Without the library
-# it takes every row count of the kernel.
-SWIGLU_STAGED_ROWS = (17, 32)
+# Without the library the interleaved gate/up product of 17 to 128 rows with its SwiGLU epilogue is the kernel that stages
+# the activations once per 64 columns (splitk_gemm.hip).  With the library it is not used: measured against the library's
+# product and the SwiGLU kernel after it, it is 5 to 10 % faster at 17 to 32 rows of the 8B shape (50 us against 55) and 10
+# to 30 % slower at the 13B and 70B shapes and at a hidden size of 3,072 (65 against 54, 200 against 184, 30 against 26).
+SWIGLU_STAGED_ROWS = (17, 128)
 
 
 def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = False, *,
                   allow_library: Optional[bool] = None) -> torch.Tensor:
     """silu(x.Wg^T) * (x.Wu^T) for w_gate_up = [Wg; Wu] ([2F, K]), or the two interleaved in
-    blocks of 8 rows (interleave_gate_up).  The decode-sized bf16 case is one kernel, and so are the
-    interleaved case at SWIGLU_STAGED_ROWS and without the library; every other case is the product
-    followed by the SwiGLU kernel."""
+    blocks of 8 rows (interleave_gate_up).  The decode-sized bf16 case is one kernel, and so is the
+    interleaved case without the library; every other case is the product followed by the SwiGLU
+    kernel."""
     require_gpu()
     _dev(x, "x", dims=2)
     _dev(w_gate_up, "w_gate_up", x.dtype, 2)
@@ -406,8 +406,8 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = 
         return torch.empty((0, F), dtype=x.dtype, device=x.device)
     ldx, ldw = _rows(x, "x"), _rows(w_gate_up, "w_gate_up")
     aligned = x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0
-    lo, hi = SWIGLU_STAGED_ROWS if allow_library else (SWIGLU_STAGED_ROWS[0], 128)
-    if (x.dtype == torch.bfloat16 and interleaved and aligned and lo <= M <= hi
+    lo, hi = SWIGLU_STAGED_ROWS
+    if (x.dtype == torch.bfloat16 and interleaved and aligned and not allow_library and lo <= M <= hi
             and _fn("splitk_gemm", "bn_splitk_gemm_supports")(M, 2 * F, K, ldx, ldw)):
         y = torch.empty((M, F), dtype=x.dtype, device=x.device)
         _check(_fn("splitk_gemm", "bn_splitk_gemm_swiglu")(x.data_ptr(), w_gate_up.data_ptr(), y.data_ptr(), M, F, K, ldx, ldw,
@@ -431,7 +431,12 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = 
 # --------------------------------------------------------------------------------------
 # Set False (or BITNET_NO_FUSED_NORM=1) to keep every norm a kernel of its own.
 SPLIT_SUMS = os.environ.get("BITNET_NO_SPLIT_SUMS", "") in ("", "0")
-SPLIT_SUM_ROWS = (17, 128)      # rows for which a product that ends a part is left as partial sums
+# Where a product that ends a part is left as partial sums (splitk_gemm) instead of going to the library: from 64 to 128
+# rows and K at least twice N, the shape of a feed-forward's last product.  Measured on nine layer shapes (hidden 2,048
+# to 8,192) with the kernels of the next norm included: there it is 15 to 45 % faster than the library's product (8B:
+# 36 us against 45 at 64 rows, 44 against 80 at 128; 70B: 119 against 148, 141 against 210), while below 64 rows and for
+# square matrices the two are within 10 % of each other with the sign depending on the shape.
+SPLIT_SUM_ROWS = (64, 128)
 
 
 @dataclass
@@ -452,7 +457,7 @@ class PartialSums:
 def can_split_sums(M: int, N: int, K: int, dtype) -> bool:
     """Whether a product of these sizes whose result goes to the residual stream is done as partial sums."""
     return (SPLIT_SUMS and dtype == torch.bfloat16 and SPLIT_SUM_ROWS[0] <= M <= SPLIT_SUM_ROWS[1] and K % 8 == 0
-            and K >= 8 and N >= 1)
+            and K >= 2 * N and N >= 1)
 
 
 def linear_partial_sums(x: torch.Tensor, w: torch.Tensor) -> PartialSums:

@@ -32,8 +32,8 @@ class Linear:
 
     def lazy(self, x: torch.Tensor):
         """The product in the form in which it reaches a residual stream cheapest (bf16, no bias): a LazyDelta at
-        decode sizes, where it can add itself to the stream; partial sums over ranges of K (ops.PartialSums) at up
-        to 128 rows, which the kernel of the next norm adds up; else its result."""
+        decode sizes, where it can add itself to the stream; partial sums over ranges of K (ops.PartialSums), which the
+        kernel of the next norm adds up, where ops.can_split_sums says so; else its result."""
         from .base import LazyDelta
         M, (N, K) = x.shape[0], self.weight.shape
         plain = (self.bias is None and x.dim() == 2 and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16

@@ -200,16 +200,17 @@ def test_products_with_the_norm_folded_in_refuse_what_they_cannot_take():
 @pytest.mark.parametrize("M", [1, 17, 33, 64, 100, 128])
 @pytest.mark.parametrize("N,K", [(4096, 4096), (200, 328), (72, 1000), (136, 16), (264, 3592)])
 def test_products_left_as_partial_sums(M, N, K):
-    """A product that ends a part at 17 to 128 rows: float32 partial sums over ranges of K, which the kernel of the
-    next norm (or the plain add) adds to the stream in slab order.  The sums are exact up to their order; the norm
-    is the plain formula on the sum."""
+    """A product left as float32 partial sums over ranges of K, which the kernel of the next norm (or the plain add)
+    adds to the stream in slab order (the dispatcher does so for a part's last product from 64 to 128 rows when K is
+    at least twice N; the kernel takes 1 to 128 rows of any shape).  The sums are exact up to their order; the norm is
+    the plain formula on the sum."""
     ops = _ops()
     eps = 1e-6
     x, w = _rand((M, K), torch.bfloat16, 41), _rand((N, K), torch.bfloat16, 42, 0.05)
     stream = _rand((M, N), torch.float32, 43, 2.0)
     norm_w = _rand((N,), torch.float32, 44) * 0.2 + 1.0
     ref = x.double() @ w.double().t()
-    assert ops.can_split_sums(M, N, K, torch.bfloat16) == (17 <= M <= 128)
+    assert ops.can_split_sums(M, N, K, torch.bfloat16) == (64 <= M <= 128 and K >= 2 * N)
     parts = ops.linear_partial_sums(x.cuda(), w.cuda())
     assert parts.slabs.dtype == torch.float32 and tuple(parts.shape) == (M, N)
     assert rel_err(parts.slabs.sum(dim=0), ref.float()) < 1e-5
@@ -236,8 +237,10 @@ def test_products_left_as_partial_sums(M, N, K):
 
 def test_partial_sums_refuse_what_they_cannot_take():
     ops = _ops()
-    assert not ops.can_split_sums(16, 64, 64, torch.bfloat16) and not ops.can_split_sums(129, 64, 64, torch.bfloat16)
-    assert not ops.can_split_sums(64, 64, 172, torch.bfloat16) and not ops.can_split_sums(64, 64, 64, torch.float32)
+    assert ops.can_split_sums(64, 64, 128, torch.bfloat16) and ops.can_split_sums(128, 64, 512, torch.bfloat16)
+    assert not ops.can_split_sums(63, 64, 128, torch.bfloat16) and not ops.can_split_sums(129, 64, 128, torch.bfloat16)
+    assert not ops.can_split_sums(64, 64, 120, torch.bfloat16)             # K below twice N
+    assert not ops.can_split_sums(64, 64, 172, torch.bfloat16) and not ops.can_split_sums(64, 64, 128, torch.float32)
     z = lambda *shape: torch.zeros(*shape, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(ops.KernelError):
         ops.linear_partial_sums(z(129, 64), z(64, 64))                 # more rows than the staged block holds
@@ -311,8 +314,9 @@ def test_gemm_mfma_swiglu(M, F, K, width):
 @pytest.mark.parametrize("M", [1, 17, 24, 33, 48, 100, 128])
 @pytest.mark.parametrize("F,K", [(8, 8), (328, 120), (1000, 512), (520, 4096), (136, 16)])
 def test_swiglu_product_with_staged_activations(M, F, K):
-    """The gate/up product of 17 to 128 rows with the SwiGLU epilogue (gate and up rows interleaved in blocks of 8,
-    activations staged once per workgroup): against the exact result, and where the dispatcher sends it."""
+    """The gate/up product of up to 128 rows with the SwiGLU epilogue (gate and up rows interleaved in blocks of 8,
+    activations staged once per workgroup): against the exact result, and that the dispatcher uses it when it may
+    not call the library."""
     ops = _ops()
     from bitnet_c_amd.csrc import build
     from ctypes import c_void_p
@@ -328,9 +332,7 @@ def test_swiglu_product_with_staged_activations(M, F, K):
     assert rc == 0
     assert close(y.float(), want, torch.bfloat16)
     lo, hi = ops.SWIGLU_STAGED_ROWS
-    if lo <= M <= hi:
-        assert torch.equal(ops.linear_swiglu(xd, wi, True), y)
-    if lo <= M:
+    if lo <= M <= hi:                              # without the library this is the kernel of these row counts
         assert torch.equal(ops.linear_swiglu(xd, wi, True, allow_library=False), y)
 
 
