@@ -4,8 +4,8 @@ Fields and defaults follow the reference's loader (src/model.c:238-310): kv head
 default to heads (:252-254), rope_theta to 10000 (:259-260), the norm's eps to 1e-5
 (:264-266), head size to hidden/heads unless given (:285-287); heads must be a multiple
 of kv heads (:299-302).  The reference's SIMD-only checks (hidden % 128, head % 16;
-:303-310) are properties of its kernels, not of the architecture; what the kernels here
-need is checked by the parts that use them.
+:303-310) are properties of its kernels, not of the architecture and are not taken over; the one limit of the kernels here that a
+config.json can break (a head size above ops.MAX_HEAD_DIM) is reported with the other errors.
 """
 from __future__ import annotations
 
@@ -94,6 +94,10 @@ class LlamaConfig:
                               f"num_key_value_heads {kv_heads}")
         if head_dim % 2:
             raise ConfigError(f"config.json: head_dim {head_dim} must be even (rotation pairs)")
+        from ..ops import MAX_HEAD_DIM
+        if head_dim > MAX_HEAD_DIM:
+            raise ConfigError(f"config.json: head_dim {head_dim} is more than the attention kernels take "
+                              f"(every even head size up to {MAX_HEAD_DIM})")
         act = raw.get("hidden_act", "silu")
         if act != "silu":
             raise ConfigError(f"config.json: hidden_act {act!r} is not supported (supported: 'silu')")

@@ -1,5 +1,7 @@
-// Attention over the paged cache for any head size (a multiple of 8, up to 256), any
-// number of heads and kv groups, float32 or bf16 cache, written on the vector ALUs.
+// Attention over the paged cache for any even head size up to 256, any number of heads and
+// kv groups, float32 or bf16 cache, written on the vector ALUs.  Head sizes whose rows are
+// not whole 16-byte groups are staged element by element and padded with zeros in shared
+// memory to the next multiple of 8, which changes no sum.
 // It serves the float32 path, every shape the matrix-core kernels do not take, and
 // both phases: a workgroup owns up to RT "rows", a row being one (query token, query
 // head) pair that shares one kv head; decode is the case of one query token per
@@ -58,6 +60,7 @@ template <typename T, int RT>
 __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int hs = a.hs, KT = a.KT, GT = a.GT;
+    const int hsp = (hs + 7) & ~7;                       // the head size padded to whole groups of 8
     const int QT = RT / GT;
     const int G = a.H / a.Hkv;
     const int n_head_tiles = (G + GT - 1) / GT;
@@ -76,9 +79,9 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
     if (n_tok > QT) n_tok = QT;
 
     // shared memory
-    const int kstride = hs + 16 / (int)sizeof(T);        // elements; keeps rows 16-byte aligned
-    float* q_s = reinterpret_cast<float*>(smem_raw);     // [RT][hs]
-    float* s_s = q_s + RT * hs;                          // [RT][KT] scores
+    const int kstride = hsp + 16 / (int)sizeof(T);       // elements; keeps rows 16-byte aligned
+    float* q_s = reinterpret_cast<float*>(smem_raw);     // [RT][hsp], zero beyond hs
+    float* s_s = q_s + RT * hsp;                         // [RT][KT] scores
     float* p_s = s_s + RT * KT;                          // [KT][RT] probabilities
     float* m_s = p_s + KT * RT;                          // [16] running max
     float* l_s = m_s + 16;                               // [16] running sum
@@ -87,12 +90,12 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
     T* v_s = k_s + KT * kstride;
 
     // rows: r = i*GT + g  ->  token tok0+i, head kvh*G + ht*GT + g
-    for (int idx = tid; idx < RT * hs; idx += ATT_THREADS) {
-        const int r = idx / hs, d = idx - r * hs;
+    for (int idx = tid; idx < RT * hsp; idx += ATT_THREADS) {
+        const int r = idx / hsp, d = idx - r * hsp;
         const int i = r / GT, g = r - i * GT;
         const int hg = ht * GT + g;
         float v = 0.f;
-        if (i < n_tok && hg < G && pos0 >= 0) {
+        if (d < hs && i < n_tok && hg < G && pos0 >= 0) {
             const T* qp = reinterpret_cast<const T*>(a.q) + (size_t)(tok0 + i) * a.q_stride +
                           (size_t)(kvh * G + hg) * hs;
             v = to_f32(qp[d]);
@@ -100,6 +103,9 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
         q_s[idx] = v;
     }
     if (tid < 16) { m_s[tid] = -INFINITY; l_s[tid] = 0.f; a_s[tid] = 1.f; }
+    const bool whole_groups = (hs * (int)sizeof(T)) % 16 == 0;      // rows of 16-byte groups in the pages
+    if (hsp != hs)                                                  // the padding of the staged rows stays zero
+        for (int idx = tid; idx < 2 * KT * kstride; idx += ATT_THREADS) k_s[idx] = from_f32<T>(0.f);
 
     // keys this workgroup visits
     int lo = 0, hi = 0;
@@ -121,7 +127,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
 
     const int P = ATT_THREADS / KT;          // threads per key in phase A: 4, 8 or 16
     const int ja = tid / P, pa = tid - ja * P;
-    const int n_chunks = hs / 4;
+    const int n_chunks = hsp / 4;
     const int lane = tid & 63, wave = tid >> 6;
     __syncthreads();
 
@@ -133,13 +139,23 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
             const int vec_per_row = hs * (int)sizeof(T) / 16;
             const uint4* kg = reinterpret_cast<const uint4*>(reinterpret_cast<const T*>(a.k_pages) + base);
             const uint4* vg = reinterpret_cast<const uint4*>(reinterpret_cast<const T*>(a.v_pages) + base);
-            for (int idx = tid; idx < KT * vec_per_row; idx += ATT_THREADS) {
+            for (int idx = tid; whole_groups && idx < KT * vec_per_row; idx += ATT_THREADS) {
                 const int j = idx / vec_per_row, c = idx - j * vec_per_row;
                 uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
                 if (j0 + j < hi) { kv = kg[idx]; if (!a.v_transposed) vv = vg[idx]; }   // rows not yet written stay zero
                 *reinterpret_cast<uint4*>(reinterpret_cast<unsigned char*>(k_s + j * kstride) + c * 16) = kv;
                 if (!a.v_transposed)
                     *reinterpret_cast<uint4*>(reinterpret_cast<unsigned char*>(v_s + j * kstride) + c * 16) = vv;
+            }
+            if (!whole_groups) {
+                const T* ke = reinterpret_cast<const T*>(a.k_pages) + base;
+                const T* ve = reinterpret_cast<const T*>(a.v_pages) + base;
+                for (int idx = tid; idx < KT * hs; idx += ATT_THREADS) {
+                    const int j = idx / hs, d = idx - j * hs;
+                    const bool in = j0 + j < hi;
+                    k_s[j * kstride + d] = in ? ke[idx] : from_f32<T>(0.f);
+                    if (!a.v_transposed) v_s[j * kstride + d] = in ? ve[idx] : from_f32<T>(0.f);
+                }
             }
             if (a.v_transposed) {
                 const T* vt = reinterpret_cast<const T*>(a.v_pages) + ((size_t)page * a.Hkv + kvh) * hs * BN_PAGE +
@@ -162,7 +178,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
                 Vec4<T>::load(kr + c * 4, kv);
 #pragma unroll
                 for (int r = 0; r < RT; ++r) {
-                    const float4 qv = *reinterpret_cast<const float4*>(q_s + r * hs + c * 4);
+                    const float4 qv = *reinterpret_cast<const float4*>(q_s + r * hsp + c * 4);
                     dot[r] = fmaf(kv[0], qv.x, dot[r]);
                     dot[r] = fmaf(kv[1], qv.y, dot[r]);
                     dot[r] = fmaf(kv[2], qv.z, dot[r]);
@@ -295,7 +311,8 @@ __global__ void attn_combine_kernel(T* __restrict__ out, int out_stride, const f
 }
 
 static size_t attn_smem_bytes(int RT, int hs, int KT, int elt) {
-    return (size_t)(RT * hs + 2 * RT * KT + 48) * sizeof(float) + (size_t)2 * KT * (hs * elt + 16);
+    const int hsp = (hs + 7) & ~7;
+    return (size_t)(RT * hsp + 2 * RT * KT + 48) * sizeof(float) + (size_t)2 * KT * (hsp * elt + 16);
 }
 
 template <typename T, int RT>
@@ -320,11 +337,15 @@ static int launch_rows_rt(const AttnArgs& a, int RT, int n_tiles, hipStream_t s)
     return BN_ERR_ARG;
 }
 
-// Largest key tile (64, 32, 16) whose shared memory stays within 64 KB; 0 if none does.
-extern "C" int bn_attn_rows_key_tile(int dtype, int RT, int hs) {
+// Keys per tile: the largest of 64, 32, 16 whose shared memory stays within 64 KB for the widest
+// workgroup (16 rows); 0 if none does.  It is a function of the cache type and the head size alone,
+// never of the rows a launch happens to hold: a query's keys are then cut into the same tiles, and
+// its sums formed in the same order, whether it arrives alone, in a prompt or in a batch (the
+// reference keeps one order per kernel, src/transformer/gqa_scalar.c:61-121).
+extern "C" int bn_attn_rows_key_tile(int dtype, int hs) {
     const int elt = dtype == BN_DT_F32 ? 4 : 2;
     for (int kt = 64; kt >= 16; kt >>= 1)
-        if (attn_smem_bytes(RT, hs, kt, elt) <= 64 * 1024) return kt;
+        if (attn_smem_bytes(16, hs, kt, elt) <= 64 * 1024) return kt;
     return 0;
 }
 
@@ -338,7 +359,7 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
                             float scale, int n_splits, int chunk, float* part_o, float* part_ml,
                             int v_transposed, hipStream_t s) {
     if (n_tiles <= 0 || n_tokens <= 0 || H <= 0 || Hkv <= 0 || H % Hkv) return BN_ERR_ARG;
-    if (hs < 8 || hs > 256 || hs % 8) return BN_ERR_ARG;
+    if (hs < 2 || hs > 256 || hs % 2) return BN_ERR_ARG;
     if (GT <= 0 || GT > RT || (GT & (GT - 1)) || RT > 16 || (RT & (RT - 1))) return BN_ERR_ARG;
     if (n_splits < 1 || window < 0) return BN_ERR_ARG;
     if (n_splits > 1 && (chunk <= 0 || chunk % BN_PAGE || !part_o || !part_ml)) return BN_ERR_ARG;
@@ -352,7 +373,7 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
     a.n_splits = n_splits; a.chunk = n_splits > 1 ? chunk : 0x40000000;
     a.scale = scale;
     a.v_transposed = v_transposed;
-    a.KT = bn_attn_rows_key_tile(dtype, RT, hs);
+    a.KT = bn_attn_rows_key_tile(dtype, hs);
     if (a.KT == 0) return BN_ERR_ARG;
     int rc;
     if (dtype == BN_DT_F32) rc = launch_rows_rt<float>(a, RT, n_tiles, s);

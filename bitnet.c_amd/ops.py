@@ -46,7 +46,7 @@ _SIGNATURES = {
                              c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "attn_rows": {
-        "bn_attn_rows_key_tile": [c_int, c_int, c_int],
+        "bn_attn_rows_key_tile": [c_int, c_int],
         "bn_attn_rows": [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
                          c_void_p, c_void_p, c_int, c_void_p],
@@ -677,6 +677,9 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
             v_pages.data_ptr(), H, Hkv, hs, _stream()), "v_transposed_write")
 
 
+MAX_HEAD_DIM = 256        # the attention kernels take every even head size up to this
+
+
 def _pow2_at_least(n: int) -> int:
     p = 1
     while p < n:
@@ -702,9 +705,13 @@ def attention_row_shape(H: int, Hkv: int, decode: bool, dtype=None, hs: int = 0)
     return 16, GT, 16 // GT
 
 
-def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int):
+def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int, dtype=None):
     """(n_splits, chunk): how the keys of a decode step are cut so that the launch fills the
-    chip.  A function of the batch's shape and of max_len alone."""
+    chip.  A function of the batch's shape and of max_len alone.  A float32 cache is never split:
+    there a query's keys are summed in one order, the prompt form's, however the step was cut, so
+    that float32 logits are equal bit for bit under every cut."""
+    if dtype == torch.float32:
+        return 1, 0
     RT, GT, _ = attention_row_shape(H, Hkv, True)
     G = H // Hkv
     wgs = max(1, n_seqs * Hkv * ((G + GT - 1) // GT))
@@ -770,8 +777,8 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     T = qkv.shape[0]
     if H % Hkv or qkv.shape[1] < H * hs or out.shape != (T, H * hs) or not out.is_contiguous():
         raise KernelError(f"attention: qkv {tuple(qkv.shape)} / out {tuple(out.shape)} do not fit H={H} hs={hs}")
-    if hs % 8 or hs > 256:
-        raise KernelError(f"attention: head size {hs} is not supported (a multiple of 8, at most 256)")
+    if hs % 2 or hs < 2 or hs > MAX_HEAD_DIM:
+        raise KernelError(f"attention: head size {hs} is not supported (even, at most {MAX_HEAD_DIM})")
     if not block_table.is_contiguous():
         raise KernelError("attention: block_table must be contiguous")
     decode = tiles is None

@@ -29,9 +29,9 @@ class Attention(Part):
                  position: PartSpec, window: int = 0, bias: bool = False):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} kv heads")
-        if head_dim % 8 or head_dim > 256:
+        if head_dim % 2 or head_dim < 2 or head_dim > ops.MAX_HEAD_DIM:
             raise ValueError(f"attention: head_dim {head_dim} is not supported by the kernels "
-                             f"(a multiple of 8, at most 256)")
+                             f"(even, at most {ops.MAX_HEAD_DIM})")
         self.hidden, self.H, self.Hkv, self.hs = int(hidden), int(n_heads), int(n_kv_heads), int(head_dim)
         self.scale, self.window, self.has_bias = float(scale), int(window), bool(bias)
         self.position = POSITION_ENCODINGS.build(position)
@@ -82,7 +82,7 @@ class Attention(Part):
             if self.window:
                 n_splits, chunk = 1, 0
             else:
-                n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len)
+                n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len, h.dtype)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
                           window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
                           fused_rotate=inv_freq, fused_write=kv.writes, by_length=ctx.by_length)
@@ -92,7 +92,7 @@ class Attention(Part):
             if self.window:                   # a window is short; its keys are not split
                 n_splits, chunk = 1, 0
             else:
-                n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len)
+                n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len, h.dtype)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
                           window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
                           by_length=ctx.by_length)

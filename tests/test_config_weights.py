@@ -23,7 +23,7 @@ def test_llama_config_defaults_and_derived_sizes():
 
 @pytest.mark.parametrize("patch,word", [
     (dict(num_key_value_heads=3), "multiple"), (dict(hidden_size=0), "positive"), (dict(vocab_size=-1), "positive"),
-    (dict(hidden_act="gelu"), "hidden_act"), (dict(head_dim=15), "even"),
+    (dict(hidden_act="gelu"), "hidden_act"), (dict(head_dim=15), "even"), (dict(head_dim=258), "attention kernels take"),
     (dict(rope_scaling=dict(rope_type="yarn", factor=2.0)), "yarn"),
     (dict(rope_scaling=dict(rope_type="llama3", factor=8.0)), "low_freq_factor"),
     (dict(num_hidden_layers=None), "num_hidden_layers"), (dict(hidden_size=66, num_attention_heads=4), "head_dim"),

@@ -530,7 +530,8 @@ def _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, seed):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,Hkv,hs,window", [(4, 2, 16, 0), (5, 5, 24, 0), (6, 2, 32, 0), (8, 2, 128, 0), (32, 1, 64, 0),
                                              (2, 1, 256, 0), (4, 2, 16, 7), (4, 4, 64, 100), (20, 1, 40, 0),
-                                             (32, 8, 128, 0), (8, 8, 128, 33), (6, 2, 64, 0), (40, 2, 64, 0)])
+                                             (32, 8, 128, 0), (8, 8, 128, 33), (6, 2, 64, 0), (40, 2, 64, 0),
+                                             (3, 3, 20, 0), (4, 2, 36, 9), (2, 1, 6, 0), (6, 2, 250, 0)])
 @pytest.mark.parametrize("force_vector", [False, True])
 def test_attention_prompt_form(dtype, H, Hkv, hs, window, force_vector):
     lens_before, n_new = [0, 0, 64, 130, 5, 0], [1, 37, 64, 3, 70, 300]
@@ -566,7 +567,8 @@ def test_attention_prompt_form_with_more_workgroups_than_cus(H, Hkv, hs, T):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,Hkv,hs,window", [(4, 2, 16, 0), (5, 5, 24, 0), (8, 2, 128, 0), (12, 4, 64, 0),
                                              (16, 1, 32, 0), (4, 2, 16, 50), (8, 8, 64, 129), (32, 8, 128, 0),
-                                             (40, 2, 128, 0), (6, 6, 128, 70)])
+                                             (40, 2, 128, 0), (6, 6, 128, 70), (3, 3, 20, 0), (4, 2, 36, 50),
+                                             (2, 1, 6, 0)])
 @pytest.mark.parametrize("force_splits", [1, 0, 5])
 @pytest.mark.parametrize("force_vector", [False, True])
 def test_attention_decode_form(dtype, H, Hkv, hs, window, force_splits, force_vector):

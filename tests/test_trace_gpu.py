@@ -72,7 +72,10 @@ def test_replay_three_ways(model_folders, tmp_path, name, dtype):
     for k in reqs:
         got = torch.cat([read_logits(out, s, vocab) for s in where[k]])
         assert rel_err(got, ref[k]) < TOL[dtype], k
-        assert rel_err(got, whole[k]) < (1e-5 if dtype == torch.float32 else TOL[dtype]), k
+        if dtype == torch.float32:               # one order of summation per query, however the tokens were cut
+            assert torch.equal(got, whole[k]), k
+        else:
+            assert rel_err(got, whole[k]) < TOL[dtype], k
 
     # (3) batches of unequal lengths; the prompts are the first part of each request, the rest is
     #     decoded one by one; shorter requests end earlier; the second batch uses the first one's slots
@@ -108,7 +111,10 @@ def test_replay_three_ways(model_folders, tmp_path, name, dtype):
     for k in reqs:
         g = torch.cat(got[k])
         assert rel_err(g, ref[k]) < TOL[dtype], k
-        assert rel_err(g, whole[k]) < (1e-5 if dtype == torch.float32 else TOL[dtype]), k
+        if dtype == torch.float32:               # nor does the batch, or the place in the cache, change a bit
+            assert torch.equal(g, whole[k]), k
+        else:
+            assert rel_err(g, whole[k]) < TOL[dtype], k
 
 
 def test_steps_without_wanted_logits_write_no_file(model_folders, tmp_path):
