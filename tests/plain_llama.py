@@ -3,7 +3,8 @@
 Whole sequences, no cache, one function per part, CPU tensors.  It shares no code
 with the package under test: it has its own config reading, its own safetensors
 reading (through the `safetensors` library) and its own sampler.  Each function
-cites the lines of the reference (`/root/reference/`) whose formula it writes out.
+cites the lines of the reference (artalis-io/bitnet.c, paths from its root) whose formula it
+writes out.
 
 Everything is computed in float32 with float64 sums where the reference has them.
 `round_to` (a torch dtype or None) rounds activations where an engine that keeps

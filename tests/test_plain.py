@@ -81,10 +81,35 @@ def test_llama3_scaling_limits():
     f = pl.rope_inv_freq(64, 500000.0, sc)
     assert torch.all(f[1:] < f[:-1])                                                        # still decreasing
     assert torch.all(f <= base * (1 + 1e-6)) and torch.all(f >= base / 8.0 * (1 - 1e-6))
-    # continuity at both thresholds: a wavelength just inside the band is close to the band's end value
-    w = 2 * math.pi / base.double()
-    lo_edge, hi_edge = 64 / 1.0, 64 / 4.0
-    assert any(hi_edge < x < lo_edge for x in w.tolist()), "the test configuration has no band member"
+
+
+def test_llama3_scaling_is_continuous_at_both_thresholds():
+    """A wavelength a hair inside the interpolated band gets (almost) the value of the region next to it:
+    at orig/high_freq_factor the unscaled frequency, at orig/low_freq_factor the frequency divided by
+    `factor`.  The interpolation weights the other way round (or a band taken in wavelength instead of
+    orig/wavelength) jumps by the factor at an edge; the middle of the band lies strictly between."""
+    hd, theta, i = 64, 500000.0, 9
+    base = float(theta ** (-2.0 * i / hd))
+    wavelen = 2 * math.pi / base
+    sc = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0)
+    eps = 1e-7
+
+    def scaled(orig):
+        return float(pl.rope_inv_freq(hd, theta, dict(sc, original_max_position_embeddings=orig)).double()[i])
+
+    # wavelength == orig/high: orig = 4 * wavelength.  A little more orig: the wavelength is short (unscaled);
+    # a little less: it is just inside the band
+    short, inside = scaled(4.0 * wavelen * (1 + eps)), scaled(4.0 * wavelen * (1 - eps))
+    assert abs(short - base) < 1e-6 * base
+    assert abs(inside - base) < 1e-5 * base                       # not base / 8
+    # wavelength == orig/low: orig = wavelength.  A little less orig: the wavelength is long (divided by the
+    # factor); a little more: just inside the band
+    long_, inside = scaled(wavelen * (1 - eps)), scaled(wavelen * (1 + eps))
+    assert abs(long_ - base / 8.0) < 1e-6 * base
+    assert abs(inside - base / 8.0) < 1e-5 * base                 # not base
+    # the middle of the band in orig/wavelength (2.5 between 1 and 4): smooth = 0.5
+    mid = scaled(2.5 * wavelen)
+    assert abs(mid - 0.5 * (base / 8.0 + base)) < 1e-5 * base
 
 
 def test_attention_reference_vector():
@@ -121,11 +146,12 @@ def test_attention_window():
     full = pl.attention(q, k, v, 0.3)
     win = pl.attention(q, k, v, 0.3, window=4)
     assert torch.allclose(win[:4], full[:4], atol=1e-6)            # the window is not full yet
-    only = pl.attention(q[8:9], k[5:9], v[5:9], 0.3)               # query 8 sees keys 5..8 (no rope here)
-    # the one query must be the last of its four keys: run it as a 4-token sequence's last row
-    four = pl.attention(torch.cat([q[5:8], q[8:9]]), k[5:9], v[5:9], 0.3)
+    # query 8 sees keys 5..8 (no rope here): the last row of the four-token sequence 5..8
+    four = pl.attention(q[5:9], k[5:9], v[5:9], 0.3)
     assert torch.allclose(win[8], four[3], atol=1e-6) and not torch.allclose(win[8], full[8], atol=1e-4)
-    del only
+    # a window of one position: every query sees itself alone, the output is its own value row
+    one = pl.attention(q, k, v, 0.3, window=1)
+    assert torch.allclose(one, v.repeat_interleave(1, dim=1), atol=1e-6)
 
 
 def test_swiglu_reference_vector():
@@ -173,6 +199,46 @@ def test_layer_order_and_residual_with_zero_output_matrices():
     assert torch.allclose(pl.forward(c, W, toks), want, atol=1e-6)
 
 
+def test_the_feed_forward_reads_the_stream_after_the_attention_add():
+    """x += attention(norm(x)) comes first and the feed-forward reads the sum (src/transformer/cpu.c:939, then
+    :1247).  Here the embeddings are zero in dimension 0, only the attention's output matrix writes it, and
+    gate and up read nothing else: with parallel residuals (both parts reading the layer's input) the
+    feed-forward would see zero there and add nothing, so its output matrix could not matter."""
+    from conftest import TINY_A
+    c, W = _tiny(dict(TINY_A, num_hidden_layers=1), 8)
+    W["model.embed_tokens.weight"][:, 0] = 0.0
+    p = "model.layers.0."
+    wo = torch.zeros_like(W[p + "self_attn.o_proj.weight"])
+    wo[0] = W[p + "self_attn.o_proj.weight"][0] * 40.0            # the attention writes dimension 0 only
+    W[p + "self_attn.o_proj.weight"] = wo
+    for n in ("mlp.gate_proj.weight", "mlp.up_proj.weight"):
+        w = torch.zeros_like(W[p + n])
+        w[:, 0] = 1.0 + W[p + n][:, 0].abs() * 10.0                # gate and up read dimension 0 only
+        W[p + n] = w
+    toks = [3, 200, 17, 5, 9]
+    with_ffn = pl.forward(c, W, toks)
+    W0 = dict(W)
+    W0[p + "mlp.down_proj.weight"] = torch.zeros_like(W[p + "mlp.down_proj.weight"])
+    without = pl.forward(c, W0, toks)
+    assert float((with_ffn - without).abs().max()) > 1e-2 * float(without.abs().max())
+    # by hand for the last token: the stream after the add, normed, through the gated unit
+    x = W["model.embed_tokens.weight"][toks]
+    H, Hkv, hs = c["heads"], c["kv_heads"], c["head_dim"]
+    xb = pl.rmsnorm(x, W[p + "input_layernorm.weight"], c["eps"])
+    pos = torch.arange(len(toks))
+    f = pl.rope_inv_freq(hs, c["theta"])
+    q = pl.apply_rope((xb @ W[p + "self_attn.q_proj.weight"].t()).view(-1, H, hs), pos, f)
+    k = pl.apply_rope((xb @ W[p + "self_attn.k_proj.weight"].t()).view(-1, Hkv, hs), pos, f)
+    v = (xb @ W[p + "self_attn.v_proj.weight"].t()).view(-1, Hkv, hs)
+    x1 = x + pl.attention(q, k, v, 1 / math.sqrt(hs)).reshape(len(toks), H * hs) @ wo.t()
+    assert float(x1[:, 0].abs().min()) > 0 and torch.equal(x1[:, 1:], x[:, 1:])
+    h = pl.rmsnorm(x1, W[p + "post_attention_layernorm.weight"], c["eps"])
+    x2 = x1 + (torch.nn.functional.silu(h @ W[p + "mlp.gate_proj.weight"].t()) * (h @ W[p + "mlp.up_proj.weight"].t())) \
+        @ W[p + "mlp.down_proj.weight"].t()
+    want = pl.rmsnorm(x2, W["model.norm.weight"], c["eps"]) @ W["lm_head.weight"].t()
+    assert torch.allclose(with_ffn, want, atol=1e-5, rtol=1e-4)
+
+
 def test_tied_output_is_the_embedding_matrix():
     from conftest import TINY_B
     c, W = _tiny(TINY_B, 5)
@@ -192,8 +258,30 @@ def test_positions_shift_when_only_distances_count():
     a = pl.forward(c, W, toks, pos0=0)
     b = pl.forward(c, W, toks, pos0=37)
     assert torch.allclose(a, b, atol=2e-5)
-    # and a wrong pairing would break exactly this: rotate interleaved pairs instead
-    assert not torch.allclose(a, pl.forward(c, W, toks[::-1]), atol=1e-3)
+
+
+def test_the_shift_of_positions_shows_a_rotation_that_is_not_relative(monkeypatch):
+    """What the invariance above catches: a key rotated by another angle than a query at the same position
+    (here: keys not rotated at all, and keys rotated the other way round) makes the logits depend on where the
+    sequence starts.  The same shift on the faulty forms changes the logits by far more than the bound above."""
+    from conftest import TINY_A
+    c, W = _tiny(TINY_A, 6)
+    toks = [9, 8, 7, 6, 5, 4]
+    real = pl.apply_rope
+    H, Hkv = c["heads"], c["kv_heads"]
+    assert H != Hkv                                               # queries and keys are told apart by their head count
+
+    def keys_unrotated(x, positions, inv_freq):
+        return x.clone().to(torch.float32) if x.shape[1] == Hkv else real(x, positions, inv_freq)
+
+    def keys_backwards(x, positions, inv_freq):
+        return real(x, -positions if x.shape[1] == Hkv else positions, inv_freq)
+
+    for bad in (keys_unrotated, keys_backwards):
+        monkeypatch.setattr(pl, "apply_rope", bad)
+        a, b = pl.forward(c, W, toks, pos0=0), pl.forward(c, W, toks, pos0=37)
+        assert float((a - b).abs().max()) > 1e-3, bad.__name__
+    monkeypatch.setattr(pl, "apply_rope", real)
 
 
 def test_prefix_logits_do_not_depend_on_the_future():
@@ -215,6 +303,70 @@ def test_sampler_reference_cases():
     hits = sum(pl.sample(torch.tensor([10.0, 0.0, 0.0, 0.0]), 1.0, 0.5, rng) == 0 for _ in range(100))
     assert hits > 80
     assert pl.sample(torch.tensor([1.0, 1.0, 1.0]), 0.0, 0.9, rng) == 0          # first of equal maxima
+
+
+class _Fixed:
+    """Stands in for the generator: hands out the given numbers."""
+
+    def __init__(self, *values):
+        self.values = list(values)
+
+    def next_float(self):
+        return self.values.pop(0)
+
+
+def test_top_p_nucleus_vectors():
+    """src/sampler.c:77-135 on probabilities 0.15, 0.5, 0.05, 0.3 with top-p 0.9: candidates sorted by falling
+    probability (tokens 1, 3, 0, 2), cut at the first whose running sum exceeds 0.9 (token 0 at 0.95, included),
+    and the walk compares r * 0.95, the kept sum and neither 1 nor top-p, with the running sums."""
+    logits = torch.log(torch.tensor([0.15, 0.5, 0.05, 0.3]))
+    def pick(r):
+        return pl.sample(logits, 1.0, 0.9, _Fixed(r))
+    assert pick(0.0) == 1 and pick(0.52) == 1          # 0.52 * 0.95 = 0.494 < 0.5; unscaled it would be past 0.5
+    assert pick(0.53) == 3                             # 0.5035
+    assert pick(0.55) == 3                             # 0.5225; scaled by top-p (0.495) it would still be token 1
+    assert pick(0.84) == 3 and pick(0.85) == 0         # 0.798 < 0.8 <= 0.8075
+    assert pick(0.9999) == 0                           # token 2 lies beyond the cut and is never drawn
+    # top-p outside (0, 1): the plain walk over all tokens in index order
+    assert pl.sample(logits, 1.0, 1.0, _Fixed(0.66)) == 2 and pl.sample(logits, 1.0, 0.0, _Fixed(0.14)) == 0
+    # temperature divides the logits first: at 0.5 the probabilities are squared and renormalised
+    sq = torch.tensor([0.15, 0.5, 0.05, 0.3]) ** 2
+    sq = sq / sq.sum()
+    r = float(sq[1]) / float(sq[1] + sq[3]) * 0.999    # top-p 0.9 keeps tokens 1 and 3 (0.686 + 0.247 > 0.9)
+    assert pl.sample(logits, 0.5, 0.9, _Fixed(r)) == 1 and pl.sample(logits, 0.5, 0.9, _Fixed(r * 1.002)) == 3
+
+
+def test_top_p_cutoff_only_shortens_the_sort():
+    """Tokens below (1 - p) / (n - 1) are dropped before the sort (src/sampler.c:88-98).  They could not have
+    been kept anyway: were the first token whose running sum exceeds p (not the very first of all) below the
+    cutoff, everything from it on, at most n - 1 tokens none larger than it, would weigh less than 1 - p,
+    while the sum before it is at most p.  So the draw is the same as from the nucleus built over all tokens,
+    which is what pins the rule here: random distributions, with many tokens under the cutoff, against a
+    nucleus written without any cutoff."""
+    g = torch.Generator().manual_seed(5)
+    for trial in range(200):
+        n = int(torch.randint(2, 40, (1,), generator=g))
+        logits = torch.randn(n, generator=g) * float(torch.rand(1, generator=g) * 6 + 0.5)
+        top_p = float(torch.rand(1, generator=g) * 0.9 + 0.05)
+        r = float(torch.rand(1, generator=g))
+        p = torch.softmax(logits, 0)
+        if float(p.max()) < (1.0 - top_p) / (n - 1):
+            continue                                   # every token under the cutoff: the reference reads out of bounds
+        order = sorted(range(n), key=lambda i: (-float(p[i]), i))
+        cum, kept = 0.0, []
+        for i in order:
+            kept.append(i)
+            cum += float(p[i])
+            if cum > top_p:
+                break
+        acc, want = 0.0, kept[-1]
+        for i in kept:
+            acc += float(p[i])
+            if r * cum < acc:
+                want = i
+                break
+        below = int((p < (1.0 - top_p) / (n - 1)).sum())
+        assert pl.sample(logits, 1.0, top_p, _Fixed(r)) == want, (trial, n, top_p, below)
 
 
 def test_rng_is_xorshift64star():
