@@ -22,6 +22,8 @@
 // the 4 waves take 32-key blocks in turn and merge through shared memory; long contexts are
 // also split over gridDim.z and merged by attn_mfma_combine_kernel in a fixed order.
 #include "common.h"
+#include "attn_mfma.h"
+#include <mutex>
 
 #ifndef PROMPT_NG
 #define PROMPT_NG 0           // groups of 4 waves in a workgroup of the prompt form: 1, 2, or 0 = by the size of the launch
@@ -887,4 +889,53 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
     hipLaunchKernelGGL(attn_mfma_combine_kernel, dim3(n_tokens * H), dim3(64), 0, s, (bf16*)out, out_stride, part_o,
                        part_ml, H, hs, n_splits);
     return bn_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// decode form for callers that cannot allocate (declared and described in attn_mfma.h)
+// ---------------------------------------------------------------------------------------
+// The split partials of bn_attn_mfma_decode_static.  In host code this name is a stand-in, not a device
+// address: the address on the current GPU comes from hipGetSymbolAddress, once per device, and only that
+// pointer is ever handed to a kernel.
+static __device__ __align__(256) float scratch[BN_ATTN_STATIC_SCRATCH_FLOATS];
+
+static int static_scratch(float** ptr) {
+    static std::mutex lock;
+    static float* per_device[64] = {nullptr};         // each GPU holds its own copy of the array at its own address
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= 64) return BN_ERR_ARG;
+    std::lock_guard<std::mutex> hold(lock);
+    if (per_device[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (p == nullptr) return (int)hipErrorInvalidSymbol;
+        per_device[dev] = static_cast<float*>(p);
+    }
+    *ptr = per_device[dev];
+    return 0;
+}
+
+extern "C" int bn_attn_mfma_decode_static(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
+                                          const void* vt_pages, const int* block_table, int bt_stride,
+                                          const int* seq_lens, int n_seqs, int H, int Hkv, int hs, int GT, int window,
+                                          float scale, int n_splits, int chunk, const float* inv_freq, int rotate,
+                                          int write_kv, const int* by_length, hipStream_t s) {
+    if (!seq_lens || n_seqs <= 0 || H <= 0 || n_splits < 1 || n_splits > 64 || !bn_attn_mfma_supports(hs)) return BN_ERR_ARG;
+    float* part_o = nullptr;
+    float* part_ml = nullptr;
+    if (n_splits > 1) {
+        const unsigned long long rows = (unsigned long long)n_seqs * (unsigned)H * (unsigned)n_splits;
+        if (rows * (unsigned)(hs + 2) > BN_ATTN_STATIC_SCRATCH_FLOATS) return BN_ERR_SCRATCH;
+        float* base = nullptr;
+        const int rc = static_scratch(&base);
+        if (rc != 0) return rc;
+        part_o = base;                                // [rows, hs]
+        part_ml = base + rows * (unsigned)hs;         // [rows, 2]
+    }
+    return bn_attn_mfma(q, q_stride, out, out_stride, k_pages, vt_pages, block_table, bt_stride, seq_lens, nullptr,
+                        n_seqs, n_seqs, H, Hkv, hs, GT, window, scale, n_splits, chunk, part_o, part_ml, inv_freq, rotate,
+                        write_kv, nullptr, by_length, s);
 }

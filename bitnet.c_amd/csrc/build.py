@@ -25,7 +25,7 @@ ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 SOURCES = ("elementwise", "rope_kv", "attn_rows", "attn_mfma", "gemm_tiled", "gemm_mfma", "skinny_gemm", "splitk_gemm", "sampling")
-HEADERS = ("common.h",)
+HEADERS = ("common.h", "attn_mfma.h")
 
 _libs = {}
 _lock = threading.Lock()
