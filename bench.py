@@ -103,7 +103,7 @@ def main() -> int:
     engine = bn.Engine(model, max_tokens=max(max_batch * per_seq, 4096, PREFILL + 64), max_seq_len=CONTEXT)
     L, H, Hkv, hs = cfg.num_hidden_layers, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
     kv_bytes_per_token = 2 * L * Hkv * hs * 2
-    weight_bytes = model.weight_bytes() - (0 if cfg.tie_word_embeddings else model.embedding.numel() * 2)
+    weight_bytes = model.weight_bytes()      # every weight a decode step reads once (no embedding table unless it is tied)
     rnd = random.Random(args.seed + 1)
 
     def sync():
@@ -154,6 +154,7 @@ def main() -> int:
             lg = engine.step([bn.StepEntry(slots[j], [last[j]], [0]) for j in range(batch)])
             last = ops.argmax(lg).cpu().tolist()
 
+        engine.prepare_decode(batch)          # as generation does at a batch's start: no capture inside the clock
         for _ in range(warmup):
             one()
         sync()
@@ -174,14 +175,20 @@ def main() -> int:
     value = args.batch / step_s
     bytes_step = weight_bytes + ctx_tokens * kv_bytes_per_token
     achieved = bytes_step / step_s / 1e9
-    print(f"[bench] decode b{args.batch}: {step_s * 1e3:.3f} ms/step, {value:.1f} tok/s, {achieved:.0f} GB/s",
-          file=sys.stderr, flush=True)
+    print(f"[bench] decode b{args.batch}: {step_s * 1e3:.3f} ms/step, {value:.1f} tok/s, {bytes_step / 1e9:.2f} GB a step, "
+          f"{achieved:.0f} GB/s = {achieved / HBM_GBS:.3f} of {HBM_GBS:.0f}", file=sys.stderr, flush=True)
     points = {}
     if not args.no_points:
         for b in (1, 64):
-            s_b, _ = decode(b, max(16, args.steps // 2), args.warmup)
+            s_b, ctx_b = decode(b, max(16, args.steps // 2), args.warmup)
+            bytes_b = weight_bytes + ctx_b * kv_bytes_per_token
+            gbs = bytes_b / s_b / 1e9
             points[f"decode_b{b}"] = round(b / s_b, 1)
-            print(f"[bench] decode b{b}: {s_b * 1e3:.3f} ms/step, {b / s_b:.1f} tok/s", file=sys.stderr, flush=True)
+            points[f"decode_b{b}_ms"] = round(s_b * 1e3, 4)
+            points[f"decode_b{b}_gbs"] = round(gbs, 1)
+            points[f"decode_b{b}_frac"] = round(gbs / HBM_GBS, 4)
+            print(f"[bench] decode b{b}: {s_b * 1e3:.3f} ms/step, {b / s_b:.1f} tok/s, {bytes_b / 1e9:.2f} GB a step, "
+                  f"{gbs:.0f} GB/s = {gbs / HBM_GBS:.3f} of {HBM_GBS:.0f}", file=sys.stderr, flush=True)
 
     rec = {
         "metric": f"decode tok/s @ batch {args.batch} ({shape['name']}, bf16)", "value": round(value, 1), "unit": "tok/s",
@@ -197,7 +204,7 @@ def main() -> int:
                    "prefill_tokens": PREFILL, "parallelism": "none (1 GPU)"},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_GBS, 4)},
+                     "frac": round(achieved / HBM_GBS, 4), "gb_per_step": round(bytes_step / 1e9, 3)},
         "points": points,
     }
     print(json.dumps(rec), flush=True)

@@ -7,7 +7,9 @@ same kind of storage (same kv heads, head size and window) form a *group* with s
 a page pool and block tables of its own, so a group that keeps a window of keys gives
 pages back while a sequence grows and a group that keeps all keys does not.  Beside the
 pages there is a state area: for every entry that asks for it, a tensor of fixed shape
-per slot, zero when a slot is handed out.
+per slot, zero when a slot is handed out, with one more row at index `padding_slot` that no
+sequence owns: the padding rows of a captured step address it, so that a mixer which reads
+and writes its state by the step's device-side slot ids needs no special case for them.
 
 The reference gives each request a session with contiguous [layer][position][kv_dim]
 arrays and a zeroed recurrent state (src/model_session.c:332-368, src/session.c:113-172)
@@ -24,9 +26,10 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
+from ..csrc.build import header_constant
 from ..parts.base import CacheNeed, KVNeed, KVView
 
-PAGE = 64
+PAGE = header_constant("BN_PAGE")        # positions per page: defined once, in csrc/common.h
 
 
 class CacheError(RuntimeError):
@@ -88,6 +91,7 @@ class PagedCache:
         if max_tokens < PAGE:
             raise CacheError(f"max_tokens {max_tokens} is below one page ({PAGE})")
         self.tables_version = 0          # grows whenever any sequence's list of pages changes
+        self._slot_version: Dict[int, int] = {}   # slot -> tables_version at the last change of its pages
         self.n_pages = max_tokens // PAGE
         self.max_slots = int(max_slots) if max_slots else self.n_pages
         self.dtype, self.device = dtype, device
@@ -127,7 +131,23 @@ class PagedCache:
                     shape = shape[:3] + (g.need.head_dim, PAGE)
                 g.v = torch.zeros(shape, dtype=dtype, device=device)
             for i, sn in self._state_needs.items():
-                self.states[i] = torch.zeros((self.max_slots,) + tuple(sn.shape), dtype=sn.dtype, device=device)
+                self.states[i] = torch.zeros((self.max_slots + 1,) + tuple(sn.shape), dtype=sn.dtype, device=device)
+
+    @property
+    def padding_slot(self) -> int:
+        """The row of the state area that belongs to no sequence."""
+        return self.max_slots
+
+    def _touch(self, slot: int) -> None:
+        self.tables_version += 1
+        self._slot_version[slot] = self.tables_version
+
+    def slot_version(self, slot: int) -> int:
+        """A number that changes whenever the slot's pages change or the slot is handed out again."""
+        return self._slot_version[slot]
+
+    def pages_of(self, group: int, slot: int) -> List[int]:
+        return self.groups[group].pages[slot]
 
     # ---- slots ------------------------------------------------------------------
     def alloc_slot(self) -> int:
@@ -135,7 +155,7 @@ class PagedCache:
             raise CacheFull(f"all {self.max_slots} sequence slots are in use")
         s = self._free_slots.pop()
         self._len[s] = 0
-        self.tables_version += 1
+        self._touch(s)
         for g in self.groups:
             g.pages[s] = []
         for t in self.states.values():
@@ -145,7 +165,7 @@ class PagedCache:
     def free_slot(self, slot: int) -> None:
         if slot not in self._len:
             raise CacheError(f"slot {slot} is freed but is not in use")
-        self.tables_version += 1
+        self._touch(slot)
         for g in self.groups:
             g.pool.give_back([p for p in g.pages.pop(slot) if p >= 0])
         del self._len[slot]
@@ -185,7 +205,20 @@ class PagedCache:
         for g, s, need in plan:
             if need:
                 g.pages[s].extend(g.pool.take(need))
-                self.tables_version += 1
+                self._touch(s)
+
+    def unreserve(self, slots: Sequence[int]) -> None:
+        """Gives back what reserve() took for a step that did not run: every page beyond the slot's length."""
+        for s in slots:
+            if s not in self._len:
+                continue
+            keep = (self._len[s] + PAGE - 1) // PAGE
+            for g in self.groups:
+                pl = g.pages[s]
+                if len(pl) > keep:
+                    g.pool.give_back([p for p in pl[keep:] if p >= 0])
+                    del pl[keep:]
+                    self._touch(s)
 
     def commit(self, slots: Sequence[int], n_new: Sequence[int]) -> None:
         """The step has run: lengths grow; groups that keep a window give back the pages that
@@ -200,7 +233,7 @@ class PagedCache:
                         if pl[i] >= 0 and PAGE * i + PAGE - 1 < first_visible:
                             g.pool.give_back([pl[i]])
                             pl[i] = -1
-                            self.tables_version += 1
+                            self._touch(s)
 
     # ---- views ------------------------------------------------------------------
     def group_of(self, entry: int) -> Optional[int]:

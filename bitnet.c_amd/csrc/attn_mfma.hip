@@ -25,10 +25,6 @@
 #include "attn_mfma.h"
 #include <mutex>
 
-#ifndef PROMPT_NG
-#define PROMPT_NG 0           // groups of 4 waves in a workgroup of the prompt form: 1, 2, or 0 = by the size of the launch
-#endif
-
 static int compute_units() {
     static int n[64] = {0};                 // per device
     int dev = 0;
@@ -65,16 +61,17 @@ struct MfmaArgs {
     // decode form only.  rotate != 0: q (and the new key) arrive unrotated and are rotated here,
     // angle = position * inv_freq[i], pairs (i, i + HS/2).  write_kv != 0: the workgroup whose keys
     // include the new position stores the new key (rotated) and value into the pages first.
-    // counters != null: the last workgroup of a (sequence, kv head) to finish merges the splits
-    // itself (no combine launch); the counters are zero between launches.
     const float* inv_freq;
     int rotate, write_kv;
-    int* counters;
     // by_length != null: the sequences ordered by length, longest first.  Workgroups are handed out
     // in that order, every other run of `order_period` sequences backwards: when the launch puts
     // two workgroups on every CU, the ones that share a CU are then a long and a short sequence.
     const int* by_length;
     int order_period;
+    // max_len != null (decode form, n_splits > 1): the longest sequence's key count lives in device memory and
+    // the keys per split follow from it (bn_split_chunk) instead of from `chunk`: a captured launch then adapts
+    // its splits to the lengths of every replay.
+    const int* max_len;
 };
 
 __device__ __forceinline__ bf16x8 ld16(const bf16* p) {
@@ -626,7 +623,6 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
     __shared__ float m_s[4][16], l_s[4][16];
     __shared__ float o_s[4][HS][17];                    // [wave][dim][col], padded
     __shared__ float cos_s[HALF], sin_s[HALF];
-    __shared__ int ticket_s;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
     const int G = a.H / a.Hkv, GT = a.GT;
@@ -654,7 +650,8 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
     const bool ok = n < GT && hg < G && L > 0;
     const int head = kvh * G + hg;
     const int lo_key = a.window > 0 ? max(0, L - a.window) : 0;
-    const int k_lo = max(lo_key, split * a.chunk), k_hi = min(L, (split + 1) * a.chunk);   // [k_lo, k_hi)
+    const int chunk = a.max_len ? bn_split_chunk(uniform_load(a.max_len, 0), a.n_splits) : a.chunk;
+    const int k_lo = max(lo_key, split * chunk), k_hi = min(L, (split + 1) * chunk);       // [k_lo, k_hi)
     const bf16* row = a.q + (size_t)seq * a.q_stride;
 
     if (a.rotate && L > 0) {
@@ -760,46 +757,6 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
             if (dim == 0) { a.part_ml[prow * 2] = (M == -INFINITY) ? -INFINITY : M * LN2; a.part_ml[prow * 2 + 1] = den; }
         }
     }
-    if (a.n_splits == 1 || a.counters == nullptr) return;
-    // the last workgroup of this (sequence, kv head, head tile) to arrive merges all splits, in split order
-    __threadfence();
-    __syncthreads();
-    int* counter = a.counters + ((size_t)seq * gridDim.x + blockIdx.x);
-    if (threadIdx.x == 0) ticket_s = atomicAdd(counter, 1);
-    __syncthreads();
-    if (ticket_s != a.n_splits - 1) return;
-    __threadfence();
-    if (threadIdx.x == 0) *counter = 0;                     // ready for the next launch
-    for (int idx = threadIdx.x; idx < HS * GT; idx += 256) {
-        const int col = idx / HS, dim = idx - col * HS;
-        const int hg2 = ht * GT + col;
-        if (hg2 >= G) continue;
-        const int hd = kvh * G + hg2;
-        const size_t prow = ((size_t)seq * a.H + hd) * a.n_splits;
-        const float* ml = a.part_ml + prow * 2;
-        float M = -INFINITY;
-        for (int sp = 0; sp < a.n_splits; ++sp) M = fmaxf(M, ml[2 * sp]);
-        float num = 0.f, den = 0.f;
-        if (M != -INFINITY) {
-            for (int s0 = 0; s0 < a.n_splits; s0 += 8) {
-                float v[8], wgt[8], ls[8];
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const bool in = s0 + j < a.n_splits;
-                    v[j] = in ? a.part_o[(prow + s0 + j) * HS + dim] : 0.f;
-                    wgt[j] = in ? ml[2 * (s0 + j)] : -INFINITY;
-                    ls[j] = in ? ml[2 * (s0 + j) + 1] : 0.f;
-                }
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float e = wgt[j] == -INFINITY ? 0.f : expf(wgt[j] - M);
-                    num = fmaf(e, v[j], num);
-                    den = fmaf(e, ls[j], den);
-                }
-            }
-        }
-        a.out[(size_t)seq * a.out_stride + (size_t)hd * HS + dim] = __float2bfloat16(den > 0.f ? num / den : 0.f);
-    }
 }
 
 // out[row, d] = sum_s e^{m_s - m} o_s[d] / sum_s e^{m_s - m} l_s: one wave per row, the weights
@@ -823,10 +780,14 @@ __global__ __launch_bounds__(64) void attn_mfma_combine_kernel(bf16* __restrict_
         const float* po = part_o + (size_t)row * n_splits * hs + d;
         for (int s0 = 0; s0 < n_splits; s0 += 8) {
             float v[8];
+            float wj[8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] = (s0 + j < n_splits) ? po[(size_t)(s0 + j) * hs] : 0.f;   // loads first
+            for (int j = 0; j < 8; ++j) {                                  // loads first; a split without keys is not read
+                wj[j] = __shfl(w, min(s0 + j, 63), BN_WAVE);
+                v[j] = (s0 + j < n_splits && wj[j] != 0.f) ? po[(size_t)(s0 + j) * hs] : 0.f;
+            }
 #pragma unroll
-            for (int j = 0; j < 8; ++j) num = fmaf(__shfl(w, min(s0 + j, 63), BN_WAVE), v[j], num);      // then split order
+            for (int j = 0; j < 8; ++j) num = fmaf(wj[j], v[j], num);      // then split order
         }
         out[(size_t)tok * out_stride + (size_t)head * hs + d] = __float2bfloat16(num * inv);
     }
@@ -842,12 +803,13 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
                             const void* vt_pages, const int* block_table, int bt_stride, const int* seq_lens,
                             const int* tiles, int n_tiles, int n_tokens, int H, int Hkv, int hs, int GT,
                             int window, float scale, int n_splits, int chunk, float* part_o, float* part_ml,
-                            const float* inv_freq, int rotate, int write_kv, int* counters, const int* by_length,
-                            hipStream_t s) {
+                            const float* inv_freq, int rotate, int write_kv, const int* by_length,
+                            const int* max_len, hipStream_t s) {
     if (!bn_attn_mfma_supports(hs) || n_tiles <= 0 || n_tokens <= 0 || H <= 0 || Hkv <= 0 || H % Hkv) return BN_ERR_ARG;
     if (GT <= 0 || GT > 16 || (GT & (GT - 1)) || window < 0 || n_splits < 1 || n_splits > 64) return BN_ERR_ARG;
-    if (n_splits > 1 && (chunk <= 0 || chunk % BN_PAGE || !part_o || !part_ml)) return BN_ERR_ARG;
+    if (n_splits > 1 && (!part_o || !part_ml || (!max_len && (chunk <= 0 || chunk % BN_PAGE)))) return BN_ERR_ARG;
     if (!tiles && !seq_lens) return BN_ERR_ARG;
+    if (max_len && tiles) return BN_ERR_ARG;                               // decode form only
     if (q_stride % 8 || out_stride % 4 || (((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)vt_pages) & 15) ||
         ((uintptr_t)out & 7))
         return BN_ERR_ARG;
@@ -862,7 +824,8 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
     a.q_stride = q_stride; a.out_stride = out_stride; a.bt_stride = bt_stride;
     a.H = H; a.Hkv = Hkv; a.GT = GT; a.window = window; a.scale = scale;
     a.n_splits = n_splits; a.chunk = n_splits > 1 ? chunk : 0x40000000;
-    a.inv_freq = inv_freq; a.rotate = rotate; a.write_kv = write_kv; a.counters = counters;
+    a.inv_freq = inv_freq; a.rotate = rotate; a.write_kv = write_kv;
+    a.max_len = n_splits > 1 ? max_len : nullptr;
     // the order matters only when the launch holds more workgroups than CUs and no sequence is split
     const int wgs_per_seq = Hkv * n_head_tiles;
     a.by_length = (!tiles && n_splits == 1 && (long long)n_tiles * wgs_per_seq > compute_units()) ? by_length : nullptr;
@@ -872,8 +835,7 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
         // Two wave groups halve the chain of key blocks of a workgroup but not the work of its CU:
         // they pay (measured 19 % at 1,024 tokens of the 8B shape) only while there are no more
         // workgroups than CUs, so that each has a CU to itself.
-        int ng = PROMPT_NG;
-        if (ng == 0) ng = ((long long)grid.x * grid.y <= compute_units()) ? 2 : 1;
+        const int ng = ((long long)grid.x * grid.y <= compute_units()) ? 2 : 1;
         if (hs == 64 && ng == 2) hipLaunchKernelGGL((attn_mfma_prompt_kernel<64, 4, 2>), grid, dim3(512), 0, s, a);
         else if (hs == 64) hipLaunchKernelGGL((attn_mfma_prompt_kernel<64, 4, 1>), grid, dim3(256), 0, s, a);
         else if (ng == 2) hipLaunchKernelGGL((attn_mfma_prompt_kernel<128, 2, 2>), grid, dim3(512), 0, s, a);
@@ -885,7 +847,7 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
     if (hs == 64) hipLaunchKernelGGL(attn_mfma_decode_kernel<64>, grid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL(attn_mfma_decode_kernel<128>, grid, dim3(256), 0, s, a);
     int rc = bn_launch_status();
-    if (rc != 0 || n_splits == 1 || counters != nullptr) return rc;
+    if (rc != 0 || n_splits == 1) return rc;
     hipLaunchKernelGGL(attn_mfma_combine_kernel, dim3(n_tokens * H), dim3(64), 0, s, (bf16*)out, out_stride, part_o,
                        part_ml, H, hs, n_splits);
     return bn_launch_status();
@@ -937,5 +899,5 @@ extern "C" int bn_attn_mfma_decode_static(const void* q, int q_stride, void* out
     }
     return bn_attn_mfma(q, q_stride, out, out_stride, k_pages, vt_pages, block_table, bt_stride, seq_lens, nullptr,
                         n_seqs, n_seqs, H, Hkv, hs, GT, window, scale, n_splits, chunk, part_o, part_ml, inv_freq, rotate,
-                        write_kv, nullptr, by_length, s);
+                        write_kv, by_length, nullptr, s);
 }

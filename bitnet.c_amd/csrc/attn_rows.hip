@@ -37,6 +37,8 @@ struct AttnArgs {
     int n_splits, chunk;      // keys per split, a multiple of BN_PAGE
     int v_transposed;         // V pages are [page, kv_head, hs, BN_PAGE]
     float scale;
+    const int* max_len;       // != null (decode form, n_splits > 1): the longest sequence's key count in device
+                              // memory; the keys per split follow from it (bn_split_chunk) instead of from `chunk`
 };
 
 template <typename T> struct Vec4;
@@ -112,8 +114,9 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
     if (pos0 >= 0 && n_tok > 0) {
         hi = pos0 + n_tok;                                        // exclusive
         lo = a.window > 0 ? max(0, pos0 + 1 - a.window) : 0;      // first key of the first row
-        lo = max(lo, split * a.chunk);
-        hi = min(hi, (split + 1) * a.chunk);
+        const int chunk = a.max_len ? bn_split_chunk(*a.max_len, a.n_splits) : a.chunk;
+        lo = max(lo, split * chunk);
+        hi = min(hi, (split + 1) * chunk);
     }
 
     // phase C ownership: thread -> (jp, dp): keys jp, jp+JP, ...; output dims 2dp, 2dp+1
@@ -357,14 +360,16 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
                             int bt_stride, const int* seq_lens, const int* tiles, int n_tiles,
                             int n_tokens, int H, int Hkv, int hs, int RT, int GT, int window,
                             float scale, int n_splits, int chunk, float* part_o, float* part_ml,
-                            int v_transposed, hipStream_t s) {
+                            int v_transposed, const int* max_len, hipStream_t s) {
     if (n_tiles <= 0 || n_tokens <= 0 || H <= 0 || Hkv <= 0 || H % Hkv) return BN_ERR_ARG;
     if (hs < 2 || hs > 256 || hs % 2) return BN_ERR_ARG;
     if (GT <= 0 || GT > RT || (GT & (GT - 1)) || RT > 16 || (RT & (RT - 1))) return BN_ERR_ARG;
     if (n_splits < 1 || window < 0) return BN_ERR_ARG;
-    if (n_splits > 1 && (chunk <= 0 || chunk % BN_PAGE || !part_o || !part_ml)) return BN_ERR_ARG;
+    if (n_splits > 1 && (!part_o || !part_ml || (!max_len && (chunk <= 0 || chunk % BN_PAGE)))) return BN_ERR_ARG;
     if (!tiles && !seq_lens) return BN_ERR_ARG;
+    if (max_len && tiles) return BN_ERR_ARG;
     AttnArgs a;
+    a.max_len = n_splits > 1 ? max_len : nullptr;
     a.q = q; a.out = out; a.k_pages = k_pages; a.v_pages = v_pages;
     a.block_table = block_table; a.seq_lens = seq_lens; a.tiles = tiles;
     a.part_o = part_o; a.part_ml = part_ml;

@@ -31,6 +31,17 @@ _libs = {}
 _lock = threading.Lock()
 
 
+def header_constant(name: str, header: str = "common.h") -> int:
+    """The integer that `#define name value` of a header gives: sizes that the kernels and the host code
+    share (the cache's page length) are written down once, in the header."""
+    import re
+    with open(os.path.join(HERE, header)) as f:
+        m = re.search(rf"^#define\s+{re.escape(name)}\s+\(?(-?\d+)u?\)?\s*(?://.*)?$", f.read(), re.M)
+    if m is None:
+        raise BuildError(f"{header} does not define {name} as an integer")
+    return int(m.group(1))
+
+
 class BuildError(RuntimeError):
     pass
 

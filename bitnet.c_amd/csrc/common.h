@@ -6,7 +6,10 @@
 #include <stdint.h>
 
 #define BN_WAVE 64
-#define BN_PAGE 64            // tokens per cache page; the Python side uses the same number
+#define BN_PAGE 64            // tokens per cache page; the Python side reads this line (csrc/build.py: header_constant)
+// Decode attention splits a sequence's keys over workgroups in runs of at least this many pages: shorter
+// runs cost more in merging than they gain in parallelism (measured at batch 1, 8 and 64 of an 8B shape).
+#define BN_SPLIT_MIN_PAGES 4
 
 // error codes returned by the extern "C" entry points (0 = ok, >0 = hipError_t)
 #define BN_ERR_ARG   (-1)     // an argument the kernel cannot take (size, alignment)
@@ -65,6 +68,15 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
     float t = scratch[0];
     for (int i = 1; i < nw; ++i) t = fmaxf(t, scratch[i]);
     return t;
+}
+
+// Keys per split of a decode step whose longest sequence holds max_len keys, cut into n_splits runs of whole
+// pages (the same rule as ops.decode_splits): the kernels use it when the length arrives in device memory.
+__host__ __device__ __forceinline__ int bn_split_chunk(int max_len, int n_splits) {
+    const int pages = max_len > 0 ? (max_len + BN_PAGE - 1) / BN_PAGE : 1;
+    int per = (pages + n_splits - 1) / n_splits;
+    if (per < BN_SPLIT_MIN_PAGES) per = BN_SPLIT_MIN_PAGES;
+    return per * BN_PAGE;
 }
 
 static inline int bn_launch_status() { return (int)hipGetLastError(); }

@@ -21,10 +21,9 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Callable, List, Optional, Sequence
 
+from ..cache import PAGE
 from ..sampling.sampler import SamplingParams, SequenceSampler
 from .step import StepEntry
-
-PAGE = 64
 
 
 @dataclass
@@ -90,8 +89,11 @@ def generate(engine, requests: Sequence[Request], sample_fn: Callable, batch_siz
     batches, errors = plan_batches(requests, batch_size, cap, engine.max_seq_len)
     for i, msg in errors.items():
         results[i].finish = msg
+    prepare = getattr(engine, "prepare_decode", None)
     for batch in batches:
         live: List[_Live] = []
+        if prepare is not None and any(requests[i].max_new_tokens > 1 for i in batch):
+            prepare(len(batch))          # whatever the decode steps will need is made now, not between two tokens
         try:
             for i in batch:
                 r = requests[i]

@@ -40,8 +40,12 @@ class StepContext:
     """Device-side description of one step, shared by all parts."""
 
     def __init__(self, device, act_dtype, tokens, positions, seq_index, seq_lens, want_rows, slots_dev,
-                 is_decode, slots, n_new, pos0, by_length=None):
+                 is_decode, slots, n_new, pos0, by_length=None, max_len_dev=None, captured=False):
         self.device, self.act_dtype = device, act_dtype
+        # captured: the step is being recorded into a HIP graph and will be replayed with other sequences: only
+        # the device tensors (tokens, positions, seq_lens, slot_ids, ...) are valid then, the host lists are not.
+        # max_len_dev: in a captured step, a device int32 with the longest sequence's key count of each replay
+        self.captured, self.max_len_dev = captured, max_len_dev
         # decode steps: the rows ordered by sequence length, longest first (a hint for kernels that
         # balance their workgroups by it; None = no hint)
         self.by_length = by_length
@@ -109,6 +113,9 @@ def _by_length(lens) -> List[int]:
     return sorted(range(len(lens)), key=lambda i: (-lens[i], i))
 
 
+MAX_GRAPH_ROWS = 64       # decode steps of more sequences than this run eagerly
+
+
 def _bucket(n: int) -> int:
     b = 1
     while b < n:
@@ -117,38 +124,40 @@ def _bucket(n: int) -> int:
 
 
 class _DecodeGraph:
-    """A captured decode step for up to `rows` sequences whose block tables have `width`
-    columns.  Inputs live in one int32 buffer that is refilled before every replay."""
+    """A captured decode step for up to `rows` sequences.  The block tables are as wide as the engine's longest
+    sequence and the split plan of attention follows the longest sequence of each replay through a device-side
+    integer, so a graph is made for a number of rows and nothing else: no step of a generation waits for a
+    capture because a sequence has grown.  The step's integers live in pinned buffers that are refilled
+    before every replay; a row of the block tables is rewritten only when its sequence's pages have changed."""
 
-    def __init__(self, engine: "Engine", rows: int, width: int):
-        self.rows, self.width = rows, width
-        dev = engine.device
-        n_groups = len(engine.cache.groups)
-        self.n_ints = 6 * rows + n_groups * rows * width
-        self.host = torch.zeros(self.n_ints, dtype=torch.int32).pin_memory()
+    N_FIELDS = 7            # tokens, positions, sequence index, lengths, wanted rows, order by length, slot ids
+
+    def __init__(self, engine: "Engine", rows: int):
+        self.rows, self.width = rows, engine.max_pages
+        dev, cache = engine.device, engine.cache
+        n_groups = len(cache.groups)
+        self.host = torch.zeros(self.N_FIELDS * rows + 1, dtype=torch.int32).pin_memory()
         self.host_np = self.host.numpy()                      # the same memory
         self.host_np[2 * rows:3 * rows] = range(rows)         # row b is sequence b
         self.host_np[4 * rows:5 * rows] = range(rows)         # wanted rows: all
-        self._tables_key = None
-        self.dev = torch.zeros(self.n_ints, dtype=torch.int32, device=dev)
+        self.dev = torch.zeros(self.host.numel(), dtype=torch.int32, device=dev)
+        self.host_tables = torch.zeros((max(n_groups, 1), rows, self.width), dtype=torch.int32).pin_memory()
+        self.tables_np = self.host_tables.numpy()
+        self.dev_tables = torch.zeros(self.host_tables.shape, dtype=torch.int32, device=dev)
+        self.row_keys = [None] * rows                         # (slot, version of its pages) that a table row holds
+        self.tables_dirty = True
         self.copied = torch.cuda.Event()
         self.copied.record()
-        o = 0
-
-        def take(n):
-            nonlocal o
-            v = self.dev[o:o + n]
-            o += n
-            return v
-
-        self.tokens, self.positions, self.seq_index = take(rows), take(rows), take(rows)
-        self.seq_lens, self.want, self.by_length = take(rows), take(rows), take(rows)
-        self.tables = {g: take(rows * width).view(rows, width) for g in range(n_groups)}
-        views = [engine.cache.view(i, self.tables, width * PAGE) for i in range(len(engine.model.plan.schedule))]
+        f = [self.dev[k * rows:(k + 1) * rows] for k in range(self.N_FIELDS)]
+        self.tokens, self.positions, self.seq_index, self.seq_lens, self.want, self.by_length, self.slot_ids = f
+        self.max_len = self.dev[self.N_FIELDS * rows:self.N_FIELDS * rows + 1]
+        self.tables = {g: self.dev_tables[g] for g in range(n_groups)}
+        views = [cache.view(i, self.tables, self.width * PAGE) for i in range(len(engine.model.plan.schedule))]
         self.ctx = StepContext(dev, engine.model.dtype, self.tokens, self.positions, self.seq_index, self.seq_lens,
-                               self.want, None, True, [-1] * rows, [1] * rows, [0] * rows, by_length=self.by_length)
-        # padding rows everywhere: the warm-up and the capture run touch no sequence's pages
-        self.fill([-1] * rows, [0] * rows, [0] * rows, engine)
+                               self.want, self.slot_ids, True, [-1] * rows, [1] * rows, [0] * rows,
+                               by_length=self.by_length, max_len_dev=self.max_len, captured=True)
+        # padding rows everywhere: the warm-up and the capture run touch no sequence's pages or state
+        self.fill([], [], [], engine)
         self.upload()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -157,33 +166,38 @@ class _DecodeGraph:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
+        with torch.cuda.graph(self.graph, pool=engine.graph_pool):
             self.logits = engine.model.forward(self.ctx, views)
 
     def fill(self, slots, tokens, lens_after, engine):
-        """Writes the step's integers into the pinned buffer.  The block tables are rewritten only
-        when the slots or any sequence's pages have changed since the last fill."""
-        rows, h = self.rows, self.host_np
+        """Writes the step's integers into the pinned buffers."""
+        rows, h, cache = self.rows, self.host_np, engine.cache
         self.copied.synchronize()
         n = len(slots)
         h[0:rows] = 0
         h[0:n] = tokens
         h[rows:2 * rows] = -1                                         # padding rows: position -1
-        h[rows:rows + n] = [l - 1 if s >= 0 else -1 for s, l in zip(slots, lens_after)]
-        h[3 * rows:4 * rows] = 0
-        h[3 * rows:3 * rows + n] = [max(l, 0) for l in lens_after]
+        h[rows:rows + n] = [l - 1 for l in lens_after]
+        h[3 * rows:4 * rows] = 0                                      # and no keys
+        h[3 * rows:3 * rows + n] = lens_after
         h[5 * rows:6 * rows] = _by_length(list(lens_after) + [0] * (rows - n))
-        key = (tuple(slots), engine.cache.tables_version)
-        if key != self._tables_key:
-            o = 6 * rows
-            for g in range(len(engine.cache.groups)):
-                bt = engine.cache.block_table(g, list(slots) + [-1] * (rows - n), self.width)
-                h[o:o + rows * self.width] = bt[:, :self.width].reshape(-1).numpy()
-                o += rows * self.width
-            self._tables_key = key
+        h[6 * rows:7 * rows] = cache.padding_slot                     # their state is the row that no sequence owns
+        h[6 * rows:6 * rows + n] = slots
+        h[7 * rows] = max(lens_after) if n else 0
+        for r, s in enumerate(slots):
+            key = (s, cache.slot_version(s))
+            if key != self.row_keys[r]:
+                for g in range(len(cache.groups)):
+                    pl = cache.pages_of(g, s)
+                    self.tables_np[g, r, :len(pl)] = pl
+                self.row_keys[r] = key
+                self.tables_dirty = True
 
     def upload(self):
         self.dev.copy_(self.host, non_blocking=True)
+        if self.tables_dirty:
+            self.dev_tables.copy_(self.host_tables, non_blocking=True)
+            self.tables_dirty = False
         self.copied.record()
 
     def run(self):
@@ -205,13 +219,19 @@ class Engine:
         if model.plan.max_positions:
             limit = min(limit, model.plan.max_positions)
         self.max_seq_len = min(limit, max_seq_len) if max_seq_len else limit
+        self.max_pages = (self.max_seq_len + PAGE - 1) // PAGE
         self.vocab_size = model.plan.vocab_size
-        ops.attention_counters(self.device)          # made before any graph capture
-        # a mixer that keeps a state addresses it by the host's slot list, which a replayed graph
-        # cannot see: such models run their decode steps eagerly
-        self.use_graphs = use_graphs and all(n.state is None for n in needs)
+        # A replayed graph sees device memory only.  A mixer that keeps a state can decode under graphs when it
+        # addresses the state by the step's device-side slot ids (StateNeed.device_addressed); one that walks the
+        # host's slot list cannot, and a model with such a mixer runs its decode steps eagerly.
+        self.use_graphs = use_graphs and all(n.state is None or n.state.device_addressed for n in needs)
         self.tap = None                     # see StepContext.tap; while it is set, steps run without graphs
-        self._graphs: Dict[tuple, _DecodeGraph] = {}
+        # One captured step per number of rows (1, 2, 4 .. MAX_GRAPH_ROWS): at most seven, made at a batch's
+        # start (prepare_decode) or at first use.  They share one memory pool: what a capture frees, the next
+        # reuses, and each keeps only its own inputs and logits ([rows, vocab] float32).
+        self._graphs: Dict[int, _DecodeGraph] = {}
+        self.graph_pool = torch.cuda.graph_pool_handle() if self.use_graphs else None
+        self.graphs_built = 0
         self.steps_run = 0
 
     # ---- construction ---------------------------------------------------------------
@@ -276,10 +296,14 @@ class Engine:
         except CacheFull as err:
             raise StepError(str(err)) from None
         is_decode = all(n == 1 for n in n_new)
-        if is_decode and self.use_graphs and self.tap is None and len(entries) <= 64:
-            logits = self._step_graph(entries, slots, pos0)
-        else:
-            logits = self._step_eager(entries, slots, n_new, pos0, is_decode)
+        try:
+            if is_decode and self.use_graphs and self.tap is None and len(entries) <= MAX_GRAPH_ROWS:
+                logits = self._step_graph(entries, slots, pos0)
+            else:
+                logits = self._step_eager(entries, slots, n_new, pos0, is_decode)
+        except BaseException:
+            self.cache.unreserve(slots)          # the step did not happen: its pages go back
+            raise
         self.cache.commit(slots, n_new)
         self.steps_run += 1
         return logits
@@ -321,15 +345,28 @@ class Engine:
         views = [self.cache.view(i, d_tables, max_len) for i in range(len(self.model.plan.schedule))]
         return self.model.forward(ctx, views)
 
+    def prepare_decode(self, n_seqs: int) -> None:
+        """Captures, now, every graph that decode steps of up to n_seqs sequences will replay (the batch
+        shrinks as sequences end), so that no later step waits for a capture.  Does nothing for what is there."""
+        if not self.use_graphs or self.tap is not None:
+            return
+        rows = _bucket(min(max(n_seqs, 1), MAX_GRAPH_ROWS))
+        while rows >= 1:
+            self._graph_for(rows)
+            rows //= 2
+
+    def _graph_for(self, rows: int) -> _DecodeGraph:
+        g = self._graphs.get(rows)
+        if g is None:
+            g = _DecodeGraph(self, rows)
+            self._graphs[rows] = g
+            self.graphs_built += 1
+        return g
+
     def _step_graph(self, entries, slots, pos0):
         B = len(entries)
         lens_after = [p + 1 for p in pos0]
-        width = _bucket(max((l + PAGE - 1) // PAGE for l in lens_after))
-        key = (_bucket(B), width)
-        g = self._graphs.get(key)
-        if g is None:
-            g = _DecodeGraph(self, key[0], width)
-            self._graphs[key] = g
+        g = self._graph_for(_bucket(B))
         g.fill(slots, [int(e.tokens[0]) for e in entries], lens_after, self)
         g.upload()
         logits = g.run()

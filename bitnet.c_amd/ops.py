@@ -17,7 +17,8 @@ import torch
 
 from .csrc import build as _build
 
-PAGE = 64                     # tokens per cache page (BN_PAGE in csrc/common.h)
+PAGE = _build.header_constant("BN_PAGE")                         # tokens per cache page: defined once, in csrc/common.h
+SPLIT_MIN_PAGES = _build.header_constant("BN_SPLIT_MIN_PAGES")   # shortest run of pages that decode attention splits off
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 
 
@@ -49,7 +50,7 @@ _SIGNATURES = {
         "bn_attn_rows_key_tile": [c_int, c_int],
         "bn_attn_rows": [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
-                         c_void_p, c_void_p, c_int, c_void_p],
+                         c_void_p, c_void_p, c_int, c_void_p, c_void_p],
     },
     "attn_mfma": {
         "bn_attn_mfma_supports": [c_int],
@@ -716,33 +717,19 @@ def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int, dtype=None):
     G = H // Hkv
     wgs = max(1, n_seqs * Hkv * ((G + GT - 1) // GT))
     pages = max(1, (max_len + PAGE - 1) // PAGE)
-    # about 512 workgroups, but no split shorter than 4 pages: below that the merging costs more
-    # than the parallelism gains (measured at batch 1, 8 and 64 of the 8B shape)
-    want = max(1, min(pages // 4, 64, (512 + wgs - 1) // wgs))
+    # about 512 workgroups, but no split shorter than SPLIT_MIN_PAGES pages: below that the merging costs
+    # more than the parallelism gains (measured at batch 1, 8 and 64 of the 8B shape)
+    want = max(1, min(pages // SPLIT_MIN_PAGES, 64, (512 + wgs - 1) // wgs))
     chunk = ((pages + want - 1) // want) * PAGE
     n_splits = (pages * PAGE + chunk - 1) // chunk
     return n_splits, chunk
 
 
-_COUNTERS = {}
-_N_COUNTERS = 65536
-# Merging the splits inside the decode kernel (the last workgroup to arrive does it) saves a launch
-# but needs fences of device scope in every workgroup, which on this chip write back and
-# invalidate a whole L2 each; measured slower than the separate combine launch, so it is off.
-MERGE_SPLITS_IN_KERNEL = False
-
-
-def attention_counters(device) -> torch.Tensor:
-    """Zeroed int32 counters that the decode attention kernel uses to find the last workgroup of a
-    (sequence, kv head); the kernel leaves them zero.  One buffer per device: attention launches
-    that overlap on one device (two streams) would race on it.  Create it outside a graph capture."""
-    device = torch.device(device)
-    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
-    t = _COUNTERS.get(key)
-    if t is None:
-        t = torch.zeros(_N_COUNTERS, dtype=torch.int32, device=device)
-        _COUNTERS[key] = t
-    return t
+def split_chunk(max_len: int, n_splits: int) -> int:
+    """Keys per split when a launch of n_splits splits meets sequences of up to max_len keys (bn_split_chunk of
+    csrc/common.h): what the kernels compute themselves when the length comes in device memory."""
+    pages = max(1, (max_len + PAGE - 1) // PAGE)
+    return max(SPLIT_MIN_PAGES, (pages + n_splits - 1) // n_splits) * PAGE
 
 
 def can_fuse_decode(dtype, H: int, Hkv: int, hs: int) -> bool:
@@ -753,7 +740,8 @@ def can_fuse_decode(dtype, H: int, Hkv: int, hs: int) -> bool:
 def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
               block_table: torch.Tensor, H: int, Hkv: int, hs: int, scale: float, *, window: int = 0,
               tiles=None, qt: int = 0, seq_lens=None, n_splits: int = 1, chunk: int = 0,
-              force_vector: bool = False, fused_rotate=None, fused_write: bool = False, by_length=None) -> None:
+              force_vector: bool = False, fused_rotate=None, fused_write: bool = False, by_length=None,
+              max_len_dev=None) -> None:
     """Causal attention of the (rotated) Q heads in qkv over the paged cache.
 
     Prompt form: `tiles` [n, 4] int32 = (sequence, first token row, tokens (<= qt), position of
@@ -768,7 +756,10 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     fused_write: the new K, V of every row (from qkv) are stored at position seq_lens - 1 first.
     by_length (decode form, optional): [B] int32, a permutation of the rows, longest sequence
     first; the matrix-core kernel hands out its workgroups in that order when a launch puts several
-    on every CU, so that long and short sequences share CUs.  It changes no result."""
+    on every CU, so that long and short sequences share CUs.  It changes no result.
+    max_len_dev (decode form, optional): a device int32 holding the longest sequence's key count; with
+    n_splits > 1 the kernels then cut the keys into n_splits runs of split_chunk(max_len, n_splits) and
+    `chunk` is not used, so that one captured launch serves every length up to the block table's width."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(out, "out", qkv.dtype, 2)
@@ -798,6 +789,11 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     if T == 0 or n_tiles == 0:
         return
     part_o = part_ml = None
+    if max_len_dev is not None:
+        _dev(max_len_dev, "max_len_dev", torch.int32)
+        if not decode or max_len_dev.numel() != 1:
+            raise KernelError("attention: max_len_dev is one int32 and belongs to the decode form")
+        chunk = split_chunk(block_table.shape[1] * PAGE, n_splits)         # of the longest sequence the table can hold
     if n_splits > 1:
         if chunk <= 0 or chunk % PAGE:
             raise KernelError(f"attention: chunk {chunk} must be a positive multiple of {PAGE}")
@@ -827,24 +823,20 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     if fused_write and qkv.shape[1] < (H + 2 * Hkv) * hs:
         raise KernelError("attention: fused cache write needs the K and V heads in qkv")
     if use_mfma:
-        counters = None
-        if (MERGE_SPLITS_IN_KERNEL and decode and n_splits > 1
-                and T * Hkv * ((H // Hkv + GT - 1) // GT) <= _N_COUNTERS):
-            counters = attention_counters(qkv.device)
         _check(_fn("attn_mfma", "bn_attn_mfma")(
             qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * hs, k_pages.data_ptr(), v_pages.data_ptr(),
             block_table.data_ptr(), block_table.shape[1], sl, tl, n_tiles, T, H, Hkv, hs, GT, int(window),
             float(scale), int(n_splits), int(chunk), po, pm,
             fused_rotate.data_ptr() if fused_rotate is not None else None, int(fused_rotate is not None),
-            int(bool(fused_write)), counters.data_ptr() if counters is not None else None,
-            by_length.data_ptr() if by_length is not None else None, _stream()),
+            int(bool(fused_write)), by_length.data_ptr() if by_length is not None else None,
+            max_len_dev.data_ptr() if max_len_dev is not None else None, _stream()),
             "attention(mfma)")
         return
     _check(_fn("attn_rows", "bn_attn_rows")(
         _code(qkv.dtype), qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * hs,
         k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1],
         sl, tl, n_tiles, T, H, Hkv, hs, RT, GT, int(window), float(scale), int(n_splits), int(chunk),
-        po, pm, int(vt), _stream()), "attention")
+        po, pm, int(vt), max_len_dev.data_ptr() if max_len_dev is not None else None, _stream()), "attention")
 
 
 # --------------------------------------------------------------------------------------
@@ -912,16 +904,5 @@ def sample(logits: torch.Tensor, temperature: float, top_p: float, uniforms=None
         return out
     probs = torch.empty((B, V), dtype=torch.float32, device=logits.device)
     _check(_fn("sampling", "bn_sample")(logits.data_ptr(), ld, B, V, probs.data_ptr(), uniforms.data_ptr(),
-                                        float(temperature), float(top_p), out.data_ptr(), _stream()), "sample")
-    return out
-    probs = None
-    if temperature != 0.0:
-        _dev(uniforms, "uniforms", torch.float32, 1)
-        if uniforms.numel() != B or not uniforms.is_contiguous():
-            raise KernelError("sample: one uniform number per row")
-        probs = torch.empty((B, V), dtype=torch.float32, device=logits.device)
-    _check(_fn("sampling", "bn_sample")(logits.data_ptr(), ld, B, V,
-                                        probs.data_ptr() if probs is not None else None,
-                                        uniforms.data_ptr() if probs is not None else None,
                                         float(temperature), float(top_p), out.data_ptr(), _stream()), "sample")
     return out

@@ -85,7 +85,8 @@ class Attention(Part):
                 n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len, h.dtype)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
                           window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
-                          fused_rotate=inv_freq, fused_write=kv.writes, by_length=ctx.by_length)
+                          fused_rotate=inv_freq, fused_write=kv.writes, by_length=ctx.by_length,
+                          max_len_dev=ctx.max_len_dev if n_splits > 1 else None)
             return last(out)
         self.position.encode_and_store(qkv, ctx, H, Hkv, hs, kv)
         if ctx.is_decode:
@@ -95,7 +96,7 @@ class Attention(Part):
                 n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len, h.dtype)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
                           window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
-                          by_length=ctx.by_length)
+                          by_length=ctx.by_length, max_len_dev=ctx.max_len_dev if n_splits > 1 else None)
         else:
             _, _, qt = ops.attention_row_shape(H, Hkv, False, h.dtype, hs)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,

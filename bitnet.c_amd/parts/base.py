@@ -69,9 +69,13 @@ class KVNeed:
 
 @dataclass(frozen=True)
 class StateNeed:
-    """A state of fixed size per sequence, zero when the sequence starts."""
+    """A state of fixed size per sequence, zero when the sequence starts.  device_addressed: the mixer reads
+    and writes it through the step's device-side slot ids only (ctx.slot_ids; padding rows carry the id of a
+    row that no sequence owns), never through the host's slot list, so its decode steps can be replayed from
+    a captured graph."""
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+    device_addressed: bool = False
 
 
 @dataclass(frozen=True)
@@ -129,7 +133,7 @@ class KVView:
     v_pages: Optional[torch.Tensor] = None
     block_table: Optional[torch.Tensor] = None  # [B, W] int32, this step's sequences
     writes: bool = True                         # False: the entry reads another entry's cache
-    state: Optional[torch.Tensor] = None        # [max_slots, *shape] fixed-size state, by slot
+    state: Optional[torch.Tensor] = None        # [max_slots + 1, *shape] fixed-size state, by slot
     max_len: int = 0                            # bound of the key count in this step (sizes the splits)
 
 

@@ -135,7 +135,7 @@ def test_window_group_gives_pages_back_while_the_sequence_grows():
 def test_state_area_is_zero_for_a_new_slot():
     needs = [CacheNeed(kv=KVNeed(1, 8), state=StateNeed((3, 2)))]
     c = _cache(needs=needs, max_tokens=64 * 4, device="cpu", max_slots=3)
-    assert c.states[0].shape == (3, 3, 2)
+    assert c.states[0].shape == (3 + 1, 3, 2) and c.padding_slot == 3      # one more row, which no sequence owns
     s = c.alloc_slot()
     c.states[0][s] += 5.0
     c.free_slot(s)
@@ -147,3 +147,21 @@ def test_state_area_is_zero_for_a_new_slot():
         c.alloc_slot()
     with pytest.raises(CacheFull):
         c.alloc_slot()
+
+
+def test_pages_of_a_step_that_did_not_run_go_back():
+    c = _cache(max_tokens=64 * 6, device=None)
+    a, b = c.alloc_slot(), c.alloc_slot()
+    c.reserve([a, b], [70, 10])
+    c.commit([a, b], [70, 10])
+    free, va, vb = c.groups[0].pool.n_free, c.slot_version(a), c.slot_version(b)
+    c.reserve([a, b], [60, 120])                   # a: 130 positions = one more page; b: 130 = two more
+    assert c.groups[0].pool.n_free == free - 3 and c.slot_version(a) != va
+    c.unreserve([a, b])                            # the step failed: nothing of it stays
+    assert c.groups[0].pool.n_free == free and len(c.pages_of(0, a)) == 2 and len(c.pages_of(0, b)) == 1
+    assert (c.length(a), c.length(b)) == (70, 10) and c.slot_version(b) != vb
+    c.check()
+    c.unreserve([a, b, 99])                        # nothing to give back, an unknown slot: no harm
+    c.check()
+    c.reserve([a], [1])                            # position 70 lies in a page the slot holds already
+    assert c.groups[0].pool.n_free == free

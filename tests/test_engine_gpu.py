@@ -284,6 +284,103 @@ def test_errors_change_nothing(model_folders):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "E"])
+def test_a_step_that_mixes_single_tokens_and_a_chunk_all_past_position_zero(model_folders, name, dtype):
+    """One step with a sequence that goes on by one token, a sequence that goes on by a chunk of 37 tokens
+    (across a page's edge), another single token, and a new sequence's whole prompt: every row of every one
+    matches the plain implementation, and in float32 the bits of the same rows run alone."""
+    from bitnet_c_amd import StepEntry
+    folder = model_folders(name, dtype)
+    eng = make_engine(folder, dtype, max_tokens=2048)
+    r_one, r_chunk, r_two, r_new = _requests(eng.vocab_size, 41, [72, 100, 6, 20])
+    a, b, c, d = (eng.new_sequence() for _ in range(4))
+    eng.step([StepEntry(a, r_one[:71], []), StepEntry(b, r_chunk[:40], []), StepEntry(c, r_two[:5], [])])
+    out = eng.step([StepEntry(a, r_one[71:], [0]), StepEntry(b, r_chunk[40:77], list(range(37))),
+                    StepEntry(c, r_two[5:], [0]), StepEntry(d, r_new, [19, 0])])
+    assert out.shape[0] == 1 + 37 + 1 + 2
+    want = [plain_logits(folder, r_one, dtype)[71:72], plain_logits(folder, r_chunk, dtype)[40:77],
+            plain_logits(folder, r_two, dtype)[5:6], plain_logits(folder, r_new, dtype)[[19, 0]]]
+    o = 0
+    for w in want:
+        assert rel_err(out[o:o + w.shape[0]], w) < TOL[dtype], o
+        o += w.shape[0]
+    # the chunk goes on: its later tokens see what the mixed step stored
+    rest = eng.step([StepEntry(b, r_chunk[77:], list(range(23)))])
+    assert rel_err(rest, plain_logits(folder, r_chunk, dtype)[77:]) < TOL[dtype]
+    for x in (a, b, c, d):
+        eng.release(x)
+    if dtype == torch.float32:
+        s = eng.new_sequence()
+        eng.step([StepEntry(s, r_chunk[:40], [])])
+        alone = eng.step([StepEntry(s, r_chunk[40:77], list(range(37)))])
+        eng.release(s)
+        assert torch.equal(alone, out[1:38])
+    eng.cache.check()
+
+
+def test_a_step_that_fails_halfway_leaves_nothing_behind(model_folders):
+    """An error inside the forward pass (here: raised by a tap in the second layer) after the step's pages
+    were taken: the pages go back, the lengths stay, and the same step runs afterwards as if nothing had been."""
+    from bitnet_c_amd import StepEntry
+    folder = model_folders("A", torch.float32)
+    eng = make_engine(folder, torch.float32, max_tokens=64 * 6)
+    toks = _requests(eng.vocab_size, 43, [200])[0]
+    s = eng.new_sequence()
+    eng.step([StepEntry(s, toks[:60], [])])
+    free = eng.cache.groups[0].pool.n_free
+
+    def tap(point, entry, stream, ctx):
+        if entry == 1:
+            raise RuntimeError("boom")
+    eng.tap = tap
+    for n in (1, 100):                                       # a decode step and a chunk of two more pages
+        with pytest.raises(RuntimeError):
+            eng.step([StepEntry(s, toks[60:60 + n], [0])])
+        assert eng.length(s) == 60 and eng.cache.groups[0].pool.n_free == free
+        eng.cache.check()
+    eng.tap = None
+    got = torch.cat([eng.step([StepEntry(s, toks[60:160], list(range(100)))]), eng.step([StepEntry(s, [toks[160]], [0])])])
+    assert rel_err(got, plain_logits(folder, toks[:161], torch.float32)[60:]) < TOL[torch.float32]
+    eng.release(s)
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_graphs_are_made_at_a_batch_s_start_and_never_between_tokens(model_folders, dtype):
+    """prepare_decode(n) captures what decode steps of up to n sequences replay; afterwards sequences grow
+    through page edges and through every power of two of pages, end one by one (the batch shrinks from five
+    rows to one), and no further capture happens; the logits stay the plain ones all the way."""
+    from bitnet_c_amd import StepEntry
+    folder = model_folders("C", dtype)                       # position limit 2,048
+    eng = make_engine(folder, dtype, max_tokens=64 * 40, max_seq_len=1100)
+    assert eng.max_pages == 18
+    rnd = random.Random(44)
+    ends = [1040, 80, 300, 20, 131]
+    reqs = [[rnd.randrange(eng.vocab_size) for _ in range(n)] for n in ends]
+    eng.prepare_decode(len(reqs))
+    built = eng.graphs_built
+    assert sorted(eng._graphs) == [1, 2, 4, 8] and built == 4
+    slots = [eng.new_sequence() for _ in reqs]
+    fed = [10, 3, 60, 1, 64]
+    eng.step([StepEntry(s, r[:f], []) for s, r, f in zip(slots, reqs, fed)])
+    got = [[] for _ in reqs]
+    live = list(range(len(reqs)))
+    while live:
+        out = eng.step([StepEntry(slots[i], [reqs[i][fed[i]]], [0]) for i in live])
+        for r, i in enumerate(live):
+            got[i].append(out[r:r + 1])
+            fed[i] += 1
+        for i in [i for i in live if fed[i] == ends[i]]:
+            eng.release(slots[i])
+        live = [i for i in live if fed[i] < ends[i]]
+    assert eng.graphs_built == built
+    for i, r in enumerate(reqs):
+        n = len(got[i])
+        assert rel_err(torch.cat(got[i]), plain_logits(folder, r, dtype)[-n:]) < TOL[dtype], i
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_far_key_through_the_engine(model_folders, dtype, tmp_path):
     """Weights made so that a fault shows: in a one-layer model whose q and k projections pick out
     one embedding dimension each and whose positions are not rotated there (the lowest frequency at
@@ -441,9 +538,10 @@ def test_forty_sequences_of_unequal_lengths_with_eight_kv_heads(model_folders, g
 def test_cuts_and_batches_agree_at_the_benchmark_layer_sizes():
     """Two layers of the Llama-3.1-8B shape (bfloat16, random weights made on the device): the
     kernels at their real sizes, where a prompt's products go to the library and a decoded token's
-    to the streaming kernel.  There is no plain run at this size; the same request whole, with its
-    last 32 tokens one by one, and inside a batch of unequal partners must agree within the
-    bfloat16 tolerance, and all of them with a float32 engine on the same (bfloat16) weights."""
+    to the streaming kernel.  The same request whole, with its last 32 tokens one by one, and inside a
+    batch of unequal partners: a float32 engine on the same (bfloat16) weights gives equal bits all three
+    ways and agrees with the plain implementation, run on the CPU at this width; the bfloat16 engine
+    agrees with them within what rounding looks like at this width."""
     import bitnet_c_amd as bn
     from bitnet_c_amd.config import architecture_for
     from bitnet_c_amd.engine import DecoderModel
@@ -461,10 +559,21 @@ def test_cuts_and_batches_agree_at_the_benchmark_layer_sizes():
         model = DecoderModel(plan, dtype, "cuda:0")
         model.load(tensors)
         engines[dtype] = bn.Engine(model, max_tokens=4096)
-    del tensors
     rnd = random.Random(31)
     toks, p1, p2 = ([rnd.randrange(cfg.vocab_size) for _ in range(n)] for n in (300, 70, 513))
     last = list(range(268, 300))
+    # the plain implementation at this width, on the CPU, in float32 on the same (bfloat16) weights: all 300
+    # tokens through the two layers, the final norm and the output matrix for the last 32 only
+    W = {k: v.float().cpu() for k, v in tensors.items()}
+    del tensors
+    c = dict(dim=cfg.hidden_size, ffn=cfg.intermediate_size, layers=2, heads=32, kv_heads=8, head_dim=128,
+             vocab=cfg.vocab_size, theta=cfg.rope_theta, eps=cfg.rms_norm_eps, tied=False, rope_scaling=raw["rope_scaling"])
+    x = W["model.embed_tokens.weight"][torch.tensor(toks)]
+    inv = pl.rope_inv_freq(128, c["theta"], c["rope_scaling"])
+    for l in range(2):
+        x = pl.decoder_layer(x, torch.arange(300), W, l, c, inv)
+    plain_ref = pl.linear(pl.rmsnorm(x[268:], W["model.norm.weight"], c["eps"]), W["lm_head.weight"])
+    del W
 
     def run(eng):
         s = eng.new_sequence()
@@ -487,6 +596,7 @@ def test_cuts_and_batches_agree_at_the_benchmark_layer_sizes():
 
     ref = run(engines[torch.float32])
     assert torch.equal(ref[1], ref[0]) and torch.equal(ref[2], ref[0])     # float32: no cut changes a bit
+    assert rel_err(ref[0], plain_ref) < TOL[torch.float32]                 # and they are the plain implementation's
     got = run(engines[torch.bfloat16])
     # 32 x 128,256 logits: the largest of four million differences is no measure (rounding noise of
     # standard deviation s has its largest value near 5.5 s there).  What rounding looks like at this

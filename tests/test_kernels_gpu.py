@@ -482,6 +482,109 @@ def test_rope_kv_write(dtype, H, Hkv, hs, rope_dims):
     assert torch.equal(vp4.cpu().float(), vp_first.contiguous())
 
 
+FAR_POSITIONS = [8191, 8192, 65535, 131071]
+LLAMA3_8B_SCALING = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                         original_max_position_embeddings=8192)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rope_kv_write_at_far_positions(dtype):
+    """Positions around and far beyond the frequency table's original_max_position_embeddings, with the rescaled
+    table of the 8B configuration: angles of up to 131,071 radians, where float32 holds the angle to 2^-7 and the
+    range reduction of sine and cosine does the rest.  Against the plain rotation; and the plain rotation at a
+    neighbouring position or with the unscaled table is far away, so neither mistake could pass."""
+    ops = _ops()
+    H, Hkv, hs = 4, 2, 128
+    inv = pl.rope_inv_freq(hs, 500000.0, LLAMA3_8B_SCALING)
+    T = len(FAR_POSITIONS)
+    qkv = _rand((T, (H + 2 * Hkv) * hs), dtype, 480)
+    pos = torch.tensor(FAR_POSITIONS, dtype=torch.int32)
+    bt = torch.zeros((T, 2048), dtype=torch.int32)
+    for t, p in enumerate(FAR_POSITIONS):
+        bt[t, p // 64] = t + 1                                   # page 0 stays untouched
+    vt = dtype == torch.bfloat16
+    kp = torch.zeros((T + 1, Hkv, 64, hs), dtype=dtype).cuda()
+    vp = torch.zeros((T + 1, Hkv, hs, 64) if vt else (T + 1, Hkv, 64, hs), dtype=dtype).cuda()
+    g = qkv.clone().cuda()
+    ops.rope_kv_write(g, pos.cuda(), H, Hkv, hs, inv_freq=inv.cuda(), rope_dims=hs,
+                      seq_index=torch.arange(T, dtype=torch.int32).cuda(), block_table=bt.cuda(), k_pages=kp, v_pages=vp)
+    q_in = qkv[:, :H * hs].float().view(T, H, hs)
+    k_in = qkv[:, H * hs:(H + Hkv) * hs].float().view(T, Hkv, hs)
+    q_ref, k_ref = pl.apply_rope(q_in, pos, inv), pl.apply_rope(k_in, pos, inv)
+    got_q = g[:, :H * hs].float().view(T, H, hs).cpu()
+    assert close(got_q, q_ref, dtype)
+    for t, p in enumerate(FAR_POSITIONS):
+        assert close(kp[t + 1, :, p % 64].float().cpu(), k_ref[t], dtype), p
+    assert float(kp[0].float().abs().sum()) == 0.0
+    assert rel_err(pl.apply_rope(q_in, pos - 1, inv), q_ref) > 0.5                               # a position off by one
+    assert rel_err(pl.apply_rope(q_in, pos, pl.rope_inv_freq(hs, 500000.0)), q_ref) > 0.5        # the table not rescaled
+
+
+def test_decode_attention_rotates_and_stores_at_far_positions():
+    """The decode kernel's own rotation, angle = (length - 1) * f_i, at lengths 8,192 to 131,072 with the rescaled
+    table of the 8B configuration.  Each sequence's cache holds one marked key 1,000 positions back, rotated for
+    its position by the plain implementation; query and new key carry the same raw vector, so the marked key's
+    score is sum |q_i|^2 cos(1000 f_i) and shares the weight with the new key only when the query was turned by
+    the right angle.  The stored key is the plain rotation, and the output the plain attention over all keys."""
+    ops = _ops()
+    dtype, H, Hkv, hs = torch.bfloat16, 4, 1, 128
+    inv = pl.rope_inv_freq(hs, 500000.0, LLAMA3_8B_SCALING)
+    scale = hs ** -0.5
+    B = len(FAR_POSITIONS)
+    g = torch.Generator().manual_seed(490)
+    raw = torch.zeros(hs)
+    for i in (3, 17, 30, 41, 52, 63):                             # pairs of fast and of slow (rescaled) frequencies
+        raw[i], raw[i + hs // 2] = 4.5, -3.0
+    raw[0], raw[hs // 2] = 6.0, -3.0                              # the fastest pair turns by one radian a position
+    new_key = 0.762 * raw          # so that the new key's score equals the marked key's (sum |q_i|^2 cos(1000 f_i))
+    qkv = torch.zeros((B, (H + 2 * Hkv) * hs))
+    for h in range(H):
+        qkv[:, h * hs:(h + 1) * hs] = raw * (1.0 - 0.05 * h)
+    qkv[:, H * hs:(H + 1) * hs] = new_key
+    qkv[:, (H + 1) * hs:] = torch.randn(B, hs, generator=g)
+    qkv = qkv.to(dtype)
+    seqs_k, seqs_v, refs, new_keys = [], [], [], []
+    for b, p in enumerate(FAR_POSITIONS):
+        L = p + 1
+        far = p - 1000
+        k = torch.zeros((L, Hkv, hs))
+        k[far, 0] = pl.apply_rope(raw.view(1, 1, hs), torch.tensor([far]), inv)[0, 0]
+        k_new = pl.apply_rope(qkv[b, H * hs:(H + 1) * hs].float().view(1, 1, hs), torch.tensor([p]), inv)[0, 0]
+        k[p, 0] = k_new
+        k = k.to(dtype)
+        v = torch.randn((L, Hkv, hs), generator=g).to(dtype)
+        v[p, 0] = qkv[b, (H + 1) * hs:]
+        q = pl.apply_rope(qkv[b, :H * hs].float().view(1, H, hs), torch.tensor([p]), inv)[0].to(dtype).double()
+        sc = (q @ k[:, 0].double().t()) * scale                    # [H, L]
+        w = torch.softmax(sc, dim=1)
+        # the marked key and the new one hold nearly all the weight (scores near 15 against 131,072 keys at 0),
+        # and share it
+        assert float((w[:, far] + w[:, p]).min()) > 0.8 and float(w[:, far].min()) > 0.25 and float(w[:, p].min()) > 0.25
+        refs.append((w @ v[:, 0].double()).reshape(H * hs).float())
+        new_keys.append(k[p, 0].float())
+        kk, vv = k.clone(), v.clone()
+        kk[p], vv[p] = float("nan"), float("nan")                  # the kernel must write this place itself
+        seqs_k.append(kk)
+        seqs_v.append(vv)
+    kp, vp, bt = _paged(seqs_k, seqs_v, dtype, sum((p + 64) // 64 for p in FAR_POSITIONS) + 2, 491)
+    kp, vp, bt = kp.cuda(), vp.cuda(), bt.cuda()
+    lens = torch.tensor([p + 1 for p in FAR_POSITIONS], dtype=torch.int32).cuda()
+    n_splits, chunk = ops.decode_splits(B, H, Hkv, bt.shape[1] * 64)
+    out = torch.full((B, H * hs), float("nan"), dtype=dtype).cuda()
+    ops.attention(qkv.cuda(), out, kp, vp, bt, H, Hkv, hs, scale, seq_lens=lens, n_splits=n_splits, chunk=chunk,
+                  fused_rotate=inv.cuda(), fused_write=True)
+    assert mfma_close(out.float(), torch.stack(refs))
+    for b, p in enumerate(FAR_POSITIONS):
+        page = int(bt[b, p // 64])
+        assert close(kp[page, 0, p % 64].float().cpu(), new_keys[b], dtype), p
+        assert torch.equal(vp[page, 0, :, p % 64].cpu(), qkv[b, (H + 1) * hs:]), p
+    # the same query turned for the position before would have weighted the two keys otherwise
+    q_off = pl.apply_rope(qkv[0, :hs].float().view(1, 1, hs), torch.tensor([FAR_POSITIONS[0] - 1]), inv)[0, 0]
+    k_far = seqs_k[0][FAR_POSITIONS[0] - 1000, 0].float()
+    q_on = pl.apply_rope(qkv[0, :hs].float().view(1, 1, hs), torch.tensor([FAR_POSITIONS[0]]), inv)[0, 0]
+    assert abs(float(q_off @ k_far) - float(q_on @ k_far)) * scale > 1.0
+
+
 def test_rope_reference_vector_on_device():
     # test/test_transformer.c:636-643 through the kernel: angles pi/2 and 0
     ops = _ops()
@@ -849,13 +952,10 @@ def test_repeat_penalty_on_device():
 
 @pytest.mark.parametrize("H,Hkv,hs,window", [(32, 8, 128, 0), (8, 2, 64, 0), (16, 1, 128, 0), (6, 6, 64, 90), (4, 4, 128, 0)])
 @pytest.mark.parametrize("force_splits", [1, 0, 7])
-@pytest.mark.parametrize("merge_in_kernel", [False, True])
-def test_decode_attention_that_rotates_and_stores_itself(H, Hkv, hs, window, force_splits, merge_in_kernel, monkeypatch):
+def test_decode_attention_that_rotates_and_stores_itself(H, Hkv, hs, window, force_splits):
     """The decode kernel doing rope_kv_write's work: unrotated qkv in, the new key and value stored,
-    against rope_kv_write followed by the same attention; run twice in a row, since it leaves its
-    counters behind for the next launch."""
+    against rope_kv_write followed by the same attention; run twice in a row."""
     ops = _ops()
-    monkeypatch.setattr(ops, "MERGE_SPLITS_IN_KERNEL", merge_in_kernel)
     dtype = torch.bfloat16
     lens_before = [0, 63, 64, 700, 129, 300, 31]
     B = len(lens_before)
@@ -895,4 +995,35 @@ def test_decode_attention_that_rotates_and_stores_itself(H, Hkv, hs, window, for
         assert torch.equal(torch.nan_to_num(v2.float(), nan=-7.0).cpu(), torch.nan_to_num(v1.float(), nan=-7.0).cpu())
         assert mfma_close(got[:B].float(), want[:B].float())
         assert float(got[B:].float().abs().sum()) == 0.0
-        assert int(ops.attention_counters("cuda:0").abs().sum()) == 0
+
+
+@pytest.mark.parametrize("dtype,H,Hkv,hs", [(torch.bfloat16, 8, 2, 128), (torch.bfloat16, 6, 3, 48), (torch.bfloat16, 4, 4, 64)])
+def test_decode_attention_with_the_longest_length_in_device_memory(dtype, H, Hkv, hs):
+    """The form a captured step uses: a fixed number of splits and a block table as wide as the longest sequence
+    the engine allows, the keys per split derived inside the kernel from a device-side integer.  Whatever the
+    longest sequence of a launch is, the result is the plain one; and with the integer equal to what the
+    table's width gives, it is bit for bit the result of the host-side plan."""
+    lens_before = [0, 63, 64, 700, 129, 300]
+    B = len(lens_before)
+    ops, qkv, kp, vp, bt, ref, scale = _attn_case(dtype, H, Hkv, hs, lens_before, [1] * B, 0, 230)
+    wide = torch.zeros((B, 40), dtype=torch.int32).cuda()                  # room for 2,560 keys a sequence
+    wide[:, :bt.shape[1]] = bt
+    lens = torch.tensor([p + 1 for p in lens_before], dtype=torch.int32).cuda()
+    check = (lambda o: mfma_close(o, ref)) if ops.mfma_attention(dtype, hs) else (lambda o: close(o, ref, dtype))
+    n_splits, _ = ops.decode_splits(B, H, Hkv, 40 * 64)
+    assert n_splits > 1
+    outs = {}
+    for max_len in (701, 1000, 2560):
+        out = torch.full((B, H * hs), float("nan"), dtype=dtype).cuda()
+        ops.attention(qkv, out, kp, vp, wide, H, Hkv, hs, scale, seq_lens=lens, n_splits=n_splits,
+                      max_len_dev=torch.tensor([max_len], dtype=torch.int32).cuda())
+        assert check(out.float()), max_len
+        outs[max_len] = out
+    host = torch.full((B, H * hs), float("nan"), dtype=dtype).cuda()
+    ops.attention(qkv, host, kp, vp, wide, H, Hkv, hs, scale, seq_lens=lens, n_splits=n_splits,
+                  chunk=ops.split_chunk(2560, n_splits))
+    assert torch.equal(host, outs[2560])
+    with pytest.raises(ops.KernelError):                                   # the prompt form has no such integer
+        ops.attention(qkv, host, kp, vp, wide, H, Hkv, hs, scale, tiles=torch.zeros((1, 4), dtype=torch.int32).cuda(),
+                      qt=ops.attention_row_shape(H, Hkv, False, dtype, hs)[2],
+                      max_len_dev=torch.tensor([5], dtype=torch.int32).cuda())

@@ -372,6 +372,113 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
     assert rel_err(again, plain(reqs[1])) < TOL[torch.float32]
 
 
+def test_a_state_mixer_that_addresses_its_state_on_the_device_decodes_under_graphs(tmp_path):
+    """The same toy recurrence written against the step's device-side slot ids (ctx.slot_ids) instead of the
+    host's slot list, and declared so (StateNeed.device_addressed): its decode steps are captured and
+    replayed, padding rows read and write the state row that no sequence owns, and the logits are those of
+    the eager engine, bit for bit, with sequences that end at different steps and a slot that is used again."""
+    from bitnet_c_amd import Engine, StepEntry
+    from bitnet_c_amd.config import Architecture, register_architecture
+    from bitnet_c_amd.config.base import _ARCHITECTURES
+    from bitnet_c_amd.engine import LayerPlan, ModelPlan, ScheduleEntry
+    from bitnet_c_amd.parts import BLOCKS, MIXERS, CacheNeed, ParamSpec, Part, PartSpec, StateNeed
+    from bitnet_c_amd.weights import write_model_folder
+
+    if "decay_sum_dev" not in MIXERS:
+        @MIXERS.register("decay_sum_dev")
+        class DecaySumDev(Part):
+            """s_t = decay * s_{t-1} + h_t ;  out_t = W s_t, the state addressed by ctx.slot_ids."""
+
+            def __init__(self, hidden, decay):
+                self.hidden, self.decay = hidden, decay
+
+            def tensors(self):
+                return {"w": ParamSpec((self.hidden, self.hidden))}
+
+            def load(self, tensors, device, dtype):
+                self.w = tensors["w"].to(dtype).to(device)
+
+            def cache_need(self):
+                return CacheNeed(state=StateNeed((self.hidden,), torch.float32, device_addressed=True))
+
+            def forward(self, h, ctx, kv):
+                ids = ctx.slot_ids.long()
+                if ctx.is_decode:                                   # one row a sequence: no host loop, capturable
+                    s = self.decay * kv.state.index_select(0, ids) + h.float()
+                    kv.state.index_copy_(0, ids, s)
+                    return (s @ self.w.float().t()).to(h.dtype)
+                out = torch.empty_like(h)
+                for b, (r0, n) in enumerate(ctx.row_ranges()):
+                    s = kv.state[ids[b]]
+                    for t in range(r0, r0 + n):
+                        s = self.decay * s + h[t].float()
+                        out[t] = (self.w.float() @ s).to(h.dtype)
+                    kv.state[ids[b]] = s
+                return out
+
+    @dataclass(frozen=True)
+    class DevConfig:
+        vocab_size: int
+        hidden_size: int
+        model_type: str = "toy_decay_dev"
+
+        @staticmethod
+        def from_dict(raw):
+            return DevConfig(raw["vocab_size"], raw["hidden_size"])
+
+        def to_dict(self):
+            return asdict(self)
+
+    def build(c):
+        norm = PartSpec.of("rmsnorm", dim=c.hidden_size, eps=1e-5)
+        ffn = PartSpec.of("swiglu", hidden=c.hidden_size, intermediate=2 * c.hidden_size)
+        att = PartSpec.of("attention", hidden=c.hidden_size, n_heads=2, n_kv_heads=1, head_dim=c.hidden_size // 2,
+                          scale=(c.hidden_size // 2) ** -0.5,
+                          position=PartSpec.of("rope", head_dim=c.hidden_size // 2, theta=100.0))
+        dec = PartSpec.of("decay_sum_dev", hidden=c.hidden_size, decay=0.8)
+        layers = []
+        for i, mixer in enumerate((dec, att, dec)):
+            blk = PartSpec.of("prenorm", mixer=mixer, ffn=ffn, mixer_norm=norm, ffn_norm=norm)
+            layers.append(LayerPlan(block=blk, names={local: f"layers.{i}.{local}" for local in BLOCKS.build(blk).tensors()}))
+        return ModelPlan(vocab_size=c.vocab_size, hidden_size=c.hidden_size, layers=layers,
+                         schedule=[ScheduleEntry(i) for i in range(3)], final_norm=norm,
+                         embedding_name="embed.weight", final_norm_names={"weight": "norm.weight"},
+                         lm_head_name="head.weight")
+
+    if "toy_decay_dev" not in _ARCHITECTURES:
+        register_architecture(Architecture("toy_decay_dev", DevConfig, build))
+    folder = write_model_folder(str(tmp_path / "toydev"), DevConfig(vocab_size=50, hidden_size=32), 13, torch.float32)
+    rnd = random.Random(14)
+    reqs = [[rnd.randrange(50) for _ in range(n)] for n in (20, 9, 33)]
+    n_dec = [12, 3, 7]
+    outs = []
+    for graphs in (True, False):
+        eng = Engine.from_folder(folder, dtype=torch.float32, max_tokens=512, use_graphs=graphs)
+        assert eng.use_graphs == graphs and sorted(eng.cache.states) == [0, 2]
+        got = []
+        for _ in range(2):                                  # the second round uses the first one's slots again
+            slots = [eng.new_sequence() for _ in reqs]
+            fed = [len(r) - d for r, d in zip(reqs, n_dec)]
+            eng.step([StepEntry(s, r[:f], []) for s, r, f in zip(slots, reqs, fed)])
+            live = list(range(3))
+            while live:
+                got.append(eng.step([StepEntry(slots[i], [reqs[i][fed[i]]], [0]) for i in live]).clone())
+                for i in live:
+                    fed[i] += 1
+                for i in [i for i in live if fed[i] == len(reqs[i])]:
+                    eng.release(slots[i])
+                live = [i for i in live if fed[i] < len(reqs[i])]
+        if graphs:
+            assert sorted(eng._graphs) == [1, 2, 4]         # three rows are a graph of four: one padding row
+            # the padding row worked on the spare state row and on no sequence's
+            assert float(eng.cache.states[0][eng.cache.padding_slot].abs().sum()) > 0
+        outs.append(got)
+    assert len(outs[0]) == len(outs[1]) == 24
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    assert torch.equal(torch.cat(outs[0][:12]), torch.cat(outs[0][12:]))      # the second round equals the first
+
+
 def test_a_windowed_group_beside_a_full_one_through_the_engine(tmp_path):
     """A toy architecture whose odd layers see only the last 70 positions: two cache groups with
     storage of their own; the windowed one gives pages back while sequences grow, and the logits
