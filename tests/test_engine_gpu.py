@@ -657,8 +657,12 @@ def test_graph_replays_of_a_wide_batch_at_the_benchmark_layer_sizes(n_seqs):
         d = (outs[0][k] - outs[1][k]).double()
         per_row = d.pow(2).mean(dim=1).sqrt() / rms
         assert float(per_row.max()) < 0.025, (k, per_row)
-        sd = float(d.pow(2).mean().sqrt())                           # 0: the same kernels ran on both sides
-        assert sd == 0.0 or float(d.abs().max()) / sd < 8.0, k
+        # No single value far outside the noise.  Where most kernels are the same on both sides (only the attention's
+        # split plan differs: the graph cuts for the longest sequence the engine allows) most differences are zero and
+        # the measured deviation says nothing, so the yardstick is never smaller than what rounding gives at this
+        # width when every kernel differs, 1.25 % of the logits' root mean square.
+        sd = max(float(d.pow(2).mean().sqrt()), 0.0125 * rms)
+        assert float(d.abs().max()) / sd < 8.0, k
 
 
 # Further sizes than the tiny configurations': head sizes in steps of 16 up to 256, one to 64 heads in groups of 1 to 16,
