@@ -4,6 +4,8 @@ MI355X.  One JSON line on stdout.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--shape 8b|13b|70b]
                     [--context C] [--prompt-lens LO,HI] [--prefill-tokens T]      (further lengths; not the default record)
+    python bench.py --only kernel:skinny|attention_prompt|attention_decode|gemm     (single kernels at the benchmark's
+                    layer sizes, for a profiler; nothing is timed or printed)
 
 A step is one decode step of the whole batch: the step function, greedy sampling on the
 device and the read-back of the tokens, as generation does it.  `value` is decoded
@@ -48,6 +50,95 @@ SHAPES = {
 PREFILL_TOKENS = 2048
 
 
+# ---- single kernels at the benchmark's layer sizes (Llama-3.1-8B shape, bfloat16), for profilers -------------------
+# Nothing is checked or timed here: the numerics of these kernels are in tests/test_kernels_gpu.py, their times in
+# the profiler's output.
+
+def _kernel_skinny(rows=8, copies=3):
+    """The decode products at 8 rows, every weight matrix read cold (three copies in turn)."""
+    import torch
+    from bitnet_c_amd import ops
+    shapes = [("qkv", 6144, 4096, False), ("o", 4096, 4096, False), ("gate_up", 14336, 4096, True),
+              ("down", 4096, 14336, False), ("output", 128256, 4096, False)]
+    for name, n, k, glu in shapes:
+        ws = [torch.randn((2 * n if glu else n), k, device="cuda:0", dtype=torch.bfloat16) * 0.02 for _ in range(copies)]
+        x = torch.randn(rows, k, device="cuda:0", dtype=torch.bfloat16)
+        for w in ws:
+            if glu:
+                ops.linear_swiglu(x, w, True)
+            else:
+                ops.linear(x, w, torch.float32 if name == "output" else None)
+        torch.cuda.synchronize()
+        del ws
+
+
+def _kernel_gemm(rows=2048, reps=3):
+    """The prompt products at 2,048 rows through this library's own matrix-core kernel."""
+    import torch
+    from bitnet_c_amd import ops
+    shapes = [("qkv", 6144, 4096, False), ("o", 4096, 4096, False), ("gate_up", 14336, 4096, True),
+              ("down", 4096, 14336, False)]
+    for name, n, k, glu in shapes:
+        w = torch.randn((2 * n if glu else n), k, device="cuda:0", dtype=torch.bfloat16) * 0.02
+        x = torch.randn(rows, k, device="cuda:0", dtype=torch.bfloat16)
+        for _ in range(reps):
+            ops.gemm_mfma(x, w, None, glu)
+        torch.cuda.synchronize()
+        del w
+
+
+def _kernel_cache(lengths, Hkv=8, hs=128):
+    import torch
+    pages = [(n + 63) // 64 for n in lengths]
+    kp = torch.randn(sum(pages) + 1, Hkv, 64, hs, device="cuda:0", dtype=torch.bfloat16)
+    vp = torch.randn(sum(pages) + 1, Hkv, hs, 64, device="cuda:0", dtype=torch.bfloat16)
+    bt = torch.zeros(len(lengths), max(pages), dtype=torch.int32)
+    p = 0
+    for i, n in enumerate(pages):
+        bt[i, :n] = torch.arange(p, p + n)
+        p += n
+    return kp, vp, bt.to("cuda:0")
+
+
+def _kernel_attention_prompt(H=32, Hkv=8, hs=128):
+    """Prompt attention over 2,048 and 8,192 tokens."""
+    import torch
+    from bitnet_c_amd import ops
+    for t in (2048, 8192):
+        kp, vp, bt = _kernel_cache([t], Hkv, hs)
+        qkv = torch.randn(t, (H + 2 * Hkv) * hs, device="cuda:0", dtype=torch.bfloat16)
+        out = torch.empty(t, H * hs, device="cuda:0", dtype=torch.bfloat16)
+        _, _, qt = ops.attention_row_shape(H, Hkv, False, torch.bfloat16, hs)
+        tiles = torch.tensor([(0, i, min(qt, t - i), i) for i in range(0, t, qt)], dtype=torch.int32, device="cuda:0")
+        for _ in range(3):
+            ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, hs ** -0.5, tiles=tiles, qt=qt)
+        torch.cuda.synchronize()
+
+
+def _kernel_attention_decode(H=32, Hkv=8, hs=128):
+    """Decode attention (rotation and cache write inside), batch 1, 8 and 64, unequal lengths."""
+    import torch
+    from bitnet_c_amd import ops
+    rnd = random.Random(0)
+    for b in (1, 8, 64):
+        lens = [rnd.randint(128, 2112) for _ in range(b)]
+        kp, vp, bt = _kernel_cache(lens, Hkv, hs)
+        qkv = torch.randn(b, (H + 2 * Hkv) * hs, device="cuda:0", dtype=torch.bfloat16)
+        out = torch.empty(b, H * hs, device="cuda:0", dtype=torch.bfloat16)
+        d_lens = torch.tensor(lens, dtype=torch.int32, device="cuda:0")
+        order = torch.tensor(sorted(range(b), key=lambda i: -lens[i]), dtype=torch.int32, device="cuda:0")
+        inv = torch.rand(hs // 2, device="cuda:0")
+        n_splits, chunk = ops.decode_splits(b, H, Hkv, bt.shape[1] * 64)
+        for _ in range(3):
+            ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, hs ** -0.5, seq_lens=d_lens, n_splits=n_splits, chunk=chunk,
+                          fused_rotate=inv, fused_write=True, by_length=order)
+        torch.cuda.synchronize()
+
+
+KERNEL_WORKLOADS = {"skinny": _kernel_skinny, "gemm": _kernel_gemm, "attention_prompt": _kernel_attention_prompt,
+                    "attention_decode": _kernel_attention_decode}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -59,8 +150,9 @@ def main() -> int:
                     help="fewer layers than the configuration has (named in the record)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points")
-    ap.add_argument("--only", choices=["prefill", "decode"], default=None,
-                    help="for profiling: run one phase alone (the record then lacks the other)")
+    ap.add_argument("--only", default=None, metavar="prefill|decode|kernel:NAME",
+                    help="for profiling: run one phase alone (the record then lacks the other), or single kernels at "
+                         "the benchmark's layer sizes (kernel:" + "|".join(sorted(KERNEL_WORKLOADS)) + ")")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--context", type=int, default=0, help="longest sequence (default: the shape's)")
     ap.add_argument("--prompt-lens", default=None, metavar="LO,HI", help="prompt lengths of the decode batches")
@@ -69,6 +161,14 @@ def main() -> int:
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.only and args.only.startswith("kernel:"):
+        name = args.only.split(":", 1)[1]
+        if name not in KERNEL_WORKLOADS:
+            ap.error(f"--only kernel:{name}: known kernels are {sorted(KERNEL_WORKLOADS)}")
+        KERNEL_WORKLOADS[name]()
+        return 0
+    if args.only not in (None, "prefill", "decode"):
+        ap.error("--only takes prefill, decode or kernel:NAME")
 
     import torch
 

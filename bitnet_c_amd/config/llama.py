@@ -16,6 +16,11 @@ from typing import Optional
 from .base import ConfigError, _positive_int
 
 
+# config.json's names of the gate activation -> the feed-forward part's (the reference's registry fixes SiLU for
+# this architecture, src/model_arch.c:807-810; its other kinds are reachable through the same key)
+HIDDEN_ACTS = {"silu": "silu", "gelu_pytorch_tanh": "gelu_tanh", "gelu_tanh": "gelu_tanh", "relu2": "relu2"}
+
+
 @dataclass(frozen=True)
 class RopeScaling:
     rope_type: str                          # "llama3" (or "default": none)
@@ -99,8 +104,8 @@ class LlamaConfig:
             raise ConfigError(f"config.json: head_dim {head_dim} is more than the attention kernels take "
                               f"(every even head size up to {MAX_HEAD_DIM})")
         act = raw.get("hidden_act", "silu")
-        if act != "silu":
-            raise ConfigError(f"config.json: hidden_act {act!r} is not supported (supported: 'silu')")
+        if act not in HIDDEN_ACTS:
+            raise ConfigError(f"config.json: hidden_act {act!r} is not supported (supported: {sorted(HIDDEN_ACTS)})")
         theta = raw.get("rope_theta")
         theta = 10000.0 if theta in (None, 0) else float(theta)
         eps = raw.get("rms_norm_eps")

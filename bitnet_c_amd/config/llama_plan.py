@@ -19,7 +19,7 @@ from dataclasses import asdict
 from ..engine.plan import LayerPlan, ModelPlan, ScheduleEntry
 from ..parts.base import PartSpec
 from .base import Architecture, register_architecture
-from .llama import LlamaConfig
+from .llama import HIDDEN_ACTS, LlamaConfig
 
 
 def build_llama_plan(c: LlamaConfig) -> ModelPlan:
@@ -29,7 +29,8 @@ def build_llama_plan(c: LlamaConfig) -> ModelPlan:
                         n_kv_heads=c.num_key_value_heads, head_dim=c.head_dim,
                         scale=1.0 / math.sqrt(c.head_dim),          # src/model_arch.c:141-145
                         position=position, bias=c.attention_bias)
-    ffn = PartSpec.of("swiglu", hidden=c.hidden_size, intermediate=c.intermediate_size, bias=c.mlp_bias)
+    ffn = PartSpec.of("swiglu", hidden=c.hidden_size, intermediate=c.intermediate_size, bias=c.mlp_bias,
+                      activation=HIDDEN_ACTS[c.hidden_act])
     norm = PartSpec.of("rmsnorm", dim=c.hidden_size, eps=c.rms_norm_eps)
     block = PartSpec.of("prenorm", mixer=mixer, ffn=ffn, mixer_norm=norm, ffn_norm=norm)
     layers = []

@@ -79,4 +79,20 @@ __host__ __device__ __forceinline__ int bn_split_chunk(int max_len, int n_splits
     return per * BN_PAGE;
 }
 
+// The gate's activation in a gated feed-forward, out = act(gate) * up: the kinds the reference knows
+// (src/transformer/cpu_backend.c:343-417).  silu(g) = g / (1 + exp(-g)) with the exact exponential (:356);
+// gelu in its tanh form 0.5 g (1 + tanh(0.79788456 g (1 + 0.044715 g^2))) (:27-29, without the reference's
+// rounding of g and of the result to half precision); relu2(g) = max(g, 0)^2 (:349-350).  Every kernel
+// that ends in a gated unit takes the kind as an argument.
+#define BN_ACT_SILU 0
+#define BN_ACT_GELU_TANH 1
+#define BN_ACT_RELU2 2
+#define BN_ACT_KINDS 3
+__device__ __forceinline__ float bn_gate_act(float g, int act) {
+    if (act == BN_ACT_SILU) return g / (1.0f + expf(-g));
+    if (act == BN_ACT_GELU_TANH) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * g * (1.0f + 0.044715f * g * g)));
+    const float p = fmaxf(g, 0.f);
+    return p * p;
+}
+
 static inline int bn_launch_status() { return (int)hipGetLastError(); }

@@ -3,12 +3,14 @@
 // activation type (float or bf16) that the matrix products read and write.
 #include "common.h"
 
-// x[t, :] = float(E[token[t], :]).  A token outside [0, vocab) gives a zero row, as the
+// x[t, :] = float(E[token[t], :]) * scale.  A token outside [0, vocab) gives a zero row, as the
 // reference's embedding does (src/model_embed.c:6-28, test/test_safety.c:278-315); the
-// step function rejects such tokens before it launches anything.
+// step function rejects such tokens before it launches anything.  scale is the architecture's
+// embedding multiplier (src/model_embed.c:23-27 scales by sqrt(dim) under one of its policies;
+// 1 for this architecture, which changes no bit).
 template <typename T>
 __global__ void embed_gather_kernel(float* __restrict__ x, const T* __restrict__ table,
-                                    const int* __restrict__ tokens, int dim, int vocab) {
+                                    const int* __restrict__ tokens, int dim, int vocab, float scale) {
     const int t = blockIdx.x;
     const int tok = tokens[t];
     float* row = x + (size_t)t * dim;
@@ -17,7 +19,13 @@ __global__ void embed_gather_kernel(float* __restrict__ x, const T* __restrict__
         return;
     }
     const T* src = table + (size_t)tok * dim;
-    for (int i = threadIdx.x; i < dim; i += blockDim.x) row[i] = to_f32(src[i]);
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) row[i] = to_f32(src[i]) * scale;
+}
+
+// logits = cap * tanh(logits / cap), in place (src/transformer/logits.c:325-333)
+__global__ void softcap_kernel(float* __restrict__ x, size_t n, float cap, float inv) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] = tanhf(x[i] * inv) * cap;
 }
 
 // One block per output row r.  src row = rows ? rows[r] : r.
@@ -194,11 +202,11 @@ __global__ void residual_add_parts_kernel(float* __restrict__ x, const float* __
     x[i] = v;
 }
 
-// out[t, f] = silu(gu[t, f]) * gu[t, F + f], silu(g) = g / (1 + exp(-g))
-// (src/transformer/cpu_backend.c:385-391, exact exponential)
+// out[t, f] = act(gu[t, f]) * gu[t, F + f], act one of bn_gate_act's kinds: silu(g) = g / (1 + exp(-g))
+// (src/transformer/cpu_backend.c:385-391, exact exponential), gelu, relu2
 // il8: gate and up interleaved in blocks of 8 columns (gate f at 16*(f/8) + f%8, up 8 further)
 template <typename T>
-__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gu, int F, size_t n, int il8) {
+__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gu, int F, size_t n, int il8, int act) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     size_t t = i / F;
@@ -206,11 +214,11 @@ __global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gu, int
     const size_t gi = il8 ? t * 2 * F + 16 * (f / 8) + (f % 8) : t * 2 * F + f;
     float g = to_f32(gu[gi]);
     float u = to_f32(gu[il8 ? gi + 8 : gi + F]);
-    out[i] = from_f32<T>((g / (1.0f + expf(-g))) * u);
+    out[i] = from_f32<T>(bn_gate_act(g, act) * u);
 }
 
 // the same, 8 bf16 values a thread (F a multiple of 8, 16-byte aligned rows)
-__global__ void swiglu_bf16x8_kernel(bf16* __restrict__ out, const bf16* __restrict__ gu, int F, size_t n8, int il8) {
+__global__ void swiglu_bf16x8_kernel(bf16* __restrict__ out, const bf16* __restrict__ gu, int F, size_t n8, int il8, int act) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n8) return;
     const int f8 = F / 8;
@@ -223,8 +231,8 @@ __global__ void swiglu_bf16x8_kernel(bf16* __restrict__ out, const bf16* __restr
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const float g0 = bf16lo_to_f32(gw[k]), g1 = bf16hi_to_f32(gw[k]);
-        const float r0 = (g0 / (1.0f + expf(-g0))) * bf16lo_to_f32(uw[k]);
-        const float r1 = (g1 / (1.0f + expf(-g1))) * bf16hi_to_f32(uw[k]);
+        const float r0 = bn_gate_act(g0, act) * bf16lo_to_f32(uw[k]);
+        const float r1 = bn_gate_act(g1, act) * bf16hi_to_f32(uw[k]);
         const bf16 b0 = __float2bfloat16(r0), b1 = __float2bfloat16(r1);
         ow[k] = (uint32_t)(*reinterpret_cast<const uint16_t*>(&b0)) | ((uint32_t)(*reinterpret_cast<const uint16_t*>(&b1)) << 16);
     }
@@ -240,18 +248,24 @@ __global__ void bias_add_kernel(T* __restrict__ y, const float* __restrict__ b, 
 
 template <typename T>
 static int embed_gather_t(void* x, const void* table, const int* tokens, int n_tokens, int dim,
-                          int vocab, hipStream_t s) {
+                          int vocab, float scale, hipStream_t s) {
     hipLaunchKernelGGL(embed_gather_kernel<T>, dim3(n_tokens), dim3(256), 0, s, (float*)x,
-                       (const T*)table, tokens, dim, vocab);
+                       (const T*)table, tokens, dim, vocab, scale);
     return bn_launch_status();
 }
 
 extern "C" int bn_embed_gather(int dtype, void* x, const void* table, const int* tokens, int n_tokens,
-                               int dim, int vocab, hipStream_t s) {
+                               int dim, int vocab, float scale, hipStream_t s) {
     if (n_tokens <= 0 || dim <= 0 || vocab <= 0) return BN_ERR_ARG;
-    if (dtype == BN_DT_F32) return embed_gather_t<float>(x, table, tokens, n_tokens, dim, vocab, s);
-    if (dtype == BN_DT_BF16) return embed_gather_t<bf16>(x, table, tokens, n_tokens, dim, vocab, s);
+    if (dtype == BN_DT_F32) return embed_gather_t<float>(x, table, tokens, n_tokens, dim, vocab, scale, s);
+    if (dtype == BN_DT_BF16) return embed_gather_t<bf16>(x, table, tokens, n_tokens, dim, vocab, scale, s);
     return BN_ERR_DTYPE;
+}
+
+extern "C" int bn_softcap(float* x, long long n, float cap, hipStream_t s) {
+    if (n <= 0 || !(cap > 0.f)) return BN_ERR_ARG;
+    hipLaunchKernelGGL(softcap_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, (size_t)n, cap, 1.0f / cap);
+    return bn_launch_status();
 }
 
 template <typename T, typename TD = T>
@@ -338,19 +352,19 @@ extern "C" int bn_residual_add(int dtype, void* x, const void* delta, long long 
     return bn_launch_status();
 }
 
-extern "C" int bn_swiglu(int dtype, void* out, const void* gu, int n_rows, int F, int il8, hipStream_t s) {
-    if (n_rows <= 0 || F <= 0 || (il8 && F % 8)) return BN_ERR_ARG;
+extern "C" int bn_swiglu(int dtype, void* out, const void* gu, int n_rows, int F, int il8, int act, hipStream_t s) {
+    if (n_rows <= 0 || F <= 0 || (il8 && F % 8) || act < 0 || act >= BN_ACT_KINDS) return BN_ERR_ARG;
     const size_t n = (size_t)n_rows * F;
     const unsigned blocks = (unsigned)((n + 255) / 256);
     if (dtype == BN_DT_F32)
         hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, s, (float*)out,
-                           (const float*)gu, F, n, il8);
+                           (const float*)gu, F, n, il8, act);
     else if (dtype == BN_DT_BF16 && F % 8 == 0 && !(((uintptr_t)out | (uintptr_t)gu) & 15))
         hipLaunchKernelGGL(swiglu_bf16x8_kernel, dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0, s, (bf16*)out,
-                           (const bf16*)gu, F, n / 8, il8);
+                           (const bf16*)gu, F, n / 8, il8, act);
     else if (dtype == BN_DT_BF16)
         hipLaunchKernelGGL(swiglu_kernel<bf16>, dim3(blocks), dim3(256), 0, s, (bf16*)out,
-                           (const bf16*)gu, F, n, il8);
+                           (const bf16*)gu, F, n, il8, act);
     else
         return BN_ERR_DTYPE;
     return bn_launch_status();

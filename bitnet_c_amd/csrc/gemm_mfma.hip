@@ -58,7 +58,7 @@ __device__ __forceinline__ int gm_swizzle(int row) {
 template <int BN, bool GLU8, typename TO>
 __global__ __launch_bounds__(GM_THREADS) void gemm_mfma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                                TO* __restrict__ Y, int M, int N, int K, int ldx, int ldw,
-                                                               int ldy, int tiles_m, int tiles_n, int vec) {
+                                                               int ldy, int tiles_m, int tiles_n, int vec, int act) {
     constexpr int WM = GM_BM / GM_WGM, WN = BN / GM_WGN;      // a wave's part of the tile
     constexpr int MT = WM / 16, NT = WN / 16;         // 16 x 16 result tiles of a wave: MT x NT
     constexpr int PASS = GM_THREADS / 8;              // rows staged by one pass of the workgroup
@@ -250,7 +250,8 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_mfma_kernel(const bf16* __res
                     // silu(g) * u with the hardware's exp2 and reciprocal (an ulp each, far below the result's
                     // rounding): expf and a division cost 25 vector instructions a value, a tenth of this kernel's time
                     for (int r = 0; r < 4; ++r)
-                        v[r] = v[r] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504f * v[r])) * up[r];
+                        v[r] = (act == BN_ACT_SILU ? v[r] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504f * v[r]))
+                                                   : bn_gate_act(v[r], act)) * up[r];
                     store4(Y + (size_t)m * ldy + f, v, (N >> 1) - f);
                 }
             } else if (m < M) {
@@ -261,7 +262,8 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_mfma_kernel(const bf16* __res
 }
 
 template <int BN, bool GLU8, typename TO>
-static int gm_launch(const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw, int ldy, hipStream_t s) {
+static int gm_launch(const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw, int ldy, int act,
+                     hipStream_t s) {
     auto kernel = gemm_mfma_kernel<BN, GLU8, TO>;
     const size_t smem = (size_t)2 * (GM_BM + BN) * 128;
     static bool raised = false;                       // per instantiation
@@ -277,7 +279,7 @@ static int gm_launch(const void* X, const void* W, void* Y, int M, int N, int K,
     if (grid > 0x7fffffffLL) return BN_ERR_ARG;
     const int vec = (ldy % 4 == 0 && ((uintptr_t)Y % (4 * sizeof(TO))) == 0) ? 1 : 0;
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(GM_THREADS), smem, s, (const bf16*)X, (const bf16*)W, (TO*)Y,
-                       M, N, K, ldx, ldw, ldy, tiles_m, tiles_n, vec);
+                       M, N, K, ldx, ldw, ldy, tiles_m, tiles_n, vec, act);
     return bn_launch_status();
 }
 
@@ -316,10 +318,10 @@ extern "C" int bn_gemm_mfma_supports(int M, int N, int K, int ldx, int ldw) {
 }
 
 // out_dtype: type of Y (bf16 or float32).  glu8 != 0: W has 2N rows, gate and up interleaved in
-// blocks of 8 (N a multiple of 8), and Y[M, N] = silu(gate) * up.
+// blocks of 8 (N a multiple of 8), and Y[M, N] = act(gate) * up, act one of BN_ACT_*.
 extern "C" int bn_gemm_mfma(int out_dtype, const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw,
-                            int ldy, int glu8, hipStream_t s) {
-    if (!bn_gemm_mfma_supports(M, N, K, ldx, ldw) || ldy < N) return BN_ERR_ARG;
+                            int ldy, int glu8, int act, hipStream_t s) {
+    if (!bn_gemm_mfma_supports(M, N, K, ldx, ldw) || ldy < N || act < 0 || act >= BN_ACT_KINDS) return BN_ERR_ARG;
     if (((uintptr_t)X | (uintptr_t)W) & 15) return BN_ERR_ARG;
     if (out_dtype != BN_DT_BF16 && out_dtype != BN_DT_F32) return BN_ERR_DTYPE;
     if (glu8) {
@@ -332,8 +334,8 @@ extern "C" int bn_gemm_mfma(int out_dtype, const void* X, const void* W, void* Y
     const int bn = g_force_bn ? g_force_bn : gm_pick_bn(M, N, gm_compute_units());
     const bool f32 = out_dtype == BN_DT_F32;
 #define GM_GO(BN_, GLU_)                                                                          \
-    return f32 ? gm_launch<BN_, GLU_, float>(X, W, Y, M, N, K, ldx, ldw, ldy, s)                  \
-               : gm_launch<BN_, GLU_, bf16>(X, W, Y, M, N, K, ldx, ldw, ldy, s)
+    return f32 ? gm_launch<BN_, GLU_, float>(X, W, Y, M, N, K, ldx, ldw, ldy, act, s)             \
+               : gm_launch<BN_, GLU_, bf16>(X, W, Y, M, N, K, ldx, ldw, ldy, act, s)
     if (glu8) {
         if (bn == 256) { GM_GO(256, true); }
         if (bn == 192) { GM_GO(192, true); }

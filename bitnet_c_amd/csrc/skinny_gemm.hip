@@ -9,7 +9,8 @@
 // waves and MFMA instead.
 //
 // DUAL: W holds two row blocks (gate rows n, up rows up_off + n); the epilogue writes
-// silu(gate) * up, silu(g) = g / (1 + exp(-g)) (src/transformer/cpu_backend.c:385-391).
+// act(gate) * up, act one of the kinds of bn_gate_act (silu(g) = g / (1 + exp(-g)) for this
+// architecture, src/transformer/cpu_backend.c:385-391).
 // GLU8: the same product with gate and up rows interleaved in blocks of 8 (rows 16t..16t+7 are
 // gate rows 8t..8t+7, rows 16t+8..16t+15 the up rows of the same columns): every 16-row tile holds
 // both halves of 8 result columns, so the plain kernel does it with half the loads in flight.
@@ -35,7 +36,7 @@ __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast
 template <int MT, bool DUAL, typename TO, bool GLU8 = false, bool XS = false>
 __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                            TO* __restrict__ Y, int M, int N, int K, int ldx,
-                                                           int ldw, int ldy, int up_off) {
+                                                           int ldw, int ldy, int up_off, int act) {
     constexpr int NA = DUAL ? 2 * MT : MT;            // accumulator tiles per wave
     extern __shared__ __align__(16) float red[];      // [n_waves][NA][64][4]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -126,9 +127,9 @@ __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_ke
             // columns 0..7 of the tile are gates, 8..15 the ups of the same result columns
             const float up = __shfl_xor(v, 8, BN_WAVE);
             if ((l & 8) == 0 && m < M && nn < N)
-                Y[(size_t)m * ldy + (n0 >> 1) + (l & 7)] = from_f32<TO>((v / (1.0f + expf(-v))) * up);
+                Y[(size_t)m * ldy + (n0 >> 1) + (l & 7)] = from_f32<TO>(bn_gate_act(v, act) * up);
         } else if (m < M && nn < N) {
-            const float y = DUAL ? (v / (1.0f + expf(-v))) * u : v;
+            const float y = DUAL ? bn_gate_act(v, act) * u : v;
             Y[(size_t)m * ldy + nn] = from_f32<TO>(y);
         }
     }
@@ -162,7 +163,7 @@ struct SkinnyFused {
 template <bool GLU8, bool PRE, bool RES, int SL>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, bf16* __restrict__ Y, int M, int N,
-                              int K, int ldx, int ldw, int ldy, int tile_cols, SkinnyFused f) {
+                              int K, int ldx, int ldw, int ldy, int tile_cols, int act, SkinnyFused f) {
     constexpr int NW = 8;                              // always eight waves: wave w owns rows w and w + 8 of the norm
     extern __shared__ __align__(16) float red[];       // [NW][64][4], then 16 row scales, then the staging
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -245,7 +246,7 @@ void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict
         if (GLU8) {
             const float up = __shfl_xor(v, 8, BN_WAVE);
             if ((l & 8) == 0 && m < M && nn < N)                          // GLU8: tile_cols is 16
-                Y[(size_t)m * ldy + (n0 >> 1) + (l & 7)] = __float2bfloat16((v / (1.0f + expf(-v))) * up);
+                Y[(size_t)m * ldy + (n0 >> 1) + (l & 7)] = __float2bfloat16(bn_gate_act(v, act) * up);
         } else if (RES) {
             float xn = 0.f;
             if (m < M && mine) {
@@ -301,7 +302,7 @@ extern "C" int bn_skinny_gemm_fused_tiles(int N) {
     return (N + tc - 1) / tc;
 }
 
-// X, W, Y as bn_skinny_gemm with a bf16 result and M <= 16; glu8 as dual == 2 there.
+// X, W, Y as bn_skinny_gemm with a bf16 result and M <= 16; glu8 as dual == 2 there, act the gate's activation.
 // slots_in != null (PRE): X is a stream's bf16 copy as a RES call leaves it, slots_in [M, n_slots] its rows'
 // sums of squares in parts, stream_width its number of columns; the result's rows are scaled by
 // 1/sqrt(sum / stream_width + eps).
@@ -309,10 +310,10 @@ extern "C" int bn_skinny_gemm_fused_tiles(int N) {
 // times next_weight [N], slots_out [M, bn_skinny_gemm_fused_tiles(N)] the sums of squares of its column tiles
 // (glu8 == 0, no Y).
 extern "C" int bn_skinny_gemm_fused(const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw, int ldy,
-                                    int glu8, const float* slots_in, int n_slots, int stream_width, float eps,
+                                    int glu8, int act, const float* slots_in, int n_slots, int stream_width, float eps,
                                     float* resid, int ld_resid, void* resid_bf16, int ld_rb, const float* next_weight,
                                     float* slots_out, hipStream_t s) {
-    if (!bn_skinny_gemm_supports(M, N, K, ldx, ldw) || M > 16) return BN_ERR_ARG;
+    if (!bn_skinny_gemm_supports(M, N, K, ldx, ldw) || M > 16 || act < 0 || act >= BN_ACT_KINDS) return BN_ERR_ARG;
     if (((uintptr_t)X | (uintptr_t)W) & 15) return BN_ERR_ARG;
     const bool pre = slots_in != nullptr, res = resid != nullptr;
     if (!pre && !res) return BN_ERR_ARG;
@@ -337,7 +338,7 @@ extern "C" int bn_skinny_gemm_fused(const void* X, const void* W, void* Y, int M
             if (e != hipSuccess) return (int)e;
         }
         hipLaunchKernelGGL(kernel, grid, block, smem, s, (const bf16*)X, (const bf16*)W, (bf16*)Y, M, N, K, ldx, ldw, ldy,
-                           tile_cols, f);
+                           tile_cols, act, f);
         return bn_launch_status();
     };
     const bool few = n_slots <= 256;                  // four slot loads per row and lane are enough
@@ -353,7 +354,7 @@ extern "C" int bn_skinny_gemm_fused(const void* X, const void* W, void* Y, int M
 
 template <int MT, bool DUAL, typename TO, bool GLU8 = false>
 static int launch(const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw, int ldy,
-                  int up_off, int n_waves, hipStream_t s) {
+                  int up_off, int act, int n_waves, hipStream_t s) {
     constexpr int NA = DUAL ? 2 * MT : MT;
     constexpr bool XS = MT == 1 && !DUAL;          // the two-block form has no registers to spare for it
     const size_t smem = (size_t)n_waves * NA * 64 * 4 * sizeof(float) + (XS ? (size_t)n_waves * M * SK_XROW : 0);
@@ -368,37 +369,33 @@ static int launch(const void* X, const void* W, void* Y, int M, int N, int K, in
         }
     }
     hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(n_waves * 64), smem, s,
-                       (const bf16*)X, (const bf16*)W, (TO*)Y, M, N, K, ldx, ldw, ldy, up_off);
+                       (const bf16*)X, (const bf16*)W, (TO*)Y, M, N, K, ldx, ldw, ldy, up_off, act);
     return bn_launch_status();
 }
 
 template <typename TO>
 static int launch_glu8(int MT, const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw,
-                       int ldy, int n_waves, hipStream_t s) {
+                       int ldy, int act, int n_waves, hipStream_t s) {
     switch (MT) {
-        case 1: return launch<1, false, TO, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, n_waves, s);
-        case 2: return launch<2, false, TO, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, n_waves, s);
-        case 3: return launch<3, false, TO, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, n_waves, s);
-        case 4: return launch<4, false, TO, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, n_waves, s);
+        case 1: return launch<1, false, TO, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, act, n_waves, s);
+        case 2: return launch<2, false, TO, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, act, n_waves, s);
+        case 3: return launch<3, false, TO, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, act, n_waves, s);
+        case 4: return launch<4, false, TO, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, act, n_waves, s);
     }
     return BN_ERR_ARG;
 }
 
 template <bool DUAL, typename TO>
 static int launch_mt(int MT, const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw,
-                     int ldy, int up_off, int n_waves, hipStream_t s) {
+                     int ldy, int up_off, int act, int n_waves, hipStream_t s) {
     switch (MT) {
-        case 1: return launch<1, DUAL, TO>(X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s);
-        case 2: return launch<2, DUAL, TO>(X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s);
-        case 3: return launch<3, DUAL, TO>(X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s);
-        case 4: return launch<4, DUAL, TO>(X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s);
+        case 1: return launch<1, DUAL, TO>(X, W, Y, M, N, K, ldx, ldw, ldy, up_off, act, n_waves, s);
+        case 2: return launch<2, DUAL, TO>(X, W, Y, M, N, K, ldx, ldw, ldy, up_off, act, n_waves, s);
+        case 3: return launch<3, DUAL, TO>(X, W, Y, M, N, K, ldx, ldw, ldy, up_off, act, n_waves, s);
+        case 4: return launch<4, DUAL, TO>(X, W, Y, M, N, K, ldx, ldw, ldy, up_off, act, n_waves, s);
     }
     return BN_ERR_ARG;
 }
-
-// Tuning hook: > 0 fixes the waves per workgroup (still bounded by the K chunks and by shared memory).
-static int g_force_waves = 0;
-extern "C" void bn_skinny_gemm_force_waves(int n) { g_force_waves = n; }
 
 // 1 if the kernel takes the shape, 0 if the caller must use the tiled kernel.
 extern "C" int bn_skinny_gemm_supports(int M, int N, int K, int ldx, int ldw) {
@@ -407,10 +404,11 @@ extern "C" int bn_skinny_gemm_supports(int M, int N, int K, int ldx, int ldw) {
 
 // out_dtype: type of Y (bf16 or float32).  dual == 1: N is the width of the result and W has
 // the gate rows at [0, N) and the up rows at [up_off, up_off + N).  dual == 2: W has 2N rows, gate
-// and up interleaved in blocks of 8 (N a multiple of 8); the result has N columns.
+// and up interleaved in blocks of 8 (N a multiple of 8); the result has N columns.  act: the gate's activation
+// (BN_ACT_*), used when dual != 0.
 extern "C" int bn_skinny_gemm(int out_dtype, const void* X, const void* W, void* Y, int M, int N, int K,
-                              int ldx, int ldw, int ldy, int dual, int up_off, hipStream_t s) {
-    if (!bn_skinny_gemm_supports(M, N, K, ldx, ldw) || ldy < N) return BN_ERR_ARG;
+                              int ldx, int ldw, int ldy, int dual, int up_off, int act, hipStream_t s) {
+    if (!bn_skinny_gemm_supports(M, N, K, ldx, ldw) || ldy < N || act < 0 || act >= BN_ACT_KINDS) return BN_ERR_ARG;
     if (((uintptr_t)X | (uintptr_t)W) & 15) return BN_ERR_ARG;
     if (dual == 2) {
         if (N % 8) return BN_ERR_ARG;
@@ -423,21 +421,20 @@ extern "C" int bn_skinny_gemm(int out_dtype, const void* X, const void* W, void*
     const int tiles = (N + 15) / 16;
     int n_waves = tiles >= 2048 ? 4 : (tiles >= 1024 ? 8 : 16);
     if (MT == 1 && dual != 1) n_waves = 8;        // staged activations: measured best at every size (several workgroups per CU)
-    if (g_force_waves > 0) n_waves = g_force_waves;
     const int k_chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
     while (n_waves > 1 && n_waves / 2 >= k_chunks) n_waves >>= 1;
     while (n_waves > 1 && n_waves * NA > 48) n_waves >>= 1;
     if (dual == 1 && MT >= 3 && n_waves > 8) n_waves = 8;      // that variant is built for 512 threads
     if (dual == 2) {
-        if (out_dtype == BN_DT_BF16) return launch_glu8<bf16>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, n_waves, s);
-        if (out_dtype == BN_DT_F32) return launch_glu8<float>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, n_waves, s);
+        if (out_dtype == BN_DT_BF16) return launch_glu8<bf16>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, act, n_waves, s);
+        if (out_dtype == BN_DT_F32) return launch_glu8<float>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, act, n_waves, s);
         return BN_ERR_DTYPE;
     }
     if (out_dtype == BN_DT_BF16)
-        return dual ? launch_mt<true, bf16>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s)
-                    : launch_mt<false, bf16>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s);
+        return dual ? launch_mt<true, bf16>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, up_off, act, n_waves, s)
+                    : launch_mt<false, bf16>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, up_off, act, n_waves, s);
     if (out_dtype == BN_DT_F32)
-        return dual ? launch_mt<true, float>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s)
-                    : launch_mt<false, float>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, up_off, n_waves, s);
+        return dual ? launch_mt<true, float>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, up_off, act, n_waves, s)
+                    : launch_mt<false, float>(MT, X, W, Y, M, N, K, ldx, ldw, ldy, up_off, act, n_waves, s);
     return BN_ERR_DTYPE;
 }

@@ -27,11 +27,12 @@ __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast
 #define SG_XROW 528                   // bytes of a staged row of X: 512 + 16, so that the 16 rows a read touches spread over the banks
 #define SG_MAX_ROWS 128
 
-// GLU: P is unused and Y [M, N / 2] (row stride ldy) takes silu(gate) * up; else Y is unused and P takes the partial sums.
+// GLU: P is unused and Y [M, N / 2] (row stride ldy) takes act(gate) * up (bn_gate_act); else Y is unused and P takes
+// the partial sums.
 template <int MT, int NWV, bool GLU>
 __global__ __launch_bounds__(NWV * 64) void splitk_gemm_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                                float* __restrict__ P, bf16* __restrict__ Y, int M, int N, int K,
-                                                               int ldx, int ldw, int ldy, int k_per_split) {
+                                                               int ldx, int ldw, int ldy, int k_per_split, int act) {
     extern __shared__ __align__(16) unsigned char xs[];       // [2][MT * 16][SG_XROW]
     constexpr int ROWS = MT * 16;
     constexpr int RP = NWV * 2;                               // rows staged per pass of the workgroup (32 threads a row)
@@ -111,7 +112,7 @@ __global__ __launch_bounds__(NWV * 64) void splitk_gemm_kernel(const bf16* __res
                 const float up = __shfl_xor(v, 8, BN_WAVE);
                 const int m = mt * 16 + 4 * g + r;
                 if ((i & 8) == 0 && m < M && n0 + i < N)
-                    Y[(size_t)m * ldy + (n0 >> 1) + i] = __float2bfloat16((v / (1.0f + expf(-v))) * up);
+                    Y[(size_t)m * ldy + (n0 >> 1) + i] = __float2bfloat16(bn_gate_act(v, act) * up);
             }
         return;
     }
@@ -172,15 +173,16 @@ extern "C" int bn_splitk_gemm(const void* X, const void* W, float* P, int M, int
     const dim3 grid((N + SG_COLS - 1) / SG_COLS, splits), block(SG_WAVES * 64);
     const size_t smem = (size_t)2 * MT * 16 * SG_XROW;
     auto go = [&](auto kernel) {
-        static bool raised = false;               // per instantiation of this lambda, that is per kernel
-        if (smem > 64 * 1024 && !raised) {        // more than the default limit of dynamic shared memory
+        // Every instantiation decays to the same pointer type, so this lambda exists once: the flags are kept per MT.
+        static bool raised[SG_MAX_ROWS / 16 + 1] = {false};
+        if (smem > 64 * 1024 && !raised[MT]) {    // more than the default limit of dynamic shared memory
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e != hipSuccess) return (int)e;
-            raised = true;
+            raised[MT] = true;
         }
         hipLaunchKernelGGL(kernel, grid, block, smem, s, (const bf16*)X, (const bf16*)W, P, (bf16*)nullptr, M, N, K, ldx, ldw, 0,
-                           kps);
+                           kps, 0);
         return bn_launch_status();
     };
     switch (MT) {
@@ -196,10 +198,11 @@ extern "C" int bn_splitk_gemm(const void* X, const void* W, float* P, int M, int
     return BN_ERR_ARG;
 }
 
-// Y[M, F] (bf16, row stride ldy) = silu(X . Wg^T) * (X . Wu^T) for W [2F, K] with gate and up rows interleaved in blocks
-// of 8 (F a multiple of 8); X, W as above.
+// Y[M, F] (bf16, row stride ldy) = act(X . Wg^T) * (X . Wu^T) for W [2F, K] with gate and up rows interleaved in blocks
+// of 8 (F a multiple of 8); X, W as above; act one of BN_ACT_*.
 extern "C" int bn_splitk_gemm_swiglu(const void* X, const void* W, void* Y, int M, int F, int K, int ldx, int ldw, int ldy,
-                                     hipStream_t s) {
+                                     int act, hipStream_t s) {
+    if (act < 0 || act >= BN_ACT_KINDS) return BN_ERR_ARG;
     if (F < 8 || F % 8 || F > (1 << 29) || !bn_splitk_gemm_supports(M, 2 * F, K, ldx, ldw) || !X || !W || !Y || ldy < F)
         return BN_ERR_ARG;
     if (((uintptr_t)X | (uintptr_t)W) & 15) return BN_ERR_ARG;
@@ -208,15 +211,15 @@ extern "C" int bn_splitk_gemm_swiglu(const void* X, const void* W, void* Y, int 
     const dim3 grid((N + SG_GLU_WAVES * 16 - 1) / (SG_GLU_WAVES * 16), 1), block(SG_GLU_WAVES * 64);
     const size_t smem = (size_t)2 * MT * 16 * SG_XROW;
     auto go = [&](auto kernel) {
-        static bool raised = false;               // per instantiation of this lambda, that is per kernel
-        if (smem > 64 * 1024 && !raised) {        
+        static bool raised[SG_MAX_ROWS / 16 + 1] = {false};       // per MT, as above
+        if (smem > 64 * 1024 && !raised[MT]) {
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e != hipSuccess) return (int)e;
-            raised = true;
+            raised[MT] = true;
         }
         hipLaunchKernelGGL(kernel, grid, block, smem, s, (const bf16*)X, (const bf16*)W, (float*)nullptr, (bf16*)Y, M, N, K, ldx,
-                           ldw, ldy, kps);
+                           ldw, ldy, kps, act);
         return bn_launch_status();
     };
     switch (MT) {

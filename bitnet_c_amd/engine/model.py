@@ -71,11 +71,14 @@ class DecoderModel:
     def forward(self, ctx, views) -> torch.Tensor:
         """ctx: the step's StepContext; views[i]: the KVView of schedule entry i.
         Returns float32 logits [len(ctx.want_rows), vocab]."""
-        x = ops.embed_gather(self.embedding, ctx.tokens)          # src/model_embed.c:6-28
+        x = ops.embed_gather(self.embedding, ctx.tokens, self.plan.embedding_multiplier)    # src/model_embed.c:6-28
         stream = ResidualStream(x)
         for i, e in enumerate(self.plan.schedule):
             ctx.entry = i
             self.blocks[e.layer].forward(stream, ctx, views[i])
         # final norm on the wanted rows only, then the output matrix (src/transformer/logits.c:249-314)
         h = stream.normed(self.final_norm, self.dtype, rows=ctx.want_rows)
-        return ops.linear(h, self.lm_head, torch.float32)
+        logits = ops.linear(h, self.lm_head, torch.float32)
+        if self.plan.logit_softcap > 0:                            # src/transformer/logits.c:325-333
+            ops.softcap_(logits, self.plan.logit_softcap)
+        return logits

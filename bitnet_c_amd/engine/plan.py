@@ -41,8 +41,14 @@ class ModelPlan:
     lm_head_name: Optional[str]          # None: the output matrix is the embedding matrix (tied)
     max_positions: int = 0               # 0: no limit from the architecture
     stop_ids: tuple = ()
+    # What some architectures put around the blocks (the reference: src/model_embed.c:23-27 scales the embedding
+    # row, src/transformer/logits.c:325-333 bounds the logits); 1 and 0 leave this architecture's values as they are.
+    embedding_multiplier: float = 1.0    # the embedding row times this before the first block
+    logit_softcap: float = 0.0           # > 0: logits = cap * tanh(logits / cap)
 
     def validate(self) -> None:
+        if not self.embedding_multiplier > 0 or self.logit_softcap < 0:
+            raise ValueError("the embedding multiplier must be positive and the logit soft-cap 0 (none) or positive")
         for i, e in enumerate(self.schedule):
             if not 0 <= e.layer < len(self.layers):
                 raise ValueError(f"schedule entry {i} names layer {e.layer}; there are {len(self.layers)}")

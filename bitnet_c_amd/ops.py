@@ -28,7 +28,8 @@ class KernelError(RuntimeError):
 
 _SIGNATURES = {
     "elementwise": {
-        "bn_embed_gather": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "bn_embed_gather": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
+        "bn_softcap": [c_void_p, c_longlong, c_float, c_void_p],
         "bn_add_rmsnorm": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p],
         "bn_residual_add": [c_int, c_void_p, c_void_p, c_longlong, c_void_p],
         "bn_add_rmsnorm_parts": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
@@ -37,7 +38,7 @@ _SIGNATURES = {
         "bn_add_rmsnorm_parts_pieces": [c_int],
         "bn_add_rmsnorm_parts_wide": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_float,
                                       c_void_p],
-        "bn_swiglu": [c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "bn_swiglu": [c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "bn_bias_add": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
     },
     "rope_kv": {
@@ -65,14 +66,15 @@ _SIGNATURES = {
     },
     "gemm_mfma": {
         "bn_gemm_mfma_supports": [c_int, c_int, c_int, c_int, c_int],
-        "bn_gemm_mfma": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bn_gemm_mfma": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                         c_void_p],
     },
     "skinny_gemm": {
         "bn_skinny_gemm_supports": [c_int, c_int, c_int, c_int, c_int],
         "bn_skinny_gemm": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                           c_int, c_void_p],
+                           c_int, c_int, c_void_p],
         "bn_skinny_gemm_fused_tiles": [c_int],
-        "bn_skinny_gemm_fused": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+        "bn_skinny_gemm_fused": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                  c_void_p, c_int, c_int, c_float, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                  c_void_p],
     },
@@ -80,7 +82,7 @@ _SIGNATURES = {
         "bn_splitk_gemm_supports": [c_int, c_int, c_int, c_int, c_int],
         "bn_splitk_gemm_splits": [c_int, c_int],
         "bn_splitk_gemm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-        "bn_splitk_gemm_swiglu": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bn_splitk_gemm_swiglu": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "sampling": {
         "bn_argmax": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
@@ -160,12 +162,25 @@ def _code(dtype) -> int:
     return _DT[dtype]
 
 
+# The gate's activation of a gated feed-forward, out = act(gate) * up (BN_ACT_* of csrc/common.h): every kernel that
+# ends in a gated unit takes the kind as an argument.
+ACTIVATIONS = {"silu": _build.header_constant("BN_ACT_SILU"), "gelu_tanh": _build.header_constant("BN_ACT_GELU_TANH"),
+               "relu2": _build.header_constant("BN_ACT_RELU2")}
+
+
+def _act(name: str) -> int:
+    if name not in ACTIVATIONS:
+        raise KernelError(f"unknown gate activation {name!r}; the kernels take {sorted(ACTIVATIONS)}")
+    return ACTIVATIONS[name]
+
+
 # --------------------------------------------------------------------------------------
 # row-wise kernels
 # --------------------------------------------------------------------------------------
 
-def embed_gather(table: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
-    """float32 rows of the embedding table for int32 token ids."""
+def embed_gather(table: torch.Tensor, tokens: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """float32 rows of the embedding table for int32 token ids, times `scale` (an architecture's embedding
+    multiplier; 1 changes no bit)."""
     require_gpu()
     _dev(table, "table", dims=2)
     _dev(tokens, "tokens", torch.int32, 1)
@@ -174,9 +189,19 @@ def embed_gather(table: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
     n, dim = tokens.numel(), table.shape[1]
     x = torch.empty((n, dim), dtype=torch.float32, device=table.device)
     _check(_fn("elementwise", "bn_embed_gather")(_code(table.dtype), x.data_ptr(), table.data_ptr(),
-                                                 tokens.data_ptr(), n, dim, table.shape[0], _stream()),
+                                                 tokens.data_ptr(), n, dim, table.shape[0], float(scale), _stream()),
            "embed_gather")
     return x
+
+
+def softcap_(logits: torch.Tensor, cap: float) -> None:
+    """In place: cap * tanh(logits / cap), float32 (an architecture's bound on its logits; cap > 0)."""
+    require_gpu()
+    _dev(logits, "logits", torch.float32)
+    if not logits.is_contiguous() or not cap > 0:
+        raise KernelError("softcap: contiguous float32 logits and a positive cap")
+    if logits.numel():
+        _check(_fn("elementwise", "bn_softcap")(logits.data_ptr(), logits.numel(), float(cap), _stream()), "softcap")
 
 
 def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor, eps: float, out_dtype,
@@ -244,9 +269,9 @@ def residual_add(x: torch.Tensor, delta) -> None:
                                                  x.numel(), _stream()), "residual_add")
 
 
-def swiglu(gu: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
-    """[T, 2F] (gate | up) -> silu(gate) * up, [T, F].  interleaved: gate and up columns
-    alternate in blocks of 8 (see interleave_gate_up)."""
+def swiglu(gu: torch.Tensor, interleaved: bool = False, activation: str = "silu") -> torch.Tensor:
+    """[T, 2F] (gate | up) -> act(gate) * up, [T, F].  interleaved: gate and up columns
+    alternate in blocks of 8 (see interleave_gate_up).  activation: one of ACTIVATIONS."""
     require_gpu()
     _dev(gu, "gu", dims=2)
     if not gu.is_contiguous() or gu.shape[1] % 2:
@@ -256,7 +281,7 @@ def swiglu(gu: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
     if interleaved and F % 8:
         raise KernelError("swiglu: the interleaved layout needs F to be a multiple of 8")
     _check(_fn("elementwise", "bn_swiglu")(_code(gu.dtype), out.data_ptr(), gu.data_ptr(), T, F, int(interleaved),
-                                           _stream()), "swiglu")
+                                           _act(activation), _stream()), "swiglu")
     return out
 
 
@@ -284,9 +309,9 @@ def _tiled(x, w, out_dtype):
     return y
 
 
-def gemm_mfma(x: torch.Tensor, w: torch.Tensor, out_dtype=None, glu8: bool = False) -> torch.Tensor:
+def gemm_mfma(x: torch.Tensor, w: torch.Tensor, out_dtype=None, glu8: bool = False, activation: str = "silu") -> torch.Tensor:
     """The library-free bf16 product for many rows: y[M, N] = x[M, K] . w[N, K]^T on the matrix cores,
-    or with glu8 silu(gate) * up for w = gate and up rows interleaved in blocks of 8 ([2N, K])."""
+    or with glu8 act(gate) * up for w = gate and up rows interleaved in blocks of 8 ([2N, K])."""
     require_gpu()
     _dev(x, "x", torch.bfloat16, 2)
     _dev(w, "w", torch.bfloat16, 2)
@@ -300,7 +325,8 @@ def gemm_mfma(x: torch.Tensor, w: torch.Tensor, out_dtype=None, glu8: bool = Fal
     if M == 0:
         return y
     _check(_fn("gemm_mfma", "bn_gemm_mfma")(_code(out_dtype), x.data_ptr(), w.data_ptr(), y.data_ptr(), M, N, K,
-                                            _rows(x, "x"), _rows(w, "w"), N, int(glu8), _stream()), "gemm_mfma")
+                                            _rows(x, "x"), _rows(w, "w"), N, int(glu8), _act(activation), _stream()),
+           "gemm_mfma")
     return y
 
 
@@ -357,7 +383,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, *, allow_library: O
     if small and aligned and skinny_supported(M, N, K, ldx, ldw):
         y = torch.empty((M, N), dtype=out_dtype, device=x.device)
         _check(_fn("skinny_gemm", "bn_skinny_gemm")(_code(out_dtype), x.data_ptr(), w.data_ptr(), y.data_ptr(),
-                                                    M, N, K, ldx, ldw, N, 0, 0, _stream()), "skinny_gemm")
+                                                    M, N, K, ldx, ldw, N, 0, 0, 0, _stream()), "skinny_gemm")
         return y
     if M > SKINNY_ROWS and allow_library:
         if out_dtype == torch.bfloat16:
@@ -387,11 +413,11 @@ SWIGLU_STAGED_ROWS = (17, 128)
 
 
 def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = False, *,
-                  allow_library: Optional[bool] = None) -> torch.Tensor:
-    """silu(x.Wg^T) * (x.Wu^T) for w_gate_up = [Wg; Wu] ([2F, K]), or the two interleaved in
-    blocks of 8 rows (interleave_gate_up).  The decode-sized bf16 case is one kernel, and so is the
-    interleaved case without the library; every other case is the product followed by the SwiGLU
-    kernel."""
+                  allow_library: Optional[bool] = None, activation: str = "silu") -> torch.Tensor:
+    """act(x.Wg^T) * (x.Wu^T) for w_gate_up = [Wg; Wu] ([2F, K]), or the two interleaved in
+    blocks of 8 rows (interleave_gate_up); act is silu unless `activation` names another of
+    ACTIVATIONS.  The decode-sized bf16 case is one kernel, and so is the interleaved case without
+    the library; every other case is the product followed by the gated-unit kernel."""
     require_gpu()
     _dev(x, "x", dims=2)
     _dev(w_gate_up, "w_gate_up", x.dtype, 2)
@@ -412,19 +438,19 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = 
             and _fn("splitk_gemm", "bn_splitk_gemm_supports")(M, 2 * F, K, ldx, ldw)):
         y = torch.empty((M, F), dtype=x.dtype, device=x.device)
         _check(_fn("splitk_gemm", "bn_splitk_gemm_swiglu")(x.data_ptr(), w_gate_up.data_ptr(), y.data_ptr(), M, F, K, ldx, ldw,
-                                                           F, _stream()), "splitk_gemm(glu)")
+                                                           F, _act(activation), _stream()), "splitk_gemm(glu)")
         return y
     if (x.dtype == torch.bfloat16 and (M <= SKINNY_ROWS or (M <= 64 and not allow_library))
             and aligned and skinny_supported(M, F, K, ldx, ldw)):
         y = torch.empty((M, F), dtype=x.dtype, device=x.device)
         _check(_fn("skinny_gemm", "bn_skinny_gemm")(_code(x.dtype), x.data_ptr(), w_gate_up.data_ptr(),
                                                     y.data_ptr(), M, F, K, ldx, ldw, F, 2 if interleaved else 1, F,
-                                                    _stream()), "skinny_gemm(glu)")
+                                                    _act(activation), _stream()), "skinny_gemm(glu)")
         return y
     if (x.dtype == torch.bfloat16 and interleaved and not allow_library and aligned
             and gemm_mfma_supported(M, 2 * F, K, ldx, ldw)):
-        return gemm_mfma(x, w_gate_up, x.dtype, glu8=True)
-    return swiglu(linear(x, w_gate_up, allow_library=allow_library), interleaved)
+        return gemm_mfma(x, w_gate_up, x.dtype, glu8=True, activation=activation)
+    return swiglu(linear(x, w_gate_up, allow_library=allow_library), interleaved, activation)
 
 
 # --------------------------------------------------------------------------------------
@@ -521,10 +547,11 @@ def can_fuse_norm(M: int, N: int, K: int, dtype) -> bool:
             and torch.cuda.is_available() and skinny_supported(M, N, K, K, K))
 
 
-def _fused_call(x, w, y, M, N, K, glu8, pre: Optional[DeferredNorm], resid, resid_bf16, next_weight, slots_out):
+def _fused_call(x, w, y, M, N, K, glu8, pre: Optional[DeferredNorm], resid, resid_bf16, next_weight, slots_out,
+                activation: str = "silu"):
     _check(_fn("skinny_gemm", "bn_skinny_gemm_fused")(
         x.data_ptr(), w.data_ptr(), y.data_ptr() if y is not None else None, M, N, K, _rows(x, "x"), _rows(w, "w"),
-        N if y is not None else 0, int(glu8),
+        N if y is not None else 0, int(glu8), _act(activation),
         pre.slots.data_ptr() if pre is not None else None, pre.slots.shape[1] if pre is not None else 0,
         pre.stream.shape[1] if pre is not None else 0, float(pre.eps) if pre is not None else 0.0,
         resid.data_ptr() if resid is not None else None, _rows(resid, "resid") if resid is not None else 0,
@@ -557,7 +584,7 @@ def linear_prenorm(pre: DeferredNorm, w: torch.Tensor) -> torch.Tensor:
     return y
 
 
-def linear_swiglu_prenorm(pre: DeferredNorm, w_gate_up: torch.Tensor) -> torch.Tensor:
+def linear_swiglu_prenorm(pre: DeferredNorm, w_gate_up: torch.Tensor, activation: str = "silu") -> torch.Tensor:
     """linear_swiglu(rmsnorm(stream), w) for gate and up interleaved in blocks of 8, in one kernel."""
     require_gpu()
     _dev(w_gate_up, "w_gate_up", torch.bfloat16, 2)
@@ -566,7 +593,7 @@ def linear_swiglu_prenorm(pre: DeferredNorm, w_gate_up: torch.Tensor) -> torch.T
     if w_gate_up.shape[0] % 16 or not can_fuse_norm(M, F, K, torch.bfloat16) or w_gate_up.data_ptr() % 16:
         raise KernelError(f"linear_swiglu_prenorm: {M} rows, w {tuple(w_gate_up.shape)} cannot be fused")
     y = torch.empty((M, F), dtype=torch.bfloat16, device=w_gate_up.device)
-    _fused_call(pre.scaled, w_gate_up, y, M, F, K, True, pre, None, None, None, None)
+    _fused_call(pre.scaled, w_gate_up, y, M, F, K, True, pre, None, None, None, None, activation)
     return y
 
 

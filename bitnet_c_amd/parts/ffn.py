@@ -1,5 +1,6 @@
-"""Dense gated feed-forward: down(silu(gate(x)) * up(x)), silu(g) = g / (1 + exp(-g))
-(src/transformer/cpu.c:1270-1303, src/transformer/cpu_backend.c:385-391).  Gate and up
+"""Dense gated feed-forward: down(act(gate(x)) * up(x)); act is a parameter, silu(g) = g / (1 + exp(-g)) for this
+architecture (src/transformer/cpu.c:1270-1303, src/transformer/cpu_backend.c:385-391; the reference's other kinds,
+tanh-gelu and relu^2, cpu_backend.c:343-417, are the kernels' other values).  Gate and up
 are stored stacked (as the reference's GPU upload stacks them, include/backend_model.h:22)
 so that one product computes both, with gate and up rows alternating in blocks of 8 when the
 width allows it, so that the decode kernel finds both halves of a result column in one tile;
@@ -13,13 +14,16 @@ from .base import FEED_FORWARDS, ParamSpec, Part
 from .linear import Linear
 
 
+@FEED_FORWARDS.register("gated")
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(Part):
     takes_deferred_norm = True      # forward accepts an ops.DeferredNorm for h
     gives_lazy_delta = True         # forward(..., lazy_ok=True) may return a LazyDelta
 
-    def __init__(self, hidden: int, intermediate: int, bias: bool = False):
-        self.hidden, self.F, self.has_bias = int(hidden), int(intermediate), bool(bias)
+    def __init__(self, hidden: int, intermediate: int, bias: bool = False, activation: str = "silu"):
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"feed-forward: unknown activation {activation!r}; known: {sorted(ops.ACTIVATIONS)}")
+        self.hidden, self.F, self.has_bias, self.activation = int(hidden), int(intermediate), bool(bias), activation
         self.gate_up, self.down = Linear(), Linear()
 
     def tensors(self):
@@ -49,11 +53,11 @@ class SwiGLU(Part):
             w = self.gate_up.weight
             if (not self.has_bias and self.interleaved and w.dtype == torch.bfloat16
                     and ops.can_fuse_norm(h.shape[0], self.F, self.hidden, w.dtype)):
-                act = ops.linear_swiglu_prenorm(h, w)
+                act = ops.linear_swiglu_prenorm(h, w, self.activation)
                 return self.down.lazy(act) if lazy_ok else self.down(act)
             h = h.materialize()
         if self.has_bias:
-            act = ops.swiglu(self.gate_up(h), self.interleaved)
+            act = ops.swiglu(self.gate_up(h), self.interleaved, self.activation)
         else:
-            act = ops.linear_swiglu(h, self.gate_up.weight, self.interleaved)
+            act = ops.linear_swiglu(h, self.gate_up.weight, self.interleaved, activation=self.activation)
         return self.down.lazy(act) if lazy_ok else self.down(act)

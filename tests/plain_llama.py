@@ -49,6 +49,7 @@ def read_config(folder: str) -> dict:
     c["eps"] = float(raw.get("rms_norm_eps") or 1e-5)         # src/model.c:264-266
     c["tied"] = bool(raw.get("tie_word_embeddings", False))   # src/model.c:453,486-493
     c["rope_scaling"] = raw.get("rope_scaling")
+    c["act"] = raw.get("hidden_act", "silu")                  # SiLU for this architecture (src/model_arch.c:807-810)
     c["max_pos"] = int(raw.get("max_position_embeddings", 0))
     return c
 
@@ -155,9 +156,23 @@ def silu(g: torch.Tensor) -> torch.Tensor:
     return g / (1.0 + torch.exp(-g))
 
 
-def swiglu(g: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
-    """hb[i] = silu(hb[i]) * hb2[i] (src/transformer/cpu_backend.c:385-391)."""
-    return silu(g) * u
+def gelu_tanh(g: torch.Tensor) -> torch.Tensor:
+    """0.5 g (1 + tanh(0.7978845608 g (1 + 0.044715 g^2))) (src/transformer/cpu_backend.c:27-29, without its
+    rounding of g and of the result to half precision)."""
+    return 0.5 * g * (1.0 + torch.tanh(0.7978845608028654 * g * (1.0 + 0.044715 * g * g)))
+
+
+def relu2(g: torch.Tensor) -> torch.Tensor:
+    """max(g, 0)^2 (src/transformer/cpu_backend.c:349-350)."""
+    return torch.clamp(g, min=0.0) ** 2
+
+
+GATE_ACTIVATIONS = {"silu": silu, "gelu_pytorch_tanh": gelu_tanh, "gelu_tanh": gelu_tanh, "relu2": relu2}
+
+
+def swiglu(g: torch.Tensor, u: torch.Tensor, act: str = "silu") -> torch.Tensor:
+    """hb[i] = act(hb[i]) * hb2[i], act = silu for this architecture (src/transformer/cpu_backend.c:365-391)."""
+    return GATE_ACTIVATIONS[act](g) * u
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None = None) -> torch.Tensor:
@@ -168,11 +183,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None = None) -> t
     return y if b is None else y + b.to(F32)
 
 
-def feed_forward(xb: torch.Tensor, wg, wu, wd, round_to=None, bg=None, bu=None, bd=None) -> torch.Tensor:
-    """gate, up -> silu(gate)*up -> down (src/transformer/cpu.c:1270-1303)."""
+def feed_forward(xb: torch.Tensor, wg, wu, wd, round_to=None, bg=None, bu=None, bd=None, act: str = "silu") -> torch.Tensor:
+    """gate, up -> act(gate)*up -> down (src/transformer/cpu.c:1270-1303)."""
     g = _rt(linear(xb, wg, bg), round_to)
     u = _rt(linear(xb, wu, bu), round_to)
-    h = _rt(swiglu(g, u), round_to)
+    h = _rt(swiglu(g, u, act), round_to)
     return _rt(linear(h, wd, bd), round_to)
 
 
@@ -199,23 +214,29 @@ def decoder_layer(x, positions, W, l, c, inv_freq, round_to=None, window=None):
     xb = _rt(rmsnorm(x, W[p + "post_attention_layernorm.weight"], c["eps"]), round_to)
     x = x + feed_forward(xb, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"],
                          W[p + "mlp.down_proj.weight"], round_to, b("mlp.gate_proj.bias"), b("mlp.up_proj.bias"),
-                         b("mlp.down_proj.bias"))
+                         b("mlp.down_proj.bias"), c.get("act", "silu"))
     return x
 
 
-def forward(c: dict, W: dict, tokens, round_to=None, pos0: int = 0) -> torch.Tensor:
+def forward(c: dict, W: dict, tokens, round_to=None, pos0: int = 0, emb_scale: float = 1.0,
+            softcap: float = 0.0) -> torch.Tensor:
     """Logits [T, vocab] (float32) of one whole sequence.  Embedding row, layers, final
     norm, output matrix or the embedding matrix when tied
-    (src/model_embed.c:6-28, src/transformer.c:128-169, src/transformer/logits.c:249-314)."""
+    (src/model_embed.c:6-28, src/transformer.c:128-169, src/transformer/logits.c:249-314).
+    emb_scale multiplies the embedding row (src/model_embed.c:23-27) and softcap > 0 bounds the
+    logits, tanh(logit / cap) * cap (src/transformer/logits.c:325-333); this architecture uses neither."""
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     positions = torch.arange(pos0, pos0 + tokens.numel())
     inv_freq = rope_inv_freq(c["head_dim"], c["theta"], c["rope_scaling"])
-    x = W["model.embed_tokens.weight"][tokens].to(F32)
+    x = W["model.embed_tokens.weight"][tokens].to(F32) * emb_scale
     for l in range(c["layers"]):
         x = decoder_layer(x, positions, W, l, c, inv_freq, round_to)
     xn = _rt(rmsnorm(x, W["model.norm.weight"], c["eps"]), round_to)
     out_w = W["model.embed_tokens.weight"] if c["tied"] else W["lm_head.weight"]
-    return linear(xn, out_w)
+    logits = linear(xn, out_w)
+    if softcap > 0.0:
+        logits = torch.tanh(logits * (1.0 / softcap)) * softcap
+    return logits
 
 
 # ----------------------------------------------------------------------------------

@@ -686,6 +686,41 @@ FURTHER_SIZES = [
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("act,F", [("gelu_pytorch_tanh", 264), ("relu2", 264), ("relu2", 173)])
+def test_other_gate_activations_through_the_engine(tmp_path, act, F, dtype):
+    """config.json's hidden_act reaches the feed-forward part as a parameter and the kernels as an argument:
+    prompts (the library's product and the gated-unit kernel, or the float32 kernels), then decoded tokens (the
+    streaming product's epilogue, with the norm folded in where the width allows), against the plain implementation."""
+    import bitnet_c_amd as bn
+    raw = dict(model_type="llama", vocab_size=211, hidden_size=128, intermediate_size=F, num_hidden_layers=2,
+               num_attention_heads=4, num_key_value_heads=2, head_dim=32, max_position_embeddings=512,
+               rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False, hidden_act=act)
+    folder = bn.write_model_folder(str(tmp_path / "m"), bn.LlamaConfig.from_dict(raw), 77, dtype)
+    c, W = pl.read_config(folder), pl.read_weights(folder)
+    assert c["act"] == act
+    eng = bn.Engine.from_folder(folder, dtype=dtype, max_tokens=1024)
+    assert eng.model.blocks[0].ffn.activation == {"gelu_pytorch_tanh": "gelu_tanh", "relu2": "relu2"}[act]
+    reqs = _requests(211, 78, [37, 74, 9])
+    slots = [eng.new_sequence() for _ in reqs]
+    got = [[] for _ in reqs]
+    lg = eng.step([bn.StepEntry(s, r[:-4], list(range(len(r) - 4))) for s, r in zip(slots, reqs)])
+    at = 0
+    for i, r in enumerate(reqs):
+        got[i].append(lg[at:at + len(r) - 4])
+        at += len(r) - 4
+    for t in range(4):
+        lg = eng.step([bn.StepEntry(s, [r[len(r) - 4 + t]], [0]) for s, r in zip(slots, reqs)])
+        for i in range(len(reqs)):
+            got[i].append(lg[i:i + 1].clone())
+    rounded = torch.bfloat16 if dtype == torch.bfloat16 else None
+    for i, r in enumerate(reqs):
+        want = pl.forward(c, W, r, rounded)
+        assert rel_err(torch.cat(got[i]), want) < TOL[dtype], i
+        other = pl.forward(dict(c, act="silu"), W, r, rounded)           # and it is not the default activation's result
+        assert rel_err(other, want) > 0.1
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("case", range(len(FURTHER_SIZES)))
 def test_further_sizes(tmp_path, case, dtype):
     """Unequal prompts in one step (logits at every place), then four tokens each, at sizes that the other tests

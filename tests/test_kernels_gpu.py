@@ -328,12 +328,88 @@ def test_swiglu_product_with_staged_activations(M, F, K):
     xd = x.cuda()
     y = torch.full((M, F), float("nan"), dtype=torch.bfloat16, device="cuda")
     rc = ops._fn("splitk_gemm", "bn_splitk_gemm_swiglu")(xd.data_ptr(), wi.data_ptr(), y.data_ptr(), M, F, K, K, K, F,
-                                                         torch.cuda.current_stream().cuda_stream)
+                                                         ops.ACTIVATIONS["silu"], torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     assert close(y.float(), want, torch.bfloat16)
     lo, hi = ops.SWIGLU_STAGED_ROWS
     if lo <= M <= hi:                              # without the library this is the kernel of these row counts
         assert torch.equal(ops.linear_swiglu(xd, wi, True, allow_library=False), y)
+
+
+@pytest.mark.parametrize("activation", ["gelu_tanh", "relu2", "silu"])
+def test_every_gated_epilogue_takes_the_activation(activation):
+    """The gate's activation is an argument of every kernel that ends in a gated unit: the gated-unit kernel
+    itself, the streaming product (both weight layouts), its form with the norm folded in, the product with
+    staged activations and the tiled matrix-core product.  Against the plain formula of that activation; and
+    the three activations differ from each other by far more than the tolerance."""
+    ops = _ops()
+    F, K = 328, 264
+    w = _rand((2 * F, K), torch.bfloat16, 62, 0.1)
+    wi = ops.interleave_gate_up(w[:F].cuda(), w[F:].cuda())
+
+    def want_for(x):
+        g, u = x.double() @ w[:F].double().t(), x.double() @ w[F:].double().t()
+        return pl.swiglu(g, u, activation).float()
+
+    others = [a for a in ops.ACTIVATIONS if a != activation]
+    x8 = _rand((8, K), torch.bfloat16, 61)
+    for o in others:
+        g, u = x8.double() @ w[:F].double().t(), x8.double() @ w[F:].double().t()
+        assert rel_err(pl.swiglu(g, u, o).float(), want_for(x8)) > 0.05
+    for dtype in DTYPES:                                                    # the gated-unit kernel, both layouts
+        gu = _rand((7, 2 * F), dtype, 63, 2.0)
+        want = pl.swiglu(gu[:, :F].float(), gu[:, F:].float(), activation)
+        assert close(ops.swiglu(gu.cuda(), False, activation).float(), want, dtype)
+        gi = torch.stack([gu[:, :F].reshape(7, F // 8, 8), gu[:, F:].reshape(7, F // 8, 8)], dim=2).reshape(7, 2 * F)
+        assert close(ops.swiglu(gi.contiguous().cuda(), True, activation).float(), want, dtype)
+    for M in (1, 8, 16, 40):                                                # the streaming product
+        x = _rand((M, K), torch.bfloat16, 64 + M)
+        assert close(ops.linear_swiglu(x.cuda(), w.cuda(), allow_library=False, activation=activation).float(),
+                     want_for(x), torch.bfloat16), M
+        assert close(ops.linear_swiglu(x.cuda(), wi, True, allow_library=False, activation=activation).float(),
+                     want_for(x), torch.bfloat16), M
+    for M in (24, 100):                                                     # staged activations (17 to 128 rows)
+        x = _rand((M, K), torch.bfloat16, 70 + M)
+        assert close(ops.linear_swiglu(x.cuda(), wi, True, allow_library=False, activation=activation).float(),
+                     want_for(x), torch.bfloat16), M
+    x = _rand((200, K), torch.bfloat16, 80)                                 # the tiled matrix-core product
+    assert close(ops.gemm_mfma(x.cuda(), wi, glu8=True, activation=activation).float(), want_for(x), torch.bfloat16)
+    # with the library the product is stored in bf16 first and the gated-unit kernel reads that: against the plain
+    # formula on the stored gate and up values
+    yl = ops.linear(x.cuda(), wi).float().cpu().reshape(200, F // 8, 2, 8)
+    gl, ul = yl[:, :, 0].reshape(200, F), yl[:, :, 1].reshape(200, F)
+    assert close(ops.linear_swiglu(x.cuda(), wi, True, activation=activation).float(), pl.swiglu(gl, ul, activation), torch.bfloat16)
+    # the norm folded in: a stream, its deferred norm, the gated product that applies it
+    M, D = 5, K
+    stream = _rand((M, D), torch.float32, 81, 2.0)
+    norm_w = _rand((D,), torch.float32, 82) * 0.2 + 1.0
+    act_in = _rand((M, 64), torch.bfloat16, 83)
+    w_out = _rand((D, 64), torch.bfloat16, 84, 0.1)
+    xs = stream.clone().cuda()
+    pre = ops.linear_into_stream(act_in.cuda(), w_out.cuda(), xs, norm_w.cuda(), 1e-5)
+    h = pl.rmsnorm((stream.double() + act_in.double() @ w_out.double().t()).float(), norm_w, 1e-5)
+    exact = want_for(h)
+    got = ops.linear_swiglu_prenorm(pre, wi, activation)
+    classic = ops.linear_swiglu(pre.materialize(), wi, True, activation=activation)
+    e_got, e_classic = rel_err(got.float(), exact), rel_err(classic.float(), exact)
+    assert e_got <= 2.0 * e_classic + 2.0 ** -7, (e_got, e_classic)
+    with pytest.raises(ops.KernelError):
+        ops.swiglu(_rand((2, 16), torch.float32, 1).cuda(), False, "gelu")
+
+
+def test_embedding_multiplier_and_logit_softcap_kernels():
+    ops = _ops()
+    table = _rand((50, 72), torch.bfloat16, 90)
+    toks = torch.tensor([3, 49, 0, 3], dtype=torch.int32)
+    assert torch.equal(ops.embed_gather(table.cuda(), toks.cuda()).cpu(), table[toks.long()].float())
+    got = ops.embed_gather(table.cuda(), toks.cuda(), math.sqrt(72.0))
+    assert torch.equal(got.cpu(), table[toks.long()].float() * torch.tensor(math.sqrt(72.0), dtype=torch.float32))
+    lg = _rand((5, 389), torch.float32, 91, 40.0)
+    g = lg.clone().cuda()
+    ops.softcap_(g, 30.0)
+    assert torch.allclose(g.cpu(), torch.tanh(lg / 30.0) * 30.0, atol=1e-5) and float(g.abs().max()) <= 30.0
+    with pytest.raises(ops.KernelError):
+        ops.softcap_(g, 0.0)
 
 
 def test_gemm_mfma_refuses_what_it_cannot_take():

@@ -3,6 +3,7 @@ twice, a layer that reads another layer's cache); and toy parts defined here, re
 and stepped without a change to the library's files: a mixer with a state of its own, a
 feed-forward with routing, another position encoding."""
 import json
+import math
 import os
 import random
 from dataclasses import asdict, dataclass
@@ -477,6 +478,58 @@ def test_a_state_mixer_that_addresses_its_state_on_the_device_decodes_under_grap
     for a, b in zip(*outs):
         assert torch.equal(a, b)
     assert torch.equal(torch.cat(outs[0][:12]), torch.cat(outs[0][12:]))      # the second round equals the first
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_an_architecture_with_an_embedding_multiplier_and_a_logit_softcap(tmp_path, dtype):
+    """Two fields of the plan, set by a toy architecture's builder: the embedding row times sqrt(hidden) before the
+    first block, the logits bounded by cap * tanh(logits / cap).  Prompts and decoded tokens (replayed from graphs)
+    against the plain implementation with the same two numbers."""
+    from dataclasses import replace
+    from bitnet_c_amd import Engine, StepEntry
+    from bitnet_c_amd.config import Architecture, LlamaConfig, register_architecture
+    from bitnet_c_amd.config.base import _ARCHITECTURES
+    from bitnet_c_amd.config.llama_plan import build_llama_plan
+    from bitnet_c_amd.weights import write_model_folder
+    from conftest import TINY_D
+    scale, cap = math.sqrt(TINY_D["hidden_size"]), 0.4
+
+    class CappedConfig(LlamaConfig):
+        @staticmethod
+        def from_dict(raw):
+            return CappedConfig(**{k: v for k, v in vars(LlamaConfig.from_dict(raw)).items()})
+
+        def to_dict(self):
+            return dict(LlamaConfig.to_dict(self), model_type="toy_capped", architectures=["ToyCapped"])
+
+    if "toy_capped" not in _ARCHITECTURES:
+        register_architecture(Architecture(
+            "toy_capped", CappedConfig,
+            lambda c: replace(build_llama_plan(c), embedding_multiplier=math.sqrt(c.hidden_size), logit_softcap=cap)))
+    cfg = CappedConfig.from_dict(dict(TINY_D, model_type="toy_capped"))
+    folder = write_model_folder(str(tmp_path / "capped"), cfg, 15, dtype)
+    eng = Engine.from_folder(folder, dtype=dtype, max_tokens=1024)
+    assert eng.model.plan.logit_softcap == cap and eng.use_graphs
+    c, W = pl.read_config(folder), pl.read_weights(folder)
+    rounded = torch.bfloat16 if dtype == torch.bfloat16 else None
+    rnd = random.Random(16)
+    reqs = [[rnd.randrange(cfg.vocab_size) for _ in range(n)] for n in (40, 7, 71)]
+    slots = [eng.new_sequence() for _ in reqs]
+    out = eng.step([StepEntry(s, r[:-5], list(range(len(r) - 5))) for s, r in zip(slots, reqs)])
+    got, o = [[] for _ in reqs], 0
+    for i, r in enumerate(reqs):
+        got[i].append(out[o:o + len(r) - 5])
+        o += len(r) - 5
+    for k in range(5):
+        out = eng.step([StepEntry(s, [r[len(r) - 5 + k]], [0]) for s, r in zip(slots, reqs)])
+        for i in range(3):
+            got[i].append(out[i:i + 1].clone())
+    for i, r in enumerate(reqs):
+        want = pl.forward(c, W, r, rounded, emb_scale=scale, softcap=cap)
+        assert float(want.abs().max()) > 0.5 * cap                          # the cap bites
+        assert rel_err(torch.cat(got[i]), want) < TOL[dtype], i
+        assert rel_err(pl.forward(c, W, r, rounded, emb_scale=scale), want) > 10 * TOL[dtype]
+        assert rel_err(pl.forward(c, W, r, rounded, softcap=cap), want) > 10 * TOL[dtype]
 
 
 def test_a_windowed_group_beside_a_full_one_through_the_engine(tmp_path):

@@ -162,6 +162,30 @@ def test_swiglu_reference_vector():
     assert torch.allclose(pl.swiglu(g, u), (g / (1 + torch.exp(-g))) * u, atol=0)
 
 
+def test_other_gate_activations_and_the_bounds_around_the_blocks():
+    g = torch.tensor([-3.0, -1.0, -0.25, 0.0, 0.25, 1.0, 2.0, 4.0])
+    u = torch.tensor([1.0, 0.5, 2.0, 3.0, -1.0, 1.5, -0.5, 2.0])
+    assert torch.allclose(pl.swiglu(g, u, "gelu_tanh"), torch.nn.functional.gelu(g, approximate="tanh") * u, atol=1e-6)
+    assert torch.equal(pl.swiglu(g, u, "relu2"), torch.tensor([0.0, 0, 0, 0, 0.0625, 1, 4, 16]) * u)
+    assert torch.equal(pl.swiglu(g, u), pl.swiglu(g, u, "silu"))
+    from conftest import TINY_A
+    c, W = _tiny(TINY_A, 9)
+    toks = [5, 6, 7]
+    base = pl.forward(c, W, toks)
+    # a soft-cap far above the logits changes almost nothing; a small one bounds them and keeps their order
+    assert torch.allclose(pl.forward(c, W, toks, softcap=1e4), base, atol=1e-5)
+    cap = float(base.abs().max())
+    capped = pl.forward(c, W, toks, softcap=cap)
+    assert abs(float(capped.abs().max()) - math.tanh(1.0) * cap) < 1e-5 * cap
+    assert torch.equal(capped.argsort(dim=1), base.argsort(dim=1))
+    # the embedding multiplier: the first norm takes a common factor out again (up to eps), so the logits move little
+    # with it, while a model whose first block were not normed would scale: the multiplier acts before the first block
+    W1 = dict(W)
+    W1["model.embed_tokens.weight"] = W["model.embed_tokens.weight"] * 8.0
+    W1["lm_head.weight"] = W["lm_head.weight"]
+    assert torch.allclose(pl.forward(c, W, toks, emb_scale=8.0), pl.forward(c, W1, toks), atol=1e-5)
+
+
 def _tiny(cfg, seed):
     g = torch.Generator().manual_seed(seed)
     c = dict(dim=cfg["hidden_size"], ffn=cfg["intermediate_size"], layers=cfg["num_hidden_layers"],
