@@ -429,8 +429,15 @@ __device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, con
 // same query rows and a stage is NG blocks of 32 keys, one for each group, so the chain of blocks
 // that a tile of late positions has to walk is NG times shorter; at the end the groups' partial
 // results (reference point, sum, accumulators) are merged through shared memory in group order.
+//
+// A causal tile's work grows with its position, and a launch is as long as its longest workgroup.  The
+// host hands the tiles over ordered by their number of keys, longest first, and workgroup p takes tile p
+// and then tile n - 1 - p: every workgroup walks about the same number of key blocks (a prompt of 2,048
+// tokens: 65 blocks each, half of them per wave group, where the last tile alone walks 64).  The grid is
+// one-dimensional with the kv heads running fastest: consecutive workgroups go to consecutive XCDs, so with
+// eight kv heads every XCD serves one of them and its keys and values live in one L2 only.
 template <int HS, int NT, int NG>
-__global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_mfma_prompt_kernel(MfmaArgs a) {
+__global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_mfma_prompt_kernel(MfmaArgs a, int n_tiles) {
     constexpr int DC = HS / 32, DT = HS / 16;
     constexpr int KB = 32 * NG;                           // keys per stage
     constexpr int KS = HS, VS = KB;                       // row strides (elements); both blocks swizzled, no padding
@@ -444,11 +451,13 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int n = lane & 15, g = lane >> 4;
     const int G = a.H / a.Hkv, GT = a.GT;
     const int n_head_tiles = (G + GT - 1) / GT;
-    const int kvh = blockIdx.y / n_head_tiles, ht = blockIdx.y - kvh * n_head_tiles;
-    // Later (longer) tiles start first; every other head walks the tiles the other way, so that the
-    // workgroups that share a CU while the whole launch is resident are a long one and a short one.
-    const bool ascending = blockIdx.y & 1;
-    const int* tl = a.tiles + 4 * (ascending ? blockIdx.x : gridDim.x - 1 - blockIdx.x);
+    const int hy = a.Hkv * n_head_tiles;
+    const int pair = blockIdx.x / hy, y = blockIdx.x - pair * hy;
+    const int kvh = y / n_head_tiles, ht = y - kvh * n_head_tiles;
+  for (int turn = 0; turn < 2; ++turn) {
+    const int tile = turn == 0 ? pair : n_tiles - 1 - pair;
+    if (turn == 1 && tile <= pair) break;                 // an odd number of tiles: the middle one has no partner
+    const int* tl = a.tiles + 4 * tile;
     const int seq = tl[0], tok0 = tl[1], n_tok = tl[2], pos0 = tl[3];
 
     bf16x8 q[NT][DC];
@@ -583,21 +592,24 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
                 __syncthreads();
             }
         }
-        if (grp != 0) return;
     }
+    if (grp == 0) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        if (qpos[nt] < 0) continue;
-        const float inv = l[nt] > 0.f ? 1.0f / l[nt] : 0.f;
-        bf16* o = a.out + (size_t)tok[nt] * a.out_stride + (size_t)head[nt] * HS + 4 * g;
+        for (int nt = 0; nt < NT; ++nt) {
+            if (qpos[nt] < 0) continue;
+            const float inv = l[nt] > 0.f ? 1.0f / l[nt] : 0.f;
+            bf16* o = a.out + (size_t)tok[nt] * a.out_stride + (size_t)head[nt] * HS + 4 * g;
 #pragma unroll
-        for (int t = 0; t < DT; ++t) {
-            uint2 w;
-            w.x = pack2(acc[nt][t][0] * inv, acc[nt][t][1] * inv);
-            w.y = pack2(acc[nt][t][2] * inv, acc[nt][t][3] * inv);
-            *reinterpret_cast<uint2*>(o + t * 16) = w;
+            for (int t = 0; t < DT; ++t) {
+                uint2 w;
+                w.x = pack2(acc[nt][t][0] * inv, acc[nt][t][1] * inv);
+                w.y = pack2(acc[nt][t][2] * inv, acc[nt][t][3] * inv);
+                *reinterpret_cast<uint2*>(o + t * 16) = w;
+            }
         }
     }
+    __syncthreads();                                      // the staging memory is free for the next tile
+  }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -716,6 +728,11 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
     const float scale2 = a.scale * LOG2E;
     if (k_lo < k_hi) {
         const size_t bt_row = (size_t)seq * a.bt_stride;
+        // (Keeping the next block's operands in a second set of registers while the current block is multiplied was
+        // measured and gained nothing: the CU's other waves already cover a wave's wait for its loads.)
+        // The waves take the blocks of 32 keys in turn, so that neighbouring waves ask for the two halves of a page at
+        // the same time (a wave that takes whole pages by itself was measured 10 to 20 % slower, and so was splitting
+        // the sequences of a large batch: the order by length with unsplit sequences keeps the CUs busiest).
         for (int kb = (k_lo / 32) * 32 + 32 * wave; kb < k_hi; kb += 128) {
             // the page index is the same for the whole wave: read through the scalar unit, so that it
             // does not queue behind the vector loads
@@ -831,15 +848,12 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
     a.by_length = (!tiles && n_splits == 1 && (long long)n_tiles * wgs_per_seq > compute_units()) ? by_length : nullptr;
     a.order_period = compute_units() / wgs_per_seq;
     if (tiles) {
-        const dim3 grid(n_tiles, Hkv * n_head_tiles);
-        // Two wave groups halve the chain of key blocks of a workgroup but not the work of its CU:
-        // they pay (measured 19 % at 1,024 tokens of the 8B shape) only while there are no more
-        // workgroups than CUs, so that each has a CU to itself.
-        const int ng = ((long long)grid.x * grid.y <= compute_units()) ? 2 : 1;
-        if (hs == 64 && ng == 2) hipLaunchKernelGGL((attn_mfma_prompt_kernel<64, 4, 2>), grid, dim3(512), 0, s, a);
-        else if (hs == 64) hipLaunchKernelGGL((attn_mfma_prompt_kernel<64, 4, 1>), grid, dim3(256), 0, s, a);
-        else if (ng == 2) hipLaunchKernelGGL((attn_mfma_prompt_kernel<128, 2, 2>), grid, dim3(512), 0, s, a);
-        else hipLaunchKernelGGL((attn_mfma_prompt_kernel<128, 2, 1>), grid, dim3(256), 0, s, a);
+        // workgroups of two wave groups (eight waves, one workgroup a CU), each with a pair of tiles
+        const long long wgs = (long long)((n_tiles + 1) / 2) * Hkv * n_head_tiles;
+        if (wgs > 0x7fffffff) return BN_ERR_ARG;
+        const dim3 grid((unsigned)wgs);
+        if (hs == 64) hipLaunchKernelGGL((attn_mfma_prompt_kernel<64, 4, 2>), grid, dim3(512), 0, s, a, n_tiles);
+        else hipLaunchKernelGGL((attn_mfma_prompt_kernel<128, 2, 2>), grid, dim3(512), 0, s, a, n_tiles);
         return bn_launch_status();
     }
     if (n_tiles > 65535) return BN_ERR_ARG;                 // sequences are the grid's y

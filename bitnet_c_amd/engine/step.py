@@ -81,7 +81,9 @@ class StepContext:
 
     def tiles(self, qt: int) -> torch.Tensor:
         """[n, 4] int32: (sequence, first row, rows <= qt, position of the first) covering all new
-        tokens, for the prompt form of the attention kernel."""
+        tokens, for the prompt form of the attention kernel; ordered by the number of keys a tile sees,
+        most first (the kernel pairs the first with the last, the second with the last but one, ...,
+        so that its workgroups carry equal work)."""
         t = self._tiles.get(qt)
         if t is None:
             rows, r = [], 0
@@ -89,6 +91,7 @@ class StepContext:
                 for i in range(0, n, qt):
                     rows.append((s, r + i, min(qt, n - i), p0 + i))
                 r += n
+            rows.sort(key=lambda t: -(t[3] + t[2]))
             t = torch.tensor(rows, dtype=torch.int32).reshape(-1, 4).to(self.device)
             self._tiles[qt] = t
         return t

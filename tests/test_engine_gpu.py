@@ -717,7 +717,7 @@ def test_other_gate_activations_through_the_engine(tmp_path, act, F, dtype):
         want = pl.forward(c, W, r, rounded)
         assert rel_err(torch.cat(got[i]), want) < TOL[dtype], i
         other = pl.forward(dict(c, act="silu"), W, r, rounded)           # and it is not the default activation's result
-        assert rel_err(other, want) > 0.1
+        assert rel_err(other, want) > 2 * TOL[dtype]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
