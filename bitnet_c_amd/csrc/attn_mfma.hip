@@ -665,6 +665,16 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
     const int chunk = a.max_len ? bn_split_chunk(uniform_load(a.max_len, 0), a.n_splits) : a.chunk;
     const int k_lo = max(lo_key, split * chunk), k_hi = min(L, (split + 1) * chunk);       // [k_lo, k_hi)
     const bf16* row = a.q + (size_t)seq * a.q_stride;
+    if (a.n_splits > 1 && k_lo >= k_hi) {
+        // A split without keys (a sequence shorter than the launch's longest, a padding row): it leaves "nothing seen"
+        // for the merge, which then does not read its sums, and is gone before it asks for anything else.
+        if (threadIdx.x < GT && ht * GT + threadIdx.x < G) {
+            const size_t prow = ((size_t)seq * a.H + kvh * G + ht * GT + threadIdx.x) * a.n_splits + split;
+            a.part_ml[prow * 2] = -INFINITY;
+            a.part_ml[prow * 2 + 1] = 0.f;
+        }
+        return;
+    }
 
     if (a.rotate && L > 0) {
         for (int i = threadIdx.x; i < HALF; i += 256) {
@@ -792,22 +802,28 @@ __global__ __launch_bounds__(64) void attn_mfma_combine_kernel(bf16* __restrict_
     float den = 0.f;
     for (int s = 0; s < n_splits; ++s) den = fmaf(__shfl(w, s, BN_WAVE), __shfl(ls, s, BN_WAVE), den);
     const float inv = den > 0.f ? 1.0f / den : 0.f;
-    for (int d = lane; d < hs; d += 64) {
-        float num = 0.f;
-        const float* po = part_o + (size_t)row * n_splits * hs + d;
-        for (int s0 = 0; s0 < n_splits; s0 += 8) {
-            float v[8];
-            float wj[8];
+    // dimensions lane and lane + 64 together, sixteen splits' loads in flight at once (a split without keys is not read)
+    const bool two = lane + 64 < hs;
+    float num0 = 0.f, num1 = 0.f;
+    const float* po = part_o + (size_t)row * n_splits * hs + lane;
+    for (int s0 = 0; s0 < n_splits; s0 += 16) {
+        float v0[16], v1[16], wj[16];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {                                  // loads first; a split without keys is not read
-                wj[j] = __shfl(w, min(s0 + j, 63), BN_WAVE);
-                v[j] = (s0 + j < n_splits && wj[j] != 0.f) ? po[(size_t)(s0 + j) * hs] : 0.f;
-            }
-#pragma unroll
-            for (int j = 0; j < 8; ++j) num = fmaf(wj[j], v[j], num);      // then split order
+        for (int j = 0; j < 16; ++j) {
+            wj[j] = __shfl(w, min(s0 + j, 63), BN_WAVE);
+            const bool in = s0 + j < n_splits && wj[j] != 0.f;
+            v0[j] = (in && lane < hs) ? po[(size_t)(s0 + j) * hs] : 0.f;
+            v1[j] = (in && two) ? po[(size_t)(s0 + j) * hs + 64] : 0.f;
         }
-        out[(size_t)tok * out_stride + (size_t)head * hs + d] = __float2bfloat16(num * inv);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {                                     // then the sums, in split order
+            num0 = fmaf(wj[j], v0[j], num0);
+            num1 = fmaf(wj[j], v1[j], num1);
+        }
     }
+    bf16* o = out + (size_t)tok * out_stride + (size_t)head * hs;
+    if (lane < hs) o[lane] = __float2bfloat16(num0 * inv);
+    if (two) o[lane + 64] = __float2bfloat16(num1 * inv);
 }
 
 // 1 when the matrix-core kernels take this shape
