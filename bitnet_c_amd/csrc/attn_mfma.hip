@@ -657,14 +657,33 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
         seq = a.by_length[r];
         if ((unsigned)seq >= gridDim.y) return;          // not a permutation: touch nothing
     }
-    const int L = a.seq_lens[seq];
+    // Everything that can be asked for before the sequence's length is known is asked for now (the query's heads, the
+    // frequencies, the new key and value): one wait for memory instead of one after the other.
     const int hg = ht * GT + n;
-    const bool ok = n < GT && hg < G && L > 0;
     const int head = kvh * G + hg;
+    const bf16* row = a.q + (size_t)seq * a.q_stride;
+    uint4 z[DC];
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+        z[c] = make_uint4(0, 0, 0, 0);
+        if (n < GT && hg < G) z[c] = *reinterpret_cast<const uint4*>(row + (size_t)head * HS + c * 32 + g * 8);
+    }
+    const int tid = threadIdx.x;
+    const float freq = (a.rotate && tid < HALF) ? a.inv_freq[tid] : 0.f;
+    bf16 new_k0 = __float2bfloat16(0.f), new_k1 = new_k0, new_v = new_k0;
+    if (a.write_kv) {
+        if (tid < HALF) {
+            new_k0 = row[(size_t)(a.H + kvh) * HS + tid];
+            new_k1 = row[(size_t)(a.H + kvh) * HS + tid + HALF];
+        } else if (tid < HALF + HS) {
+            new_v = row[(size_t)(a.H + a.Hkv + kvh) * HS + tid - HALF];
+        }
+    }
+    const int L = a.seq_lens[seq];
+    const bool ok = n < GT && hg < G && L > 0;
     const int lo_key = a.window > 0 ? max(0, L - a.window) : 0;
     const int chunk = a.max_len ? bn_split_chunk(uniform_load(a.max_len, 0), a.n_splits) : a.chunk;
     const int k_lo = max(lo_key, split * chunk), k_hi = min(L, (split + 1) * chunk);       // [k_lo, k_hi)
-    const bf16* row = a.q + (size_t)seq * a.q_stride;
     if (a.n_splits > 1 && k_lo >= k_hi) {
         // A split without keys (a sequence shorter than the launch's longest, a padding row): it leaves "nothing seen"
         // for the merge, which then does not read its sums, and is gone before it asks for anything else.
@@ -677,10 +696,10 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
     }
 
     if (a.rotate && L > 0) {
-        for (int i = threadIdx.x; i < HALF; i += 256) {
+        if (tid < HALF) {                                // HALF <= 64: one frequency a thread
             float sv, cv;
-            sincosf((float)(L - 1) * a.inv_freq[i], &sv, &cv);
-            cos_s[i] = cv; sin_s[i] = sv;
+            sincosf((float)(L - 1) * freq, &sv, &cv);
+            cos_s[tid] = cv; sin_s[tid] = sv;
         }
         __syncthreads();
     }
@@ -691,11 +710,9 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
         const int page = a.block_table[(size_t)seq * a.bt_stride + pos / BN_PAGE], off = pos % BN_PAGE;
         bf16* kdst = const_cast<bf16*>(a.k_pages) + (((size_t)page * a.Hkv + kvh) * BN_PAGE + off) * HS;
         bf16* vdst = const_cast<bf16*>(a.vt_pages) + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + off;
-        const bf16* kraw = row + (size_t)(a.H + kvh) * HS;
-        const bf16* vraw = row + (size_t)(a.H + a.Hkv + kvh) * HS;
         const int t = threadIdx.x;
         if (t < HALF) {
-            float k0 = __bfloat162float(kraw[t]), k1 = __bfloat162float(kraw[t + HALF]);
+            float k0 = __bfloat162float(new_k0), k1 = __bfloat162float(new_k1);
             if (a.rotate) {
                 const float c = cos_s[t], sv = sin_s[t];
                 const float r0 = k0 * c - k1 * sv, r1 = k0 * sv + k1 * c;
@@ -705,7 +722,7 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
             kdst[t + HALF] = __float2bfloat16(k1);
         } else if (t < HALF + HS) {
             const int d = t - HALF;
-            vdst[(size_t)d * BN_PAGE] = vraw[d];
+            vdst[(size_t)d * BN_PAGE] = new_v;
         }
         // only this workgroup reads what it has just stored: a fence of workgroup scope is enough
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
@@ -714,12 +731,6 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
 
     bf16x8 q[1][DC];
     {
-        uint4 z[DC];
-#pragma unroll
-        for (int c = 0; c < DC; ++c) {
-            z[c] = make_uint4(0, 0, 0, 0);
-            if (ok) z[c] = *reinterpret_cast<const uint4*>(row + (size_t)head * HS + c * 32 + g * 8);
-        }
         if (a.rotate && L > 0) {
 #pragma unroll
             for (int c = 0; c < DC / 2; ++c)      // chunk c holds pair indices c*32 + g*8 .. +7, its partners are in chunk c + DC/2
