@@ -25,6 +25,8 @@
 #include "attn_mfma.h"
 #include <mutex>
 
+#define PROMPT_BUFFERS 3      // staged key blocks of the prompt form in shared memory
+
 static int compute_units() {
     static int n[64] = {0};                 // per device
     int dev = 0;
@@ -79,6 +81,13 @@ __device__ __forceinline__ bf16x8 ld16(const bf16* p) {
 }
 // Combining a value with the ones 16 and 32 lanes away (the four lane groups of a column) without
 // going through shared memory: gfx950 swaps 16- and 32-lane halves between two registers.
+// The largest of three in one instruction; fmaxf would first bring each operand into canonical form (an instruction
+// each), which the scores out of the matrix cores do not need.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
 __device__ __forceinline__ float max_over_lane_groups(float x) {
     const unsigned b = __float_as_uint(x);
     auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
@@ -134,49 +143,38 @@ __device__ __forceinline__ int v_swizzle(int row) {
     return KEYS == 64 ? (h | ((row >> 1) & 1) << 2) : h;
 }
 
-// One 32-key block for NT column tiles.  kbase/vbase point at the block's first key inside its
-// page (row strides HS and BN_PAGE) or inside a staged copy in shared memory (KSTRIDE, VSTRIDE).  qpos/lo: per tile, this lane's column's position and first visible key (qpos < 0: no
-// such column).  key_hi: keys >= key_hi do not exist (decode: split end / length).
-// The same block for operands that come straight from the pages (the decode form: STREAM is false
-// here).  It is a copy of its own on purpose: the decode kernel is sensitive to how the compiler lays
-// this code out, and changes made for the staged form below must not move it.
-template <int HS, int NT, int KSTRIDE, int VSTRIDE, bool STREAM, bool need_mask>
+// One 32-key block for NT column tiles, operands straight from the pages (the decode form).  kbase/vbase point at
+// the block's first key inside its page (row strides HS and BN_PAGE).  qpos/lo: per tile, this lane's column's
+// position and first visible key (qpos < 0: no such column).  key_hi: keys >= key_hi do not exist (split end /
+// length).  All operands are asked for up front: they come from memory, and the latency is paid once.
+// The prompt form below has code of its own on purpose: the decode kernel is sensitive to how the compiler lays
+// this code out, and changes made for the staged form must not move it.
+template <int HS, int NT, bool need_mask>
 __device__ __forceinline__ void attend_block_direct_m(const bf16* __restrict__ kbase, const bf16* __restrict__ vbase,
-                                               int vchunk0, int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
+                                               int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
                                                float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
                                                const int (&lo)[NT], int key_hi, float scale2, int lane) {
-    // STREAM: the operands come from shared memory (short latency): fetch each one right before its
-    // products instead of all of them up front, which keeps fewer registers live.
-    constexpr int DC = HS / 32, DT = HS / 16;
+    constexpr int DC = HS / 32, DT = HS / 16, KSTRIDE = HS, VSTRIDE = BN_PAGE;
     const int i = lane & 15, g = lane >> 4;
     const int krow0 = 8 * (i >> 2) + (i & 3);        // key row of tile 0; tile 1 is 4 further
     f32x4 st[NT][2];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) { st[nt][0] = (f32x4){0.f, 0.f, 0.f, 0.f}; st[nt][1] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
-    bf16x8 ka[STREAM ? 1 : DC][2];
-    bf16x8 va[STREAM ? 1 : DT];
-    if (!STREAM) {
-#pragma unroll
-        for (int c = 0; c < DC; ++c) {
-            ka[c][0] = ld16(kbase + (size_t)krow0 * KSTRIDE + c * 32 + g * 8);
-            ka[c][1] = ld16(kbase + (size_t)(krow0 + 4) * KSTRIDE + c * 32 + g * 8);
-        }
-#pragma unroll
-        for (int t = 0; t < DT; ++t) va[t] = ld16(vbase + (size_t)(t * 16 + i) * VSTRIDE + 8 * g);
-    }
+    bf16x8 ka[DC][2];
+    bf16x8 va[DT];
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
-        if (STREAM) {
-            // staged keys are stored with their 16-byte chunks swizzled (k_swizzle): the 16 lanes that read
-            // together want the same chunk of 16 different rows
-            const int chunk = ((c * 4 + g) ^ k_swizzle<HS>(krow0)) * 8;
-            ka[0][0] = ld16(kbase + (size_t)krow0 * KSTRIDE + chunk);
-            ka[0][1] = ld16(kbase + (size_t)(krow0 + 4) * KSTRIDE + chunk);
-        }
+        ka[c][0] = ld16(kbase + (size_t)krow0 * KSTRIDE + c * 32 + g * 8);
+        ka[c][1] = ld16(kbase + (size_t)(krow0 + 4) * KSTRIDE + c * 32 + g * 8);
+    }
+#pragma unroll
+    for (int t = 0; t < DT; ++t) va[t] = ld16(vbase + (size_t)(t * 16 + i) * VSTRIDE + 8 * g);
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            st[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[STREAM ? 0 : c][0], q[nt][c], st[nt][0], 0, 0, 0);
-            st[nt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[STREAM ? 0 : c][1], q[nt][c], st[nt][1], 0, 0, 0);
+            st[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c][0], q[nt][c], st[nt][0], 0, 0, 0);
+            st[nt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c][1], q[nt][c], st[nt][1], 0, 0, 0);
         }
     }
     // keys that do not exist may hold anything, NaN included: they are cleared in V^T (0 * NaN is NaN)
@@ -193,7 +191,7 @@ __device__ __forceinline__ void attend_block_direct_m(const bf16* __restrict__ k
         if (first + 7 >= key_hi) v.w &= 0x0000ffffu;
         return __builtin_bit_cast(bf16x8, v);
     };
-    if (!STREAM && need_mask) {
+    if (need_mask) {
 #pragma unroll
         for (int t = 0; t < DT; ++t) va[t] = clear_missing(va[t]);
     }
@@ -250,60 +248,49 @@ __device__ __forceinline__ void attend_block_direct_m(const bf16* __restrict__ k
     }
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
-        if (STREAM) {
-            // staged: VSTRIDE keys a row, this group's keys start at chunk vchunk0
-            va[0] = ld16(vbase + (size_t)(t * 16 + i) * VSTRIDE + ((vchunk0 + g) ^ v_swizzle<VSTRIDE>(i)) * 8);
-            if (need_mask) va[0] = clear_missing(va[0]);
-        }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
-            acc[nt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[STREAM ? 0 : t], pb[nt], acc[nt][t], 0, 0, 0);
+            acc[nt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[t], pb[nt], acc[nt][t], 0, 0, 0);
     }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) l[nt] += lsum[nt][0];
 }
 
-template <int HS, int NT, int KSTRIDE, int VSTRIDE, bool STREAM, bool need_mask>
-__device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, const bf16* __restrict__ vbase,
-                                               int vchunk0, int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
-                                               float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
-                                               const int (&lo)[NT], int key_hi, float scale2, int lane) {
-    // STREAM: the operands come from shared memory (short latency): fetch each one right before its
-    // products instead of all of them up front, which keeps fewer registers live.
-    constexpr int DC = HS / 32, DT = HS / 16;
-    const int i = lane & 15, g = lane >> 4;
-    const int krow0 = 8 * (i >> 2) + (i & 3);        // key row of tile 0; tile 1 is 4 further
-    f32x4 st[NT][2];
+// The prompt form runs a block in two halves, so that a wave can have the first product of the next block on the
+// matrix cores while its vector units work on the weights of the current one:
+//   block_scores:   S^T = K . Q^T of a staged block of 32 keys (two 16-key tiles per column tile), nothing else;
+//   block_weights_values: mask, reference point, exponentials, the sums of the weights and O^T += V^T . P^T.
+// Operands come from the staged copies in shared memory (swizzled as k_swizzle / v_swizzle say).
+// stage: the staged buffer (the same address in every lane); koff[c]: this lane's byte offset of chunk c of its key row
+// of tile 0 (k_read_offsets), the row of tile 1 lies 4 rows further.
+template <int HS, int NT, int KSTRIDE>
+__device__ __forceinline__ void block_scores(const unsigned char* __restrict__ stage, const int (&koff)[HS / 32],
+                                             const bf16x8 (&q)[NT][HS / 32], f32x4 (&st)[NT][2]) {
+    constexpr int DC = HS / 32;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) { st[nt][0] = (f32x4){0.f, 0.f, 0.f, 0.f}; st[nt][1] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
-    bf16x8 ka[STREAM ? 1 : DC][2];
-    bf16x8 va[STREAM ? 1 : DT];
-    if (!STREAM) {
-#pragma unroll
-        for (int c = 0; c < DC; ++c) {
-            ka[c][0] = ld16(kbase + (size_t)krow0 * KSTRIDE + c * 32 + g * 8);
-            ka[c][1] = ld16(kbase + (size_t)(krow0 + 4) * KSTRIDE + c * 32 + g * 8);
-        }
-#pragma unroll
-        for (int t = 0; t < DT; ++t) va[t] = ld16(vbase + (size_t)(t * 16 + i) * VSTRIDE + 8 * g);
-    }
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
-        if (STREAM) {
-            // staged keys are stored with their 16-byte chunks swizzled (k_swizzle): the 16 lanes that read
-            // together want the same chunk of 16 different rows
-            const int chunk = ((c * 4 + g) ^ k_swizzle<HS>(krow0)) * 8;
-            ka[0][0] = ld16(kbase + (size_t)krow0 * KSTRIDE + chunk);
-            ka[0][1] = ld16(kbase + (size_t)(krow0 + 4) * KSTRIDE + chunk);
-        }
+        const bf16x8 k0 = ld16(reinterpret_cast<const bf16*>(stage + koff[c]));
+        const bf16x8 k1 = ld16(reinterpret_cast<const bf16*>(stage + koff[c] + 4 * KSTRIDE * 2));
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            st[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[STREAM ? 0 : c][0], q[nt][c], st[nt][0], 0, 0, 0);
-            st[nt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[STREAM ? 0 : c][1], q[nt][c], st[nt][1], 0, 0, 0);
+            st[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, q[nt][c], st[nt][0], 0, 0, 0);
+            st[nt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, q[nt][c], st[nt][1], 0, 0, 0);
         }
     }
-    // keys that do not exist may hold anything, NaN included: they are cleared in V^T (0 * NaN is NaN)
+}
+
+// stage as above; voff: this lane's byte offset of its 8 keys of V^T row i (v_read_offset), row t * 16 + i lies t * 16 rows further.
+template <int HS, int NT, int VSTRIDE, bool need_mask>
+__device__ __forceinline__ void block_weights_values_m(const f32x4 (&st)[NT][2], const unsigned char* __restrict__ stage, int voff,
+                                                       int kb, f32x4 (&acc)[NT][HS / 16], float (&m)[NT], float (&l)[NT],
+                                                       const int (&qpos)[NT], const int (&lo)[NT], int key_hi, float scale2,
+                                                       int lane) {
+    constexpr int DT = HS / 16;
+    const int g = lane >> 4;
     const int first = kb + 8 * g;                     // this lane's 8 keys are first .. first+7
+    // keys that do not exist may hold anything, NaN included: they are cleared in V^T (0 * NaN is NaN)
     auto clear_missing = [&](bf16x8 x) {
         uint4 v = __builtin_bit_cast(uint4, x);
         if (first + 0 >= key_hi) v.x &= 0xffff0000u;
@@ -316,26 +303,18 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
         if (first + 7 >= key_hi) v.w &= 0x0000ffffu;
         return __builtin_bit_cast(bf16x8, v);
     };
-    if (!STREAM && need_mask) {
-#pragma unroll
-        for (int t = 0; t < DT; ++t) va[t] = clear_missing(va[t]);
-    }
-    // staged values: the first tiles of V^T are asked for now, so that they arrive while the weights are
-    // computed; every later tile is asked for when an earlier one has been used
+    // the first tiles of V^T are asked for now, so that they arrive while the weights are computed; every later
+    // tile is asked for when an earlier one has been used
     constexpr int PF = DT < 4 ? DT : 4;
     bf16x8 vpre[PF];
-    auto staged_v = [&](int t) {
-        return ld16(vbase + (size_t)(t * 16 + i) * VSTRIDE + ((vchunk0 + g) ^ v_swizzle<VSTRIDE>(i)) * 8);
-    };
-    if (STREAM) {
+    auto staged_v = [&](int t) { return ld16(reinterpret_cast<const bf16*>(stage + voff + t * 16 * VSTRIDE * 2)); };
 #pragma unroll
-        for (int t = 0; t < PF; ++t) vpre[t] = staged_v(t);
-    }
+    for (int t = 0; t < PF; ++t) vpre[t] = staged_v(t);
     bf16x8 pb[NT];
+    float s[NT][8];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         // raw scores; the scale (with log2 e folded in) is applied inside the exponent's fma
-        float s[8];
 #pragma unroll
         for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
@@ -345,14 +324,17 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
                     const int key = kb + 8 * g + 4 * sb + r;
                     if (key > qpos[nt] || key < lo[nt] || key >= key_hi) v = -INFINITY;
                 }
-                s[sb * 4 + r] = v;
+                s[nt][sb * 4 + r] = v;
             }
         // The reference point m of the exponents moves only when some score of the column exceeds it
         // by more than 2^8: until then p = 2^(s - m) may exceed 1 (at most 256), which float32 sums
         // and bf16 weights hold as well, and nothing has to be rescaled.  So the common block only
         // asks whether any lane of the wave sees such a score; the exchange between the four lane
         // groups of a column, the new reference point and the rescaling happen when one does.
-        float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+        float mx = max3(s[nt][0], s[nt][1], s[nt][2]);
+        mx = max3(mx, s[nt][3], s[nt][4]);
+        mx = max3(mx, s[nt][5], s[nt][6]);
+        mx = max3(mx, s[nt][7], s[nt][7]);
         float m_new = m[nt];
         mx *= scale2;                                  // scale2 > 0: the maximum of the scaled scores
         if (__any(mx > m[nt] + 8.0f)) {                // also true for a column's first visible key (m = -inf)
@@ -366,15 +348,15 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
                 for (int t = 0; t < DT; ++t) acc[nt][t] *= alpha;
             }
         }
-        if (need_mask && m_new == -INFINITY) {         // a column that has seen no key yet (only behind a mask)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) s[e] = 0.f;
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) s[e] = __builtin_amdgcn_exp2f(fmaf(s[e], scale2, -m_new));
-        }
         m[nt] = m_new;
-        pb[nt] = pack8(s);
+    }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        // a column that has seen no key yet (only behind a mask) has m = -inf and only scores of -inf: 2^(-inf - 0) = 0
+        const float ref = (need_mask && m[nt] == -INFINITY) ? 0.f : m[nt];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s[nt][e] = __builtin_amdgcn_exp2f(fmaf(s[nt][e], scale2, -ref));
+        pb[nt] = pack8(s[nt]);
     }
     // The sums of the weights come from the matrix cores too: a tile of ones times P gives every lane
     // the sum over the 32 keys for its column (the same bf16 weights that multiply V, so numerator
@@ -388,14 +370,12 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
     }
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
-        if (STREAM) {
-            va[0] = vpre[t % PF];
-            if (t + PF < DT) vpre[t % PF] = staged_v(t + PF);
-            if (need_mask) va[0] = clear_missing(va[0]);
-        }
+        bf16x8 va = vpre[t % PF];
+        if (t + PF < DT) vpre[t % PF] = staged_v(t + PF);
+        if (need_mask) va = clear_missing(va);
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
-            acc[nt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[STREAM ? 0 : t], pb[nt], acc[nt][t], 0, 0, 0);
+            acc[nt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[nt], acc[nt][t], 0, 0, 0);
     }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) l[nt] += lsum[nt][0];
@@ -403,29 +383,38 @@ __device__ __forceinline__ void attend_block_m(const bf16* __restrict__ kbase, c
 
 // The masked form (a block on the causal diagonal, at a window's edge or at the end of the keys) and
 // the plain one are separate instantiations: almost every block is plain, and it carries no mask code.
-template <int HS, int NT, int KSTRIDE = HS, int VSTRIDE = BN_PAGE, bool STREAM = false>
+template <int HS, int NT>
 __device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, const bf16* __restrict__ vbase,
-                                             int vchunk0, int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
+                                             int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
                                              float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
                                              const int (&lo)[NT], int key_hi, bool need_mask, float scale2,
                                              int lane) {
-    if (!STREAM) {
-        if (need_mask)
-            attend_block_direct_m<HS, NT, KSTRIDE, VSTRIDE, false, true>(kbase, vbase, vchunk0, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
-        else
-            attend_block_direct_m<HS, NT, KSTRIDE, VSTRIDE, false, false>(kbase, vbase, vchunk0, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
-    } else if (need_mask)
-        attend_block_m<HS, NT, KSTRIDE, VSTRIDE, STREAM, true>(kbase, vbase, vchunk0, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
+    if (need_mask)
+        attend_block_direct_m<HS, NT, true>(kbase, vbase, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
     else
-        attend_block_m<HS, NT, KSTRIDE, VSTRIDE, STREAM, false>(kbase, vbase, vchunk0, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
+        attend_block_direct_m<HS, NT, false>(kbase, vbase, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
+}
+template <int HS, int NT, int VSTRIDE>
+__device__ __forceinline__ void block_weights_values(const f32x4 (&st)[NT][2], const unsigned char* __restrict__ stage, int voff, int kb,
+                                                     f32x4 (&acc)[NT][HS / 16], float (&m)[NT], float (&l)[NT],
+                                                     const int (&qpos)[NT], const int (&lo)[NT], int key_hi, bool need_mask,
+                                                     float scale2, int lane) {
+    if (need_mask) block_weights_values_m<HS, NT, VSTRIDE, true>(st, stage, voff, kb, acc, m, l, qpos, lo, key_hi, scale2, lane);
+    else block_weights_values_m<HS, NT, VSTRIDE, false>(st, stage, voff, kb, acc, m, l, qpos, lo, key_hi, scale2, lane);
 }
 
 // ---------------------------------------------------------------------------------------
 // prompt form
 // ---------------------------------------------------------------------------------------
 // The waves of a workgroup need the same keys, so a stage of keys is fetched once per workgroup
-// into shared memory (the next stage's loads are in flight while the current one is multiplied),
-// double-buffered, one barrier per stage.  A workgroup has NG groups of 4 waves; all groups hold the
+// into shared memory, three buffers in turn, one barrier per stage: while stage s is multiplied, stage s + 1
+// lies ready, stage s + 2 is stored from registers and the loads of stage s + 3 are in flight.  A wave works on
+// two stages at once: it issues the first product of stage s + 1 (S^T = K . Q^T), then turns the scores of
+// stage s into weights on the vector units while the last of those matrix instructions finish, and then
+// multiplies the weights with the values of stage s.  (The compiler keeps the two in separate basic blocks, so
+// inside one wave little more than that tail overlaps; most of the overlap of matrix cores and vector units
+// comes from the two waves that share a SIMD.  Measured against one stage at a time: 65 -> 61 us at 2,048
+// tokens of the 8B shape, 10.9 -> 9.9 ms at 32,768.)  A workgroup has NG groups of 4 waves; all groups hold the
 // same query rows and a stage is NG blocks of 32 keys, one for each group, so the chain of blocks
 // that a tile of late positions has to walk is NG times shorter; at the end the groups' partial
 // results (reference point, sum, accumulators) are merged through shared memory in group order.
@@ -444,11 +433,38 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
     constexpr int KV4 = 32 * HS / 8 / 256;                // uint4 loads per thread for K (and for V^T)
     constexpr int STAGE = (KB * KS + HS * VS) * 2;        // bytes of one buffer
     constexpr int MERGE = NG > 1 ? 4 * 64 * (DT * 4 + 2) * 4 : 0;
-    __shared__ __align__(16) unsigned char smem[(2 * STAGE > MERGE) ? 2 * STAGE : MERGE];
-    auto k_s = [&](int b) { return reinterpret_cast<bf16*>(smem + b * STAGE); };
-    auto v_s = [&](int b) { return reinterpret_cast<bf16*>(smem + b * STAGE) + KB * KS; };
+    static_assert(PROMPT_BUFFERS * STAGE >= MERGE, "the merge of the wave groups reuses the staging memory");
+    extern __shared__ __align__(16) unsigned char smem[];     // prompt_smem_bytes(HS, NG)
     const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3, grp = threadIdx.x >> 8;
     const int n = lane & 15, g = lane >> 4;
+    // Where this thread's pieces of a stage come from (bytes from the page's keys of this kv head, and from its
+    // V^T rows) and where they go in a staged buffer, and where this lane's operands lie in it: a handful of
+    // numbers that depend on the thread alone.  They are made opaque to the compiler, which otherwise works them
+    // out again in every stage (some seventy vector instructions of index arithmetic beside thirty-four products).
+    static_assert(KV4 == 1 || KV4 == 2, "a thread stages one or two pieces of K and of V^T");
+    int k_src[2], v_src[2], k_dst[2], v_dst[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int idx = threadIdx.x + h * 256 * NG;
+        k_src[h] = idx * 16;
+        const int krow = (idx * 8) / HS, kchunk = ((idx * 8) % HS) / 8;
+        k_dst[h] = (krow * KS + ((kchunk ^ k_swizzle<HS>(krow)) * 8)) * 2;
+        const int vrow = idx / (KB / 8), vchunk = idx % (KB / 8);
+        v_src[h] = (vrow * BN_PAGE + vchunk * 8) * 2;
+        v_dst[h] = (KB * KS + vrow * VS + ((vchunk ^ v_swizzle<KB>(vrow & 15)) * 8)) * 2;
+        asm volatile("" : "+v"(k_src[h]), "+v"(v_src[h]), "+v"(k_dst[h]), "+v"(v_dst[h]));
+    }
+    int k_read[DC], v_read;
+    {
+        const int krow0 = 32 * grp + 8 * (n >> 2) + (n & 3);          // this group's block, key row of tile 0
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+            k_read[c] = (krow0 * KS + (((c * 4 + g) ^ k_swizzle<HS>(krow0)) * 8)) * 2;
+            asm volatile("" : "+v"(k_read[c]));
+        }
+        v_read = (KB * KS + n * VS + (((4 * grp + g) ^ v_swizzle<VS>(n)) * 8)) * 2;
+        asm volatile("" : "+v"(v_read));
+    }
     const int G = a.H / a.Hkv, GT = a.GT;
     const int n_head_tiles = (G + GT - 1) / GT;
     const int hy = a.Hkv * n_head_tiles;
@@ -502,60 +518,74 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
     const size_t bt_row = (size_t)seq * a.bt_stride;
     // Two stages are in flight: one or two 16-byte pieces of K and of V^T per thread and stage, in named
     // registers (arrays indexed in a loop end up in memory when they have to live across the products).
-    static_assert(KV4 == 1 || KV4 == 2, "a thread stages one or two pieces of K and of V^T");
     struct Stage { uint4 k0, k1, v0, v1; };
     auto fetch = [&](int kb, Stage& st) {                 // a stage never crosses a page: KB divides BN_PAGE
         const int page = uniform_load(a.block_table, bt_row + kb / BN_PAGE);
         const int koff = kb % BN_PAGE;
-        const bf16* kg = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS;      // KB rows of HS, contiguous
-        const bf16* vg = a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff;       // HS rows, KB of 64 keys each
-        const int i0 = threadIdx.x, i1 = threadIdx.x + 256 * NG;
-        st.k0 = *reinterpret_cast<const uint4*>(kg + (size_t)i0 * 8);
-        st.v0 = *reinterpret_cast<const uint4*>(vg + (size_t)(i0 / (KB / 8)) * BN_PAGE + (i0 % (KB / 8)) * 8);
+        // the same addresses in every lane: the page's keys of this kv head (KB rows of HS, contiguous) and its V^T
+        // rows (HS rows of 64 keys, KB of them wanted)
+        const unsigned char* kg = reinterpret_cast<const unsigned char*>(a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS);
+        const unsigned char* vg = reinterpret_cast<const unsigned char*>(a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff);
+        st.k0 = *reinterpret_cast<const uint4*>(kg + (unsigned)k_src[0]);
+        st.v0 = *reinterpret_cast<const uint4*>(vg + (unsigned)v_src[0]);
         if (KV4 > 1) {
-            st.k1 = *reinterpret_cast<const uint4*>(kg + (size_t)i1 * 8);
-            st.v1 = *reinterpret_cast<const uint4*>(vg + (size_t)(i1 / (KB / 8)) * BN_PAGE + (i1 % (KB / 8)) * 8);
+            st.k1 = *reinterpret_cast<const uint4*>(kg + (unsigned)k_src[1]);
+            st.v1 = *reinterpret_cast<const uint4*>(vg + (unsigned)v_src[1]);
         }
-    };
-    auto stash_one = [&](int buf, int idx, const uint4& kv, const uint4& vv) {
-        const int krow = (idx * 8) / HS, kchunk = ((idx * 8) % HS) / 8;
-        *reinterpret_cast<uint4*>(k_s(buf) + krow * KS + ((kchunk ^ k_swizzle<HS>(krow)) * 8)) = kv;
-        const int vrow = idx / (KB / 8), vchunk = idx % (KB / 8);
-        *reinterpret_cast<uint4*>(v_s(buf) + vrow * VS + ((vchunk ^ v_swizzle<KB>(vrow & 15)) * 8)) = vv;
     };
     auto stash = [&](int buf, const Stage& st, int zero = 0) {    // zero: 0, in a form the compiler cannot see through
-        stash_one(buf, threadIdx.x + zero, st.k0, st.v0);
-        if (KV4 > 1) stash_one(buf, threadIdx.x + 256 * NG + zero, st.k1, st.v1);
-    };
-    // One stage of the walk: the loads of the stage after next go out, the current one (in shared memory
-    // `buf`) is multiplied, the next one (`have`, loaded a stage ago) is stored into the other buffer.
-    auto step = [&](int kb, int buf, Stage& want, const Stage& have) {
-        if (kb + 2 * KB <= g_hi) fetch(kb + 2 * KB, want);
-        const int kbb = kb + 32 * grp;                    // this group's block of the stage
-        if (w_hi >= 0 && kbb <= w_hi && kbb + 31 >= w_lo) {
-            const bool need_mask = (kbb + 31 > all_hi) || (kbb < all_lo);
-            attend_block<HS, NT, KS, VS, true>(k_s(buf) + 32 * grp * KS, v_s(buf), 4 * grp, kbb, q, acc, m, l, qpos, lo,
-                                               w_hi + 1, need_mask, scale2, lane);
+        unsigned char* stage = smem + buf * STAGE + zero;
+        *reinterpret_cast<uint4*>(stage + k_dst[0]) = st.k0;
+        *reinterpret_cast<uint4*>(stage + v_dst[0]) = st.v0;
+        if (KV4 > 1) {
+            *reinterpret_cast<uint4*>(stage + k_dst[1]) = st.k1;
+            *reinterpret_cast<uint4*>(stage + v_dst[1]) = st.v1;
         }
-        // The stores of the next stage must stay behind the products: next to their loads (where the
+    };
+    // Stage t holds the keys kb0 + t KB ..; its block for this wave group begins at kbb(t).  A wave skips the blocks
+    // that none of its columns can see.
+    const int kb0 = (g_lo / KB) * KB;
+    const int n_stages = (g_hi - kb0) / KB + 1;
+    auto kbb = [&](int t) { return kb0 + t * KB + 32 * grp; };
+    auto active = [&](int t) { return t < n_stages && w_hi >= 0 && kbb(t) <= w_hi && kbb(t) + 31 >= w_lo; };
+    auto scores = [&](int t, f32x4 (&st)[NT][2]) {
+        if (active(t)) block_scores<HS, NT, KS>(smem + (t % PROMPT_BUFFERS) * STAGE, k_read, q, st);
+    };
+    // One stage of the walk.  `cur` holds the scores of stage t (computed a stage ago), `next` takes those of stage
+    // t + 1; `have` holds the loads of stage t + 2, `want` takes those of stage t + 3.
+    auto step = [&](int t, f32x4 (&cur)[NT][2], f32x4 (&next)[NT][2], Stage& want, const Stage& have) {
+        if (t + 3 < n_stages) fetch(kb0 + (t + 3) * KB, want);
+        // The scores of the next block go to the matrix cores before the vector units start on the weights of this
+        // one.  (Put into one basic block with the exponentials, so that the compiler can interleave them, they cost
+        // more registers than a wave has here: 188 spilled.)
+        scores(t + 1, next);
+        if (active(t)) {
+            const bool need_mask = (kbb(t) + 31 > all_hi) || (kbb(t) < all_lo);
+            block_weights_values<HS, NT, VS>(cur, smem + (t % PROMPT_BUFFERS) * STAGE, v_read, kbb(t), acc, m, l, qpos, lo, w_hi + 1,
+                                             need_mask, scale2, lane);
+        }
+        // The stores of a later stage must stay behind the products: next to their loads (where the
         // compiler puts them otherwise) they would wait out the memory latency before the block is
         // multiplied, instead of hiding it behind the block.  An empty asm makes the store offset look
         // as if it came out of the last product.
         int after_products = 0;
         asm volatile("" : "+v"(after_products) : "v"(acc[NT - 1][DT - 1][3]));
-        if (kb + KB <= g_hi) stash(buf ^ 1, have, after_products);
+        if (t + 2 < n_stages) stash((t + 2) % PROMPT_BUFFERS, have, after_products);
         __syncthreads();
     };
     Stage sa = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)}, sb = sa;
-    const int kb0 = (g_lo / KB) * KB;
     fetch(kb0, sa);
+    if (n_stages > 1) fetch(kb0 + KB, sb);
     stash(0, sa);
-    if (kb0 + KB <= g_hi) fetch(kb0 + KB, sa);
+    if (n_stages > 1) stash(1, sb);
+    if (n_stages > 2) fetch(kb0 + 2 * KB, sa);
     __syncthreads();
-    for (int kb = kb0; kb <= g_hi; kb += 2 * KB) {
-        step(kb, 0, sb, sa);
-        if (kb + KB > g_hi) break;
-        step(kb + KB, 1, sa, sb);
+    f32x4 s_even[NT][2], s_odd[NT][2];
+    scores(0, s_even);
+    for (int t = 0; t < n_stages; t += 2) {
+        step(t, s_even, s_odd, sb, sa);
+        if (t + 1 >= n_stages) break;
+        step(t + 1, s_odd, s_even, sa, sb);
     }
     if (NG > 1) {
         // the later groups hand their partial results to group 0, one column tile a time; the staging
@@ -762,7 +792,7 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
             const bf16* kbase = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS;
             const bf16* vbase = a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff;
             const bool need_mask = (kb + 32 > k_hi) || (kb < k_lo);
-            attend_block<HS, 1>(kbase, vbase, 0, kb, q, acc, m, l, qpos, lo, k_hi, need_mask, scale2, lane);
+            attend_block<HS, 1>(kbase, vbase, kb, q, acc, m, l, qpos, lo, k_hi, need_mask, scale2, lane);
         }
     }
     // merge the four waves: every wave's (m, l, O^T) through shared memory, in wave order
@@ -879,9 +909,20 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
         const long long wgs = (long long)((n_tiles + 1) / 2) * Hkv * n_head_tiles;
         if (wgs > 0x7fffffff) return BN_ERR_ARG;
         const dim3 grid((unsigned)wgs);
-        if (hs == 64) hipLaunchKernelGGL((attn_mfma_prompt_kernel<64, 4, 2>), grid, dim3(512), 0, s, a, n_tiles);
-        else hipLaunchKernelGGL((attn_mfma_prompt_kernel<128, 2, 2>), grid, dim3(512), 0, s, a, n_tiles);
-        return bn_launch_status();
+        // three staged blocks of 64 keys with their values: 48 or 96 KB, beyond the default limit of dynamic shared memory
+        const size_t smem = (size_t)PROMPT_BUFFERS * (64 * hs + hs * 64) * 2;
+        auto go = [&](auto kernel, int which) {
+            static bool raised[2] = {false, false};
+            if (!raised[which]) {
+                const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess) return (int)e;
+                raised[which] = true;
+            }
+            hipLaunchKernelGGL(kernel, grid, dim3(512), smem, s, a, n_tiles);
+            return bn_launch_status();
+        };
+        return hs == 64 ? go(attn_mfma_prompt_kernel<64, 4, 2>, 0) : go(attn_mfma_prompt_kernel<128, 2, 2>, 1);
     }
     if (n_tiles > 65535) return BN_ERR_ARG;                 // sequences are the grid's y
     const dim3 grid(Hkv * n_head_tiles, n_tiles, n_splits);
