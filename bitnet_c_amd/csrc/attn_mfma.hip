@@ -422,11 +422,13 @@ __device__ __forceinline__ void block_weights_values(const f32x4 (&st)[NT][2], c
 // A causal tile's work grows with its position, and a launch is as long as its longest workgroup.  The
 // host hands the tiles over ordered by their number of keys, longest first, and workgroup p takes tile p
 // and then tile n - 1 - p: every workgroup walks about the same number of key blocks (a prompt of 2,048
-// tokens: 65 blocks each, half of them per wave group, where the last tile alone walks 64).  The grid is
+// tokens: 65 blocks each, half of them per wave group, where the last tile alone walks 64).  A launch whose tiles
+// all fit on the chip at once (paired = 0) gives every workgroup one tile: it is as long as its longest tile
+// either way, and a second tile would only add its fixed cost.  The grid is
 // one-dimensional with the kv heads running fastest: consecutive workgroups go to consecutive XCDs, so with
 // eight kv heads every XCD serves one of them and its keys and values live in one L2 only.
 template <int HS, int NT, int NG>
-__global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_mfma_prompt_kernel(MfmaArgs a, int n_tiles) {
+__global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_mfma_prompt_kernel(MfmaArgs a, int n_tiles, int paired) {
     constexpr int DC = HS / 32, DT = HS / 16;
     constexpr int KB = 32 * NG;                           // keys per stage
     constexpr int KS = HS, VS = KB;                       // row strides (elements); both blocks swizzled, no padding
@@ -470,7 +472,7 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int hy = a.Hkv * n_head_tiles;
     const int pair = blockIdx.x / hy, y = blockIdx.x - pair * hy;
     const int kvh = y / n_head_tiles, ht = y - kvh * n_head_tiles;
-  for (int turn = 0; turn < 2; ++turn) {
+  for (int turn = 0; turn <= paired; ++turn) {
     const int tile = turn == 0 ? pair : n_tiles - 1 - pair;
     if (turn == 1 && tile <= pair) break;                 // an odd number of tiles: the middle one has no partner
     const int* tl = a.tiles + 4 * tile;
@@ -905,8 +907,10 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
     a.by_length = (!tiles && n_splits == 1 && (long long)n_tiles * wgs_per_seq > compute_units()) ? by_length : nullptr;
     a.order_period = compute_units() / wgs_per_seq;
     if (tiles) {
-        // workgroups of two wave groups (eight waves, one workgroup a CU), each with a pair of tiles
-        const long long wgs = (long long)((n_tiles + 1) / 2) * Hkv * n_head_tiles;
+        // workgroups of two wave groups (eight waves, one workgroup a CU), each with a pair of tiles when there are
+        // more tiles than CUs
+        const int paired = (long long)n_tiles * wgs_per_seq > compute_units() ? 1 : 0;
+        const long long wgs = (long long)(paired ? (n_tiles + 1) / 2 : n_tiles) * wgs_per_seq;
         if (wgs > 0x7fffffff) return BN_ERR_ARG;
         const dim3 grid((unsigned)wgs);
         // three staged blocks of 64 keys with their values: 48 or 96 KB, beyond the default limit of dynamic shared memory
@@ -919,7 +923,7 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
                 if (e != hipSuccess) return (int)e;
                 raised[which] = true;
             }
-            hipLaunchKernelGGL(kernel, grid, dim3(512), smem, s, a, n_tiles);
+            hipLaunchKernelGGL(kernel, grid, dim3(512), smem, s, a, n_tiles, paired);
             return bn_launch_status();
         };
         return hs == 64 ? go(attn_mfma_prompt_kernel<64, 4, 2>, 0) : go(attn_mfma_prompt_kernel<128, 2, 2>, 1);
