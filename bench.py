@@ -109,7 +109,8 @@ def _kernel_attention_prompt(H=32, Hkv=8, hs=128):
         qkv = torch.randn(t, (H + 2 * Hkv) * hs, device="cuda:0", dtype=torch.bfloat16)
         out = torch.empty(t, H * hs, device="cuda:0", dtype=torch.bfloat16)
         _, _, qt = ops.attention_row_shape(H, Hkv, False, torch.bfloat16, hs)
-        tiles = torch.tensor([(0, i, min(qt, t - i), i) for i in range(0, t, qt)], dtype=torch.int32, device="cuda:0")
+        tiles = torch.tensor(ops.pair_tiles([(0, i, min(qt, t - i), i) for i in range(0, t, qt)]), dtype=torch.int32,
+                             device="cuda:0")
         for _ in range(3):
             ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, hs ** -0.5, tiles=tiles, qt=qt)
         torch.cuda.synchronize()

@@ -419,12 +419,14 @@ __device__ __forceinline__ void block_weights_values(const f32x4 (&st)[NT][2], c
 // that a tile of late positions has to walk is NG times shorter; at the end the groups' partial
 // results (reference point, sum, accumulators) are merged through shared memory in group order.
 //
-// A causal tile's work grows with its position, and a launch is as long as its longest workgroup.  The
-// host hands the tiles over ordered by their number of keys, longest first, and workgroup p takes tile p
-// and then tile n - 1 - p: every workgroup walks about the same number of key blocks (a prompt of 2,048
-// tokens: 65 blocks each, half of them per wave group, where the last tile alone walks 64).  A launch whose tiles
-// all fit on the chip at once (paired = 0) gives every workgroup one tile: it is as long as its longest tile
-// either way, and a second tile would only add its fixed cost.  The grid is
+// A causal tile's work grows with its position, and a launch is as long as its longest workgroup.  A workgroup
+// therefore takes two tiles, 2p and 2p + 1 of the list, and the host orders the list so that these are a long and
+// a short tile of the same sequence (the first with the last, the second with the last but one, ...): every
+// workgroup walks about the same number of key blocks (a prompt of 2,048 tokens: 65 blocks each, half of them
+// per wave group, where the last tile alone walks 64), and the workgroups that run at the same time walk the
+// keys of one sequence, which its L2 then holds.  Any order gives the same result.  A launch whose tiles all
+// fit on the chip at once (paired = 0) gives every workgroup one tile: it is as long as its longest tile either
+// way, and a second tile would only add its fixed cost.  The grid is
 // one-dimensional with the kv heads running fastest: consecutive workgroups go to consecutive XCDs, so with
 // eight kv heads every XCD serves one of them and its keys and values live in one L2 only.
 template <int HS, int NT, int NG>
@@ -473,8 +475,8 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int pair = blockIdx.x / hy, y = blockIdx.x - pair * hy;
     const int kvh = y / n_head_tiles, ht = y - kvh * n_head_tiles;
   for (int turn = 0; turn <= paired; ++turn) {
-    const int tile = turn == 0 ? pair : n_tiles - 1 - pair;
-    if (turn == 1 && tile <= pair) break;                 // an odd number of tiles: the middle one has no partner
+    const int tile = paired ? 2 * pair + turn : pair;
+    if (tile >= n_tiles) break;                           // an odd number of tiles: the last one has no partner
     const int* tl = a.tiles + 4 * tile;
     const int seq = tl[0], tok0 = tl[1], n_tok = tl[2], pos0 = tl[3];
 

@@ -81,9 +81,8 @@ class StepContext:
 
     def tiles(self, qt: int) -> torch.Tensor:
         """[n, 4] int32: (sequence, first row, rows <= qt, position of the first) covering all new
-        tokens, for the prompt form of the attention kernel; ordered by the number of keys a tile sees,
-        most first (the kernel pairs the first with the last, the second with the last but one, ...,
-        so that its workgroups carry equal work)."""
+        tokens, for the prompt form of the attention kernel, in the order that gives its workgroups
+        equal work (ops.pair_tiles)."""
         t = self._tiles.get(qt)
         if t is None:
             rows, r = [], 0
@@ -91,8 +90,7 @@ class StepContext:
                 for i in range(0, n, qt):
                     rows.append((s, r + i, min(qt, n - i), p0 + i))
                 r += n
-            rows.sort(key=lambda t: -(t[3] + t[2]))
-            t = torch.tensor(rows, dtype=torch.int32).reshape(-1, 4).to(self.device)
+            t = torch.tensor(ops.pair_tiles(rows), dtype=torch.int32).reshape(-1, 4).to(self.device)
             self._tiles[qt] = t
         return t
 

@@ -733,6 +733,35 @@ def attention_row_shape(H: int, Hkv: int, decode: bool, dtype=None, hs: int = 0)
     return 16, GT, 16 // GT
 
 
+def pair_tiles(rows: list) -> list:
+    """The order in which the prompt form of the matrix-core attention wants its tiles (sequence, first row, rows,
+    position of the first): it gives a workgroup two consecutive tiles of the list when there are more tiles than
+    CUs, and a causal tile's work grows with its position.  So a sequence's tile with the most keys is followed by
+    its tile with the fewest, the second by the last but one, and so on (equal work per workgroup); sequences follow
+    each other, longest first, so that workgroups that run together walk the same keys; the middle tiles of
+    sequences with an odd number of them are paired with each other at the end.  The result of the attention does
+    not depend on the order."""
+    by_seq = {}
+    for r in rows:
+        by_seq.setdefault(r[0], []).append(r)
+    keys = lambda r: r[3] + r[2]
+    out, single = [], []
+    for seq in sorted(by_seq, key=lambda q: -max(keys(r) for r in by_seq[q])):
+        ts = sorted(by_seq[seq], key=lambda r: -keys(r))
+        n = len(ts)
+        for p in range(n // 2):
+            out += [ts[p], ts[n - 1 - p]]
+        if n % 2:
+            single.append(ts[n // 2])
+    single.sort(key=lambda r: -keys(r))
+    n = len(single)
+    for p in range(n // 2):
+        out += [single[p], single[n - 1 - p]]
+    if n % 2:
+        out.append(single[n // 2])
+    return out
+
+
 def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int, dtype=None):
     """(n_splits, chunk): how the keys of a decode step are cut so that the launch fills the
     chip.  A function of the batch's shape and of max_len alone.  A float32 cache is never split:

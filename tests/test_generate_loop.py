@@ -136,3 +136,31 @@ def test_same_seed_same_stream_whatever_the_batch():
             out.append(vals[0])
         return out
     assert draws(0) == draws(3)
+
+
+def test_prompt_tiles_are_paired_long_with_short_inside_a_sequence():
+    # The prompt attention gives a workgroup two consecutive tiles of the list: every tile appears once, a pair
+    # belongs to one sequence and carries about the same number of keys as every other pair of that sequence, the
+    # longest sequence comes first, and the odd ones out are paired with each other at the end.
+    from bitnet_c_amd.ops import pair_tiles
+    import random
+    rnd = random.Random(3)
+    for lens in ([2048], [130], [32], [700, 64, 2048, 33], [rnd.randint(1, 3000) for _ in range(9)]):
+        qt, rows, r = 32, [], 0
+        for s, n in enumerate(lens):
+            p0 = 64 * s                                    # some sequences continue a cached prefix
+            rows += [(s, r + i, min(qt, n - i), p0 + i) for i in range(0, n, qt)]
+            r += n
+        out = pair_tiles(list(rows))
+        assert sorted(out) == sorted(rows)
+        keys = lambda t: t[3] + t[2]
+        n_paired = sum(len([t for t in rows if t[0] == s]) // 2 * 2 for s in range(len(lens)))
+        first_seq = [t[0] for t in out[:n_paired:2]]
+        assert first_seq == sorted(first_seq, key=lambda s: -max(keys(t) for t in rows if t[0] == s))
+        for a, b in zip(out[:n_paired:2], out[1:n_paired:2]):
+            assert a[0] == b[0] and keys(a) >= keys(b)
+            mine = [t for t in rows if t[0] == a[0]]
+            total = max(keys(t) for t in mine) + min(keys(t) for t in mine)
+            assert abs(keys(a) + keys(b) - total) <= qt    # long + short: the same sum for every pair
+        rest = out[n_paired:]
+        assert len({t[0] for t in rest}) == len(rest)       # one middle tile per sequence with an odd count
