@@ -241,14 +241,19 @@ def main() -> int:
     def decode(batch, steps, warmup):
         lens = [rnd.randint(len_lo, len_hi) for _ in range(batch)]
         slots = [engine.new_sequence() for _ in range(batch)]
-        # the prompts, a few sequences a step to bound the activations
+        # the prompts, a few sequences a step to bound the activations: at most 8 and at most 2^18 tokens
         last = [0] * batch
-        for i in range(0, batch, 8):
+        i = 0
+        while i < batch:
+            k = i + 1
+            while k < batch and k - i < 8 and sum(lens[i:k + 1]) <= 1 << 18:
+                k += 1
             ent = [bn.StepEntry(slots[j], [rnd.randrange(cfg.vocab_size) for _ in range(lens[j])], [lens[j] - 1])
-                   for j in range(i, min(batch, i + 8))]
+                   for j in range(i, k)]
             toks = ops.argmax(engine.step(ent)).cpu().tolist()
-            for j, t in zip(range(i, min(batch, i + 8)), toks):
+            for j, t in zip(range(i, k), toks):
                 last[j] = t
+            i = k
 
         def one():
             nonlocal last
