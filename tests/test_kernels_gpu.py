@@ -731,8 +731,9 @@ def test_attention_prompt_form(dtype, H, Hkv, hs, window, force_vector):
 
 @pytest.mark.parametrize("H,Hkv,hs,T", [(32, 8, 128, 1200), (32, 8, 64, 2200)])
 def test_attention_prompt_form_with_more_workgroups_than_cus(H, Hkv, hs, T):
-    """One long prompt: the launch has more workgroups than the chip has CUs, which is where the
-    matrix-core kernel runs its workgroups with one group of waves instead of two."""
+    """One long prompt: the launch has more tiles than the chip has CUs, which is where a workgroup of the
+    matrix-core kernel takes two tiles (the second case has an odd number of them; here they come in
+    ascending order, which the kernel must take as well as any other)."""
     dtype = torch.bfloat16
     ops, qkv, kp, vp, bt, ref, scale = _attn_case(dtype, H, Hkv, hs, [0], [T], 0, 500)
     _, _, qt = ops.attention_row_shape(H, Hkv, False, dtype, hs)
@@ -740,6 +741,26 @@ def test_attention_prompt_form_with_more_workgroups_than_cus(H, Hkv, hs, T):
     assert len(tiles) * Hkv > 256
     out = torch.full((T, H * hs), float("nan"), dtype=dtype).cuda()
     ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, scale, tiles=torch.tensor(tiles, dtype=torch.int32).cuda(), qt=qt)
+    assert mfma_close(out.float(), ref)
+
+
+@pytest.mark.parametrize("window", [0, 200])
+def test_attention_prompt_form_paired_tiles_of_several_sequences(window):
+    """Three sequences of unequal lengths, one of them continuing a cached prefix, in the order the engine hands
+    the tiles over (long with short inside a sequence), with more tiles than CUs and an odd number of them in
+    each of the sequences; with and without a window."""
+    dtype, H, Hkv, hs = torch.bfloat16, 32, 8, 128
+    lens_before, n_new = [0, 64, 0], [650, 333, 900]
+    ops, qkv, kp, vp, bt, ref, scale = _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, 300)
+    _, _, qt = ops.attention_row_shape(H, Hkv, False, dtype, hs)
+    tiles, r = [], 0
+    for s, (p0, n) in enumerate(zip(lens_before, n_new)):
+        tiles += [(s, r + i, min(qt, n - i), p0 + i) for i in range(0, n, qt)]
+        r += n
+    assert len(tiles) * Hkv > 256 and len(tiles) % 2 == 1
+    out = torch.full((qkv.shape[0], H * hs), float("nan"), dtype=dtype).cuda()
+    ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, scale, window=window,
+                  tiles=torch.tensor(ops.pair_tiles(tiles), dtype=torch.int32).cuda(), qt=qt)
     assert mfma_close(out.float(), ref)
 
 
