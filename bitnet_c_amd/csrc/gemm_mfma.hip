@@ -308,20 +308,18 @@ static int gm_pick_bn(int M, int N, int cus) {
     return pick;
 }
 
-// Tuning hook: != 0 fixes the tile width (256, 192 or 128).
-static int g_force_bn = 0;
-extern "C" void bn_gemm_mfma_force_width(int bn) { g_force_bn = (bn == 256 || bn == 192 || bn == 128) ? bn : 0; }
-
 // 1 if the kernel takes the shape.
 extern "C" int bn_gemm_mfma_supports(int M, int N, int K, int ldx, int ldw) {
     return (M >= 1 && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldx >= K && ldw >= K) ? 1 : 0;
 }
 
 // out_dtype: type of Y (bf16 or float32).  glu8 != 0: W has 2N rows, gate and up interleaved in
-// blocks of 8 (N a multiple of 8), and Y[M, N] = act(gate) * up, act one of BN_ACT_*.
+// blocks of 8 (N a multiple of 8), and Y[M, N] = act(gate) * up, act one of BN_ACT_*.  width: the tile's rows of W
+// (256, 192 or 128), or 0 for the one that suits the shape.
 extern "C" int bn_gemm_mfma(int out_dtype, const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw,
-                            int ldy, int glu8, int act, hipStream_t s) {
+                            int ldy, int glu8, int act, int width, hipStream_t s) {
     if (!bn_gemm_mfma_supports(M, N, K, ldx, ldw) || ldy < N || act < 0 || act >= BN_ACT_KINDS) return BN_ERR_ARG;
+    if (width != 0 && width != 256 && width != 192 && width != 128) return BN_ERR_ARG;
     if (((uintptr_t)X | (uintptr_t)W) & 15) return BN_ERR_ARG;
     if (out_dtype != BN_DT_BF16 && out_dtype != BN_DT_F32) return BN_ERR_DTYPE;
     if (glu8) {
@@ -331,7 +329,7 @@ extern "C" int bn_gemm_mfma(int out_dtype, const void* X, const void* W, void* Y
     // The tile width: the one with the least work on the busiest CU (rounds of workgroups over the
     // CUs times the width), a wider tile counting a little less than its width because it reads
     // less of X per result.
-    const int bn = g_force_bn ? g_force_bn : gm_pick_bn(M, N, gm_compute_units());
+    const int bn = width ? width : gm_pick_bn(M, N, gm_compute_units());
     const bool f32 = out_dtype == BN_DT_F32;
 #define GM_GO(BN_, GLU_)                                                                          \
     return f32 ? gm_launch<BN_, GLU_, float>(X, W, Y, M, N, K, ldx, ldw, ldy, act, s)             \

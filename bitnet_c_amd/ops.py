@@ -67,7 +67,7 @@ _SIGNATURES = {
     "gemm_mfma": {
         "bn_gemm_mfma_supports": [c_int, c_int, c_int, c_int, c_int],
         "bn_gemm_mfma": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                         c_void_p],
+                         c_int, c_void_p],
     },
     "skinny_gemm": {
         "bn_skinny_gemm_supports": [c_int, c_int, c_int, c_int, c_int],
@@ -309,10 +309,14 @@ def _tiled(x, w, out_dtype):
     return y
 
 
-def gemm_mfma(x: torch.Tensor, w: torch.Tensor, out_dtype=None, glu8: bool = False, activation: str = "silu") -> torch.Tensor:
+def gemm_mfma(x: torch.Tensor, w: torch.Tensor, out_dtype=None, glu8: bool = False, activation: str = "silu",
+              width: int = 0) -> torch.Tensor:
     """The library-free bf16 product for many rows: y[M, N] = x[M, K] . w[N, K]^T on the matrix cores,
-    or with glu8 act(gate) * up for w = gate and up rows interleaved in blocks of 8 ([2N, K])."""
+    or with glu8 act(gate) * up for w = gate and up rows interleaved in blocks of 8 ([2N, K]).
+    width: the tile's rows of w (256, 192 or 128); 0 lets the kernel pick by the shape."""
     require_gpu()
+    if width not in (0, 256, 192, 128):
+        raise KernelError(f"gemm_mfma: the tile width is 256, 192, 128 or 0 (any), not {width}")
     _dev(x, "x", torch.bfloat16, 2)
     _dev(w, "w", torch.bfloat16, 2)
     M, K = x.shape
@@ -325,7 +329,8 @@ def gemm_mfma(x: torch.Tensor, w: torch.Tensor, out_dtype=None, glu8: bool = Fal
     if M == 0:
         return y
     _check(_fn("gemm_mfma", "bn_gemm_mfma")(_code(out_dtype), x.data_ptr(), w.data_ptr(), y.data_ptr(), M, N, K,
-                                            _rows(x, "x"), _rows(w, "w"), N, int(glu8), _act(activation), _stream()),
+                                            _rows(x, "x"), _rows(w, "w"), N, int(glu8), _act(activation), int(width),
+                                            _stream()),
            "gemm_mfma")
     return y
 

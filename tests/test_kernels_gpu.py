@@ -262,20 +262,14 @@ def test_gemm_mfma(M, N, K, width):
     """The tiled matrix-core product, every tile width, at sizes that fill no tile: float32 results are
     the exact sums up to their order, bf16 results one rounding of them."""
     ops = _ops()
-    from bitnet_c_amd.csrc import build
     x, w = _rand((M, K), torch.bfloat16, 21), _rand((N, K), torch.bfloat16, 22, 0.05)
     ref = (x.double() @ w.double().t()).float()
-    lib = build.load("gemm_mfma")
-    lib.bn_gemm_mfma_force_width(width)
-    try:
-        y32 = ops.gemm_mfma(x.cuda(), w.cuda(), torch.float32)
-        y16 = ops.gemm_mfma(x.cuda(), w.cuda())
-        # rows of a larger buffer (a row stride above K), as the stacked projections pass them
-        xw = torch.zeros(M, K + 24, dtype=torch.bfloat16)
-        xw[:, :K] = x
-        y_strided = ops.gemm_mfma(xw.cuda()[:, :K], w.cuda(), torch.float32)
-    finally:
-        lib.bn_gemm_mfma_force_width(0)
+    y32 = ops.gemm_mfma(x.cuda(), w.cuda(), torch.float32, width=width)
+    y16 = ops.gemm_mfma(x.cuda(), w.cuda(), width=width)
+    # rows of a larger buffer (a row stride above K), as the stacked projections pass them
+    xw = torch.zeros(M, K + 24, dtype=torch.bfloat16)
+    xw[:, :K] = x
+    y_strided = ops.gemm_mfma(xw.cuda()[:, :K], w.cuda(), torch.float32, width=width)
     assert y32.dtype == torch.float32 and rel_err(y32, ref) < 1e-5
     assert y16.dtype == torch.bfloat16 and close(y16.float(), ref, torch.bfloat16)
     assert torch.equal(y_strided, y32)
@@ -289,20 +283,14 @@ def test_gemm_mfma(M, N, K, width):
 def test_gemm_mfma_swiglu(M, F, K, width):
     """The same kernel with gate and up rows interleaved in blocks of 8 and the SwiGLU epilogue."""
     ops = _ops()
-    from bitnet_c_amd.csrc import build
     x, w = _rand((M, K), torch.bfloat16, 23), _rand((2 * F, K), torch.bfloat16, 24, 0.1)
     g = x.double() @ w[:F].double().t()
     u = x.double() @ w[F:].double().t()
     want = ((g / (1 + torch.exp(-g))) * u).float()
     wi = ops.interleave_gate_up(w[:F].cuda(), w[F:].cuda())
-    lib = build.load("gemm_mfma")
-    lib.bn_gemm_mfma_force_width(width)
-    try:
-        y32 = ops.gemm_mfma(x.cuda(), wi, torch.float32, glu8=True)
-        y16 = ops.gemm_mfma(x.cuda(), wi, glu8=True)
-        via = ops.linear_swiglu(x.cuda(), wi, True, allow_library=False)
-    finally:
-        lib.bn_gemm_mfma_force_width(0)
+    y32 = ops.gemm_mfma(x.cuda(), wi, torch.float32, glu8=True, width=width)
+    y16 = ops.gemm_mfma(x.cuda(), wi, glu8=True, width=width)
+    via = ops.linear_swiglu(x.cuda(), wi, True, allow_library=False)
     assert y32.shape == (M, F) and close(y32, want, torch.float32)
     assert close(y16.float(), want, torch.bfloat16)
     if M > 128:                                    # up to 128 rows the dispatcher has another kernel for this product
