@@ -417,7 +417,8 @@ __device__ __forceinline__ void block_weights_values(const f32x4 (&st)[NT][2], c
 // tokens of the 8B shape, 10.9 -> 9.9 ms at 32,768.)  A workgroup has NG groups of 4 waves; all groups hold the
 // same query rows and a stage is NG blocks of 32 keys, one for each group, so the chain of blocks
 // that a tile of late positions has to walk is NG times shorter; at the end the groups' partial
-// results (reference point, sum, accumulators) are merged through shared memory in group order.
+// results (reference point, sum, accumulators) are merged through shared memory in group order.  NG is 2 for
+// launches of one round over the chip and 1 (with two workgroups a CU) for longer ones; the launch code says why.
 //
 // A causal tile's work grows with its position, and a launch is as long as its longest workgroup.  A workgroup
 // therefore takes two tiles, 2p and 2p + 1 of the list, and the host orders the list so that these are a long and
@@ -909,25 +910,38 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
     a.by_length = (!tiles && n_splits == 1 && (long long)n_tiles * wgs_per_seq > compute_units()) ? by_length : nullptr;
     a.order_period = compute_units() / wgs_per_seq;
     if (tiles) {
-        // workgroups of two wave groups (eight waves, one workgroup a CU), each with a pair of tiles when there are
-        // more tiles than CUs
+        // a workgroup takes a pair of tiles when there are more tiles than CUs
         const int paired = (long long)n_tiles * wgs_per_seq > compute_units() ? 1 : 0;
         const long long wgs = (long long)(paired ? (n_tiles + 1) / 2 : n_tiles) * wgs_per_seq;
         if (wgs > 0x7fffffff) return BN_ERR_ARG;
         const dim3 grid((unsigned)wgs);
-        // three staged blocks of 64 keys with their values: 48 or 96 KB, beyond the default limit of dynamic shared memory
-        const size_t smem = (size_t)PROMPT_BUFFERS * (64 * hs + hs * 64) * 2;
+        // Two groups of waves a workgroup (eight waves, one workgroup a CU) halve the chain of blocks that a tile walks,
+        // which is what a launch of one round waits for.  A launch of several rounds is faster with one group a
+        // workgroup and two workgroups a CU: they share nothing and drift apart, so that one's matrix instructions
+        // meet the other's vector work, where the two groups of one workgroup meet at a barrier in every stage and do
+        // the same thing at the same time (8 to 16 % at 8,192 tokens and for eight or 64 prompts of 128 to 2,048).
+        // It is taken from four rounds on, and from two when its rounds (of two workgroups a CU) are not much emptier
+        // than those of the wide form (6,144 tokens of one sequence are three full rounds of the wide form and one and
+        // a half of the other: 410 against 445 us).
+        const long long cus = compute_units();
+        const double fill1 = (double)wgs / (double)(((wgs + 2 * cus - 1) / (2 * cus)) * 2 * cus);
+        const double fill2 = (double)wgs / (double)(((wgs + cus - 1) / cus) * cus);
+        const int ng = (wgs >= 4 * cus || (wgs >= 2 * cus && fill1 * 1.1 >= fill2)) ? 1 : 2;
+        // three staged blocks of 32 keys a group with their values: up to 96 KB, beyond the default limit of dynamic
+        // shared memory
+        const size_t smem = (size_t)PROMPT_BUFFERS * (32 * ng * hs + hs * 32 * ng) * 2;
         auto go = [&](auto kernel, int which) {
-            static bool raised[2] = {false, false};
+            static bool raised[4] = {false, false, false, false};
             if (!raised[which]) {
                 const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
                 if (e != hipSuccess) return (int)e;
                 raised[which] = true;
             }
-            hipLaunchKernelGGL(kernel, grid, dim3(512), smem, s, a, n_tiles, paired);
+            hipLaunchKernelGGL(kernel, grid, dim3(256 * ng), smem, s, a, n_tiles, paired);
             return bn_launch_status();
         };
+        if (ng == 1) return hs == 64 ? go(attn_mfma_prompt_kernel<64, 4, 1>, 2) : go(attn_mfma_prompt_kernel<128, 2, 1>, 3);
         return hs == 64 ? go(attn_mfma_prompt_kernel<64, 4, 2>, 0) : go(attn_mfma_prompt_kernel<128, 2, 2>, 1);
     }
     if (n_tiles > 65535) return BN_ERR_ARG;                 // sequences are the grid's y
