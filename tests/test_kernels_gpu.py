@@ -732,6 +732,29 @@ def test_attention_prompt_form_with_more_workgroups_than_cus(H, Hkv, hs, T):
     assert mfma_close(out.float(), ref)
 
 
+@pytest.mark.parametrize("hs,window", [(128, 0), (128, 100), (64, 0)])
+def test_attention_prompt_form_launch_of_many_rounds(hs, window):
+    """Dozens of sequences of unequal lengths, some continuing a cached prefix: several rounds of workgroups over
+    the chip, which is where the matrix-core kernel runs one group of waves a workgroup (two workgroups a CU)."""
+    import random
+    dtype, H, Hkv = torch.bfloat16, 32, 8
+    rnd = random.Random(5)
+    n_seqs = 24 if hs == 128 else 40                   # a tile holds 32 tokens at head size 128, 64 at 64
+    n_new = [rnd.randint(300, 520) for _ in range(n_seqs)]
+    lens_before = [rnd.choice([0, 0, 64, 100]) for _ in range(n_seqs)]
+    ops, qkv, kp, vp, bt, ref, scale = _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, 700)
+    _, _, qt = ops.attention_row_shape(H, Hkv, False, dtype, hs)
+    tiles, r = [], 0
+    for s, (p0, n) in enumerate(zip(lens_before, n_new)):
+        tiles += [(s, r + i, min(qt, n - i), p0 + i) for i in range(0, n, qt)]
+        r += n
+    assert (len(tiles) + 1) // 2 * Hkv >= 4 * 256
+    out = torch.full((qkv.shape[0], H * hs), float("nan"), dtype=dtype).cuda()
+    ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, scale, window=window,
+                  tiles=torch.tensor(ops.pair_tiles(tiles), dtype=torch.int32).cuda(), qt=qt)
+    assert mfma_close(out.float(), ref)
+
+
 @pytest.mark.parametrize("window", [0, 200])
 def test_attention_prompt_form_paired_tiles_of_several_sequences(window):
     """Three sequences of unequal lengths, one of them continuing a cached prefix, in the order the engine hands
