@@ -845,19 +845,22 @@ __global__ __launch_bounds__(64) void attn_mfma_combine_kernel(bf16* __restrict_
     if (lane < n_splits) { ms = ml[2 * lane]; ls = ml[2 * lane + 1]; }
     const float M = wave_max(ms);
     const float w = (M == -INFINITY || ms == -INFINITY) ? 0.f : expf(ms - M);
+    // splits behind the last one with keys (a table much wider than the sequences are long) add nothing: stop there
+    const unsigned long long live = __ballot(w != 0.f);
+    const int n_live = live ? 64 - __builtin_clzll(live) : 0;
     float den = 0.f;
-    for (int s = 0; s < n_splits; ++s) den = fmaf(__shfl(w, s, BN_WAVE), __shfl(ls, s, BN_WAVE), den);
+    for (int s = 0; s < n_live; ++s) den = fmaf(__shfl(w, s, BN_WAVE), __shfl(ls, s, BN_WAVE), den);
     const float inv = den > 0.f ? 1.0f / den : 0.f;
     // dimensions lane and lane + 64 together, sixteen splits' loads in flight at once (a split without keys is not read)
     const bool two = lane + 64 < hs;
     float num0 = 0.f, num1 = 0.f;
     const float* po = part_o + (size_t)row * n_splits * hs + lane;
-    for (int s0 = 0; s0 < n_splits; s0 += 16) {
+    for (int s0 = 0; s0 < n_live; s0 += 16) {
         float v0[16], v1[16], wj[16];
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
             wj[j] = __shfl(w, min(s0 + j, 63), BN_WAVE);
-            const bool in = s0 + j < n_splits && wj[j] != 0.f;
+            const bool in = s0 + j < n_live && wj[j] != 0.f;
             v0[j] = (in && lane < hs) ? po[(size_t)(s0 + j) * hs] : 0.f;
             v1[j] = (in && two) ? po[(size_t)(s0 + j) * hs + 64] : 0.f;
         }
