@@ -241,7 +241,9 @@ class PagedCache:
         return None if eg is None else eg[0]
 
     def block_table(self, group: int, slots: Sequence[int], width: int = 0) -> torch.Tensor:
-        """Host int32 [len(slots), width]; a slot of -1 gives a row of zeros (padding)."""
+        """Host int32 [len(slots), width]; a slot of -1 gives a row of zeros (padding).  A page that a windowed
+        group has given back (-1 in the slot's list) appears as page 0: no kernel reads below a window, and if one
+        ever did it would read a page that exists."""
         g = self.groups[group]
         w = max([width, 1] + [len(g.pages[s]) for s in slots if s >= 0])
         bt = torch.zeros((len(slots), w), dtype=torch.int32)
@@ -249,7 +251,7 @@ class PagedCache:
             if s >= 0:
                 pl = g.pages[s]
                 if pl:
-                    bt[r, :len(pl)] = torch.tensor(pl, dtype=torch.int32)
+                    bt[r, :len(pl)] = torch.tensor(pl, dtype=torch.int32).clamp_(min=0)
         return bt
 
     def view(self, entry: int, block_tables: Dict[int, torch.Tensor], max_len: int) -> KVView:

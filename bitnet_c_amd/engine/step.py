@@ -190,7 +190,7 @@ class _DecodeGraph:
             if key != self.row_keys[r]:
                 for g in range(len(cache.groups)):
                     pl = cache.pages_of(g, s)
-                    self.tables_np[g, r, :len(pl)] = pl
+                    self.tables_np[g, r, :len(pl)] = [max(p, 0) for p in pl]     # a page given back: as block_table
                 self.row_keys[r] = key
                 self.tables_dirty = True
 
