@@ -306,8 +306,6 @@ def test_swiglu_product_with_staged_activations(M, F, K):
     activations staged once per workgroup): against the exact result, and that the dispatcher uses it when it may
     not call the library."""
     ops = _ops()
-    from bitnet_c_amd.csrc import build
-    from ctypes import c_void_p
     x, w = _rand((M, K), torch.bfloat16, 51), _rand((2 * F, K), torch.bfloat16, 52, 0.1)
     g = x.double() @ w[:F].double().t()
     u = x.double() @ w[F:].double().t()
