@@ -1,7 +1,8 @@
 """Each part alone against the plain implementation; the order of layers as data (a layer named
 twice, a layer that reads another layer's cache); and toy parts defined here, registered, built
 and stepped without a change to the library's files: a mixer with a state of its own, a
-feed-forward with routing, another position encoding."""
+feed-forward with routing, another position encoding, another norm and another arrangement of
+a layer's parts."""
 import json
 import math
 import os
@@ -750,3 +751,162 @@ def test_a_toy_feed_forward_with_routing_and_another_position_encoding(tmp_path,
         used |= set((margin > 0).flatten().tolist())
         assert rel_err(torch.cat(got[i]), want) < TOL[dtype], i
     assert used == {True, False}                                       # both experts were chosen somewhere
+
+
+def _register_parallel_toy():
+    """Another norm (mean taken out before the root mean square) and another arrangement of a layer's parts (mixer
+    and feed-forward read the same normed stream and both add to it), both defined here."""
+    from bitnet_c_amd.config import Architecture, register_architecture
+    from bitnet_c_amd.config.base import _ARCHITECTURES
+    from bitnet_c_amd.engine import LayerPlan, ModelPlan, ScheduleEntry
+    from bitnet_c_amd.parts import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, ParamSpec, Part, PartSpec
+
+    if "centered" not in NORMS:
+        @NORMS.register("centered")
+        class CenteredNorm(Part):
+            # neither deferrable nor takes_partial_sums: the stream hands it tensors, with every sum formed
+
+            def __init__(self, dim, eps):
+                self.dim, self.eps = dim, eps
+
+            def tensors(self):
+                return {"weight": ParamSpec((self.dim,), init="ones")}
+
+            def load(self, tensors, device, dtype):
+                self.weight = tensors["weight"].float().to(device)
+
+            def apply(self, x, delta, out_dtype, rows=None):
+                if rows is None:
+                    if delta is not None:
+                        x.add_(delta.float())                       # the norm's kernel is where the sum is formed
+                    xs = x
+                else:
+                    xs = x[rows.long()] if delta is None else x[rows.long()] + delta[rows.long()].float()
+                c = xs - xs.mean(dim=1, keepdim=True)
+                return (c * torch.rsqrt((c * c).mean(dim=1, keepdim=True) + self.eps) * self.weight).to(out_dtype)
+
+    if "parallel" not in BLOCKS:
+        @BLOCKS.register("parallel")
+        class ParallelBlock(Part):
+            def __init__(self, mixer, ffn, norm):
+                self.mixer, self.ffn, self.norm = MIXERS.build(mixer), FEED_FORWARDS.build(ffn), NORMS.build(norm)
+
+            def children(self):
+                return {"mixer": self.mixer, "ffn": self.ffn, "norm": self.norm}
+
+            def tensors(self):
+                return {f"{cn}.{tn}": spec for cn, c in self.children().items() for tn, spec in c.tensors().items()}
+
+            def load(self, tensors, device, dtype):
+                for cn, c in self.children().items():
+                    c.load({k[len(cn) + 1:]: v for k, v in tensors.items() if k.startswith(cn + ".")}, device, dtype)
+
+            def cache_need(self):
+                return self.mixer.cache_need()
+
+            def forward(self, stream, ctx, kv):
+                h = stream.normed(self.norm, ctx.act_dtype)
+                a = self.mixer.forward(h, ctx, kv)
+                f = self.ffn.forward(h, ctx)
+                stream.add(a)
+                stream.add(f)
+
+    @dataclass(frozen=True)
+    class ParallelConfig:
+        vocab_size: int
+        hidden_size: int
+        n_layers: int
+        model_type: str = "toy_parallel"
+
+        @staticmethod
+        def from_dict(raw):
+            return ParallelConfig(raw["vocab_size"], raw["hidden_size"], raw["n_layers"])
+
+        def to_dict(self):
+            return asdict(self)
+
+    def build(c):
+        norm = PartSpec.of("centered", dim=c.hidden_size, eps=1e-3)
+        ffn = PartSpec.of("swiglu", hidden=c.hidden_size, intermediate=56)
+        att = PartSpec.of("attention", hidden=c.hidden_size, n_heads=4, n_kv_heads=2, head_dim=12, scale=0.3,
+                          position=PartSpec.of("none"))
+        layers = []
+        for i in range(c.n_layers):
+            blk = PartSpec.of("parallel", mixer=att, ffn=ffn, norm=norm)
+            names = {local: f"layers.{i}.{local}" for local in BLOCKS.build(blk).tensors()}
+            layers.append(LayerPlan(block=blk, names=names))
+        return ModelPlan(vocab_size=c.vocab_size, hidden_size=c.hidden_size, layers=layers,
+                         schedule=[ScheduleEntry(i) for i in range(c.n_layers)], final_norm=norm,
+                         embedding_name="embed.weight", final_norm_names={"weight": "norm.weight"},
+                         lm_head_name="head.weight")
+
+    if "toy_parallel" not in _ARCHITECTURES:
+        register_architecture(Architecture("toy_parallel", ParallelConfig, build))
+    return ParallelConfig
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_toy_norm_and_another_arrangement_of_a_layer(tmp_path, dtype):
+    """A norm and a block arrangement defined in this file (registered, built from a folder, stepped in a batch of
+    unequal prompts and then token by token from graphs) against a plain computation of the same formulas."""
+    from bitnet_c_amd import Engine, StepEntry
+    from bitnet_c_amd.weights import write_model_folder
+    ParallelConfig = _register_parallel_toy()
+    cfg = ParallelConfig(vocab_size=60, hidden_size=40, n_layers=3)
+    folder = write_model_folder(str(tmp_path / "parallel"), cfg, 23, dtype)
+    eng = Engine.from_folder(folder, dtype=dtype, max_tokens=512)
+    assert eng.use_graphs
+    from safetensors.torch import load_file
+    W = {k: v.float() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    rt = None if dtype == torch.float32 else dtype
+    r_ = lambda x: x if rt is None else x.to(rt).float()
+
+    def centered(x, w):
+        c = x - x.mean(dim=1, keepdim=True)
+        return c * torch.rsqrt((c * c).mean(dim=1, keepdim=True) + 1e-3) * w
+
+    def plain(toks):
+        x = W["embed.weight"][toks]
+        n = len(toks)
+        for l in range(3):
+            p = f"layers.{l}."
+            xb = r_(centered(x, W[p + "norm.weight"]))
+            q = r_(pl.linear(xb, W[p + "mixer.wq"])).view(n, 4, 12)
+            k = r_(pl.linear(xb, W[p + "mixer.wk"])).view(n, 2, 12)
+            v = r_(pl.linear(xb, W[p + "mixer.wv"])).view(n, 2, 12)
+            a = r_(pl.linear(r_(pl.attention(q, k, v, 0.3).reshape(n, 48)), W[p + "mixer.wo"]))
+            f = pl.feed_forward(xb, W[p + "ffn.w_gate"], W[p + "ffn.w_up"], W[p + "ffn.w_down"], rt)
+            x = x + a + f                                          # both read the same xb, both add
+        return pl.linear(r_(centered(x, W["norm.weight"])), W["head.weight"])
+
+    rnd = random.Random(31)
+    reqs = [[rnd.randrange(60) for _ in range(n)] for n in (19, 3, 70)]
+    slots = [eng.new_sequence() for _ in reqs]
+    fed = [len(r) - 2 for r in reqs]
+    out = eng.step([StepEntry(s, r[:f], list(range(f))) for s, r, f in zip(slots, reqs, fed)])
+    got, o = [[] for _ in reqs], 0
+    for i, f in enumerate(fed):
+        got[i].append(out[o:o + f])
+        o += f
+    for k in range(2):
+        out = eng.step([StepEntry(s, [r[f + k]], [0]) for s, r, f in zip(slots, reqs, fed)])
+        for i in range(3):
+            got[i].append(out[i:i + 1])
+    assert eng.graphs_built >= 1
+    for i, r in enumerate(reqs):
+        assert rel_err(torch.cat(got[i]), plain(r)) < TOL[dtype], (dtype, i)
+    # the residual order matters: a sequential layer (the feed-forward reading the stream after the mixer's add)
+    # gives other logits, so the comparison above does tell the two arrangements apart
+    def sequential(toks):
+        x = W["embed.weight"][toks]
+        n = len(toks)
+        for l in range(3):
+            p = f"layers.{l}."
+            xb = centered(x, W[p + "norm.weight"])
+            q, k, v = (pl.linear(xb, W[p + "mixer." + t]).view(n, h, 12) for t, h in (("wq", 4), ("wk", 2), ("wv", 2)))
+            x = x + pl.linear(pl.attention(q, k, v, 0.3).reshape(n, 48), W[p + "mixer.wo"])
+            xb = centered(x, W[p + "norm.weight"])
+            x = x + pl.feed_forward(xb, W[p + "ffn.w_gate"], W[p + "ffn.w_up"], W[p + "ffn.w_down"], None)
+        return pl.linear(centered(x, W["norm.weight"]), W["head.weight"])
+    apart = rel_err(sequential(reqs[0]), plain(reqs[0]))
+    assert apart > 0.03 and apart > 4 * rel_err(torch.cat(got[0]), plain(reqs[0])), apart
