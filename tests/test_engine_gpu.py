@@ -611,6 +611,58 @@ def test_cuts_and_batches_agree_at_the_benchmark_layer_sizes():
         assert float(d.abs().max() / d.pow(2).mean().sqrt()) < 7.0
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_positions_beyond_the_original_context_with_the_8b_rotation_table(dtype):
+    """A sequence of 8,260 tokens with the head size, theta and llama3 scaling of the Llama-3.1-8B shape
+    (original context 8,192) at a narrow width: a prompt step that ends beyond position 8,192, then tokens one
+    by one from there (the decode kernels work the rotation out of the position themselves), against the plain
+    implementation.  With rotation in single precision an angle at position 8,200 is exact to about 5e-4, and
+    a table or a position that is off by one shows far above the tolerance."""
+    import bitnet_c_amd as bn
+    from bitnet_c_amd.config import architecture_for
+    from bitnet_c_amd.engine import DecoderModel
+    from bitnet_c_amd.weights import random_tensors
+    raw = dict(model_type="llama", vocab_size=96, hidden_size=256, intermediate_size=344,
+               num_hidden_layers=1, num_attention_heads=2, num_key_value_heads=1, head_dim=128,
+               max_position_embeddings=131072, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+               rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                 original_max_position_embeddings=8192))
+    cfg = bn.LlamaConfig.from_dict(raw)
+    plan = architecture_for(raw).build_plan(cfg)
+    tensors = random_tensors(plan.expected_tensors(), 9, dtype, device="cuda:0")
+    # queries and keys large enough that the rotation decides which keys a token attends to
+    for name in ("model.layers.0.self_attn.q_proj.weight", "model.layers.0.self_attn.k_proj.weight"):
+        tensors[name] = (tensors[name].float() * 12.0).to(dtype)
+    model = DecoderModel(plan, dtype, "cuda:0")
+    model.load(tensors)
+    eng = bn.Engine(model, max_tokens=8320 + 64)
+    T, fed = 8260, 8254
+    rnd = random.Random(12)
+    toks = [rnd.randrange(cfg.vocab_size) for _ in range(T)]
+    W = {k: v.float().cpu() for k, v in tensors.items()}
+    c = dict(dim=cfg.hidden_size, ffn=cfg.intermediate_size, layers=1, heads=2, kv_heads=1, head_dim=128,
+             vocab=cfg.vocab_size, theta=cfg.rope_theta, eps=cfg.rms_norm_eps, tied=False, rope_scaling=raw["rope_scaling"])
+    rt = None if dtype == torch.float32 else dtype
+    inv = pl.rope_inv_freq(128, c["theta"], c["rope_scaling"])
+    x = pl.decoder_layer(W["model.embed_tokens.weight"][torch.tensor(toks)], torch.arange(T), W, 0, c, inv, rt)
+    want_rows = list(range(8190, 8196)) + list(range(fed - 4, T))          # around 8,192 and at the end
+    xb = pl.rmsnorm(x[want_rows], W["model.norm.weight"], c["eps"])
+    plain_ref = pl.linear(xb if rt is None else xb.to(rt).float(), W["lm_head.weight"])
+    s = eng.new_sequence()
+    got = [eng.step([bn.StepEntry(s, toks[:fed], [r for r in want_rows if r < fed])])]
+    for t in toks[fed:]:
+        got.append(eng.step([bn.StepEntry(s, [t], [0])]))
+    got = torch.cat(got)
+    assert rel_err(got, plain_ref) < TOL[dtype], rel_err(got, plain_ref)
+    # the check can fail: with the last token one position too far the plain implementation gives other values
+    tail = W["model.embed_tokens.weight"][torch.tensor(toks[8100:])]
+    right = pl.decoder_layer(tail, torch.arange(8100, T), W, 0, c, inv, rt)
+    one_off = pl.decoder_layer(tail, torch.cat([torch.arange(8100, T - 1), torch.tensor([T])]), W, 0, c, inv, rt)
+    assert rel_err(one_off[-1:], right[-1:]) > 10 * TOL[dtype]
+    eng.release(s)
+    eng.cache.check()
+
+
 @pytest.mark.parametrize("n_seqs", [20, 50])
 def test_graph_replays_of_a_wide_batch_at_the_benchmark_layer_sizes(n_seqs):
     """20 or 50 sequences decode together at the Llama-3.1-8B layer sizes (two layers, bfloat16): 32 or 64
