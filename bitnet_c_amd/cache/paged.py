@@ -3,7 +3,8 @@
 A *slot* stands for one sequence: its length, its pages in every group, its row of the
 state area.  Keys and values live in pages of PAGE positions; a page id addresses the
 same page in every entry of its group.  Entries of the schedule whose mixers need the
-same kind of storage (same kv heads, head size and window) form a *group* with storage,
+same kind of storage (same kv heads, key and value widths, value layout and window: equal
+KVNeed) form a *group* with storage,
 a page pool and block tables of its own, so a group that keeps a window of keys gives
 pages back while a sequence grows and a group that keeps all keys does not.  Beside the
 pages there is a state area: for every entry that asks for it, a tensor of fixed shape
@@ -27,6 +28,7 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from ..csrc.build import header_constant
+from ..ops import kernel_v_layout
 from ..parts.base import CacheNeed, KVNeed, KVView
 
 PAGE = header_constant("BN_PAGE")        # positions per page: defined once, in csrc/common.h
@@ -78,8 +80,9 @@ class _Group:
     entries: List[int]                       # schedule entries that own storage here, in order
     pool: PagePool
     pages: Dict[int, List[int]]              # slot -> page of each PAGE positions (-1: given back)
-    k: Optional[torch.Tensor] = None         # [entries, pages, Hkv, PAGE, hs]
-    v: Optional[torch.Tensor] = None         # the same; in bfloat16 [entries, pages, Hkv, hs, PAGE]
+    v_transposed: bool = False               # the layout of v that the group's need asks for
+    k: Optional[torch.Tensor] = None         # [entries, pages, Hkv, PAGE, head_dim]
+    v: Optional[torch.Tensor] = None         # [entries, pages, Hkv, PAGE, v_dim], or [.., v_dim, PAGE] when v_transposed
 
 
 class PagedCache:
@@ -107,17 +110,19 @@ class PagedCache:
             if gi is None:
                 gi = len(self.groups)
                 by_need[need.kv] = gi
-                self.groups.append(_Group(need.kv, [], PagePool(self.n_pages), {}))
+                layout = need.kv.v_layout or kernel_v_layout(dtype)      # the need says how its values lie
+                self.groups.append(_Group(need.kv, [], PagePool(self.n_pages), {}, v_transposed=layout == "transposed"))
             self._entry_group.append((gi, len(self.groups[gi].entries)))
             self.groups[gi].entries.append(i)
         for i, src in enumerate(kv_from):
             if src is not None:
                 if self._entry_group[src] is None:
                     raise CacheError(f"entry {i} reads the cache of entry {src}, which keeps none")
-                if needs[i].kv is not None and needs[src].kv is not None and (
-                        needs[i].kv.n_kv_heads != needs[src].kv.n_kv_heads
-                        or needs[i].kv.head_dim != needs[src].kv.head_dim):
-                    raise CacheError(f"entry {i} reads the cache of entry {src} but their kv shapes differ")
+                a, b = needs[i].kv, needs[src].kv
+                if a is not None and b is not None and (
+                        (a.n_kv_heads, a.head_dim, a.v_dim) != (b.n_kv_heads, b.head_dim, b.v_dim)
+                        or (a.v_layout or kernel_v_layout(dtype)) != (b.v_layout or kernel_v_layout(dtype))):
+                    raise CacheError(f"entry {i} reads the cache of entry {src} but their kv shapes or layouts differ")
                 self._entry_group[i] = self._entry_group[src]
         self._free_slots = list(range(self.max_slots - 1, -1, -1))
         self._len: Dict[int, int] = {}
@@ -125,11 +130,10 @@ class PagedCache:
         self._state_needs = {i: n.state for i, n in enumerate(needs) if n.state is not None}
         if device is not None:
             for g in self.groups:
-                shape = (len(g.entries), self.n_pages, g.need.n_kv_heads, PAGE, g.need.head_dim)
-                g.k = torch.zeros(shape, dtype=dtype, device=device)
-                if dtype == torch.bfloat16:     # V transposed inside a page: [.., head_dim, PAGE]
-                    shape = shape[:3] + (g.need.head_dim, PAGE)
-                g.v = torch.zeros(shape, dtype=dtype, device=device)
+                lead = (len(g.entries), self.n_pages, g.need.n_kv_heads)
+                g.k = torch.zeros(lead + (PAGE, g.need.head_dim), dtype=dtype, device=device)
+                g.v = torch.zeros(lead + ((g.need.v_dim, PAGE) if g.v_transposed else (PAGE, g.need.v_dim)),
+                                  dtype=dtype, device=device)
             for i, sn in self._state_needs.items():
                 self.states[i] = torch.zeros((self.max_slots + 1,) + tuple(sn.shape), dtype=sn.dtype, device=device)
 
@@ -263,8 +267,8 @@ class PagedCache:
         g = self.groups[gi]
         return KVView(k_pages=g.k[idx] if g.k is not None else None,
                       v_pages=g.v[idx] if g.v is not None else None,
-                      block_table=block_tables.get(gi), writes=self.kv_from[entry] is None,
-                      state=st, max_len=max_len)
+                      v_transposed=g.v_transposed, block_table=block_tables.get(gi),
+                      writes=self.kv_from[entry] is None, state=st, max_len=max_len)
 
     def check(self) -> None:
         """No page lost, held twice or free twice; no slot both free and in use."""

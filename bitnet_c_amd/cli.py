@@ -182,10 +182,15 @@ def main(argv=None) -> int:
             print(f"[bitnet] tokenizer.json could not be loaded: {e}", file=sys.stderr)
     t0 = time.time()
     max_seq = args.maxseq
-    llm = api.load(args.model, dtype="float32" if args.fp32 else "bfloat16",
-                   max_tokens=max(64, (max_seq or 4096) * (args.batch if args.batch_file else 1)),
-                   max_seq_len=max_seq)
+    # The cache holds min(the model's context length, --maxseq) positions for every sequence of a batch, as the
+    # reference sizes its own (src/model.c:256-257), or what fits into the device's memory if that is less.
+    llm = api.load(args.model, dtype="float32" if args.fp32 else "bfloat16", max_tokens=0, max_seq_len=max_seq,
+                   n_seqs=args.batch if args.batch_file else 1)
     eng = llm.engine
+    if eng.max_seq_len < (min(max_seq, eng.model.plan.max_positions or max_seq) if max_seq
+                          else eng.model.plan.max_positions):
+        print(f"[bitnet] the cache holds sequences of up to {eng.max_seq_len} tokens (what fits into the device's "
+              f"memory beside the model); longer prompts are refused", file=sys.stderr)
     eng.tap = _dump_tap(args)
     vocab = eng.vocab_size
     cfg = llm.config

@@ -5,7 +5,7 @@ default to heads (:252-254), rope_theta to 10000 (:259-260), the norm's eps to 1
 (:264-266), head size to hidden/heads unless given (:285-287); heads must be a multiple
 of kv heads (:299-302).  The reference's SIMD-only checks (hidden % 128, head % 16;
 :303-310) are properties of its kernels, not of the architecture and are not taken over; the one limit of the kernels here that a
-config.json can break (a head size above ops.MAX_HEAD_DIM) is reported with the other errors.
+config.json can break (a head size above BN_MAX_HEAD_DIM of csrc/common.h) is reported with the other errors.
 """
 from __future__ import annotations
 
@@ -13,12 +13,15 @@ import math
 from dataclasses import asdict, dataclass
 from typing import Optional
 
+from ..csrc.build import header_constant
 from .base import ConfigError, _positive_int
 
 
-# config.json's names of the gate activation -> the feed-forward part's (the reference's registry fixes SiLU for
-# this architecture, src/model_arch.c:807-810; its other kinds are reachable through the same key)
+# config.json's names of the gate activation -> the feed-forward part's.  Which of them a config.json may name is the
+# architecture's decision (LlamaConfig.GATE_ACTIVATIONS): the reference's registry fixes SiLU for this one
+# (src/model_arch.c:807-810); the other kinds exist for architectures that declare them.
 HIDDEN_ACTS = {"silu": "silu", "gelu_pytorch_tanh": "gelu_tanh", "gelu_tanh": "gelu_tanh", "relu2": "relu2"}
+MAX_HEAD_DIM = header_constant("BN_MAX_HEAD_DIM")      # the kernels' limit, read from their header (no kernel is loaded for it)
 
 
 @dataclass(frozen=True)
@@ -80,8 +83,12 @@ class LlamaConfig:
     eos_token_id: Optional[object] = None    # an int or a list of ints
     model_type: str = "llama"
 
-    @staticmethod
-    def from_dict(raw: dict) -> "LlamaConfig":
+    # the values of hidden_act that this architecture takes; a configuration class of another architecture of the
+    # family (a subclass) widens it
+    GATE_ACTIVATIONS = ("silu",)
+
+    @classmethod
+    def from_dict(cls, raw: dict) -> "LlamaConfig":
         hidden = _positive_int(raw, "hidden_size")
         heads = _positive_int(raw, "num_attention_heads")
         kv_heads = raw.get("num_key_value_heads")
@@ -99,20 +106,20 @@ class LlamaConfig:
                               f"num_key_value_heads {kv_heads}")
         if head_dim % 2:
             raise ConfigError(f"config.json: head_dim {head_dim} must be even (rotation pairs)")
-        from ..ops import MAX_HEAD_DIM
         if head_dim > MAX_HEAD_DIM:
             raise ConfigError(f"config.json: head_dim {head_dim} is more than the attention kernels take "
                               f"(every even head size up to {MAX_HEAD_DIM})")
         act = raw.get("hidden_act", "silu")
-        if act not in HIDDEN_ACTS:
-            raise ConfigError(f"config.json: hidden_act {act!r} is not supported (supported: {sorted(HIDDEN_ACTS)})")
+        if act not in HIDDEN_ACTS or act not in cls.GATE_ACTIVATIONS:
+            raise ConfigError(f"config.json: hidden_act {act!r} is not supported by this architecture "
+                              f"(supported: {sorted(cls.GATE_ACTIVATIONS)})")
         theta = raw.get("rope_theta")
         theta = 10000.0 if theta in (None, 0) else float(theta)
         eps = raw.get("rms_norm_eps")
         eps = 1e-5 if eps in (None, 0) else float(eps)
         if not (theta > 0 and math.isfinite(theta)) or not (eps > 0 and math.isfinite(eps)):
             raise ConfigError("config.json: rope_theta and rms_norm_eps must be positive and finite")
-        return LlamaConfig(
+        return cls(
             vocab_size=_positive_int(raw, "vocab_size"),
             hidden_size=hidden,
             intermediate_size=_positive_int(raw, "intermediate_size"),

@@ -362,7 +362,7 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
                             float scale, int n_splits, int chunk, float* part_o, float* part_ml,
                             int v_transposed, const int* max_len, hipStream_t s) {
     if (n_tiles <= 0 || n_tokens <= 0 || H <= 0 || Hkv <= 0 || H % Hkv) return BN_ERR_ARG;
-    if (hs < 2 || hs > 256 || hs % 2) return BN_ERR_ARG;
+    if (hs < 2 || hs > BN_MAX_HEAD_DIM || hs % 2) return BN_ERR_ARG;
     if (GT <= 0 || GT > RT || (GT & (GT - 1)) || RT > 16 || (RT & (RT - 1))) return BN_ERR_ARG;
     if (n_splits < 1 || window < 0) return BN_ERR_ARG;
     if (n_splits > 1 && (!part_o || !part_ml || (!max_len && (chunk <= 0 || chunk % BN_PAGE)))) return BN_ERR_ARG;

@@ -10,6 +10,7 @@
 // Decode attention splits a sequence's keys over workgroups in runs of at least this many pages: shorter
 // runs cost more in merging than they gain in parallelism (measured at batch 1, 8 and 64 of an 8B shape).
 #define BN_SPLIT_MIN_PAGES 4
+#define BN_MAX_HEAD_DIM 256   // the attention kernels take every even head size up to this; the configuration reads this line too
 
 // error codes returned by the extern "C" entry points (0 = ok, >0 = hipError_t)
 #define BN_ERR_ARG   (-1)     // an argument the kernel cannot take (size, alignment)
@@ -81,9 +82,10 @@ __host__ __device__ __forceinline__ int bn_split_chunk(int max_len, int n_splits
 
 // The gate's activation in a gated feed-forward, out = act(gate) * up: the kinds the reference knows
 // (src/transformer/cpu_backend.c:343-417).  silu(g) = g / (1 + exp(-g)) with the exact exponential (:356);
-// gelu in its tanh form 0.5 g (1 + tanh(0.79788456 g (1 + 0.044715 g^2))) (:27-29, without the reference's
-// rounding of g and of the result to half precision); relu2(g) = max(g, 0)^2 (:349-350).  Every kernel
-// that ends in a gated unit takes the kind as an argument.
+// gelu in its tanh form 0.5 g (1 + tanh(0.79788456 g (1 + 0.044715 g^2))) (:27-29; the reference's function also
+// returns 0 below -10 and g above 10 and rounds g and the result to half precision, :20-30, which this one does not:
+// it is no activation of the architecture built here, and its parity with the reference is not pinned by a test);
+// relu2(g) = max(g, 0)^2 (:349-350).  Every kernel that ends in a gated unit takes the kind as an argument.
 #define BN_ACT_SILU 0
 #define BN_ACT_GELU_TANH 1
 #define BN_ACT_RELU2 2

@@ -10,6 +10,7 @@ import torch
 
 from .. import ops
 from ..parts import BLOCKS, NORMS, CacheNeed, ResidualStream
+from ..parts.linear import upload
 from .plan import ModelPlan
 
 
@@ -26,17 +27,24 @@ class DecoderModel:
 
     # ---- weights --------------------------------------------------------------------
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        """tensors: folder name -> host tensor (every name of plan.expected_tensors())."""
+        """tensors: folder name -> host (or device) tensor for every name of plan.expected_tensors(): a dict, or a
+        weights.TensorSource, whose tensors are views of the mapped file; then every layer's tensors are let go
+        (release) as soon as the layer has uploaded them, so the host never holds the model."""
         p = self.plan
+        done = getattr(tensors, "release", lambda names: None)
         for lp, blk in zip(p.layers, self.blocks):
             local = {ln: tensors[fn] for ln, fn in lp.names.items() if fn in tensors and ln in blk.tensors()}
             blk.load(local, self.device, self.dtype)
+            del local
+            done(lp.names.values())
         self.final_norm.load({ln: tensors[fn] for ln, fn in p.final_norm_names.items()}, self.device, self.dtype)
-        self.embedding = tensors[p.embedding_name].to(self.dtype).to(self.device).contiguous()
+        self.embedding = upload(tensors[p.embedding_name], self.device, self.dtype)
+        done([p.embedding_name])
         if p.lm_head_name is None:
             self.lm_head = self.embedding
         else:
-            self.lm_head = tensors[p.lm_head_name].to(self.dtype).to(self.device).contiguous()
+            self.lm_head = upload(tensors[p.lm_head_name], self.device, self.dtype)
+            done([p.lm_head_name])
 
     def weight_bytes(self) -> int:
         """Bytes of every weight a decode step reads once (the embedding table only when it is

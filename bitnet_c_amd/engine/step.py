@@ -21,7 +21,7 @@ import torch
 from .. import ops
 from ..cache import PAGE, CacheError, CacheFull, PagedCache
 from ..config import load_config
-from ..weights import load_tensors
+from ..weights import open_tensors
 from .model import DecoderModel
 
 
@@ -191,7 +191,13 @@ class _DecodeGraph:
                 for g in range(len(cache.groups)):
                     pl = cache.pages_of(g, s)
                     self.tables_np[g, r, :len(pl)] = [max(p, 0) for p in pl]     # a page given back: as block_table
+                    self.tables_np[g, r, len(pl):] = 0       # and nothing of the row's former owner stays behind it
                 self.row_keys[r] = key
+                self.tables_dirty = True
+        for r in range(n, rows):                             # rows that have become padding: the table block_table() gives
+            if self.row_keys[r] is not None:
+                self.tables_np[:, r, :] = 0
+                self.row_keys[r] = None
                 self.tables_dirty = True
 
     def upload(self):
@@ -237,14 +243,40 @@ class Engine:
 
     # ---- construction ---------------------------------------------------------------
     @staticmethod
+    def cache_bytes_per_token(model: DecoderModel) -> int:
+        """Bytes of keys and values that one cached position takes over all entries of the schedule."""
+        needs, kv_from = model.cache_needs()
+        size = torch.empty((), dtype=model.dtype).element_size()
+        return sum(n.kv.n_kv_heads * (n.kv.head_dim + n.kv.v_dim) * size
+                   for n, src in zip(needs, kv_from) if n.kv is not None and src is None)
+
+    @staticmethod
+    def tokens_that_fit(model: DecoderModel, wanted: int, share: float = 0.8) -> int:
+        """`wanted` cached positions, or as many whole pages as fit into `share` of the device memory that is free
+        now (the model is loaded already), whichever is less; at least one page."""
+        per_token = Engine.cache_bytes_per_token(model)
+        if per_token == 0:
+            return max(PAGE, wanted)
+        free, _ = torch.cuda.mem_get_info(model.device)
+        fit = int(free * share) // per_token // PAGE * PAGE
+        return max(PAGE, min(wanted, fit))
+
+    @staticmethod
     def from_folder(folder: str, dtype=torch.bfloat16, max_tokens: int = 4096, device="cuda:0",
-                    max_seq_len: int = 0, max_slots: int = 0, use_graphs: bool = True) -> "Engine":
+                    max_seq_len: int = 0, max_slots: int = 0, use_graphs: bool = True, n_seqs: int = 1) -> "Engine":
+        """max_tokens: positions that the cache holds; 0: n_seqs sequences of the longest length there can be
+        (the model's max_positions, or max_seq_len when that is less: the reference sizes its cache by
+        min(context length, --maxseq), src/model.c:256-257), or as many as fit into the free device memory."""
         ops.require_gpu()
         arch, config = load_config(folder)
         plan = arch.build_plan(config)
-        tensors = load_tensors(folder, plan.expected_tensors())
         model = DecoderModel(plan, dtype, device)
-        model.load(tensors)
+        with open_tensors(folder, plan.expected_tensors()) as tensors:      # views of the mapped file, uploaded one by one
+            model.load(tensors)
+        if max_tokens <= 0:
+            longest = min(v for v in (plan.max_positions, max_seq_len) if v > 0) if (plan.max_positions or max_seq_len) else 4096
+            per_seq = (longest + PAGE - 1) // PAGE * PAGE
+            max_tokens = Engine.tokens_that_fit(model, per_seq * max(1, n_seqs))
         eng = Engine(model, max_tokens, max_seq_len, max_slots, use_graphs)
         eng.config = config
         return eng

@@ -639,15 +639,18 @@ def linear_into_stream(x: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, w
 # position encoding + cache write, attention
 # --------------------------------------------------------------------------------------
 
-def v_transposed_for(dtype) -> bool:
-    """bf16 caches keep V transposed ([pages, Hkv, hs, PAGE]) for the matrix-core attention
-    kernels; float32 caches keep V like K ([pages, Hkv, PAGE, hs])."""
-    return dtype == torch.bfloat16
+def kernel_v_layout(dtype) -> str:
+    """The value layout (KVNeed.v_layout) that the attention kernels of this library read fastest at a cache
+    type: bf16 values transposed inside a page ([pages, Hkv, hs, PAGE]) for the matrix-core kernels, float32
+    values like the keys ([pages, Hkv, PAGE, hs]).  The vector kernel and the cache write take either layout
+    at either type; the matrix-core kernels take the transposed one alone."""
+    return "transposed" if dtype == torch.bfloat16 else "rows"
 
 
-def _check_pages(k_pages, v_pages, Hkv, hs, dtype):
-    """Checks both page tensors; returns whether V is transposed."""
-    vt = v_transposed_for(dtype)
+def _check_pages(k_pages, v_pages, Hkv, hs, dtype, v_transposed=None):
+    """Checks both page tensors against the layout that the caller names (None: kernel_v_layout of the type);
+    returns whether V is transposed.  The kernels here want values as wide as keys."""
+    vt = kernel_v_layout(dtype) == "transposed" if v_transposed is None else bool(v_transposed)
     for t, nm, shape in ((k_pages, "k_pages", (Hkv, PAGE, hs)), (v_pages, "v_pages", (Hkv, hs, PAGE) if vt else (Hkv, PAGE, hs))):
         _dev(t, nm, dtype, 4)
         if tuple(t.shape[1:]) != shape or not t.is_contiguous():
@@ -659,13 +662,14 @@ def _check_pages(k_pages, v_pages, Hkv, hs, dtype):
 
 def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, hs: int, *,
                   inv_freq=None, rope_dims: int = 0, seq_index=None, block_table=None,
-                  k_pages=None, v_pages=None, page_tiles=None) -> None:
+                  k_pages=None, v_pages=None, page_tiles=None, v_transposed=None) -> None:
     """Rotate the Q heads of qkv ([T, (H+2Hkv)*hs]) in place, rotate the K heads and store
     them and the V heads at each token's position of its sequence's pages.
     k_pages None: rotate Q only.  rope_dims 0: no rotation.  positions < 0: padding rows.
     page_tiles (optional, [n, 4] int32 = sequence, first row, rows, position of the first; each
     tile inside one page, all rows covered): transposed V pages are then filled by a kernel
-    that stores runs of positions instead of single elements."""
+    that stores runs of positions instead of single elements.
+    v_transposed: the layout of v_pages (None: kernel_v_layout of qkv's type)."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(positions, "positions", torch.int32, 1)
@@ -682,7 +686,7 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
     bt_stride = 0
     vt = False
     if k_pages is not None:
-        vt = _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype)
+        vt = _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype, v_transposed)
         _dev(seq_index, "seq_index", torch.int32, 1)
         _dev(block_table, "block_table", torch.int32, 2)
         if seq_index.numel() != T or not seq_index.is_contiguous() or not block_table.is_contiguous():
@@ -710,7 +714,7 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
             v_pages.data_ptr(), H, Hkv, hs, _stream()), "v_transposed_write")
 
 
-MAX_HEAD_DIM = 256        # the attention kernels take every even head size up to this
+MAX_HEAD_DIM = _build.header_constant("BN_MAX_HEAD_DIM")    # the attention kernels take every even head size up to this
 
 
 def _pow2_at_least(n: int) -> int:
@@ -802,7 +806,7 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
               block_table: torch.Tensor, H: int, Hkv: int, hs: int, scale: float, *, window: int = 0,
               tiles=None, qt: int = 0, seq_lens=None, n_splits: int = 1, chunk: int = 0,
               force_vector: bool = False, fused_rotate=None, fused_write: bool = False, by_length=None,
-              max_len_dev=None) -> None:
+              max_len_dev=None, v_transposed=None) -> None:
     """Causal attention of the (rotated) Q heads in qkv over the paged cache.
 
     Prompt form: `tiles` [n, 4] int32 = (sequence, first token row, tokens (<= qt), position of
@@ -820,11 +824,13 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     on every CU, so that long and short sequences share CUs.  It changes no result.
     max_len_dev (decode form, optional): a device int32 holding the longest sequence's key count; with
     n_splits > 1 the kernels then cut the keys into n_splits runs of split_chunk(max_len, n_splits) and
-    `chunk` is not used, so that one captured launch serves every length up to the block table's width."""
+    `chunk` is not used, so that one captured launch serves every length up to the block table's width.
+    v_transposed: the layout of v_pages (None: kernel_v_layout of qkv's type); values that lie like the keys go to
+    the vector kernel whatever their type."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(out, "out", qkv.dtype, 2)
-    vt = _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype)
+    vt = _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype, v_transposed)
     _dev(block_table, "block_table", torch.int32, 2)
     T = qkv.shape[0]
     if H % Hkv or qkv.shape[1] < H * hs or out.shape != (T, H * hs) or not out.is_contiguous():
@@ -834,7 +840,7 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     if not block_table.is_contiguous():
         raise KernelError("attention: block_table must be contiguous")
     decode = tiles is None
-    use_mfma = mfma_attention(qkv.dtype, hs) and not force_vector
+    use_mfma = mfma_attention(qkv.dtype, hs) and vt and not force_vector
     RT, GT, QT = attention_row_shape(H, Hkv, decode, qkv.dtype if use_mfma else None, hs)
     if decode:
         _dev(seq_lens, "seq_lens", torch.int32, 1)

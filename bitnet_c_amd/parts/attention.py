@@ -17,7 +17,7 @@ import torch
 
 from .. import ops
 from .base import MIXERS, POSITION_ENCODINGS, CacheNeed, KVNeed, ParamSpec, Part, PartSpec
-from .linear import Linear
+from .linear import Linear, upload
 
 
 @MIXERS.register("attention")
@@ -54,10 +54,11 @@ class Attention(Part):
         return t
 
     def load(self, tensors, device, dtype):
-        w = torch.cat([tensors["wq"].to(dtype), tensors["wk"].to(dtype), tensors["wv"].to(dtype)], dim=0)
+        # stacked on the device: the host holds no copy beside the file's own bytes
+        w = torch.cat([upload(tensors[n], device, dtype) for n in ("wq", "wk", "wv")], dim=0)
         b = None
         if self.has_bias:
-            b = torch.cat([tensors["bq"].float(), tensors["bk"].float(), tensors["bv"].float()])
+            b = torch.cat([upload(tensors[n], device, torch.float32) for n in ("bq", "bk", "bv")])
         self.qkv.load(w, b, device, dtype)
         self.o.load(tensors["wo"], tensors.get("bo") if self.has_bias else None, device, dtype)
         self.position.prepare(device)
@@ -77,7 +78,9 @@ class Attention(Part):
             qkv = pad
         out = torch.empty((h.shape[0], self.q_dim), dtype=h.dtype, device=h.device)
         fuse_ok, inv_freq = self.position.fusable(hs)
-        if ctx.is_decode and fuse_ok and ops.can_fuse_decode(h.dtype, H, Hkv, hs):
+        vt = kv.v_transposed
+        if (ctx.is_decode and fuse_ok and ops.can_fuse_decode(h.dtype, H, Hkv, hs)
+                and (vt is None or vt)):                        # the matrix-core kernels read transposed values
             # one kernel: rotation of Q and the new K, the cache write, attention, merge of the splits
             if self.window:
                 n_splits, chunk = 1, 0
@@ -86,7 +89,7 @@ class Attention(Part):
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
                           window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
                           fused_rotate=inv_freq, fused_write=kv.writes, by_length=ctx.by_length,
-                          max_len_dev=ctx.max_len_dev if n_splits > 1 else None)
+                          max_len_dev=ctx.max_len_dev if n_splits > 1 else None, v_transposed=vt)
             return last(out)
         self.position.encode_and_store(qkv, ctx, H, Hkv, hs, kv)
         if ctx.is_decode:
@@ -96,9 +99,11 @@ class Attention(Part):
                 n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len, h.dtype)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
                           window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
-                          by_length=ctx.by_length, max_len_dev=ctx.max_len_dev if n_splits > 1 else None)
+                          by_length=ctx.by_length, max_len_dev=ctx.max_len_dev if n_splits > 1 else None,
+                          v_transposed=vt)
         else:
-            _, _, qt = ops.attention_row_shape(H, Hkv, False, h.dtype, hs)
+            mfma = vt is None or vt                             # values that lie like the keys: the vector kernel
+            _, _, qt = ops.attention_row_shape(H, Hkv, False, h.dtype if mfma else None, hs)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
-                          window=self.window, tiles=ctx.tiles(qt), qt=qt)
+                          window=self.window, tiles=ctx.tiles(qt), qt=qt, v_transposed=vt, force_vector=not mfma)
         return last(out)

@@ -61,10 +61,30 @@ class ParamSpec:
 
 @dataclass(frozen=True)
 class KVNeed:
-    """Keys and values of every position (window 0) or of the last `window` positions."""
+    """Keys and values of every position (window 0) or of the last `window` positions, and how a page of the
+    cache holds them.  A page keeps PAGE positions of every kv head: the keys as [kv head, PAGE, head_dim]; the
+    values, v_head_dim wide (0: as wide as the keys), either the same way (v_layout "rows") or turned,
+    [kv head, v_head_dim, PAGE] ("transposed": 8 consecutive positions of one value column lie together, which is
+    what a kernel that multiplies weights by values on the matrix cores reads).  v_layout None asks for the layout
+    that this library's attention kernels read at the cache's type (ops.kernel_v_layout); a mixer with kernels or
+    torch code of its own names the layout it wants."""
     n_kv_heads: int
     head_dim: int
     window: int = 0
+    v_head_dim: int = 0
+    v_layout: Optional[str] = None
+
+    V_LAYOUTS = ("rows", "transposed")
+
+    def __post_init__(self):
+        if self.v_layout is not None and self.v_layout not in self.V_LAYOUTS:
+            raise ValueError(f"KVNeed: v_layout {self.v_layout!r} is not one of {self.V_LAYOUTS}")
+        if self.n_kv_heads < 1 or self.head_dim < 1 or self.v_head_dim < 0 or self.window < 0:
+            raise ValueError(f"KVNeed: sizes must be positive, got {self}")
+
+    @property
+    def v_dim(self) -> int:
+        return self.v_head_dim or self.head_dim
 
 
 @dataclass(frozen=True)
@@ -129,8 +149,9 @@ class Part:
 @dataclass
 class KVView:
     """What a mixer sees of the cache for one entry of the schedule in one step."""
-    k_pages: Optional[torch.Tensor] = None      # [pages, Hkv, PAGE, hs]
-    v_pages: Optional[torch.Tensor] = None
+    k_pages: Optional[torch.Tensor] = None      # [pages, Hkv, PAGE, head_dim]
+    v_pages: Optional[torch.Tensor] = None      # [pages, Hkv, PAGE, v_dim], or [pages, Hkv, v_dim, PAGE] when v_transposed
+    v_transposed: Optional[bool] = None         # the layout of v_pages (KVNeed.v_layout as the cache resolved it)
     block_table: Optional[torch.Tensor] = None  # [B, W] int32, this step's sequences
     writes: bool = True                         # False: the entry reads another entry's cache
     state: Optional[torch.Tensor] = None        # [max_slots + 1, *shape] fixed-size state, by slot

@@ -11,7 +11,7 @@ import torch
 
 from .. import ops
 from .base import FEED_FORWARDS, ParamSpec, Part
-from .linear import Linear
+from .linear import Linear, upload
 
 
 @FEED_FORWARDS.register("gated")
@@ -36,13 +36,12 @@ class SwiGLU(Part):
 
     def load(self, tensors, device, dtype):
         self.interleaved = self.F % 8 == 0
-        if self.interleaved:
-            w = ops.interleave_gate_up(tensors["w_gate"].to(dtype), tensors["w_up"].to(dtype))
-        else:
-            w = torch.cat([tensors["w_gate"].to(dtype), tensors["w_up"].to(dtype)], dim=0)
+        wg, wu = upload(tensors["w_gate"], device, dtype), upload(tensors["w_up"], device, dtype)
+        w = ops.interleave_gate_up(wg, wu) if self.interleaved else torch.cat([wg, wu], dim=0)     # on the device
+        del wg, wu
         b = None
         if self.has_bias:
-            bg, bu = tensors["b_gate"].float(), tensors["b_up"].float()
+            bg, bu = upload(tensors["b_gate"], device, torch.float32), upload(tensors["b_up"], device, torch.float32)
             b = (torch.stack([bg.reshape(-1, 8), bu.reshape(-1, 8)], dim=1).reshape(-1) if self.interleaved
                  else torch.cat([bg, bu]))
         self.gate_up.load(w, b, device, dtype)

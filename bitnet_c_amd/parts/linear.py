@@ -7,14 +7,20 @@ import torch
 from .. import ops
 
 
+def upload(t: torch.Tensor, device, dtype) -> torch.Tensor:
+    """A tensor on the device in the compute type: copied up in the type it has (a host tensor may be a view of
+    the mapped model file, which is neither converted nor copied on the host) and converted there."""
+    return t.to(device).to(dtype).contiguous()      # a tensor that is there already in that type is taken as it is
+
+
 class Linear:
     def __init__(self):
         self.weight = None
         self.bias = None
 
     def load(self, weight: torch.Tensor, bias, device, dtype):
-        self.weight = weight.to(dtype).to(device).contiguous()
-        self.bias = bias.to(torch.float32).to(device).contiguous() if bias is not None else None
+        self.weight = upload(weight, device, dtype)
+        self.bias = upload(bias, device, torch.float32) if bias is not None else None
 
     def __call__(self, x, out_dtype=None, rows: slice | None = None) -> torch.Tensor:
         """x: activations, or an ops.DeferredNorm whose norm this product applies itself when it can."""

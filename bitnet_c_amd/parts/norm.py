@@ -7,6 +7,7 @@ import torch
 
 from .. import ops
 from .base import NORMS, ParamSpec, Part
+from .linear import upload
 
 
 @NORMS.register("rmsnorm")
@@ -22,7 +23,7 @@ class RMSNorm(Part):
         return {"weight": ParamSpec((self.dim,), init="ones")}
 
     def load(self, tensors, device, dtype):
-        self.weight = tensors["weight"].to(torch.float32).to(device).contiguous()
+        self.weight = upload(tensors["weight"], device, torch.float32)
 
     def apply(self, x, delta, out_dtype, rows=None):
         return ops.add_rmsnorm(x, delta, self.weight, self.eps, out_dtype, rows)

@@ -60,7 +60,8 @@ class PositionEncoding(Part):
                           block_table=kv.block_table if kv.writes else None,
                           k_pages=kv.k_pages if kv.writes else None,
                           v_pages=kv.v_pages if kv.writes else None,
-                          page_tiles=ctx.page_tiles() if kv.writes and not ctx.is_decode else None)
+                          page_tiles=ctx.page_tiles() if kv.writes and not ctx.is_decode else None,
+                          v_transposed=kv.v_transposed)
 
 
 @POSITION_ENCODINGS.register("rope")

@@ -46,7 +46,8 @@ class SafetensorsFile:
             raise SafetensorsError(f"{path}: the header is not a JSON object")
         self._base = 8 + hlen
         self._data_len = size - self._base
-        self._mm = mmap.mmap(self._f.fileno(), 0, access=mmap.ACCESS_READ) if size else None
+        # private (copy-on-write) rather than read-only: nothing writes to it, and a tensor can share its memory
+        self._mm = mmap.mmap(self._f.fileno(), 0, access=mmap.ACCESS_COPY) if size else None
         self.entries: Dict[str, Tuple[torch.dtype, Tuple[int, ...]]] = {}
         self._spans = {}
         for name, info in header.items():
@@ -82,10 +83,36 @@ class SafetensorsFile:
         owned = bytearray(self._mm[self._base + a:self._base + b])     # one copy out of the map
         return torch.frombuffer(owned, dtype=dt).reshape(shape)
 
+    def view(self, name: str) -> torch.Tensor:
+        """The tensor as it lies in the map: no copy, no memory of its own (the reference maps its file the same way
+        and points its tensors into it, src/model.c:147).  The pages come in when they are touched; release()
+        lets them go again.  Not to be written to; it keeps the map alive for as long as it lives."""
+        dt, shape = self.entries[name]
+        a, b = self._spans[name]
+        if a == b:
+            return torch.empty(shape, dtype=dt)
+        if (self._base + a) % torch.empty((), dtype=dt).element_size():
+            return self.read(name)                          # not aligned for its type in the file: a copy is
+        return torch.frombuffer(self._mm, dtype=dt, count=(b - a) // torch.empty((), dtype=dt).element_size(),
+                                offset=self._base + a).reshape(shape)
+
+    def release(self, name: str) -> None:
+        """Tells the system that the tensor's pages are not needed any more (they are read again from the file
+        if they are): what was touched of it stops counting as this process's memory."""
+        a, b = self._spans[name]
+        ps = mmap.PAGESIZE
+        lo = -(-(self._base + a) // ps) * ps               # whole pages inside the span only: neighbours may be in use
+        hi = (self._base + b) // ps * ps
+        if hi > lo and self._mm is not None and hasattr(self._mm, "madvise"):
+            try:
+                self._mm.madvise(mmap.MADV_DONTNEED, lo, hi - lo)
+            except (OSError, ValueError, AttributeError):
+                pass                                        # advice only
+
     def close(self) -> None:
-        if self._mm is not None:
-            self._mm.close()
-            self._mm = None
+        # The map is not unmapped here but when nothing refers to it any more: a tensor from view() shares its memory
+        # and holds a reference to it, and unmapping under such a tensor would leave it pointing nowhere.
+        self._mm = None
         self._f.close()
 
     def __enter__(self):

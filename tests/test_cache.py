@@ -114,6 +114,32 @@ def test_groups_by_need_and_shared_entries():
         _cache(needs=[CacheNeed(), CacheNeed(kv=full)], kv_from=[None, 0])
 
 
+def test_a_need_names_the_width_and_the_layout_of_its_values():
+    """The layout of a page is the mixer's to say (KVNeed): values of another width than the keys, lying like the
+    keys or turned, at either type; needs that differ in it get storage of their own, and an entry cannot read the
+    cache of an entry whose layout differs."""
+    plain, wide = KVNeed(2, 16), KVNeed(2, 16, v_head_dim=40, v_layout="rows")
+    turned, rows = KVNeed(2, 16, v_layout="transposed"), KVNeed(2, 16, v_layout="rows")
+    needs = [CacheNeed(kv=n) for n in (plain, wide, turned, rows, wide)]
+    for dtype in (torch.float32, torch.bfloat16):
+        c = PagedCache(needs, [None] * 5, 64 * 4, dtype=dtype, device="cpu")
+        shapes = [(tuple(g.k.shape[2:]), tuple(g.v.shape[2:]), g.v_transposed, g.entries) for g in c.groups]
+        own = (2, 16, PAGE) if dtype == torch.bfloat16 else (2, PAGE, 16)      # no layout named: the kernels' for the type
+        assert ((2, PAGE, 16), own, dtype == torch.bfloat16, [0]) in shapes
+        assert ((2, PAGE, 16), (2, PAGE, 40), False, [1, 4]) in shapes
+        # a named layout that is the kernels' own for the type shares no storage with the unnamed need: the need differs
+        assert ((2, PAGE, 16), (2, 16, PAGE), True, [2]) in shapes and ((2, PAGE, 16), (2, PAGE, 16), False, [3]) in shapes
+        tables = {g: torch.zeros(1, 1, dtype=torch.int32) for g in range(len(c.groups))}
+        assert c.view(1, tables, 64).v_transposed is False and c.view(2, tables, 64).v_transposed is True
+        assert c.view(1, tables, 64).v_pages.shape == (4, 2, PAGE, 40)
+    with pytest.raises(CacheError, match="layouts differ"):
+        PagedCache([CacheNeed(kv=wide), CacheNeed(kv=plain)], [None, 0], 64 * 4, device=None)
+    with pytest.raises(CacheError, match="layouts differ"):
+        PagedCache([CacheNeed(kv=turned), CacheNeed(kv=rows)], [None, 0], 64 * 4, device=None)
+    with pytest.raises(ValueError):
+        KVNeed(2, 16, v_layout="columns")
+
+
 def test_window_group_gives_pages_back_while_the_sequence_grows():
     full, win = KVNeed(1, 8), KVNeed(1, 8, window=70)
     c = _cache(needs=[CacheNeed(kv=full), CacheNeed(kv=win)], max_tokens=64 * 10)

@@ -172,6 +172,72 @@ def test_sharded_folder(tmp_path):
     assert float(t["a"].sum()) == 2.0 and t["b"].shape == (3,)
 
 
+def test_a_model_is_read_tensor_by_tensor_without_holding_it(tmp_path):
+    """open_tensors gives views of the mapped files and release() lets their pages go: walking a sharded folder of
+    24 tensors of 4 MB the way a model is uploaded (take a layer's tensors, use them, release them) raises the
+    process's peak memory by less than two tensors, where reading the folder whole (load_tensors) raises it by the
+    folder's size.  Measured in a fresh process with resource.getrusage, whose peak only ever grows."""
+    import subprocess
+    import sys
+    from bitnet_c_amd.weights import write_file
+    d = str(tmp_path)
+    names, wm = [], {}
+    for shard in range(3):
+        fn = f"model-0000{shard + 1}-of-00003.safetensors"
+        part = {f"t{shard}_{i}": torch.full((1024, 1024), float(8 * shard + i), dtype=torch.float32) for i in range(8)}
+        write_file(os.path.join(d, fn), part)
+        names += list(part)
+        wm.update({n: fn for n in part})
+    with open(os.path.join(d, "model.safetensors.index.json"), "w") as f:
+        json.dump({"weight_map": wm}, f)
+    script = f"""
+import resource, sys, torch
+sys.path.insert(0, {os.path.dirname(os.path.dirname(os.path.abspath(__file__)))!r})
+from bitnet_c_amd.weights import TensorSpec, load_tensors, open_tensors
+names = {names!r}
+exp = {{n: TensorSpec(n, (1024, 1024)) for n in names}}
+peak = lambda: resource.getrusage(resource.RUSAGE_SELF).ru_maxrss * 1024
+torch.zeros(1 << 20).sum()                       # whatever the first use of torch brings in
+p0 = peak()
+total = 0.0
+with open_tensors({d!r}, exp) as src:
+    for i in range(0, len(names), 2):            # two tensors at a time, as a layer's
+        pair = [src[n] for n in names[i:i + 2]]
+        total += sum(float(t.sum()) for t in pair)
+        del pair
+        src.release(names[i:i + 2])
+p1 = peak()
+whole = load_tensors({d!r}, exp)
+p2 = peak()
+print(total, p1 - p0, p2 - p1)
+"""
+    out = subprocess.run([sys.executable, "-c", script], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr[-2000:]
+    total, streamed, held = (float(v) for v in out.stdout.split())
+    assert total == sum(range(24)) * 1024 * 1024
+    one = 4 << 20
+    assert streamed <= 2 * 2 * one + (4 << 20), streamed      # two tensors in use at a time, and some slack
+    assert held >= 16 * one, held                              # the measure can tell: the whole folder is 24 tensors
+
+
+def test_views_of_the_map_are_the_file_s_bytes(tmp_path):
+    from bitnet_c_amd.weights import SafetensorsFile, TensorSpec, open_tensors, write_file
+    d = str(tmp_path)
+    a = torch.arange(5, dtype=torch.bfloat16)                  # 10 bytes: what follows it is not aligned for 4-byte types
+    b = torch.arange(12, dtype=torch.float32).view(3, 4)
+    h = torch.arange(6, dtype=torch.float16).view(2, 3)
+    write_file(os.path.join(d, "model.safetensors"), {"a": a, "b": b, "h": h})
+    with SafetensorsFile(os.path.join(d, "model.safetensors")) as f:
+        assert torch.equal(f.view("a"), a) and torch.equal(f.view("b"), b)
+    with open_tensors(d, {"a": TensorSpec("a", (5,)), "b": TensorSpec("b", (3, 4)), "h": TensorSpec("h", (2, 3))}) as src:
+        assert set(src) == {"a", "b", "h"} and len(src) == 3 and "zz" not in src
+        assert torch.equal(src["b"], b) and src["h"].dtype == torch.float32 and torch.equal(src["h"], h.float())
+        kept = src["a"]
+        src.release(["a", "b", "zz"])                          # advice only; the bytes are read again when asked for
+        assert torch.equal(src["a"], a)
+    assert torch.equal(kept, a)                                # a view that outlives the source keeps the map alive
+
+
 def test_rope_frequencies_match_the_plain_implementation():
     import plain_llama as pl
     from bitnet_c_amd.parts.position import rope_frequencies

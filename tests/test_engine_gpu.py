@@ -744,10 +744,21 @@ def test_other_gate_activations_through_the_engine(tmp_path, act, F, dtype):
     prompts (the library's product and the gated-unit kernel, or the float32 kernels), then decoded tokens (the
     streaming product's epilogue, with the norm folded in where the width allows), against the plain implementation."""
     import bitnet_c_amd as bn
-    raw = dict(model_type="llama", vocab_size=211, hidden_size=128, intermediate_size=F, num_hidden_layers=2,
+    from bitnet_c_amd.config import Architecture, ConfigError, register_architecture
+    from bitnet_c_amd.config.llama import HIDDEN_ACTS
+    from bitnet_c_amd.config.llama_plan import build_llama_plan
+
+    # this architecture's config.json takes silu alone; another architecture of the family declares what it takes
+    class OtherGateConfig(bn.LlamaConfig):
+        GATE_ACTIVATIONS = tuple(HIDDEN_ACTS)
+
+    register_architecture(Architecture("other_gate_test", OtherGateConfig, build_llama_plan), replace=True)
+    raw = dict(model_type="other_gate_test", vocab_size=211, hidden_size=128, intermediate_size=F, num_hidden_layers=2,
                num_attention_heads=4, num_key_value_heads=2, head_dim=32, max_position_embeddings=512,
                rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False, hidden_act=act)
-    folder = bn.write_model_folder(str(tmp_path / "m"), bn.LlamaConfig.from_dict(raw), 77, dtype)
+    with pytest.raises(ConfigError, match="hidden_act"):
+        bn.LlamaConfig.from_dict(dict(raw, model_type="llama"))
+    folder = bn.write_model_folder(str(tmp_path / "m"), OtherGateConfig.from_dict(raw), 77, dtype)
     c, W = pl.read_config(folder), pl.read_weights(folder)
     assert c["act"] == act
     eng = bn.Engine.from_folder(folder, dtype=dtype, max_tokens=1024)

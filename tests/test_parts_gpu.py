@@ -910,3 +910,192 @@ def test_a_toy_norm_and_another_arrangement_of_a_layer(tmp_path, dtype):
         return pl.linear(centered(x, W["norm.weight"]), W["head.weight"])
     apart = rel_err(sequential(reqs[0]), plain(reqs[0]))
     assert apart > 0.03 and apart > 4 * rel_err(torch.cat(got[0]), plain(reqs[0])), apart
+
+
+# ---------------------------------------------------------------------------------------
+# the layout of a cache page is the mixer's to say (KVNeed): values wider than keys, and the
+# library's own attention over values that lie like the keys in bfloat16
+# ---------------------------------------------------------------------------------------
+
+def test_a_toy_mixer_whose_values_are_wider_than_its_keys(tmp_path):
+    """One-head attention with keys of 8 and values of 24 columns, written in the test with torch over the pages
+    that the cache gives it: the cache allocates what the need says ([.., PAGE, 24] beside [.., PAGE, 8]) and nothing
+    in the library is edited for it.  Prompts of unequal lengths, tokens one by one, a slot that is used again."""
+    from bitnet_c_amd import Engine, StepEntry
+    from bitnet_c_amd.cache import PAGE
+    from bitnet_c_amd.config import Architecture, register_architecture
+    from bitnet_c_amd.config.base import _ARCHITECTURES
+    from bitnet_c_amd.engine import LayerPlan, ModelPlan, ScheduleEntry
+    from bitnet_c_amd.parts import BLOCKS, MIXERS, CacheNeed, KVNeed, ParamSpec, Part, PartSpec
+    from bitnet_c_amd.weights import write_model_folder
+    DK, DV = 8, 24
+
+    if "wide_values" not in MIXERS:
+        @MIXERS.register("wide_values")
+        class WideValues(Part):
+            def __init__(self, hidden):
+                self.hidden = hidden
+
+            def tensors(self):
+                return {"wq": ParamSpec((DK, self.hidden)), "wk": ParamSpec((DK, self.hidden)),
+                        "wv": ParamSpec((DV, self.hidden)), "wo": ParamSpec((self.hidden, DV))}
+
+            def load(self, tensors, device, dtype):
+                self.w = {k: v.float().to(device) for k, v in tensors.items()}
+
+            def cache_need(self):
+                return CacheNeed(kv=KVNeed(1, DK, v_head_dim=DV, v_layout="rows"))
+
+            def forward(self, h, ctx, kv):
+                assert kv.v_transposed is False and kv.v_pages.shape[1:] == (1, PAGE, DV)
+                x = h.float()
+                q, k, v = x @ self.w["wq"].t(), x @ self.w["wk"].t(), x @ self.w["wv"].t()
+                pos, seq = ctx.positions.long(), ctx.seq_index.long()
+                page = kv.block_table.long()[seq, pos // PAGE]
+                kv.k_pages[page, 0, pos % PAGE] = k.to(kv.k_pages.dtype)
+                kv.v_pages[page, 0, pos % PAGE] = v.to(kv.v_pages.dtype)
+                out = torch.empty((h.shape[0], DV), dtype=torch.float32, device=h.device)
+                for b, ((r0, n), p0) in enumerate(zip(ctx.row_ranges(), ctx.pos0)):
+                    L = p0 + n
+                    pages = kv.block_table.long()[b, :(L + PAGE - 1) // PAGE]
+                    K = kv.k_pages[pages, 0].reshape(-1, DK)[:L].float()
+                    V = kv.v_pages[pages, 0].reshape(-1, DV)[:L].float()
+                    sc = (q[r0:r0 + n] @ K.t()) * DK ** -0.5
+                    keys = torch.arange(L, device=h.device)[None, :]
+                    sc = sc.masked_fill(keys > (p0 + torch.arange(n, device=h.device))[:, None], float("-inf"))
+                    out[r0:r0 + n] = torch.softmax(sc, dim=-1) @ V
+                return (out @ self.w["wo"].t()).to(h.dtype)
+
+    @dataclass(frozen=True)
+    class WideConfig:
+        vocab_size: int
+        hidden_size: int
+        model_type: str = "toy_wide_values"
+
+        @staticmethod
+        def from_dict(raw):
+            return WideConfig(raw["vocab_size"], raw["hidden_size"])
+
+        def to_dict(self):
+            return asdict(self)
+
+    def build(c):
+        norm = PartSpec.of("rmsnorm", dim=c.hidden_size, eps=1e-5)
+        ffn = PartSpec.of("swiglu", hidden=c.hidden_size, intermediate=2 * c.hidden_size)
+        att = PartSpec.of("attention", hidden=c.hidden_size, n_heads=2, n_kv_heads=1, head_dim=DK,
+                          scale=DK ** -0.5, position=PartSpec.of("rope", head_dim=DK, theta=100.0))
+        layers = []
+        for i, mixer in enumerate((PartSpec.of("wide_values", hidden=c.hidden_size), att)):
+            blk = PartSpec.of("prenorm", mixer=mixer, ffn=ffn, mixer_norm=norm, ffn_norm=norm)
+            layers.append(LayerPlan(block=blk, names={n: f"layers.{i}.{n}" for n in BLOCKS.build(blk).tensors()}))
+        return ModelPlan(vocab_size=c.vocab_size, hidden_size=c.hidden_size, layers=layers,
+                         schedule=[ScheduleEntry(0), ScheduleEntry(1)], final_norm=norm, embedding_name="embed.weight",
+                         final_norm_names={"weight": "norm.weight"}, lm_head_name="head.weight")
+
+    if "toy_wide_values" not in _ARCHITECTURES:
+        register_architecture(Architecture("toy_wide_values", WideConfig, build))
+    folder = write_model_folder(str(tmp_path / "wide"), WideConfig(vocab_size=50, hidden_size=32), 21, torch.float32)
+    eng = Engine.from_folder(folder, dtype=torch.float32, max_tokens=512, use_graphs=False)
+    # two groups: the toy mixer's pages (values of 24 columns) and the attention's (keys and values of 8)
+    shapes = sorted((tuple(g.k.shape[2:]), tuple(g.v.shape[2:])) for g in eng.cache.groups)
+    assert shapes == [((1, PAGE, DK), (1, PAGE, DK)), ((1, PAGE, DK), (1, PAGE, DV))]
+
+    from safetensors.torch import load_file
+    W = load_file(os.path.join(folder, "model.safetensors"))
+
+    def plain(toks):
+        x = W["embed.weight"][toks]
+        n = len(toks)
+        pos = torch.arange(n)
+        for l in range(2):
+            p = f"layers.{l}."
+            xb = pl.rmsnorm(x, W[p + "mixer_norm.weight"], 1e-5)
+            if l == 0:
+                q, k, v = (pl.linear(xb, W[p + "mixer.w" + c]) for c in "qkv")
+                sc = (q @ k.t()) * DK ** -0.5
+                sc = sc.masked_fill(torch.arange(n)[None, :] > torch.arange(n)[:, None], float("-inf"))
+                o = pl.softmax(sc) @ v                                  # [n, DV]: one head, values of their own width
+            else:
+                inv = pl.rope_inv_freq(DK, 100.0)
+                q = pl.apply_rope(pl.linear(xb, W[p + "mixer.wq"]).view(n, 2, DK), pos, inv)
+                k = pl.apply_rope(pl.linear(xb, W[p + "mixer.wk"]).view(n, 1, DK), pos, inv)
+                o = pl.attention(q, k, pl.linear(xb, W[p + "mixer.wv"]).view(n, 1, DK), DK ** -0.5).reshape(n, 2 * DK)
+            x = x + pl.linear(o, W[p + "mixer.wo"])
+            xb = pl.rmsnorm(x, W[p + "ffn_norm.weight"], 1e-5)
+            x = x + pl.feed_forward(xb, W[p + "ffn.w_gate"], W[p + "ffn.w_up"], W[p + "ffn.w_down"])
+        return pl.linear(pl.rmsnorm(x, W["norm.weight"], 1e-5), W["head.weight"])
+
+    rnd = random.Random(22)
+    reqs = [[rnd.randrange(50) for _ in range(n)] for n in (70, 9, 131)]
+    for round_ in range(2):                                   # the second round runs in slots that were used before
+        slots = [eng.new_sequence() for _ in reqs]
+        fed = [len(r) - 3 for r in reqs]
+        out = eng.step([StepEntry(s, r[:f], list(range(f))) for s, r, f in zip(slots, reqs, fed)])
+        got, o = [[] for _ in reqs], 0
+        for i, f in enumerate(fed):
+            got[i].append(out[o:o + f])
+            o += f
+        for k in range(3):
+            out = eng.step([StepEntry(s, [r[f + k]], [0]) for s, r, f in zip(slots, reqs, fed)])
+            for i in range(3):
+                got[i].append(out[i:i + 1])
+        for i, r in enumerate(reqs):
+            assert rel_err(torch.cat(got[i]), plain(r)) < TOL[torch.float32], (round_, i)
+        for s in slots:
+            eng.release(s)
+        eng.cache.check()
+        reqs = reqs[::-1]
+
+
+@pytest.mark.parametrize("dtype,layout", [(torch.bfloat16, "rows"), (torch.float32, "transposed")])
+@pytest.mark.parametrize("hs", [64, 24])
+def test_the_attention_part_over_the_layout_that_is_not_its_kernels_own(dtype, layout, hs):
+    """An attention whose need names the other layout of the values (bfloat16 values lying like the keys, float32
+    values turned): the cache write and the vector kernel take either, the matrix-core kernels are not used, and the
+    result is the plain attention's."""
+    from bitnet_c_amd.cache import PAGE, PagedCache
+    from bitnet_c_amd.parts import MIXERS, CacheNeed, KVNeed, PartSpec
+    from bitnet_c_amd.parts.attention import Attention
+
+    class OtherLayout(Attention):
+        def cache_need(self):
+            return CacheNeed(kv=KVNeed(self.Hkv, self.hs, self.window, v_layout=layout))
+
+    H, Hkv, hidden, scale = 4, 2, 48, 0.2
+    att = OtherLayout(hidden, H, Hkv, hs, scale, PartSpec.of("rope", head_dim=hs, theta=5000.0))
+    t = {k: _rand(v.shape, 40 + i, 0.15).to(dtype) for i, (k, v) in enumerate(att.tensors().items())}
+    att.load(t, DEV, dtype)
+    cache = PagedCache([att.cache_need()], [None], 64 * 8, dtype=dtype, device=DEV)
+    assert cache.groups[0].v.shape[2:] == ((Hkv, hs, PAGE) if layout == "transposed" else (Hkv, PAGE, hs))
+    lens = [70, 5, 130]
+    hs_in = [_rand((n, hidden), 50 + i).to(dtype) for i, n in enumerate(lens)]
+    slots = [cache.alloc_slot() for _ in lens]
+    got = [[] for _ in lens]
+    fed = [n - 3 for n in lens]
+    ctx, tables, max_len = _ctx(cache, slots, fed, dtype)
+    out = att.forward(torch.cat([h[:f] for h, f in zip(hs_in, fed)]).to(DEV), ctx, cache.view(0, tables, max_len))
+    cache.commit(slots, fed)
+    o = 0
+    for i, f in enumerate(fed):
+        got[i].append(out[o:o + f])
+        o += f
+    for step in range(3):
+        ctx, tables, max_len = _ctx(cache, slots, [1] * 3, dtype)
+        out = att.forward(torch.cat([h[f + step:f + step + 1] for h, f in zip(hs_in, fed)]).to(DEV), ctx,
+                          cache.view(0, tables, max_len))
+        cache.commit(slots, [1] * 3)
+        for i in range(3):
+            got[i].append(out[i:i + 1])
+    rt = None if dtype == torch.float32 else dtype
+    r = (lambda x: x) if rt is None else (lambda x: x.to(rt).float())
+    inv = pl.rope_inv_freq(hs, 5000.0)
+    for i, n in enumerate(lens):
+        h = hs_in[i].float()
+        pos = torch.arange(n)
+
+        def whole(r):
+            q = r(pl.apply_rope(r(pl.linear(h, t["wq"].float())).view(n, H, hs), pos, inv))
+            k = r(pl.apply_rope(r(pl.linear(h, t["wk"].float())).view(n, Hkv, hs), pos, inv))
+            v = r(pl.linear(h, t["wv"].float())).view(n, Hkv, hs)
+            return r(pl.linear(r(pl.attention(q, k, v, scale).reshape(n, H * hs)), t["wo"].float()))
+        assert part_close(torch.cat(got[i]).float(), whole(r), dtype, whole(lambda x: x)), i
