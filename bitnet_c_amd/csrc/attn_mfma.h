@@ -25,7 +25,9 @@ extern "C" {
 // BN_ERR_SCRATCH and launches nothing.  Every call on a GPU shares that GPU's array: calls that
 // overlap on one GPU (two streams, two threads) race on it, so keep them on one stream.  Nothing in
 // the array has to start at zero (every partial that the merge reads is written first by the same
-// call), and the array keeps the last call's contents.
+// call), and the array keeps the last call's contents.  The first call on a GPU looks the array's
+// address up (hipGetSymbolAddress, under a lock), which is no stream operation: a caller that records
+// graphs makes one call outside any capture first; every later call only launches kernels.
 int bn_attn_mfma_decode_static(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
                                const void* vt_pages, const int* block_table, int bt_stride, const int* seq_lens,
                                int n_seqs, int H, int Hkv, int hs, int GT, int window, float scale, int n_splits,

@@ -70,6 +70,13 @@ struct MfmaArgs {
     // two workgroups on every CU, the ones that share a CU are then a long and a short sequence.
     const int* by_length;
     int order_period;
+    // row_ssq != null (decode form with rotate): q, the new key and the new value of row b are what a product made of
+    // an RMSNorm's input times the norm's weights, without the norm's factor (a deferred norm).  The factor
+    // 1/sqrt(sum of row_ssq[b][0..n_pieces) / ssq_width + eps) multiplies the whole row, so it is applied here: folded
+    // into the rotation's cosines and sines for q and the key, a multiplication for the value.
+    const float* row_ssq;
+    int n_pieces;
+    float inv_ssq_width, ssq_eps;
     // max_len != null (decode form, n_splits > 1): the longest sequence's key count lives in device memory and
     // the keys per split follow from it (bn_split_chunk) instead of from `chunk`: a captured launch then adapts
     // its splits to the lengths of every replay.
@@ -480,6 +487,7 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
     if (tile >= n_tiles) break;                           // an odd number of tiles: the last one has no partner
     const int* tl = a.tiles + 4 * tile;
     const int seq = tl[0], tok0 = tl[1], n_tok = tl[2], pos0 = tl[3];
+    if (n_tok <= 0) continue;                             // an empty tile (a list padded to a fixed length): the whole workgroup skips it
 
     bf16x8 q[NT][DC];
     int qpos[NT], lo[NT], head[NT], tok[NT];
@@ -705,6 +713,12 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
     }
     const int tid = threadIdx.x;
     const float freq = (a.rotate && tid < HALF) ? a.inv_freq[tid] : 0.f;
+    float row_scale = 1.0f;
+    if (a.row_ssq) {                                     // the same few floats in every thread, added in piece order
+        float ss = 0.f;
+        for (int p = 0; p < a.n_pieces; ++p) ss += a.row_ssq[(size_t)seq * a.n_pieces + p];
+        row_scale = 1.0f / sqrtf(ss * a.inv_ssq_width + a.ssq_eps);
+    }
     bf16 new_k0 = __float2bfloat16(0.f), new_k1 = new_k0, new_v = new_k0;
     if (a.write_kv) {
         if (tid < HALF) {
@@ -734,7 +748,7 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
         if (tid < HALF) {                                // HALF <= 64: one frequency a thread
             float sv, cv;
             sincosf((float)(L - 1) * freq, &sv, &cv);
-            cos_s[tid] = cv; sin_s[tid] = sv;
+            cos_s[tid] = cv * row_scale; sin_s[tid] = sv * row_scale;
         }
         __syncthreads();
     }
@@ -757,7 +771,7 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
             kdst[t + HALF] = __float2bfloat16(k1);
         } else if (t < HALF + HS) {
             const int d = t - HALF;
-            vdst[(size_t)d * BN_PAGE] = new_v;
+            vdst[(size_t)d * BN_PAGE] = a.row_ssq ? __float2bfloat16(__bfloat162float(new_v) * row_scale) : new_v;
         }
         // only this workgroup reads what it has just stored: a fence of workgroup scope is enough
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
@@ -881,13 +895,15 @@ extern "C" int bn_attn_mfma_supports(int hs) { return (hs == 64 || hs == 128) ? 
 // query tokens per tile of the prompt form, for GT heads per group
 extern "C" int bn_attn_mfma_prompt_tokens(int hs, int GT) { return (hs == 64 ? 256 : 128) / GT; }
 
-extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
+static int attn_mfma_launch(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
                             const void* vt_pages, const int* block_table, int bt_stride, const int* seq_lens,
                             const int* tiles, int n_tiles, int n_tokens, int H, int Hkv, int hs, int GT,
                             int window, float scale, int n_splits, int chunk, float* part_o, float* part_ml,
                             const float* inv_freq, int rotate, int write_kv, const int* by_length,
-                            const int* max_len, hipStream_t s) {
+                            const int* max_len, const float* row_ssq, int n_pieces, int ssq_width, float ssq_eps,
+                            hipStream_t s) {
     if (!bn_attn_mfma_supports(hs) || n_tiles <= 0 || n_tokens <= 0 || H <= 0 || Hkv <= 0 || H % Hkv) return BN_ERR_ARG;
+    if (row_ssq && (tiles || !rotate || n_pieces < 1 || n_pieces > 64 || ssq_width < 1)) return BN_ERR_ARG;   // decode form, rotating
     if (GT <= 0 || GT > 16 || (GT & (GT - 1)) || window < 0 || n_splits < 1 || n_splits > 64) return BN_ERR_ARG;
     if (n_splits > 1 && (!part_o || !part_ml || (!max_len && (chunk <= 0 || chunk % BN_PAGE)))) return BN_ERR_ARG;
     if (!tiles && !seq_lens) return BN_ERR_ARG;
@@ -907,6 +923,7 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
     a.H = H; a.Hkv = Hkv; a.GT = GT; a.window = window; a.scale = scale;
     a.n_splits = n_splits; a.chunk = n_splits > 1 ? chunk : 0x40000000;
     a.inv_freq = inv_freq; a.rotate = rotate; a.write_kv = write_kv;
+    a.row_ssq = row_ssq; a.n_pieces = n_pieces; a.inv_ssq_width = row_ssq ? 1.0f / (float)ssq_width : 0.f; a.ssq_eps = ssq_eps;
     a.max_len = n_splits > 1 ? max_len : nullptr;
     // the order matters only when the launch holds more workgroups than CUs and no sequence is split
     const int wgs_per_seq = Hkv * n_head_tiles;
@@ -956,6 +973,31 @@ extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stri
     hipLaunchKernelGGL(attn_mfma_combine_kernel, dim3(n_tokens * H), dim3(64), 0, s, (bf16*)out, out_stride, part_o,
                        part_ml, H, hs, n_splits);
     return bn_launch_status();
+}
+
+extern "C" int bn_attn_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
+                            const void* vt_pages, const int* block_table, int bt_stride, const int* seq_lens,
+                            const int* tiles, int n_tiles, int n_tokens, int H, int Hkv, int hs, int GT,
+                            int window, float scale, int n_splits, int chunk, float* part_o, float* part_ml,
+                            const float* inv_freq, int rotate, int write_kv, const int* by_length,
+                            const int* max_len, hipStream_t s) {
+    return attn_mfma_launch(q, q_stride, out, out_stride, k_pages, vt_pages, block_table, bt_stride, seq_lens, tiles, n_tiles,
+                            n_tokens, H, Hkv, hs, GT, window, scale, n_splits, chunk, part_o, part_ml, inv_freq, rotate,
+                            write_kv, by_length, max_len, nullptr, 0, 0, 0.f, s);
+}
+
+// The decode form (tiles none, rotate on) over rows whose RMSNorm was left undone: q, the new key and the new value of
+// row b still lack the factor 1/sqrt(sum of row_ssq[b][0..n_pieces) / ssq_width + eps), which is applied here.
+extern "C" int bn_attn_mfma_scaled(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
+                                   const void* vt_pages, const int* block_table, int bt_stride, const int* seq_lens,
+                                   int n_seqs, int H, int Hkv, int hs, int GT, int window, float scale, int n_splits,
+                                   int chunk, float* part_o, float* part_ml, const float* inv_freq, int write_kv,
+                                   const int* by_length, const int* max_len, const float* row_ssq, int n_pieces,
+                                   int ssq_width, float ssq_eps, hipStream_t s) {
+    if (!row_ssq) return BN_ERR_ARG;
+    return attn_mfma_launch(q, q_stride, out, out_stride, k_pages, vt_pages, block_table, bt_stride, seq_lens, nullptr, n_seqs,
+                            n_seqs, H, Hkv, hs, GT, window, scale, n_splits, chunk, part_o, part_ml, inv_freq, 1, write_kv,
+                            by_length, max_len, row_ssq, n_pieces, ssq_width, ssq_eps, s);
 }
 
 // ---------------------------------------------------------------------------------------

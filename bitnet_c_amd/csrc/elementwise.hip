@@ -164,6 +164,45 @@ __global__ __launch_bounds__(256) void sum_parts_kernel(float* __restrict__ x, c
     if (threadIdx.x == 0) ssq[(size_t)row * gridDim.x + blockIdx.x] = ss;
 }
 
+// The sum for a norm that its consumer applies itself: x += delta (n_parts float32 slabs in slab order, or one tensor of
+// type TD when n_parts is 1; none when delta is null), the bf16 copy of the new x times the next norm's weights, and the
+// piece's sum of squares to ssq[row][piece].  The consumer multiplies its result's rows by 1/sqrt(sum / dim + eps)
+// (src/transformer/rmsnorm_scalar.c:4-13: the factor is the same for a whole row, so it commutes with the product).
+template <typename TD>
+__global__ __launch_bounds__(256) void sum_deferred_kernel(float* __restrict__ x, const TD* __restrict__ delta, int n_parts,
+                                                           size_t part_stride, const float* __restrict__ w,
+                                                           bf16* __restrict__ scaled, float* __restrict__ ssq, int dim) {
+    __shared__ float scratch[16];
+    const int row = blockIdx.y, i = blockIdx.x * SP_PIECE + threadIdx.x * 4;
+    const bool in = i < dim;                                  // dim is a multiple of 4
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (in) {
+        float* xr = x + (size_t)row * dim + i;
+        v = *reinterpret_cast<const float4*>(xr);
+        if (delta) {
+            const TD* pr = delta + (size_t)row * dim + i;
+            if (sizeof(TD) == 4) {
+#pragma unroll 8
+                for (int p = 0; p < n_parts; ++p) {
+                    const float4 d = *reinterpret_cast<const float4*>(pr + (size_t)p * part_stride);
+                    v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+                }
+            } else {
+                const uint2 d = *reinterpret_cast<const uint2*>(pr);
+                v.x += bf16lo_to_f32(d.x); v.y += bf16hi_to_f32(d.x); v.z += bf16lo_to_f32(d.y); v.w += bf16hi_to_f32(d.y);
+            }
+            *reinterpret_cast<float4*>(xr) = v;
+        }
+        const float4 wv = *reinterpret_cast<const float4*>(w + i);
+        bf16 t[4] = {from_f32<bf16>(v.x * wv.x), from_f32<bf16>(v.y * wv.y), from_f32<bf16>(v.z * wv.z), from_f32<bf16>(v.w * wv.w)};
+        *reinterpret_cast<uint2*>(scaled + (size_t)row * dim + i) = *reinterpret_cast<const uint2*>(t);
+    }
+    float ss = 0.f;
+    ss += v.x * v.x; ss += v.y * v.y; ss += v.z * v.z; ss += v.w * v.w;
+    ss = block_sum(ss, scratch);
+    if (threadIdx.x == 0) ssq[(size_t)row * gridDim.x + blockIdx.x] = ss;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void rmsnorm_ssq_kernel(const float* __restrict__ x, const float* __restrict__ ssq,
                                                           int n_pieces, const float* __restrict__ w, T* __restrict__ out,
@@ -233,6 +272,32 @@ __global__ void swiglu_bf16x8_kernel(bf16* __restrict__ out, const bf16* __restr
         const float g0 = bf16lo_to_f32(gw[k]), g1 = bf16hi_to_f32(gw[k]);
         const float r0 = bn_gate_act(g0, act) * bf16lo_to_f32(uw[k]);
         const float r1 = bn_gate_act(g1, act) * bf16hi_to_f32(uw[k]);
+        const bf16 b0 = __float2bfloat16(r0), b1 = __float2bfloat16(r1);
+        ow[k] = (uint32_t)(*reinterpret_cast<const uint16_t*>(&b0)) | ((uint32_t)(*reinterpret_cast<const uint16_t*>(&b1)) << 16);
+    }
+    *reinterpret_cast<uint4*>(out + t * F + f) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
+// The gated unit behind a product whose norm was deferred: gate and up (interleaved in blocks of 8 columns) are both
+// multiplied by the row's 1/sqrt(sum of the ssq pieces / width + eps) first, in float32, then act(gate) * up.
+__global__ void swiglu_scaled_bf16x8_kernel(bf16* __restrict__ out, const bf16* __restrict__ gu, int F, size_t n8, int il8,
+                                            int act, const float* __restrict__ ssq, int n_pieces, float inv_width, float eps) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n8) return;
+    const int f8 = F / 8;
+    const size_t t = i / f8;
+    const int f = (int)(i - t * f8) * 8;
+    float ss = 0.f;
+    for (int p = 0; p < n_pieces; ++p) ss += ssq[t * n_pieces + p];          // in piece order: the same in every thread
+    const float sc = 1.0f / sqrtf(ss * inv_width + eps);
+    const uint4 g = *reinterpret_cast<const uint4*>(gu + t * 2 * F + (il8 ? 2 * f : f));
+    const uint4 u = *reinterpret_cast<const uint4*>(gu + t * 2 * F + (il8 ? 2 * f + 8 : F + f));
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float r0 = bn_gate_act(bf16lo_to_f32(gw[k]) * sc, act) * (bf16lo_to_f32(uw[k]) * sc);
+        const float r1 = bn_gate_act(bf16hi_to_f32(gw[k]) * sc, act) * (bf16hi_to_f32(uw[k]) * sc);
         const bf16 b0 = __float2bfloat16(r0), b1 = __float2bfloat16(r1);
         ow[k] = (uint32_t)(*reinterpret_cast<const uint16_t*>(&b0)) | ((uint32_t)(*reinterpret_cast<const uint16_t*>(&b1)) << 16);
     }
@@ -328,6 +393,39 @@ extern "C" int bn_add_rmsnorm_parts_wide(int dtype, void* x, const float* parts,
         hipLaunchKernelGGL(rmsnorm_ssq_kernel<float>, dim3(total_rows), dim3(256), 0, s, (const float*)x, ssq, pieces, w, (float*)out, dim, eps);
     else
         hipLaunchKernelGGL(rmsnorm_ssq_kernel<bf16>, dim3(total_rows), dim3(256), 0, s, (const float*)x, ssq, pieces, w, (bf16*)out, dim, eps);
+    return bn_launch_status();
+}
+
+// x[total_rows, dim] (float32) += delta, scaled [total_rows, dim] (bf16) = the new x times w, ssq [total_rows, pieces] the
+// sums of squares of the pieces of bn_add_rmsnorm_parts_pieces(dim).  delta: null, or n_parts float32 slabs
+// [n_parts][total_rows][dim] (delta_dtype float32), or one bf16 tensor (delta_dtype bf16, n_parts 1).
+extern "C" int bn_sum_deferred(int delta_dtype, void* x, const void* delta, int n_parts, int total_rows, const float* w,
+                               void* scaled, float* ssq, int dim, hipStream_t s) {
+    if (dim <= 0 || dim % 4 || total_rows < 1 || total_rows > 65535 || !x || !w || !scaled || !ssq) return BN_ERR_ARG;
+    if (delta && (n_parts < 1 || (delta_dtype == BN_DT_BF16 && n_parts != 1))) return BN_ERR_ARG;
+    if (((uintptr_t)x | (uintptr_t)delta | (uintptr_t)w | (uintptr_t)scaled) & 15) return BN_ERR_ARG;
+    const dim3 grid(bn_add_rmsnorm_parts_pieces(dim), total_rows);
+    const size_t stride = (size_t)total_rows * dim;
+    if (delta_dtype == BN_DT_F32)
+        hipLaunchKernelGGL(sum_deferred_kernel<float>, grid, dim3(256), 0, s, (float*)x, (const float*)delta, n_parts, stride, w,
+                           (bf16*)scaled, ssq, dim);
+    else if (delta_dtype == BN_DT_BF16)
+        hipLaunchKernelGGL(sum_deferred_kernel<bf16>, grid, dim3(256), 0, s, (float*)x, (const bf16*)delta, n_parts, stride, w,
+                           (bf16*)scaled, ssq, dim);
+    else
+        return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+// bn_swiglu for bf16 with gate and up interleaved in blocks of 8, both multiplied first by the rows' deferred norm factors
+// 1/sqrt(sum of ssq[row][0..n_pieces) / width + eps).
+extern "C" int bn_swiglu_scaled(void* out, const void* gu, int n_rows, int F, int act, const float* ssq, int n_pieces,
+                                int width, float eps, hipStream_t s) {
+    if (n_rows <= 0 || F <= 0 || F % 8 || act < 0 || act >= BN_ACT_KINDS || !ssq || n_pieces < 1 || width < 1) return BN_ERR_ARG;
+    if (((uintptr_t)out | (uintptr_t)gu) & 15) return BN_ERR_ARG;
+    const size_t n8 = (size_t)n_rows * F / 8;
+    hipLaunchKernelGGL(swiglu_scaled_bf16x8_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, s, (bf16*)out,
+                       (const bf16*)gu, F, n8, 1, act, ssq, n_pieces, 1.0f / (float)width, eps);
     return bn_launch_status();
 }
 

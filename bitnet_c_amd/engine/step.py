@@ -73,8 +73,10 @@ class StepContext:
 
     def page_tiles(self) -> torch.Tensor:
         """[n, 4] int32: the new tokens cut at page boundaries (sequence, first row, rows, position of
-        the first), for kernels that store a page's positions together."""
+        the first), for kernels that store a page's positions together.  A list may end in tiles of no rows."""
         if self._page_tiles is None:
+            if self.captured:
+                raise StepError("this captured step was recorded without a list of page tiles")
             self._page_tiles = torch.tensor(_page_tiles(self.n_new, self.pos0),
                                             dtype=torch.int32).reshape(-1, 4).to(self.device)
         return self._page_tiles
@@ -82,15 +84,12 @@ class StepContext:
     def tiles(self, qt: int) -> torch.Tensor:
         """[n, 4] int32: (sequence, first row, rows <= qt, position of the first) covering all new
         tokens, for the prompt form of the attention kernel, in the order that gives its workgroups
-        equal work (ops.pair_tiles)."""
+        equal work (ops.pair_tiles).  A list may end in tiles of no rows."""
         t = self._tiles.get(qt)
         if t is None:
-            rows, r = [], 0
-            for s, (n, p0) in enumerate(zip(self.n_new, self.pos0)):
-                for i in range(0, n, qt):
-                    rows.append((s, r + i, min(qt, n - i), p0 + i))
-                r += n
-            t = torch.tensor(ops.pair_tiles(rows), dtype=torch.int32).reshape(-1, 4).to(self.device)
+            if self.captured:
+                raise StepError(f"this captured step was recorded without a list of tiles of {qt} tokens")
+            t = torch.tensor(_query_tiles(self.n_new, self.pos0, qt), dtype=torch.int32).reshape(-1, 4).to(self.device)
             self._tiles[qt] = t
         return t
 
@@ -109,12 +108,23 @@ def _page_tiles(n_new, pos0) -> List[tuple]:
     return rows
 
 
+def _query_tiles(n_new, pos0, qt: int) -> List[tuple]:
+    """(sequence, first row, rows <= qt, position of the first) covering every sequence's new tokens, in the order
+    in which the prompt form of attention wants them (ops.pair_tiles)."""
+    rows, r = [], 0
+    for s, (n, p0) in enumerate(zip(n_new, pos0)):
+        for i in range(0, n, qt):
+            rows.append((s, r + i, min(qt, n - i), p0 + i))
+        r += n
+    return ops.pair_tiles(rows)
+
+
 def _by_length(lens) -> List[int]:
     """The rows ordered by length, longest first (ties by row)."""
     return sorted(range(len(lens)), key=lambda i: (-lens[i], i))
 
 
-MAX_GRAPH_ROWS = 64       # decode steps of more sequences than this run eagerly
+MAX_GRAPH_ROWS = 256      # rows of the largest captured decode step; a step of more sequences is replayed in pieces of this size
 
 
 def _bucket(n: int) -> int:
@@ -212,6 +222,124 @@ class _DecodeGraph:
         return self.logits
 
 
+MAX_PROMPT_GRAPH_ROWS = 8192      # prompt steps of more tokens than this run eagerly: their launches are a small part of them
+MAX_PROMPT_GRAPHS = 12            # captured prompt steps that an engine keeps; the one unused for longest goes first
+
+
+def _row_bucket(n: int) -> int:
+    """Token rows of the captured step that serves a prompt step of n tokens: the padding is at most an eighth."""
+    unit = 64 if n <= 512 else 128 if n <= 2048 else 512
+    return -(-n // unit) * unit
+
+
+class _PromptGraph:
+    """A captured prompt step (or a mixed one: some sequences with many tokens, some with one) for up to `rows`
+    tokens of up to `seqs` sequences with up to `wants` wanted places.  Everything that differs between the steps it
+    serves is device memory that is filled before a replay: tokens, positions (-1 for the padding rows, which write
+    nothing), the sequence of every row, lengths, wanted rows, slot ids, the block tables at the engine's full
+    width, and the tile lists of the attention kernels and of the cache write, padded with tiles of no rows.  So a
+    prompt step costs the host one copy and one launch instead of some hundred launches (the reference runs its
+    batched prompt pass from one call as well, src/transformer/prefill.c:1228-1962)."""
+
+    def __init__(self, engine: "Engine", rows: int, seqs: int, wants: int, qts: Sequence[int], page_tiles: bool):
+        self.rows, self.seqs, self.wants, self.width = rows, seqs, wants, engine.max_pages
+        dev, cache = engine.device, engine.cache
+        n_groups = len(cache.groups)
+        self.n_tiles = {qt: -(-rows // qt) + seqs for qt in qts}         # every sequence may end in a tile that is not full
+        self.n_page_tiles = -(-rows // PAGE) + 2 * seqs if page_tiles else 0
+        sizes = [rows, rows, rows, seqs, wants, seqs] + [4 * self.n_tiles[qt] for qt in qts] + [4 * self.n_page_tiles]
+        self.offsets = [0]
+        for n in sizes:
+            self.offsets.append(self.offsets[-1] + n)
+        self.host = torch.zeros(max(self.offsets[-1], 1), dtype=torch.int32).pin_memory()
+        self.host_np = self.host.numpy()
+        self.dev = torch.zeros(self.host.numel(), dtype=torch.int32, device=dev)
+        f = [self.dev[a:b] for a, b in zip(self.offsets[:-1], self.offsets[1:])]
+        self.tokens, self.positions, self.seq_index, self.seq_lens, self.want, self.slot_ids = f[:6]
+        self.host_tables = torch.zeros((max(n_groups, 1), seqs, self.width), dtype=torch.int32).pin_memory()
+        self.tables_np = self.host_tables.numpy()
+        self.dev_tables = torch.zeros(self.host_tables.shape, dtype=torch.int32, device=dev)
+        self.row_keys = [None] * seqs
+        self.tables_dirty = True
+        self.copied = torch.cuda.Event()
+        self.copied.record()
+        self.tables = {g: self.dev_tables[g] for g in range(n_groups)}
+        views = [cache.view(i, self.tables, self.width * PAGE) for i in range(len(engine.model.plan.schedule))]
+        self.ctx = StepContext(dev, engine.model.dtype, self.tokens, self.positions, self.seq_index, self.seq_lens,
+                               self.want, self.slot_ids, False, [-1] * seqs, [0] * seqs, [0] * seqs, captured=True)
+        self.qts = tuple(qts)
+        for k, qt in enumerate(self.qts):
+            self.ctx._tiles[qt] = f[6 + k].view(-1, 4)
+        if page_tiles:
+            self.ctx._page_tiles = f[6 + len(self.qts)].view(-1, 4)
+        self.fill([], [], [], [], [], engine)                  # padding everywhere: the two runs below touch no sequence
+        self.upload()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            engine.model.forward(self.ctx, views)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, pool=engine.graph_pool):
+            self.logits = engine.model.forward(self.ctx, views)
+
+    def fill(self, slots, tokens, n_new, pos0, want, engine):
+        """tokens: the flattened new tokens; want: rows of the flattened batch."""
+        h, o, cache = self.host_np, self.offsets, engine.cache
+        self.copied.synchronize()
+        T, B = len(tokens), len(slots)
+        h[o[0]:o[1]] = 0
+        h[o[0]:o[0] + T] = tokens
+        h[o[1]:o[2]] = -1
+        h[o[2]:o[3]] = 0
+        r = 0
+        for b, (n, p0) in enumerate(zip(n_new, pos0)):
+            h[o[1] + r:o[1] + r + n] = range(p0, p0 + n)
+            h[o[2] + r:o[2] + r + n] = b
+            r += n
+        h[o[3]:o[4]] = 0
+        h[o[3]:o[3] + B] = [p + n for p, n in zip(pos0, n_new)]
+        h[o[4]:o[5]] = 0
+        h[o[4]:o[4] + len(want)] = want
+        h[o[5]:o[6]] = cache.padding_slot
+        h[o[5]:o[5] + B] = slots
+        for k, qt in enumerate(self.qts):
+            flat = [v for t in _query_tiles(n_new, pos0, qt) for v in t]
+            h[o[6 + k]:o[7 + k]] = 0
+            h[o[6 + k]:o[6 + k] + len(flat)] = flat
+        if self.n_page_tiles:
+            k = 6 + len(self.qts)
+            flat = [v for t in _page_tiles(n_new, pos0) for v in t]
+            h[o[k]:o[k + 1]] = 0
+            h[o[k]:o[k] + len(flat)] = flat
+        for r, s in enumerate(slots):
+            key = (s, cache.slot_version(s))
+            if key != self.row_keys[r]:
+                for g in range(len(cache.groups)):
+                    pl = cache.pages_of(g, s)
+                    self.tables_np[g, r, :len(pl)] = [max(p, 0) for p in pl]
+                    self.tables_np[g, r, len(pl):] = 0
+                self.row_keys[r] = key
+                self.tables_dirty = True
+        for r in range(B, self.seqs):
+            if self.row_keys[r] is not None:
+                self.tables_np[:, r, :] = 0
+                self.row_keys[r] = None
+                self.tables_dirty = True
+
+    def upload(self):
+        self.dev.copy_(self.host, non_blocking=True)
+        if self.tables_dirty:
+            self.dev_tables.copy_(self.host_tables, non_blocking=True)
+            self.tables_dirty = False
+        self.copied.record()
+
+    def run(self):
+        self.graph.replay()
+        return self.logits
+
+
 class Engine:
     """A model, its cache and the step function over both."""
 
@@ -233,11 +361,20 @@ class Engine:
         # host's slot list cannot, and a model with such a mixer runs its decode steps eagerly.
         self.use_graphs = use_graphs and all(n.state is None or n.state.device_addressed for n in needs)
         self.tap = None                     # see StepContext.tap; while it is set, steps run without graphs
-        # One captured step per number of rows (1, 2, 4 .. MAX_GRAPH_ROWS): at most seven, made at a batch's
+        # One captured step per number of rows (1, 2, 4 .. MAX_GRAPH_ROWS): at most nine, made at a batch's
         # start (prepare_decode) or at first use.  They share one memory pool: what a capture frees, the next
         # reuses, and each keeps only its own inputs and logits ([rows, vocab] float32).
         self._graphs: Dict[int, _DecodeGraph] = {}
         self.graph_pool = torch.cuda.graph_pool_handle() if self.use_graphs else None
+        # Prompt steps are captured too, per (token rows, sequences, wanted places) rounded up to buckets: the first
+        # step of a bucket runs eagerly (and shows which tile lists the model's parts ask for), the second is recorded,
+        # every later one is a replay.  Only when every part of the model says that its prompt work can be recorded
+        # (Part.prompt_capturable); prompt_graphs False keeps prompt steps eager.
+        self.prompt_graphs = (all(getattr(b, "prompt_capturable", False) for b in model.blocks)
+                              and getattr(model.final_norm, "prompt_capturable", False))
+        self._prompt_graphs: Dict[tuple, _PromptGraph] = {}     # in order of last use
+        self._prompt_seen: Dict[tuple, int] = {}
+        self._prompt_lists = None                                # (tile sizes asked for, page tiles asked for) of an eager prompt step
         self.graphs_built = 0
         self.steps_run = 0
 
@@ -329,9 +466,16 @@ class Engine:
         except CacheFull as err:
             raise StepError(str(err)) from None
         is_decode = all(n == 1 for n in n_new)
+        graphs = self.use_graphs and self.tap is None
         try:
-            if is_decode and self.use_graphs and self.tap is None and len(entries) <= MAX_GRAPH_ROWS:
-                logits = self._step_graph(entries, slots, pos0)
+            if is_decode and graphs:
+                # the sequences of a decode step do not depend on each other: more of them than the largest captured
+                # step holds are replayed in pieces
+                pieces = [self._step_graph(entries[i:i + MAX_GRAPH_ROWS], slots[i:i + MAX_GRAPH_ROWS], pos0[i:i + MAX_GRAPH_ROWS])
+                          for i in range(0, len(entries), MAX_GRAPH_ROWS)]
+                logits = pieces[0] if len(pieces) == 1 else torch.cat(pieces)
+            elif not is_decode and graphs and self.prompt_graphs and self._prompt_bucket_ready(entries, n_new):
+                logits = self._step_prompt_graph(entries, slots, n_new, pos0)
             else:
                 logits = self._step_eager(entries, slots, n_new, pos0, is_decode)
         except BaseException:
@@ -376,7 +520,60 @@ class Engine:
         ctx.tap = self.tap
         max_len = max(lens_after)
         views = [self.cache.view(i, d_tables, max_len) for i in range(len(self.model.plan.schedule))]
-        return self.model.forward(ctx, views)
+        logits = self.model.forward(ctx, views)
+        if not is_decode:
+            self._prompt_lists = (tuple(sorted(ctx._tiles)), ctx._page_tiles is not None)
+        return logits
+
+    # ---- captured prompt steps ----------------------------------------------------------
+    @staticmethod
+    def _prompt_key(entries, n_new):
+        wants = sum(len(e.want) for e in entries)
+        return _row_bucket(sum(n_new)), _bucket(len(entries)), _bucket(wants) if wants else 0
+
+    def _prompt_bucket_ready(self, entries, n_new) -> bool:
+        """Whether this prompt step is replayed from a graph: its bucket has been seen before (the first step of a
+        bucket runs eagerly: one-off prompts never pay for a capture)."""
+        if sum(n_new) > MAX_PROMPT_GRAPH_ROWS:
+            return False
+        key = self._prompt_key(entries, n_new)
+        if key in self._prompt_graphs:
+            return True
+        seen = self._prompt_seen.get(key, 0)
+        self._prompt_seen[key] = seen + 1
+        return seen >= 1 and self._prompt_lists is not None
+
+    def prepare_prompt(self, n_tokens: int, n_seqs: int = 1, n_wanted: int = 1) -> None:
+        """Captures, now, the graph that prompt steps of this size replay (a server does it for the sizes it
+        expects, a benchmark before its clock starts).  Needs one eager prompt step to have run before."""
+        if not (self.use_graphs and self.prompt_graphs and self.tap is None) or n_tokens > MAX_PROMPT_GRAPH_ROWS:
+            return
+        if self._prompt_lists is None:
+            raise StepError("prepare_prompt: run one prompt step first (it shows which tile lists the model's parts use)")
+        self._prompt_graph_for((_row_bucket(n_tokens), _bucket(n_seqs), _bucket(n_wanted) if n_wanted else 0))
+
+    def _prompt_graph_for(self, key) -> _PromptGraph:
+        g = self._prompt_graphs.pop(key, None)
+        if g is None:
+            while len(self._prompt_graphs) >= MAX_PROMPT_GRAPHS:
+                self._prompt_graphs.pop(next(iter(self._prompt_graphs)))        # the one unused for longest
+            qts, page_tiles = self._prompt_lists
+            g = _PromptGraph(self, key[0], key[1], key[2], qts, page_tiles)
+            self.graphs_built += 1
+        self._prompt_graphs[key] = g                                            # most recently used last
+        return g
+
+    def _step_prompt_graph(self, entries, slots, n_new, pos0):
+        g = self._prompt_graph_for(self._prompt_key(entries, n_new))
+        tokens = [int(t) for e in entries for t in e.tokens]
+        want, row = [], 0
+        for e, n in zip(entries, n_new):
+            want += [row + int(w) for w in e.want]
+            row += n
+        g.fill(slots, tokens, n_new, pos0, want, self)
+        g.upload()
+        logits = g.run()
+        return logits[:len(want)].clone()
 
     def prepare_decode(self, n_seqs: int) -> None:
         """Captures, now, every graph that decode steps of up to n_seqs sequences will replay (the batch

@@ -39,6 +39,8 @@ _SIGNATURES = {
         "bn_add_rmsnorm_parts_wide": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_float,
                                       c_void_p],
         "bn_swiglu": [c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "bn_sum_deferred": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
+        "bn_swiglu_scaled": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_float, c_void_p],
         "bn_bias_add": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
     },
     "rope_kv": {
@@ -56,6 +58,9 @@ _SIGNATURES = {
     "attn_mfma": {
         "bn_attn_mfma_supports": [c_int],
         "bn_attn_mfma_prompt_tokens": [c_int, c_int],
+        "bn_attn_mfma_scaled": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
+                                c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p],
         "bn_attn_mfma": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p,
                          c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p],
@@ -468,7 +473,8 @@ SPLIT_SUMS = os.environ.get("BITNET_NO_SPLIT_SUMS", "") in ("", "0")
 # to 8,192) with the kernels of the next norm included: there it is 15 to 45 % faster than the library's product (8B:
 # 36 us against 45 at 64 rows, 44 against 80 at 128; 70B: 119 against 148, 141 against 210), while below 64 rows and for
 # square matrices the two are within 10 % of each other with the sign depending on the shape.
-SPLIT_SUM_ROWS = (64, 128)
+SPLIT_SUM_ROWS = (17, 128)
+SPLIT_SUM_SQUARE_WIDTH = 6144     # square products (an output projection) up to this width as well: see can_split_sums
 
 
 @dataclass
@@ -488,8 +494,9 @@ class PartialSums:
 
 def can_split_sums(M: int, N: int, K: int, dtype) -> bool:
     """Whether a product of these sizes whose result goes to the residual stream is done as partial sums."""
-    return (SPLIT_SUMS and dtype == torch.bfloat16 and SPLIT_SUM_ROWS[0] <= M <= SPLIT_SUM_ROWS[1] and K % 8 == 0
-            and K >= 2 * N and N >= 1)
+    if not (SPLIT_SUMS and dtype == torch.bfloat16 and SPLIT_SUM_ROWS[0] <= M <= SPLIT_SUM_ROWS[1] and K % 8 == 0 and N >= 1):
+        return False
+    return K >= 2 * N or (K >= N and N <= SPLIT_SUM_SQUARE_WIDTH)
 
 
 def linear_partial_sums(x: torch.Tensor, w: torch.Tensor) -> PartialSums:
@@ -546,6 +553,59 @@ class DeferredNorm:
         return add_rmsnorm(self.stream, None, self.weight, self.eps, out_dtype or self.scaled.dtype, rows)
 
 
+DEFER_ROWS = (17, 128)    # row counts at which a norm is left to its consumer through sum_deferred (below: the fused products)
+
+
+def can_sum_deferred(M: int, D: int, dtype) -> bool:
+    """Whether the residual stream of M rows of D columns leaves the norm of a consumer that asks for it undone
+    (sum_deferred) instead of norming the rows itself."""
+    return FUSE_NORMS and dtype == torch.bfloat16 and DEFER_ROWS[0] <= M <= DEFER_ROWS[1] and D % 8 == 0 and D >= 8
+
+
+def sum_deferred(x: torch.Tensor, delta, weight: torch.Tensor, eps: float) -> DeferredNorm:
+    """x (float32 [M, D], in place) += delta (a bf16 or float32 tensor, PartialSums, or None), and what the next norm
+    (weights `weight`, `eps`) needs of the new x for a consumer that applies it itself: the bf16 copy times the weights
+    and the rows' sums of squares in pieces of 1,024 columns.  One kernel over the whole chip."""
+    require_gpu()
+    _dev(x, "x", torch.float32, 2)
+    _dev(weight, "weight", torch.float32, 1)
+    M, D = x.shape
+    if not x.is_contiguous() or weight.numel() != D or not weight.is_contiguous() or D % 4 or M < 1 or M > 65535:
+        raise KernelError(f"sum_deferred: x {tuple(x.shape)} must be contiguous with a width that is a multiple of 4, "
+                          f"weight have {D} elements")
+    n_parts, dptr, ddt = 0, None, 0
+    if isinstance(delta, PartialSums):
+        if tuple(delta.shape) != (M, D) or not delta.slabs.is_contiguous():
+            raise KernelError(f"sum_deferred: partial sums {tuple(delta.shape)} do not match x {tuple(x.shape)}")
+        n_parts, dptr, ddt = delta.slabs.shape[0], delta.slabs.data_ptr(), _DT[torch.float32]
+    elif delta is not None:
+        _dev(delta, "delta", dims=2)
+        if tuple(delta.shape) != (M, D) or not delta.is_contiguous() or delta.dtype not in _DT:
+            raise KernelError(f"sum_deferred: delta {tuple(delta.shape)} ({delta.dtype}) does not match x {tuple(x.shape)}")
+        n_parts, dptr, ddt = 1, delta.data_ptr(), _DT[delta.dtype]
+    scaled = torch.empty((M, D), dtype=torch.bfloat16, device=x.device)
+    slots = torch.empty((M, _fn("elementwise", "bn_add_rmsnorm_parts_pieces")(D)), dtype=torch.float32, device=x.device)
+    _check(_fn("elementwise", "bn_sum_deferred")(ddt, x.data_ptr(), dptr, n_parts, M, weight.data_ptr(), scaled.data_ptr(),
+                                                 slots.data_ptr(), D, _stream()), "sum_deferred")
+    return DeferredNorm(scaled, slots, x, weight, float(eps))
+
+
+def swiglu_scaled(gu: torch.Tensor, pre: DeferredNorm, activation: str = "silu") -> torch.Tensor:
+    """act(s * gate) * (s * up) for gu = [T, 2F] (bf16, gate and up interleaved in blocks of 8) that is the product of a
+    deferred norm's copy with the gate and up weights; s the rows' 1/sqrt(mean + eps)."""
+    require_gpu()
+    _dev(gu, "gu", torch.bfloat16, 2)
+    T, F = gu.shape[0], gu.shape[1] // 2
+    if not gu.is_contiguous() or gu.shape[1] % 16 or pre.slots.shape[0] != T or not pre.slots.is_contiguous():
+        raise KernelError(f"swiglu_scaled: gu {tuple(gu.shape)} / slots {tuple(pre.slots.shape)} do not fit")
+    out = torch.empty((T, F), dtype=gu.dtype, device=gu.device)
+    if T:
+        _check(_fn("elementwise", "bn_swiglu_scaled")(out.data_ptr(), gu.data_ptr(), T, F, _act(activation), pre.slots.data_ptr(),
+                                                      pre.slots.shape[1], pre.stream.shape[1], float(pre.eps), _stream()),
+               "swiglu_scaled")
+    return out
+
+
 def can_fuse_norm(M: int, N: int, K: int, dtype) -> bool:
     """Whether a product of these sizes can take a norm into its kernel (either side of it)."""
     return (dtype == torch.bfloat16 and 1 <= M <= FUSED_ROWS and K % 8 == 0 and N >= 1
@@ -595,6 +655,10 @@ def linear_swiglu_prenorm(pre: DeferredNorm, w_gate_up: torch.Tensor, activation
     _dev(w_gate_up, "w_gate_up", torch.bfloat16, 2)
     F, K = w_gate_up.shape[0] // 2, w_gate_up.shape[1]
     M = _check_deferred(pre, K)
+    if M > FUSED_ROWS and w_gate_up.shape[0] % 16 == 0 and LIBRARY_PRODUCTS:
+        # more rows than the fused kernel takes: the library's product of the copy, and the norm's factor in the
+        # kernel of the gated unit, which runs anyway
+        return swiglu_scaled(torch.matmul(pre.scaled, w_gate_up.t()), pre, activation)
     if w_gate_up.shape[0] % 16 or not can_fuse_norm(M, F, K, torch.bfloat16) or w_gate_up.data_ptr() % 16:
         raise KernelError(f"linear_swiglu_prenorm: {M} rows, w {tuple(w_gate_up.shape)} cannot be fused")
     y = torch.empty((M, F), dtype=torch.bfloat16, device=w_gate_up.device)
@@ -694,7 +758,8 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
         bt_stride = block_table.shape[1]
     if T == 0:
         return
-    tiled_v = (page_tiles is not None and k_pages is not None and vt and hs % 8 == 0 and stride % 8 == 0
+    tiled_v = (page_tiles is not None and k_pages is not None and vt and qkv.dtype == torch.bfloat16     # a bf16 kernel
+               and hs % 8 == 0 and stride % 8 == 0
                and qkv.data_ptr() % 16 == 0 and hs * (PAGE + 2) * 2 <= 65536 and Hkv <= 65535)
     if tiled_v:
         _dev(page_tiles, "page_tiles", torch.int32, 2)
@@ -771,6 +836,10 @@ def pair_tiles(rows: list) -> list:
     return out
 
 
+# Workgroups that a decode attention launch aims for when it cuts the keys (two for every CU of this chip).
+DECODE_TARGET_WGS = int(os.environ.get("BITNET_DECODE_WGS", "512"))
+
+
 def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int, dtype=None):
     """(n_splits, chunk): how the keys of a decode step are cut so that the launch fills the
     chip.  A function of the batch's shape and of max_len alone.  A float32 cache is never split:
@@ -784,7 +853,7 @@ def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int, dtype=None):
     pages = max(1, (max_len + PAGE - 1) // PAGE)
     # about 512 workgroups, but no split shorter than SPLIT_MIN_PAGES pages: below that the merging costs
     # more than the parallelism gains (measured at batch 1, 8 and 64 of the 8B shape)
-    want = max(1, min(pages // SPLIT_MIN_PAGES, 64, (512 + wgs - 1) // wgs))
+    want = max(1, min(pages // SPLIT_MIN_PAGES, 64, (DECODE_TARGET_WGS + wgs - 1) // wgs))
     chunk = ((pages + want - 1) // want) * PAGE
     n_splits = (pages * PAGE + chunk - 1) // chunk
     return n_splits, chunk
@@ -806,7 +875,7 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
               block_table: torch.Tensor, H: int, Hkv: int, hs: int, scale: float, *, window: int = 0,
               tiles=None, qt: int = 0, seq_lens=None, n_splits: int = 1, chunk: int = 0,
               force_vector: bool = False, fused_rotate=None, fused_write: bool = False, by_length=None,
-              max_len_dev=None, v_transposed=None) -> None:
+              max_len_dev=None, v_transposed=None, row_scale: Optional["DeferredNorm"] = None) -> None:
     """Causal attention of the (rotated) Q heads in qkv over the paged cache.
 
     Prompt form: `tiles` [n, 4] int32 = (sequence, first token row, tokens (<= qt), position of
@@ -826,7 +895,10 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     n_splits > 1 the kernels then cut the keys into n_splits runs of split_chunk(max_len, n_splits) and
     `chunk` is not used, so that one captured launch serves every length up to the block table's width.
     v_transposed: the layout of v_pages (None: kernel_v_layout of qkv's type); values that lie like the keys go to
-    the vector kernel whatever their type."""
+    the vector kernel whatever their type.
+    row_scale (decode form on the matrix cores with fused_rotate): a DeferredNorm whose factor the rows of qkv still
+    lack (qkv is the product of its bf16 copy with the stacked weights); the kernel multiplies q and the new key and
+    value of every row by it."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(out, "out", qkv.dtype, 2)
@@ -889,6 +961,21 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
             raise KernelError(f"attention: fused rotation needs {hs // 2} frequencies (full rotary)")
     if fused_write and qkv.shape[1] < (H + 2 * Hkv) * hs:
         raise KernelError("attention: fused cache write needs the K and V heads in qkv")
+    if row_scale is not None:
+        if not (use_mfma and decode and fused_rotate is not None):
+            raise KernelError("attention: a deferred norm's factor is applied by the decode form on the matrix cores "
+                              "with the rotation inside the kernel, and by nothing else")
+        _dev(row_scale.slots, "row_scale.slots", torch.float32, 2)
+        if row_scale.slots.shape[0] != T or not row_scale.slots.is_contiguous() or not 1 <= row_scale.slots.shape[1] <= 64:
+            raise KernelError(f"attention: row_scale slots {tuple(row_scale.slots.shape)} do not fit {T} rows (1 to 64 pieces)")
+        _check(_fn("attn_mfma", "bn_attn_mfma_scaled")(
+            qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * hs, k_pages.data_ptr(), v_pages.data_ptr(),
+            block_table.data_ptr(), block_table.shape[1], sl, T, H, Hkv, hs, GT, int(window), float(scale), int(n_splits),
+            int(chunk), po, pm, fused_rotate.data_ptr(), int(bool(fused_write)),
+            by_length.data_ptr() if by_length is not None else None,
+            max_len_dev.data_ptr() if max_len_dev is not None else None, row_scale.slots.data_ptr(),
+            row_scale.slots.shape[1], row_scale.stream.shape[1], float(row_scale.eps), _stream()), "attention(mfma, scaled)")
+        return
     if use_mfma:
         _check(_fn("attn_mfma", "bn_attn_mfma")(
             qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * hs, k_pages.data_ptr(), v_pages.data_ptr(),

@@ -22,6 +22,10 @@ from .linear import Linear, upload
 
 @MIXERS.register("attention")
 class Attention(Part):
+    @property
+    def prompt_capturable(self) -> bool:      # a prompt step is read from the context's device tensors alone
+        return getattr(self.position, "prompt_capturable", False)
+
     takes_deferred_norm = True      # forward accepts an ops.DeferredNorm for h
     gives_lazy_delta = True         # forward(..., lazy_ok=True) may return a LazyDelta
 
@@ -69,6 +73,19 @@ class Attention(Part):
     def forward(self, h, ctx, kv, lazy_ok: bool = False):
         H, Hkv, hs = self.H, self.Hkv, self.hs
         last = self.o.lazy if lazy_ok else self.o
+        fuse_ok, inv_freq = self.position.fusable(hs)
+        vt = kv.v_transposed
+        decode_fused = (ctx.is_decode and fuse_ok and ops.can_fuse_decode(self.qkv.weight.dtype, H, Hkv, hs)
+                        and (vt is None or vt))                 # the matrix-core kernels read transposed values
+        row_scale = None
+        if isinstance(h, ops.DeferredNorm) and h.shape[0] > ops.FUSED_ROWS:
+            # More rows than the fused product takes.  When the decode kernel rotates by itself it can apply the norm's
+            # factor as well (it multiplies whole rows of q, k and v): the library's product of the copy, then that
+            # kernel.  Else the norm is applied the plain way.
+            if decode_fused and inv_freq is not None and not self.has_bias and kv.writes and ops.LIBRARY_PRODUCTS:
+                row_scale, h = h, h.scaled
+            else:
+                h = h.materialize()
         if kv.writes:
             qkv = self.qkv(h)                                   # [T, (H + 2 Hkv) hs]
         else:
@@ -77,10 +94,7 @@ class Attention(Part):
             pad[:, :self.q_dim] = qkv
             qkv = pad
         out = torch.empty((h.shape[0], self.q_dim), dtype=h.dtype, device=h.device)
-        fuse_ok, inv_freq = self.position.fusable(hs)
-        vt = kv.v_transposed
-        if (ctx.is_decode and fuse_ok and ops.can_fuse_decode(h.dtype, H, Hkv, hs)
-                and (vt is None or vt)):                        # the matrix-core kernels read transposed values
+        if decode_fused:
             # one kernel: rotation of Q and the new K, the cache write, attention, merge of the splits
             if self.window:
                 n_splits, chunk = 1, 0
@@ -89,7 +103,7 @@ class Attention(Part):
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
                           window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
                           fused_rotate=inv_freq, fused_write=kv.writes, by_length=ctx.by_length,
-                          max_len_dev=ctx.max_len_dev if n_splits > 1 else None, v_transposed=vt)
+                          max_len_dev=ctx.max_len_dev if n_splits > 1 else None, v_transposed=vt, row_scale=row_scale)
             return last(out)
         self.position.encode_and_store(qkv, ctx, H, Hkv, hs, kv)
         if ctx.is_decode:

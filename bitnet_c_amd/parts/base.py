@@ -139,6 +139,12 @@ BLOCKS = Registry("block")
 class Part:
     """Base of all parts: no tensors, nothing to load."""
 
+    # Whether the part's work on a prompt step can be recorded into a graph and replayed for other sequences: it reads
+    # the step from the device tensors of its context alone (tokens, positions, seq_index, seq_lens, slot_ids, tiles(),
+    # page_tiles(), the block tables), never from the host lists (slots, n_new, pos0, row_ranges()), and never waits for
+    # the device.  The parts of this library say True; a part that does not say so keeps its model's prompt steps eager.
+    prompt_capturable = False
+
     def tensors(self) -> Dict[str, ParamSpec]:
         return {}
 
@@ -206,6 +212,15 @@ class ResidualStream:
                 and getattr(norm, "deferrable", False)):
             deferred = self.pending.linear.into_stream(self.pending.act, self.x, norm.weight, norm.eps)
             if deferred is not None:
+                self.pending = None
+                return deferred
+        if (rows is None and getattr(consumer, "takes_deferred_norm", False) and getattr(norm, "deferrable", False)
+                and not isinstance(self.pending, LazyDelta)):
+            from .. import ops
+            if ops.can_sum_deferred(self.x.shape[0], self.x.shape[1], out_dtype) and self.x.is_contiguous():
+                # more rows than the fused products take: one kernel adds the pending output (a tensor or partial sums)
+                # and leaves the norm's factor to the consumer's own kernels
+                deferred = ops.sum_deferred(self.x, self.pending, norm.weight, norm.eps)
                 self.pending = None
                 return deferred
         delta = self._pending_tensor()

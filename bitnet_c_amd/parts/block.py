@@ -15,6 +15,10 @@ class PreNormBlock(Part):
         self.mixer_norm = NORMS.build(mixer_norm)
         self.ffn_norm = NORMS.build(ffn_norm)
 
+    @property
+    def prompt_capturable(self) -> bool:
+        return all(getattr(c, "prompt_capturable", False) for c in self.children().values())
+
     def children(self):
         return {"mixer": self.mixer, "ffn": self.ffn, "mixer_norm": self.mixer_norm, "ffn_norm": self.ffn_norm}
 

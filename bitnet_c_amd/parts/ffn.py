@@ -17,6 +17,7 @@ from .linear import Linear, upload
 @FEED_FORWARDS.register("gated")
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(Part):
+    prompt_capturable = True    # a prompt step is read from the context's device tensors alone
     takes_deferred_norm = True      # forward accepts an ops.DeferredNorm for h
     gives_lazy_delta = True         # forward(..., lazy_ok=True) may return a LazyDelta
 
@@ -50,8 +51,10 @@ class SwiGLU(Part):
     def forward(self, h, ctx, lazy_ok: bool = False):
         if isinstance(h, ops.DeferredNorm):
             w = self.gate_up.weight
+            M = h.shape[0]
             if (not self.has_bias and self.interleaved and w.dtype == torch.bfloat16
-                    and ops.can_fuse_norm(h.shape[0], self.F, self.hidden, w.dtype)):
+                    and (ops.can_fuse_norm(M, self.F, self.hidden, w.dtype)
+                         or (M > ops.FUSED_ROWS and ops.LIBRARY_PRODUCTS and w.data_ptr() % 16 == 0))):
                 act = ops.linear_swiglu_prenorm(h, w, self.activation)
                 return self.down.lazy(act) if lazy_ok else self.down(act)
             h = h.materialize()

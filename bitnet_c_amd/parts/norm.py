@@ -12,6 +12,7 @@ from .linear import upload
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Part):
+    prompt_capturable = True    # a prompt step is read from the context's device tensors alone
     deferrable = True        # a product may fold this norm around itself (weight and eps are all it needs)
     takes_partial_sums = True    # apply() accepts ops.PartialSums as the delta
 

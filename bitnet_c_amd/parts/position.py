@@ -66,6 +66,7 @@ class PositionEncoding(Part):
 
 @POSITION_ENCODINGS.register("rope")
 class RotaryEncoding(PositionEncoding):
+    prompt_capturable = True    # a prompt step is read from the context's device tensors alone
     def __init__(self, head_dim: int, theta: float, rope_dims: int = 0, scaling=None):
         self.head_dim = int(head_dim)
         self.rope_dims = int(rope_dims) or self.head_dim
@@ -82,5 +83,6 @@ class RotaryEncoding(PositionEncoding):
 
 @POSITION_ENCODINGS.register("none")
 class NoEncoding(PositionEncoding):
+    prompt_capturable = True    # a prompt step is read from the context's device tensors alone
     def __init__(self, head_dim: int = 0):
         self.rope_dims = 0

@@ -558,7 +558,7 @@ def test_cuts_and_batches_agree_at_the_benchmark_layer_sizes():
     for dtype in (torch.bfloat16, torch.float32):
         model = DecoderModel(plan, dtype, "cuda:0")
         model.load(tensors)
-        engines[dtype] = bn.Engine(model, max_tokens=4096)
+        engines[dtype] = bn.Engine(model, max_tokens=16384)
     rnd = random.Random(31)
     toks, p1, p2 = ([rnd.randrange(cfg.vocab_size) for _ in range(n)] for n in (300, 70, 513))
     last = list(range(268, 300))
@@ -591,24 +591,42 @@ def test_cuts_and_batches_agree_at_the_benchmark_layer_sizes():
             rows.append(o[:1])
         for x in (a, b, c):
             eng.release(x)
+        # the prompt in two steps, the second of 100 tokens: at 64 to 128 rows a feed-forward's last product is left
+        # as partial sums over ranges of K (4,096 x 14,336 here) that the kernels of the next norm add up
+        s = eng.new_sequence()
+        eng.step([bn.StepEntry(s, toks[:200], [])])
+        chunk = eng.step([bn.StepEntry(s, toks[200:], list(range(68, 100)))])
+        eng.release(s)
+        # twenty sequences that decode together, sequence j from the first 268 + j tokens: steps of 20 rows (a
+        # captured step of 32 rows, whose products have more rows than one tile of the matrix cores); row j of
+        # step k holds the logits at position 268 + j + k
+        seqs = [eng.new_sequence() for _ in range(20)]
+        eng.step([bn.StepEntry(q, toks[:268 + j], []) for j, q in enumerate(seqs)])
+        wide = torch.cat([eng.step([bn.StepEntry(q, [toks[268 + j + k]], [0]) for j, q in enumerate(seqs)])
+                          for k in range(12)])
+        for q in seqs:
+            eng.release(q)
         eng.cache.check()
-        return whole, one_by_one, torch.cat(rows)
+        return whole, one_by_one, torch.cat(rows), chunk, wide
 
+    wide_rows = torch.tensor([j + k for k in range(12) for j in range(20)], device="cuda:0")
     ref = run(engines[torch.float32])
     assert torch.equal(ref[1], ref[0]) and torch.equal(ref[2], ref[0])     # float32: no cut changes a bit
+    assert torch.equal(ref[3], ref[0]) and torch.equal(ref[4], ref[0][wide_rows])
     assert rel_err(ref[0], plain_ref) < TOL[torch.float32]                 # and they are the plain implementation's
     got = run(engines[torch.bfloat16])
+    assert engines[torch.bfloat16]._graphs.keys() >= {1, 4, 32}           # the decode steps were replayed from graphs
     # 32 x 128,256 logits: the largest of four million differences is no measure (rounding noise of
     # standard deviation s has its largest value near 5.5 s there).  What rounding looks like at this
     # width: a difference of about 1.4 % of the logits' root mean square, the same in every row, with
     # no value far outside it.  A fault (a wrong key, a lost column) breaks one of the three.
     rms = float(ref[0].double().pow(2).mean().sqrt())
-    for g in got:
-        d = (g - ref[0]).double()
+    for i, g in enumerate(got):
+        d = (g - (ref[0][wide_rows] if i == 4 else ref[0])).double()
         per_row = d.pow(2).mean(dim=1).sqrt() / rms
-        assert float(per_row.max()) < 0.025, per_row
-        assert float(per_row.max() / per_row.min()) < 2.0, per_row
-        assert float(d.abs().max() / d.pow(2).mean().sqrt()) < 7.0
+        assert float(per_row.max()) < 0.025, (i, per_row)
+        assert float(per_row.max() / per_row.min()) < 2.0, (i, per_row)
+        assert float(d.abs().max() / d.pow(2).mean().sqrt()) < 7.0, i
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -661,6 +679,79 @@ def test_positions_beyond_the_original_context_with_the_8b_rotation_table(dtype)
     assert rel_err(one_off[-1:], right[-1:]) > 10 * TOL[dtype]
     eng.release(s)
     eng.cache.check()
+
+
+@pytest.mark.parametrize("H,Hkv,lens", [(8, 8, [700]), (8, 8, [300, 9, 1500]), (40, 40, [520, 70])])
+def test_decoding_with_the_split_plan_of_a_very_long_context(H, Hkv, lens):
+    """An engine whose sequences may grow to 131,072 tokens cuts the keys of a captured decode step for that length:
+    up to 64 runs, of which a sequence of some hundred tokens fills the first few and leaves the rest empty, with heads
+    of 128 that have a kv head each.  bfloat16 (float32 never splits its keys), against the plain implementation, with
+    one key among the hundreds made to stand out so that a run that is lost or merged twice shows."""
+    import bitnet_c_amd as bn
+    from bitnet_c_amd import ops
+    from bitnet_c_amd.config import architecture_for
+    from bitnet_c_amd.engine import DecoderModel
+    from bitnet_c_amd.weights import random_tensors
+    dtype = torch.bfloat16
+    raw = dict(model_type="llama", vocab_size=96, hidden_size=64, intermediate_size=136, num_hidden_layers=2,
+               num_attention_heads=H, num_key_value_heads=Hkv, head_dim=128, max_position_embeddings=131072,
+               rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+    cfg = bn.LlamaConfig.from_dict(raw)
+    plan = architecture_for(raw).build_plan(cfg)
+    tensors = random_tensors(plan.expected_tensors(), 19, dtype, device="cuda:0")
+    for name in ("model.layers.0.self_attn.q_proj.weight", "model.layers.0.self_attn.k_proj.weight"):
+        tensors[name] = (tensors[name].float() * 14.0).to(dtype)          # scores that tell keys apart
+    model = DecoderModel(plan, dtype, "cuda:0")
+    model.load(tensors)
+    eng = bn.Engine(model, max_tokens=131072 + 4096)
+    assert eng.max_seq_len == 131072
+    n_splits, _ = ops.decode_splits(len(lens), H, Hkv, eng.max_seq_len, dtype)
+    assert n_splits >= (64 if H * len(lens) <= 8 else 4)
+    n_dec = 6
+    reqs = _requests(96, 77, [n + n_dec for n in lens])
+    W = {k: v.float().cpu() for k, v in tensors.items()}
+    c = dict(dim=64, ffn=136, layers=2, heads=H, kv_heads=Hkv, head_dim=128, vocab=96, theta=cfg.rope_theta,
+             eps=cfg.rms_norm_eps, tied=False, rope_scaling=None, act="silu")
+    slots = [eng.new_sequence() for _ in reqs]
+    eng.step([bn.StepEntry(s, r[:-n_dec], []) for s, r in zip(slots, reqs)])
+    got = [[] for _ in reqs]
+    for t in range(n_dec):
+        lg = eng.step([bn.StepEntry(s, [r[len(r) - n_dec + t]], [0]) for s, r in zip(slots, reqs)])
+        for i in range(len(reqs)):
+            got[i].append(lg[i:i + 1].clone())
+    assert eng._graphs, "the decode steps were meant to be replayed from a graph"
+    for i, r in enumerate(reqs):
+        want = pl.forward(c, W, r, dtype)[-n_dec:]
+        assert rel_err(torch.cat(got[i]), want) < TOL[dtype], (i, len(r))
+    for s in slots:
+        eng.release(s)
+    eng.cache.check()
+
+
+def test_decode_steps_of_many_sequences_are_replayed_from_graphs(model_folders):
+    """300 sequences decode together: more than the largest captured step holds (256 rows), so the step is replayed in
+    two pieces (256 rows and 64 rows for the other 44); then 70 of them go on (a captured step of 128 rows).  float32:
+    equal, bit for bit, to an engine that runs every step without graphs."""
+    import bitnet_c_amd as bn
+    folder = model_folders("A", torch.float32)
+    reqs = _requests(256, 91, [1 + i % 9 for i in range(300)])
+    outs = []
+    for graphs in (True, False):
+        eng = bn.Engine.from_folder(folder, dtype=torch.float32, max_tokens=64 * 320, use_graphs=graphs)
+        slots = [eng.new_sequence() for _ in reqs]
+        got = [eng.step([bn.StepEntry(s, r, [len(r) - 1]) for s, r in zip(slots, reqs)])]
+        for k in range(2):
+            got.append(eng.step([bn.StepEntry(s, [(7 * i + k) % 256], [0]) for i, s in enumerate(slots)]))
+        for s in slots[70:]:
+            eng.release(s)
+        for k in range(2):
+            got.append(eng.step([bn.StepEntry(s, [(5 * i + k) % 256], [0]) for i, s in enumerate(slots[:70])]))
+        eng.cache.check()
+        outs.append(got)
+        if graphs:
+            assert set(eng._graphs) == {256, 64, 128}
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
 
 
 @pytest.mark.parametrize("n_seqs", [20, 50])
@@ -734,6 +825,8 @@ FURTHER_SIZES = [
     (20, 3, 3, 60, 100, 101, 2, False, False, True, [1, 40, 17, 70]),
     (36, 4, 2, 72, 173, 131, 1, True, False, False, [33, 2, 100]),
     (6, 6, 1, 30, 50, 61, 2, False, True, False, [5, 64, 65]),
+    # forty heads of 128 with a kv head each (no grouping: one useful column in a tile of the matrix cores)
+    (128, 40, 40, 160, 264, 389, 2, False, False, False, [200, 7, 130, 70, 33, 19, 100, 65]),
 ]
 
 

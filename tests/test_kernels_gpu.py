@@ -198,19 +198,20 @@ def test_products_with_the_norm_folded_in_refuse_what_they_cannot_take():
 
 
 @pytest.mark.parametrize("M", [1, 17, 33, 64, 100, 128])
-@pytest.mark.parametrize("N,K", [(4096, 4096), (200, 328), (72, 1000), (136, 16), (264, 3592)])
+@pytest.mark.parametrize("N,K", [(4096, 4096), (200, 328), (72, 1000), (136, 16), (264, 3592), (4096, 14336)])
 def test_products_left_as_partial_sums(M, N, K):
     """A product left as float32 partial sums over ranges of K, which the kernel of the next norm (or the plain add)
-    adds to the stream in slab order (the dispatcher does so for a part's last product from 64 to 128 rows when K is
-    at least twice N; the kernel takes 1 to 128 rows of any shape).  The sums are exact up to their order; the norm is
-    the plain formula on the sum."""
+    adds to the stream in slab order (the dispatcher does so for a part's last product from 17 to 128 rows when K is
+    at least twice N, or at least N for widths up to 6,144; the kernel takes 1 to 128 rows of any shape), among them
+    the last product of a feed-forward of the 8B shape (4,096 x 14,336).  The sums are exact up to their order; the
+    norm is the plain formula on the sum."""
     ops = _ops()
     eps = 1e-6
     x, w = _rand((M, K), torch.bfloat16, 41), _rand((N, K), torch.bfloat16, 42, 0.05)
     stream = _rand((M, N), torch.float32, 43, 2.0)
     norm_w = _rand((N,), torch.float32, 44) * 0.2 + 1.0
     ref = x.double() @ w.double().t()
-    assert ops.can_split_sums(M, N, K, torch.bfloat16) == (64 <= M <= 128 and K >= 2 * N)
+    assert ops.can_split_sums(M, N, K, torch.bfloat16) == (17 <= M <= 128 and K % 8 == 0 and (K >= 2 * N or (K >= N and N <= 6144)))
     parts = ops.linear_partial_sums(x.cuda(), w.cuda())
     assert parts.slabs.dtype == torch.float32 and tuple(parts.shape) == (M, N)
     assert rel_err(parts.slabs.sum(dim=0), ref.float()) < 1e-5
@@ -233,6 +234,92 @@ def test_products_left_as_partial_sums(M, N, K):
     xs = stream.clone().cuda()
     ops.residual_add(xs, parts)
     assert rel_err(xs, want_x.float()) < 1e-5
+
+
+@pytest.mark.parametrize("M", [17, 64, 128])
+@pytest.mark.parametrize("D", [4096, 264, 5120])
+@pytest.mark.parametrize("kind", ["none", "bf16", "f32", "slabs"])
+def test_a_norm_left_to_its_consumer(M, D, kind):
+    """sum_deferred: the stream takes what a part has produced (nothing, a tensor, or partial sums), and a consumer
+    gets the bf16 copy of the new stream times the norm's weights with the rows' sums of squares in pieces.  What
+    the consumers make of it is the plain norm: materialize(), and the gated unit whose kernel applies the factor
+    to a product of the copy (act(s g) * (s u), s = 1/sqrt(mean + eps))."""
+    ops = _ops()
+    eps = 1e-5
+    stream = _rand((M, D), torch.float32, 61, 2.0)
+    norm_w = _rand((D,), torch.float32, 62) * 0.2 + 1.0
+    delta, add = None, torch.zeros(M, D, dtype=torch.float64)
+    if kind == "bf16":
+        delta = _rand((M, D), torch.bfloat16, 63)
+        add = delta.double()
+        delta = delta.cuda()
+    elif kind == "f32":
+        delta = _rand((M, D), torch.float32, 63)
+        add = delta.double()
+        delta = delta.cuda()
+    elif kind == "slabs":
+        slabs = _rand((3, M, D), torch.float32, 63)
+        add = slabs.double().sum(dim=0)
+        delta = ops.PartialSums(slabs.cuda())
+    want_x = (stream.double() + add).float()
+    xs = stream.clone().cuda()
+    pre = ops.sum_deferred(xs, delta, norm_w.cuda(), eps)
+    assert rel_err(xs, want_x) < 1e-6
+    assert tuple(pre.scaled.shape) == (M, D) and pre.scaled.dtype == torch.bfloat16
+    assert tuple(pre.slots.shape) == (M, (D + 1023) // 1024)
+    assert close(pre.scaled.float(), want_x * norm_w, torch.bfloat16)
+    assert rel_err(pre.slots.sum(dim=1), want_x.double().pow(2).sum(dim=1).float()) < 1e-5
+    normed = pl.rmsnorm(want_x, norm_w, eps)
+    assert close(pre.materialize().float(), normed, torch.bfloat16)
+    # the gated unit over a product of the copy: 2F columns, gate and up interleaved in blocks of 8
+    F = 48
+    gu = _rand((M, 2 * F), torch.bfloat16, 64, 3.0)
+    got = ops.swiglu_scaled(gu.cuda(), pre, "silu")
+    sc = 1.0 / torch.sqrt(want_x.double().pow(2).mean(dim=1) + eps)
+    g8 = gu.double().view(M, F // 8, 2, 8) * sc[:, None, None, None]
+    want = (g8[:, :, 0] / (1.0 + torch.exp(-g8[:, :, 0])) * g8[:, :, 1]).reshape(M, F)
+    assert close(got.float(), want.float(), torch.bfloat16)
+    assert ops.can_sum_deferred(M, D, torch.bfloat16) and not ops.can_sum_deferred(16, D, torch.bfloat16)
+    assert not ops.can_sum_deferred(M, D, torch.float32)
+    with pytest.raises(ops.KernelError):
+        ops.sum_deferred(xs, _rand((M, D + 4), torch.bfloat16, 1).cuda(), norm_w.cuda(), eps)
+
+
+@pytest.mark.parametrize("H,Hkv,hs,n_splits", [(8, 2, 128, 1), (8, 2, 128, 3), (6, 6, 64, 2)])
+def test_decode_attention_applies_a_deferred_norm_s_factor(H, Hkv, hs, n_splits):
+    """Rows of q, k, v that lack their norm's factor (a product of a deferred norm's copy): the decode kernel that
+    rotates and stores by itself multiplies it in.  With factors that are powers of two nothing is rounded
+    differently, so the output and the stored keys and values equal, bit for bit, those of the same rows with the
+    factor applied beforehand."""
+    ops = _ops()
+    dtype = torch.bfloat16
+    lens = [1, 64, 65, 300, 190]
+    B = len(lens)
+    seqs_k = [_rand((l, Hkv, hs), dtype, 70 + i) for i, l in enumerate(lens)]
+    seqs_v = [_rand((l, Hkv, hs), dtype, 80 + i) for i, l in enumerate(lens)]
+    kp, vp, bt = _paged(seqs_k, seqs_v, dtype, sum((l + 63) // 64 for l in lens) + 2, 90)
+    qkv = _rand((B, (H + 2 * Hkv) * hs), dtype, 91)
+    factor = torch.tensor([0.5, 2.0, 4.0, 0.25, 1.0])
+    raw = (qkv.float() / factor[:, None]).to(dtype)
+    assert torch.equal((raw.float() * factor[:, None]).to(dtype), qkv)
+    slots = torch.zeros(B, 3)
+    slots[:, 1] = 4.0 / factor ** 2                            # width 4, eps 0: 1 / sqrt(sum of the slots / 4) is the factor
+    pre = ops.DeferredNorm(raw.cuda(), slots.cuda(), torch.zeros(B, 4).cuda(), None, 0.0)
+    inv = pl.rope_inv_freq(hs, 10000.0).cuda()
+    d_lens = torch.tensor(lens, dtype=torch.int32).cuda()
+    chunk = ((bt.shape[1] + n_splits - 1) // n_splits) * 64
+    outs = []
+    for rows, rs in ((qkv, None), (raw, pre)):
+        k_pages, v_pages = kp.clone().cuda(), vp.clone().cuda()
+        out = torch.full((B, H * hs), float("nan"), dtype=dtype).cuda()
+        ops.attention(rows.cuda(), out, k_pages, v_pages, bt.cuda(), H, Hkv, hs, hs ** -0.5, seq_lens=d_lens,
+                      n_splits=n_splits, chunk=chunk if n_splits > 1 else 0, fused_rotate=inv, fused_write=True, row_scale=rs)
+        outs.append((out.cpu(), k_pages.cpu(), v_pages.cpu()))
+    for a, b in zip(*outs):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))        # bits: the pages hold NaN where nothing was written
+    assert not bool(outs[0][0].isnan().any())
+    with pytest.raises(ops.KernelError):                                       # only where the kernel rotates by itself
+        ops.attention(raw.cuda(), out, k_pages, v_pages, bt.cuda(), H, Hkv, hs, hs ** -0.5, seq_lens=d_lens, row_scale=pre)
 
 
 def test_partial_sums_refuse_what_they_cannot_take():

@@ -90,18 +90,66 @@ def test_decode_attention_without_allocation_equals_the_allocating_entry_point()
                               part_o.data_ptr(), part_ml.data_ptr(), None, 0, 0, None, None, stream)
         assert rc == 0
         got = torch.full((B, H * hs), float("nan"), dtype=torch.bfloat16, device="cuda")
-        before = torch.cuda.memory_allocated()
-        rc = lib.bn_attn_mfma_decode_static(q.data_ptr(), H * hs, got.data_ptr(), H * hs, kp.data_ptr(), vp.data_ptr(),
-                                            bt.data_ptr(), bt.shape[1], d_lens.data_ptr(), B, H, Hkv, hs, GT, 0, scale,
-                                            n_splits, chunk, None, 0, 0, None, stream)
-        assert rc == 0
-        assert torch.cuda.memory_allocated() == before
+
+        def static_call(out):
+            return lib.bn_attn_mfma_decode_static(q.data_ptr(), H * hs, out.data_ptr(), H * hs, kp.data_ptr(), vp.data_ptr(),
+                                                  bt.data_ptr(), bt.shape[1], d_lens.data_ptr(), B, H, Hkv, hs, GT, 0, scale,
+                                                  n_splits, chunk, None, 0, 0, None,
+                                                  torch.cuda.current_stream().cuda_stream)
+        assert static_call(got) == 0
         torch.cuda.synchronize()
         assert torch.equal(got.cpu(), want.cpu()), seed
+        # It allocates nothing: the call goes past torch's allocator, so what is compared is the driver's own count of
+        # free device memory, around a call after the one that looked the array's address up.
+        again = torch.full((B, H * hs), float("nan"), dtype=torch.bfloat16, device="cuda")
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        assert static_call(again) == 0
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
+        assert torch.equal(again.cpu(), want.cpu()), seed
+        # Under graph capture (a caller that cannot allocate): recorded after the warm call, replayed three times with
+        # eager work between the replays, every replay the eager result.
+        captured = torch.full((B, H * hs), float("nan"), dtype=torch.bfloat16, device="cuda")
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            rc = static_call(captured)
+        assert rc == 0
+        for replay in range(3):
+            captured.fill_(float("nan"))
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(captured.cpu(), want.cpu()), (seed, replay)
+            assert static_call(again) == 0                     # the array's contents between replays do not matter
+            torch.cuda.synchronize()
         # and both are the plain formula's result within the rounding of the bf16 softmax weights
         ref = _plain(q, ks, vs, H, Hkv, hs, scale)
         assert bool(((got.float().cpu() - ref).abs() <= ref.abs() * 2.0 ** -8 + 5 * 2.0 ** -9).all()), seed
-    # more partials than the array holds: refused, nothing launched, the output untouched
+    # The limit from both sides: the most partials that fit (419 sequences x 11 heads x 7 splits x 130 floats are 114
+    # floats short of the array; the head size plus two never divides its size) run and equal the allocating entry
+    # point's result; one sequence more is refused.
+    H2, n_splits2, chunk2 = 11, 7, 64
+    rnd = random.Random(5)
+    lens2 = [rnd.randrange(1, 7 * 64 + 1) for _ in range(420)]
+    q2, kp2, vp2, bt2, d_lens2, _, _ = _case(3, lens2, H2, H2, hs)
+    assert 419 * H2 * n_splits2 * (hs + 2) <= SCRATCH_FLOATS < 420 * H2 * n_splits2 * (hs + 2)
+    po = torch.empty((419 * H2 * n_splits2, hs), dtype=torch.float32, device="cuda")
+    pm = torch.empty((419 * H2 * n_splits2, 2), dtype=torch.float32, device="cuda")
+    want2 = torch.zeros((420, H2 * hs), dtype=torch.bfloat16, device="cuda")
+    got2 = torch.zeros((420, H2 * hs), dtype=torch.bfloat16, device="cuda")
+    assert lib.bn_attn_mfma(q2.data_ptr(), H2 * hs, want2.data_ptr(), H2 * hs, kp2.data_ptr(), vp2.data_ptr(), bt2.data_ptr(),
+                            bt2.shape[1], d_lens2.data_ptr(), None, 419, 419, H2, H2, hs, 1, 0, scale, n_splits2, chunk2,
+                            po.data_ptr(), pm.data_ptr(), None, 0, 0, None, None, stream) == 0
+    fits = lambda n, out: lib.bn_attn_mfma_decode_static(
+        q2.data_ptr(), H2 * hs, out.data_ptr(), H2 * hs, kp2.data_ptr(), vp2.data_ptr(), bt2.data_ptr(), bt2.shape[1],
+        d_lens2.data_ptr(), n, H2, H2, hs, 1, 0, scale, n_splits2, chunk2, None, 0, 0, None, stream)
+    assert fits(419, got2) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(got2.cpu(), want2.cpu()) and float(got2[:419].float().abs().sum()) > 0
+    assert fits(420, got2) == ERR_SCRATCH
+    torch.cuda.synchronize()
+    assert float(got2[419].float().abs().sum()) == 0.0            # nothing was launched for the call that was refused
+    # far more partials than the array holds: refused, nothing launched, the output untouched
     B = SCRATCH_FLOATS // (H * 64 * (hs + 2)) + 1
     out = torch.zeros((1, H * hs), dtype=torch.bfloat16, device="cuda")
     rc = lib.bn_attn_mfma_decode_static(q.data_ptr(), H * hs, out.data_ptr(), H * hs, kp.data_ptr(), vp.data_ptr(),
