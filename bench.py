@@ -285,6 +285,11 @@ def main() -> int:
           f"{achieved:.0f} GB/s = {achieved / HBM_GBS:.3f} of {HBM_GBS:.0f}", file=sys.stderr, flush=True)
     points = {}
     if not args.no_points:
+        for n in (128, 512):                  # short prompts: a step is the weights once and the host's work, not the matrix cores
+            prefill_once(n)
+            prefill_once(n)
+            points[f"prefill_{n}_ms"] = round(sorted(prefill_once(n) for _ in range(5))[2] * 1e3, 3)
+            print(f"[bench] prefill of {n} tokens: {points[f'prefill_{n}_ms']} ms", file=sys.stderr, flush=True)
         for b in (1, 64):
             s_b, ctx_b = decode(b, max(16, args.steps // 2), args.warmup)
             bytes_b = weight_bytes + ctx_b * kv_bytes_per_token

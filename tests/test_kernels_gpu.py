@@ -325,8 +325,11 @@ def test_decode_attention_applies_a_deferred_norm_s_factor(H, Hkv, hs, n_splits)
 def test_partial_sums_refuse_what_they_cannot_take():
     ops = _ops()
     assert ops.can_split_sums(64, 64, 128, torch.bfloat16) and ops.can_split_sums(128, 64, 512, torch.bfloat16)
-    assert not ops.can_split_sums(63, 64, 128, torch.bfloat16) and not ops.can_split_sums(129, 64, 128, torch.bfloat16)
-    assert not ops.can_split_sums(64, 64, 120, torch.bfloat16)             # K below twice N
+    assert ops.can_split_sums(17, 64, 128, torch.bfloat16) and ops.can_split_sums(64, 64, 64, torch.bfloat16)
+    assert not ops.can_split_sums(16, 64, 128, torch.bfloat16) and not ops.can_split_sums(129, 64, 128, torch.bfloat16)
+    assert not ops.can_split_sums(64, 64, 56, torch.bfloat16)              # K below N
+    assert not ops.can_split_sums(64, 8192, 8192, torch.bfloat16)          # a square product wider than the rule's bound
+    assert ops.can_split_sums(64, 8192, 16384, torch.bfloat16)             # K twice N: any width
     assert not ops.can_split_sums(64, 64, 172, torch.bfloat16) and not ops.can_split_sums(64, 64, 128, torch.float32)
     z = lambda *shape: torch.zeros(*shape, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(ops.KernelError):

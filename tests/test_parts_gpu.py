@@ -78,8 +78,8 @@ def test_norm_and_feed_forward_parts(dtype):
 
 @pytest.mark.parametrize("T", [8, 40, 64, 128, 200])
 def test_a_feed_forward_s_last_product_reaches_the_stream_in_every_form(T):
-    """bfloat16: at 8 rows the last product adds itself to the stream and leaves the norm deferred, at 64 and 128
-    rows it comes as partial sums over ranges of K that the kernels of the next norm add up, at 40 and 200 rows as a
+    """bfloat16: at 8 rows the last product adds itself to the stream and leaves the norm deferred, at 40, 64 and 128
+    rows it comes as partial sums over ranges of K that the kernels of the next norm add up, at 200 rows as a
     tensor.  The stream and the normed rows are the plain formulas' in every form; a norm that knows only tensors
     (defined here) gets the sum formed for it."""
     from bitnet_c_amd import ops
@@ -94,7 +94,7 @@ def test_a_feed_forward_s_last_product_reaches_the_stream_in_every_form(T):
     norm.load({"weight": nw}, DEV, dtype)
     h, x0 = _rand((T, D), 7).to(dtype), _rand((T, D), 8, 2.0)
     delta = ffn.forward(h.to(DEV), None, lazy_ok=True)
-    kind = LazyDelta if T <= 16 else ops.PartialSums if 64 <= T <= 128 else torch.Tensor
+    kind = LazyDelta if T <= 16 else ops.PartialSums if 17 <= T <= 128 else torch.Tensor
     assert isinstance(delta, kind), type(delta)
     if kind is ops.PartialSums:
         assert delta.slabs.shape[0] == 4
@@ -118,6 +118,20 @@ def test_a_feed_forward_s_last_product_reaches_the_stream_in_every_form(T):
         assert rel_err(stream.x, exact_x.float()) < 2e-2
         assert part_close(got.float(), pl.rmsnorm(exact_x.float(), nw, 1e-5).to(dtype).float(), dtype,
                           pl.rmsnorm(exact_x.float(), nw, 1e-5))
+    if 17 <= T <= 128:
+        # a consumer that applies the norm itself gets it undone: one kernel forms the sum and leaves the factor
+        stream = ResidualStream(x0.clone().to(DEV))
+        stream.add(ffn.forward(h.to(DEV), None, lazy_ok=True))
+        pre = stream.normed(norm, dtype, consumer=ffn)
+        assert isinstance(pre, ops.DeferredNorm) and stream.pending is None
+        assert rel_err(stream.x, exact_x.float()) < 2e-2
+        assert part_close(pre.materialize().float(), pl.rmsnorm(exact_x.float(), nw, 1e-5).to(dtype).float(), dtype,
+                          pl.rmsnorm(exact_x.float(), nw, 1e-5))
+        # and the feed-forward that consumes it gives what it gives for the normed rows
+        plain_in = pl.rmsnorm(exact_x.float(), nw, 1e-5)
+        want = pl.feed_forward(plain_in.to(dtype).float(), t["w_gate"].float(), t["w_up"].float(), t["w_down"].float(), dtype)
+        exact = pl.feed_forward(plain_in, t["w_gate"].float(), t["w_up"].float(), t["w_down"].float())
+        assert part_close(ffn.forward(pre, None).float(), want, dtype, exact)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
