@@ -227,7 +227,11 @@ MAX_PROMPT_GRAPHS = 12            # captured prompt steps that an engine keeps; 
 
 
 def _row_bucket(n: int) -> int:
-    """Token rows of the captured step that serves a prompt step of n tokens: the padding is at most an eighth."""
+    """Token rows of the captured step that serves a prompt step of n tokens: 16 and 32 (up to 16 rows the products are
+    the fused ones of a decode step, and rows cost time there), then multiples of 64 up to 512, of 128 up to 2,048, of
+    512 beyond: from 64 tokens on the padding is at most an eighth."""
+    if n <= 32:
+        return 16 if n <= 16 else 32
     unit = 64 if n <= 512 else 128 if n <= 2048 else 512
     return -(-n // unit) * unit
 

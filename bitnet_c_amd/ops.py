@@ -474,7 +474,8 @@ SPLIT_SUMS = os.environ.get("BITNET_NO_SPLIT_SUMS", "") in ("", "0")
 # 36 us against 45 at 64 rows, 44 against 80 at 128; 70B: 119 against 148, 141 against 210), while below 64 rows and for
 # square matrices the two are within 10 % of each other with the sign depending on the shape.
 SPLIT_SUM_ROWS = (17, 128)
-SPLIT_SUM_SQUARE_WIDTH = 6144     # square products (an output projection) up to this width as well: see can_split_sums
+# square products (an output projection) up to this width as well: see can_split_sums
+SPLIT_SUM_SQUARE_WIDTH = int(os.environ.get("BITNET_SPLIT_SQUARE_WIDTH", "6144"))
 
 
 @dataclass

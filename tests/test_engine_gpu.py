@@ -728,6 +728,64 @@ def test_decoding_with_the_split_plan_of_a_very_long_context(H, Hkv, lens):
     eng.cache.check()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_prompt_steps_are_replayed_from_graphs(model_folders, name, dtype, monkeypatch):
+    """The first prompt step of a bucket (token rows, sequences, wanted places) runs eagerly, the second is recorded,
+    later ones are replays with other sequences, other lengths inside the bucket, other places in the cache and other
+    wanted rows: continuations of a prompt, mixed steps (a sequence with one token beside one with many), steps that
+    want nothing.  float32: every step equals, bit for bit, the same step of an engine that never records prompt steps;
+    bfloat16: within rounding (the padded step may pick another product kernel).  The graphs that an engine keeps are
+    bounded: the one unused for longest goes."""
+    import bitnet_c_amd as bn
+    from bitnet_c_amd.engine import step as step_mod
+    monkeypatch.setattr(step_mod, "MAX_PROMPT_GRAPHS", 3)
+    folder = model_folders(name, dtype)
+    vocab = pl.read_config(folder)["vocab"]
+    engines = [bn.Engine.from_folder(folder, dtype=dtype, max_tokens=64 * 64) for _ in range(2)]
+    engines[1].prompt_graphs = False
+    assert engines[0].prompt_graphs
+    rnd = random.Random(5)
+    toks = lambda n: [rnd.randrange(vocab) for _ in range(n)]
+    # (new sequences' prompt lengths, continuation lengths of the sequences that live, single tokens for live sequences)
+    script = [([40, 9], [], 0), ([33, 20], [], 0), ([50, 3], [], 0),           # bucket (64 rows, 2 seqs): eager, recorded, replayed
+              ([], [30, 31], 0), ([], [17, 5], 2),                              # continuations; then mixed with two decoding rows
+              ([100], [], 0), ([90], [], 0), ([70], [], 0),                    # (128, 1)
+              ([3], [], 0), ([9], [], 0), ([16], [], 0),                        # (16, 1)
+              ([20, 20, 20, 4], [], 0), ([10, 30, 1, 23], [], 0), ([5, 5, 5, 49], [], 0),   # (64, 4)
+              ([44, 4], [], 0)]                                                  # (64, 2) again: its graph was dropped meanwhile
+    outs = [[], []]
+    for which, eng in enumerate(engines):
+        rnd.seed(5)
+        live = []
+        for new, cont, singles in script:
+            ent = []
+            for n in new:
+                s = eng.new_sequence()
+                live.append(s)
+                ent.append(bn.StepEntry(s, toks(n), [0, n - 1] if n > 1 else [0]))
+            older = [s for s in live if s not in [e.slot for e in ent]]
+            for n, s in zip(cont, older):
+                ent.append(bn.StepEntry(s, toks(n), [n // 2]))
+            for s in older[len(cont):len(cont) + singles]:
+                ent.append(bn.StepEntry(s, toks(1), []))                      # a row that decodes, and wants nothing
+            outs[which].append(eng.step(ent))
+            if len(live) > 6:                                                  # slots are given back and used again
+                for s in live[:4]:
+                    eng.release(s)
+                live = live[4:]
+        eng.cache.check()
+    eng = engines[0]
+    assert eng.graphs_built >= 5 and len(eng._prompt_graphs) <= 3
+    assert (64, 2, 4) in eng._prompt_seen and not engines[1]._prompt_graphs
+    for i, (a, b) in enumerate(zip(*outs)):
+        assert a.shape == b.shape
+        if dtype == torch.float32:
+            assert torch.equal(a, b), i
+        else:
+            assert rel_err(a, b) < TOL[dtype], i
+
+
 def test_decode_steps_of_many_sequences_are_replayed_from_graphs(model_folders):
     """300 sequences decode together: more than the largest captured step holds (256 rows), so the step is replayed in
     two pieces (256 rows and 64 rows for the other 44); then 70 of them go on (a captured step of 128 rows).  float32:
