@@ -468,14 +468,16 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = 
 # --------------------------------------------------------------------------------------
 # Set False (or BITNET_NO_FUSED_NORM=1) to keep every norm a kernel of its own.
 SPLIT_SUMS = os.environ.get("BITNET_NO_SPLIT_SUMS", "") in ("", "0")
-# Where a product that ends a part is left as partial sums (splitk_gemm) instead of going to the library: from 64 to 128
-# rows and K at least twice N, the shape of a feed-forward's last product.  Measured on nine layer shapes (hidden 2,048
-# to 8,192) with the kernels of the next norm included: there it is 15 to 45 % faster than the library's product (8B:
-# 36 us against 45 at 64 rows, 44 against 80 at 128; 70B: 119 against 148, 141 against 210), while below 64 rows and for
-# square matrices the two are within 10 % of each other with the sign depending on the shape.
+# Where a product that ends a part is left as partial sums (splitk_gemm) instead of going to the library: from 17 to 128
+# rows when K is at least twice N, the shape of a feed-forward's last product.  Measured on nine layer shapes (hidden 2,048
+# to 8,192) with the kernels of the next norm included: from 64 rows on it is 15 to 45 % faster than the library's product
+# (8B: 36 us against 45 at 64 rows, 44 against 80 at 128; 70B: 119 against 148, 141 against 210); below 64 rows the two
+# products are equal within a tenth, and the partial sums win by the kernel that they save: one kernel adds them to
+# the stream and leaves the next norm to its consumer (sum_deferred), where the library's product needs the add and the
+# norm.  Square products (an output projection) as well up to SPLIT_SUM_SQUARE_WIDTH columns: 12 + 5 us against 15 + 5 at
+# 64 rows of the 8B shape; at widths of 5,120 and 8,192 whole decode steps were equal within the noise of a run or slower.
 SPLIT_SUM_ROWS = (17, 128)
-# square products (an output projection) up to this width as well: see can_split_sums
-SPLIT_SUM_SQUARE_WIDTH = int(os.environ.get("BITNET_SPLIT_SQUARE_WIDTH", "6144"))
+SPLIT_SUM_SQUARE_WIDTH = int(os.environ.get("BITNET_SPLIT_SQUARE_WIDTH", "4096"))
 
 
 @dataclass

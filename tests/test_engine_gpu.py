@@ -812,6 +812,55 @@ def test_decode_steps_of_many_sequences_are_replayed_from_graphs(model_folders):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("n_tokens", [2048, 2000, 128])
+def test_graph_replays_of_a_prompt_step_at_the_benchmark_layer_sizes(n_tokens):
+    """A prompt step at the Llama-3.1-8B layer sizes (two layers, bfloat16) recorded into a graph: its products are the
+    library's at their real sizes (the kernel the library picks for 2,048 rows of the feed-forward splits its work over
+    the chip and keeps partial results in a work buffer), and a node that clears such a buffer inside a graph has to
+    give the right result on every replay, not only on the first.  The same prompt in a new slot five times, other
+    prompt steps and synchronisations between; the first run is eager, the second is the capture, the rest are replays;
+    each is compared with the plain run of an engine that records nothing."""
+    import bitnet_c_amd as bn
+    from bitnet_c_amd.config import architecture_for
+    from bitnet_c_amd.engine import DecoderModel
+    from bitnet_c_amd.weights import random_tensors
+    raw = dict(model_type="llama", vocab_size=128256, hidden_size=4096, intermediate_size=14336,
+               num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+               max_position_embeddings=131072, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+    cfg = bn.LlamaConfig.from_dict(raw)
+    plan = architecture_for(raw).build_plan(cfg)
+    model = DecoderModel(plan, torch.bfloat16, "cuda:0")
+    model.load(random_tensors(plan.expected_tensors(), 3, torch.bfloat16, device="cuda:0"))
+    engines = [bn.Engine(model, max_tokens=8192, max_seq_len=4096) for _ in range(2)]
+    engines[1].prompt_graphs = False
+    rnd = random.Random(41)
+    toks = [rnd.randrange(cfg.vocab_size) for _ in range(n_tokens)]
+    other = [rnd.randrange(cfg.vocab_size) for _ in range(700)]
+    want = list(range(n_tokens - 4, n_tokens))
+
+    def run(eng):
+        s = eng.new_sequence()
+        out = eng.step([bn.StepEntry(s, toks, want)])
+        eng.release(s)
+        return out
+
+    ref = run(engines[1])
+    rms = float(ref.double().pow(2).mean().sqrt())
+    for k in range(5):
+        got = run(engines[0])
+        d = (got - ref).double()
+        # the same kernels on the same rows: at most the rounding of a product whose sums the library forms in another order
+        assert float(d.pow(2).mean().sqrt()) / rms < 0.01, k
+        assert float(d.abs().max()) / rms < 0.1, k
+        s = engines[0].new_sequence()                    # eager work of another size and a synchronisation between the replays
+        engines[0].step([bn.StepEntry(s, other[:300 + 100 * k], [0])])
+        engines[0].release(s)
+        torch.cuda.synchronize()
+    assert len(engines[0]._prompt_graphs) >= 1 and not engines[1]._prompt_graphs
+    for e in engines:
+        e.cache.check()
+
+
 @pytest.mark.parametrize("n_seqs", [20, 50])
 def test_graph_replays_of_a_wide_batch_at_the_benchmark_layer_sizes(n_seqs):
     """20 or 50 sequences decode together at the Llama-3.1-8B layer sizes (two layers, bfloat16): 32 or 64

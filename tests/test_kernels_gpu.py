@@ -202,7 +202,7 @@ def test_products_with_the_norm_folded_in_refuse_what_they_cannot_take():
 def test_products_left_as_partial_sums(M, N, K):
     """A product left as float32 partial sums over ranges of K, which the kernel of the next norm (or the plain add)
     adds to the stream in slab order (the dispatcher does so for a part's last product from 17 to 128 rows when K is
-    at least twice N, or at least N for widths up to 6,144; the kernel takes 1 to 128 rows of any shape), among them
+    at least twice N, or at least N for widths up to 4,096; the kernel takes 1 to 128 rows of any shape), among them
     the last product of a feed-forward of the 8B shape (4,096 x 14,336).  The sums are exact up to their order; the
     norm is the plain formula on the sum."""
     ops = _ops()
@@ -211,7 +211,7 @@ def test_products_left_as_partial_sums(M, N, K):
     stream = _rand((M, N), torch.float32, 43, 2.0)
     norm_w = _rand((N,), torch.float32, 44) * 0.2 + 1.0
     ref = x.double() @ w.double().t()
-    assert ops.can_split_sums(M, N, K, torch.bfloat16) == (17 <= M <= 128 and K % 8 == 0 and (K >= 2 * N or (K >= N and N <= 6144)))
+    assert ops.can_split_sums(M, N, K, torch.bfloat16) == (17 <= M <= 128 and K % 8 == 0 and (K >= 2 * N or (K >= N and N <= 4096)))
     parts = ops.linear_partial_sums(x.cuda(), w.cuda())
     assert parts.slabs.dtype == torch.float32 and tuple(parts.shape) == (M, N)
     assert rel_err(parts.slabs.sum(dim=0), ref.float()) < 1e-5
@@ -328,7 +328,7 @@ def test_partial_sums_refuse_what_they_cannot_take():
     assert ops.can_split_sums(17, 64, 128, torch.bfloat16) and ops.can_split_sums(64, 64, 64, torch.bfloat16)
     assert not ops.can_split_sums(16, 64, 128, torch.bfloat16) and not ops.can_split_sums(129, 64, 128, torch.bfloat16)
     assert not ops.can_split_sums(64, 64, 56, torch.bfloat16)              # K below N
-    assert not ops.can_split_sums(64, 8192, 8192, torch.bfloat16)          # a square product wider than the rule's bound
+    assert not ops.can_split_sums(64, 5120, 5120, torch.bfloat16)          # a square product wider than the rule's bound
     assert ops.can_split_sums(64, 8192, 16384, torch.bfloat16)             # K twice N: any width
     assert not ops.can_split_sums(64, 64, 172, torch.bfloat16) and not ops.can_split_sums(64, 64, 128, torch.float32)
     z = lambda *shape: torch.zeros(*shape, dtype=torch.bfloat16, device="cuda")
