@@ -39,7 +39,19 @@ struct AttnArgs {
     float scale;
     const int* max_len;       // != null (decode form, n_splits > 1): the longest sequence's key count in device
                               // memory; the keys per split follow from it (bn_split_chunk) instead of from `chunk`
+    int fold;                 // > 0: keys are summed in runs of `fold` positions (a multiple of BN_PAGE, counted from
+                              // position 0) and the runs folded in order (fold_factors, fold_value below); a split is then one run
 };
+
+// The fold of one run of keys into the sums of the runs before it: (M, L, O) <- (M, L, O) + (m, l, o) with both sides
+// rescaled to the larger maximum.  Every place that folds calls these two functions, and their operations are written out
+// (no contraction left to the compiler), so the same runs give the same bits wherever they are folded.
+__device__ __forceinline__ void fold_factors(float M, float m, float& m2, float& fa, float& fb) {
+    m2 = fmaxf(M, m);
+    fa = expf(M - m2);                                   // 0 when nothing was there before (M = -inf)
+    fb = expf(m - m2);
+}
+__device__ __forceinline__ float fold_value(float O, float fa, float o, float fb) { return __fmaf_rn(O, fa, __fmul_rn(o, fb)); }
 
 template <typename T> struct Vec4;
 template <> struct Vec4<float> {
@@ -88,7 +100,11 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
     float* m_s = p_s + KT * RT;                          // [16] running max
     float* l_s = m_s + 16;                               // [16] running sum
     float* a_s = l_s + 16;                               // [16] rescale of this tile
-    T* k_s = reinterpret_cast<T*>(a_s + 16);             // [KT][kstride]
+    float* Mt_s = a_s + 16;                              // [16] fold mode: maximum and sum over the runs folded so far,
+    float* Lt_s = Mt_s + 16;                             // [16]
+    float* fa_s = Lt_s + 16;                             // [16] and the factors of the fold that is under way
+    float* fb_s = fa_s + 16;                             // [16]
+    T* k_s = reinterpret_cast<T*>(fb_s + 16);            // [KT][kstride]
     T* v_s = k_s + KT * kstride;
 
     // rows: r = i*GT + g  ->  token tok0+i, head kvh*G + ht*GT + g
@@ -104,7 +120,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
         }
         q_s[idx] = v;
     }
-    if (tid < 16) { m_s[tid] = -INFINITY; l_s[tid] = 0.f; a_s[tid] = 1.f; }
+    if (tid < 16) { m_s[tid] = -INFINITY; l_s[tid] = 0.f; a_s[tid] = 1.f; Mt_s[tid] = -INFINITY; Lt_s[tid] = 0.f; }
     const bool whole_groups = (hs * (int)sizeof(T)) % 16 == 0;      // rows of 16-byte groups in the pages
     if (hsp != hs)                                                  // the padding of the staged rows stays zero
         for (int idx = tid; idx < 2 * KT * kstride; idx += ATT_THREADS) k_s[idx] = from_f32<T>(0.f);
@@ -127,6 +143,56 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
     float acc[RT][2];
 #pragma unroll
     for (int r = 0; r < RT; ++r) { acc[r][0] = 0.f; acc[r][1] = 0.f; }
+
+    // fold mode: the sums over the runs folded so far (the threads with jp == 0 hold them)
+    float tot[RT][2];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) { tot[r][0] = 0.f; tot[r][1] = 0.f; }
+    // Adds the JP partial accumulators up in a fixed order, through `scratch` ([RT][hs] floats that nobody else uses now);
+    // the threads with jp == 0 then hold the sums.
+    auto sum_partials = [&](float* scratch) {
+        for (int src = 1; src < JP; ++src) {
+            if (c_active && jp == src) {
+#pragma unroll
+                for (int r = 0; r < RT; ++r) { scratch[r * hs + 2 * dp] = acc[r][0]; scratch[r * hs + 2 * dp + 1] = acc[r][1]; }
+            }
+            __syncthreads();
+            if (jp == 0) {
+#pragma unroll
+                for (int r = 0; r < RT; ++r) { acc[r][0] += scratch[r * hs + 2 * dp]; acc[r][1] += scratch[r * hs + 2 * dp + 1]; }
+            }
+            __syncthreads();
+        }
+    };
+    // The end of a run of keys: its sums join the sums of the runs before it, and the next run starts from nothing.  The
+    // staged keys are not needed any more when this is called (a barrier has passed): their memory is the scratch.
+    auto fold_run = [&]() {
+        sum_partials(reinterpret_cast<float*>(k_s));
+        if (tid < RT) {
+            const float m = m_s[tid];
+            float fa = 1.f, fb = 0.f;
+            if (m != -INFINITY) {                         // a run of which this row saw no key changes nothing
+                float m2;
+                fold_factors(Mt_s[tid], m, m2, fa, fb);
+                Lt_s[tid] = fold_value(Lt_s[tid], fa, l_s[tid], fb);
+                Mt_s[tid] = m2;
+            }
+            fa_s[tid] = fa; fb_s[tid] = fb;
+            m_s[tid] = -INFINITY; l_s[tid] = 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+            if (jp == 0 && fb_s[r] != 0.f) {
+                tot[r][0] = fold_value(tot[r][0], fa_s[r], acc[r][0], fb_s[r]);
+                tot[r][1] = fold_value(tot[r][1], fa_s[r], acc[r][1], fb_s[r]);
+            }
+            acc[r][0] = 0.f; acc[r][1] = 0.f;
+        }
+        if (hsp != hs)                                    // the scratch lay over the staged rows, whose padding is zero
+            for (int idx = tid; idx < 2 * KT * kstride; idx += ATT_THREADS) k_s[idx] = from_f32<T>(0.f);
+        __syncthreads();
+    };
 
     const int P = ATT_THREADS / KT;          // threads per key in phase A: 4, 8 or 16
     const int ja = tid / P, pa = tid - ja * P;
@@ -252,20 +318,17 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
             }
         }
         __syncthreads();
+        // a run of keys ends here and more keys follow (one workgroup walks several runs: a prompt step, or a decode step
+        // whose keys are not split): fold it
+        if (a.fold > 0 && a.n_splits == 1 && (j0 + KT) % a.fold == 0 && j0 + KT < hi) fold_run();
     }
 
-    // ---- sum the JP partial accumulators in a fixed order (q_s is free now) ----
-    for (int src = 1; src < JP; ++src) {
-        if (c_active && jp == src) {
-#pragma unroll
-            for (int r = 0; r < RT; ++r) { q_s[r * hs + 2 * dp] = acc[r][0]; q_s[r * hs + 2 * dp + 1] = acc[r][1]; }
-        }
-        __syncthreads();
-        if (jp == 0) {
-#pragma unroll
-            for (int r = 0; r < RT; ++r) { acc[r][0] += q_s[r * hs + 2 * dp]; acc[r][1] += q_s[r * hs + 2 * dp + 1]; }
-        }
-        __syncthreads();
+    const bool folded = a.fold > 0 && a.n_splits == 1;
+    if (folded) {
+        fold_run();                                       // the last run; the result is in tot, Mt_s, Lt_s
+    } else {
+        // ---- sum the JP partial accumulators in a fixed order (q_s is free now) ----
+        sum_partials(q_s);
     }
     if (jp != 0) return;
 #pragma unroll
@@ -277,11 +340,11 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
         const int head = kvh * G + hg;
         const size_t tok = (size_t)(tok0 + i);
         if (a.n_splits == 1) {
-            const float l = l_s[r];
+            const float l = folded ? Lt_s[r] : l_s[r];
             const float inv = l > 0.f ? 1.0f / l : 0.f;
             T* o = reinterpret_cast<T*>(a.out) + tok * a.out_stride + (size_t)head * hs + 2 * dp;
-            o[0] = from_f32<T>(acc[r][0] * inv);
-            o[1] = from_f32<T>(acc[r][1] * inv);
+            o[0] = from_f32<T>(__fmul_rn(folded ? tot[r][0] : acc[r][0], inv));
+            o[1] = from_f32<T>(__fmul_rn(folded ? tot[r][1] : acc[r][1], inv));
         } else {
             const size_t row = (tok * a.H + head) * a.n_splits + split;
             a.part_o[row * hs + 2 * dp] = acc[r][0];
@@ -313,9 +376,33 @@ __global__ void attn_combine_kernel(T* __restrict__ out, int out_stride, const f
     }
 }
 
+// The merge of a decode step whose keys were split in runs (fold mode): the runs' sums folded in run order with the
+// operations of fold_factors and fold_value, which is what a workgroup that walks all runs by itself does; runs without keys are passed over.
+template <typename T>
+__global__ void attn_fold_kernel(T* __restrict__ out, int out_stride, const float* __restrict__ part_o,
+                                 const float* __restrict__ part_ml, int H, int hs, int n_splits) {
+    const int row = blockIdx.x;               // token*H + head
+    const int tok = row / H, head = row - tok * H;
+    const float* ml = part_ml + (size_t)row * n_splits * 2;
+    for (int d = threadIdx.x; d < hs; d += blockDim.x) {
+        float M = -INFINITY, L = 0.f, O = 0.f;
+        for (int s = 0; s < n_splits; ++s) {
+            const float m = ml[2 * s];
+            if (m == -INFINITY) continue;
+            float m2, fa, fb;
+            fold_factors(M, m, m2, fa, fb);
+            L = fold_value(L, fa, ml[2 * s + 1], fb);
+            O = fold_value(O, fa, part_o[((size_t)row * n_splits + s) * hs + d], fb);
+            M = m2;
+        }
+        const float inv = L > 0.f ? 1.0f / L : 0.f;
+        out[(size_t)tok * out_stride + (size_t)head * hs + d] = from_f32<T>(__fmul_rn(O, inv));
+    }
+}
+
 static size_t attn_smem_bytes(int RT, int hs, int KT, int elt) {
     const int hsp = (hs + 7) & ~7;
-    return (size_t)(RT * hsp + 2 * RT * KT + 48) * sizeof(float) + (size_t)2 * KT * (hsp * elt + 16);
+    return (size_t)(RT * hsp + 2 * RT * KT + 112) * sizeof(float) + (size_t)2 * KT * (hsp * elt + 16);
 }
 
 template <typename T, int RT>
@@ -360,8 +447,10 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
                             int bt_stride, const int* seq_lens, const int* tiles, int n_tiles,
                             int n_tokens, int H, int Hkv, int hs, int RT, int GT, int window,
                             float scale, int n_splits, int chunk, float* part_o, float* part_ml,
-                            int v_transposed, const int* max_len, hipStream_t s) {
+                            int v_transposed, const int* max_len, int fold, hipStream_t s) {
     if (n_tiles <= 0 || n_tokens <= 0 || H <= 0 || Hkv <= 0 || H % Hkv) return BN_ERR_ARG;
+    // fold mode: runs of whole pages; a split is one run, and the runs' length does not follow the longest sequence
+    if (fold < 0 || fold % BN_PAGE || (fold > 0 && n_splits > 1 && (chunk != fold || max_len))) return BN_ERR_ARG;
     if (hs < 2 || hs > BN_MAX_HEAD_DIM || hs % 2) return BN_ERR_ARG;
     if (GT <= 0 || GT > RT || (GT & (GT - 1)) || RT > 16 || (RT & (RT - 1))) return BN_ERR_ARG;
     if (n_splits < 1 || window < 0) return BN_ERR_ARG;
@@ -378,6 +467,7 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
     a.n_splits = n_splits; a.chunk = n_splits > 1 ? chunk : 0x40000000;
     a.scale = scale;
     a.v_transposed = v_transposed;
+    a.fold = fold;
     a.KT = bn_attn_rows_key_tile(dtype, hs);
     if (a.KT == 0) return BN_ERR_ARG;
     int rc;
@@ -385,6 +475,15 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
     else if (dtype == BN_DT_BF16) rc = launch_rows_rt<bf16>(a, RT, n_tiles, s);
     else return BN_ERR_DTYPE;
     if (rc != 0 || n_splits == 1) return rc;
+    if (fold > 0) {
+        if (dtype == BN_DT_F32)
+            hipLaunchKernelGGL(attn_fold_kernel<float>, dim3(n_tokens * H), dim3(64), 0, s, (float*)out, out_stride, part_o,
+                               part_ml, H, hs, n_splits);
+        else
+            hipLaunchKernelGGL(attn_fold_kernel<bf16>, dim3(n_tokens * H), dim3(64), 0, s, (bf16*)out, out_stride, part_o,
+                               part_ml, H, hs, n_splits);
+        return bn_launch_status();
+    }
     if (dtype == BN_DT_F32)
         hipLaunchKernelGGL(attn_combine_kernel<float>, dim3(n_tokens * H), dim3(64), 0, s, (float*)out,
                            out_stride, part_o, part_ml, H, hs, n_splits);

@@ -10,6 +10,10 @@
 // Decode attention splits a sequence's keys over workgroups in runs of at least this many pages: shorter
 // runs cost more in merging than they gain in parallelism (measured at batch 1, 8 and 64 of an 8B shape).
 #define BN_SPLIT_MIN_PAGES 4
+// A float32 cache's keys are summed in runs of this many positions (whole pages, counted from position 0), each run by
+// itself and the runs folded in order: a decode step then spreads a long sequence's runs over workgroups and still forms
+// every sum in the order in which a prompt step forms it, so that float32 logits do not depend on how a sequence was cut.
+#define BN_F32_FOLD_KEYS 2048
 #define BN_MAX_HEAD_DIM 256   // the attention kernels take every even head size up to this; the configuration reads this line too
 
 // error codes returned by the extern "C" entry points (0 = ok, >0 = hipError_t)

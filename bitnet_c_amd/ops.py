@@ -18,6 +18,7 @@ import torch
 from .csrc import build as _build
 
 PAGE = _build.header_constant("BN_PAGE")                         # tokens per cache page: defined once, in csrc/common.h
+F32_FOLD_KEYS = _build.header_constant("BN_F32_FOLD_KEYS")       # a float32 cache's keys are summed in runs of this many
 SPLIT_MIN_PAGES = _build.header_constant("BN_SPLIT_MIN_PAGES")   # shortest run of pages that decode attention splits off
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 
@@ -53,7 +54,7 @@ _SIGNATURES = {
         "bn_attn_rows_key_tile": [c_int, c_int],
         "bn_attn_rows": [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
-                         c_void_p, c_void_p, c_int, c_void_p, c_void_p],
+                         c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p],
     },
     "attn_mfma": {
         "bn_attn_mfma_supports": [c_int],
@@ -845,11 +846,11 @@ DECODE_TARGET_WGS = int(os.environ.get("BITNET_DECODE_WGS", "512"))
 
 def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int, dtype=None):
     """(n_splits, chunk): how the keys of a decode step are cut so that the launch fills the
-    chip.  A function of the batch's shape and of max_len alone.  A float32 cache is never split:
-    there a query's keys are summed in one order, the prompt form's, however the step was cut, so
-    that float32 logits are equal bit for bit under every cut."""
+    chip.  A function of the batch's shape and of max_len alone.  A float32 cache is cut in runs of F32_FOLD_KEYS
+    positions whatever the batch: both forms of the float32 kernel sum a query's keys run by run and fold the runs in
+    order, so a decode step may give every run a workgroup and float32 logits stay equal bit for bit under every cut."""
     if dtype == torch.float32:
-        return 1, 0
+        return max(1, (max_len + F32_FOLD_KEYS - 1) // F32_FOLD_KEYS), F32_FOLD_KEYS
     RT, GT, _ = attention_row_shape(H, Hkv, True)
     G = H // Hkv
     wgs = max(1, n_seqs * Hkv * ((G + GT - 1) // GT))
@@ -931,6 +932,11 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     if T == 0 or n_tiles == 0:
         return
     part_o = part_ml = None
+    fold = F32_FOLD_KEYS if qkv.dtype == torch.float32 else 0       # float32: runs of keys folded in order, in both forms
+    if fold:
+        if decode and n_splits > 1 and chunk != fold:
+            raise KernelError(f"attention: a float32 cache's keys are split in runs of {fold}, not {chunk}")
+        max_len_dev = None                                          # and the runs do not follow the longest sequence
     if max_len_dev is not None:
         _dev(max_len_dev, "max_len_dev", torch.int32)
         if not decode or max_len_dev.numel() != 1:
@@ -942,8 +948,8 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
         if n_splits * chunk < block_table.shape[1] * PAGE:
             raise KernelError(f"attention: {n_splits} splits of {chunk} keys do not cover the "
                               f"{block_table.shape[1]} pages of the block table")
-        if n_splits > 64:
-            raise KernelError("attention: at most 64 splits")
+        if n_splits > (1024 if fold else 64):
+            raise KernelError("attention: at most 64 splits (1,024 runs of a float32 cache)")
         part_o = torch.empty((T * H * n_splits, hs), dtype=torch.float32, device=qkv.device)
         part_ml = torch.empty((T * H * n_splits, 2), dtype=torch.float32, device=qkv.device)
     po = part_o.data_ptr() if part_o is not None else None
@@ -993,7 +999,7 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
         _code(qkv.dtype), qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * hs,
         k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1],
         sl, tl, n_tiles, T, H, Hkv, hs, RT, GT, int(window), float(scale), int(n_splits), int(chunk),
-        po, pm, int(vt), max_len_dev.data_ptr() if max_len_dev is not None else None, _stream()), "attention")
+        po, pm, int(vt), max_len_dev.data_ptr() if max_len_dev is not None else None, int(fold), _stream()), "attention")
 
 
 # --------------------------------------------------------------------------------------

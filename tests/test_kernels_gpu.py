@@ -882,9 +882,11 @@ def test_attention_decode_form(dtype, H, Hkv, hs, window, force_splits, force_ve
     lens = torch.tensor([p + 1 for p in lens_before] + [0, 0], dtype=torch.int32).cuda()
     max_len = bt.shape[1] * 64
     if force_splits == 0:
-        n_splits, chunk = ops.decode_splits(B + 2, H, Hkv, max_len)
+        n_splits, chunk = ops.decode_splits(B + 2, H, Hkv, max_len, dtype)
     elif force_splits == 1:
         n_splits, chunk = 1, 0
+    elif dtype == torch.float32:
+        pytest.skip("a float32 cache's keys are cut in the kernel's own runs and no others")
     else:
         chunk = ((max_len + force_splits - 1) // force_splits + 63) // 64 * 64
         n_splits = (max_len + chunk - 1) // chunk
@@ -937,7 +939,8 @@ def test_attention_finds_a_far_key(dtype):
         q[0, :, 0] = 16.0                                   # score 256 * scale at `far`, about 0 elsewhere
         kp, vp, bt = _paged([k], [v], dtype, 20, far)
         qkv = q.reshape(1, H * hs).contiguous().cuda()
-        for n_splits, chunk in ((1, 0), (4, 256), (15, 64)):
+        # (a float32 cache's keys are cut in the kernel's own runs of 2,048 and no others)
+        for n_splits, chunk in ((1, 0), (4, 256), (15, 64)) if dtype == torch.bfloat16 else ((1, 0), (1, ops.F32_FOLD_KEYS)):
             out = torch.empty((1, H * hs), dtype=dtype).cuda()
             ops.attention(qkv, out, kp.cuda(), vp.cuda(), bt.cuda(), H, Hkv, hs, 1 / math.sqrt(hs),
                           seq_lens=torch.tensor([L], dtype=torch.int32).cuda(), n_splits=n_splits, chunk=chunk)
@@ -1024,12 +1027,30 @@ def test_attention_over_a_long_context(dtype, H, Hkv, hs):
     ref = plain_rows(L - n_new)
     check(out, ref)
     # one decoded token at the last position, split as the engine splits it
-    n_splits, chunk = ops.decode_splits(1, H, Hkv, bt.shape[1] * 64)
+    n_splits, chunk = ops.decode_splits(1, H, Hkv, bt.shape[1] * 64, dtype)
     assert n_splits > 1
     out1 = torch.full((1, H * hs), float("nan"), dtype=dtype).cuda()
     ops.attention(qkv[-1:].contiguous(), out1, kp, vp, bt, H, Hkv, hs, scale,
                   seq_lens=torch.tensor([L], dtype=torch.int32).cuda(), n_splits=n_splits, chunk=chunk)
     check(out1, ref[-1:])
+    if dtype == torch.float32:
+        # float32 keys are summed in runs of 2,048 that are folded in order, by one workgroup that walks them all (the
+        # prompt form, a decode row that is not split) or by a workgroup a run and the fold kernel: the same bits
+        assert (n_splits, chunk) == ((bt.shape[1] * 64 + ops.F32_FOLD_KEYS - 1) // ops.F32_FOLD_KEYS, ops.F32_FOLD_KEYS)
+        assert torch.equal(out1, out[-1:])
+        out2 = torch.full((1, H * hs), float("nan"), dtype=dtype).cuda()
+        ops.attention(qkv[-1:].contiguous(), out2, kp, vp, bt, H, Hkv, hs, scale,
+                      seq_lens=torch.tensor([L], dtype=torch.int32).cuda(), n_splits=1, chunk=0)
+        assert torch.equal(out2, out1)
+        wide = torch.zeros((1, 2048), dtype=torch.int32).cuda()            # a table for 131,072 keys: 64 runs, most of them empty
+        wide[:, :bt.shape[1]] = bt
+        out3 = torch.full((1, H * hs), float("nan"), dtype=dtype).cuda()
+        ops.attention(qkv[-1:].contiguous(), out3, kp, vp, wide, H, Hkv, hs, scale,
+                      seq_lens=torch.tensor([L], dtype=torch.int32).cuda(), n_splits=64, chunk=ops.F32_FOLD_KEYS)
+        assert torch.equal(out3, out1)
+        with pytest.raises(ops.KernelError):                               # runs of another length are refused
+            ops.attention(qkv[-1:].contiguous(), out3, kp, vp, bt, H, Hkv, hs, scale,
+                          seq_lens=torch.tensor([L], dtype=torch.int32).cuda(), n_splits=5, chunk=4096)
 
 
 # ---------------------------------------------------------------------------------------
