@@ -136,8 +136,28 @@ def _kernel_attention_decode(H=32, Hkv=8, hs=128):
         torch.cuda.synchronize()
 
 
+def _kernel_mid(rows=64, copies=3):
+    """The products of a decode step of 64 rows, every weight matrix read cold: gate/up through this library's own kernel
+    with the SwiGLU epilogue (what runs when the library may not be called) and through the library, the feed-forward's
+    last product and the output projection as partial sums."""
+    import torch
+    from bitnet_c_amd import ops
+    x = torch.randn(rows, 4096, device="cuda:0", dtype=torch.bfloat16)
+    ws = [torch.randn(28672, 4096, device="cuda:0", dtype=torch.bfloat16) * 0.02 for _ in range(copies)]
+    for w in ws:
+        ops.linear_swiglu(x, w, True, allow_library=False)
+    for w in ws:
+        ops.swiglu(torch.matmul(x, w.t()), True)
+    del ws
+    for n, k in ((4096, 14336), (4096, 4096)):
+        xs = torch.randn(rows, k, device="cuda:0", dtype=torch.bfloat16)
+        for _ in range(copies):
+            ops.linear_partial_sums(xs, torch.randn(n, k, device="cuda:0", dtype=torch.bfloat16) * 0.02)
+    torch.cuda.synchronize()
+
+
 KERNEL_WORKLOADS = {"skinny": _kernel_skinny, "gemm": _kernel_gemm, "attention_prompt": _kernel_attention_prompt,
-                    "attention_decode": _kernel_attention_decode}
+                    "attention_decode": _kernel_attention_decode, "mid": _kernel_mid}
 
 
 def main() -> int:

@@ -225,6 +225,14 @@ __global__ __launch_bounds__(256) void rmsnorm_ssq_kernel(const float* __restric
     }
 }
 
+// out[r, :] = x[rows[r], :] in type T: the wanted rows of the stream for an output matrix that no norm precedes
+template <typename T>
+__global__ void gather_rows_kernel(T* __restrict__ out, const float* __restrict__ x, const int* __restrict__ rows, int dim) {
+    const float* xr = x + (size_t)rows[blockIdx.x] * dim;
+    T* o = out + (size_t)blockIdx.x * dim;
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) o[i] = from_f32<T>(xr[i]);
+}
+
 // x[t, :] += delta[t, :]   (src/transformer/cpu_backend.c:252-256)
 template <typename T>
 __global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__ delta, size_t n) {
@@ -325,6 +333,15 @@ extern "C" int bn_embed_gather(int dtype, void* x, const void* table, const int*
     if (dtype == BN_DT_F32) return embed_gather_t<float>(x, table, tokens, n_tokens, dim, vocab, scale, s);
     if (dtype == BN_DT_BF16) return embed_gather_t<bf16>(x, table, tokens, n_tokens, dim, vocab, scale, s);
     return BN_ERR_DTYPE;
+}
+
+// out [n_rows, dim] (dtype) = the rows `rows` of x [., dim] (float32)
+extern "C" int bn_gather_rows(int dtype, void* out, const float* x, const int* rows, int n_rows, int dim, hipStream_t s) {
+    if (n_rows <= 0 || dim <= 0 || !out || !x || !rows) return BN_ERR_ARG;
+    if (dtype == BN_DT_F32) hipLaunchKernelGGL(gather_rows_kernel<float>, dim3(n_rows), dim3(256), 0, s, (float*)out, x, rows, dim);
+    else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(gather_rows_kernel<bf16>, dim3(n_rows), dim3(256), 0, s, (bf16*)out, x, rows, dim);
+    else return BN_ERR_DTYPE;
+    return bn_launch_status();
 }
 
 extern "C" int bn_softcap(float* x, long long n, float cap, hipStream_t s) {

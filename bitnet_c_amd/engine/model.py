@@ -21,7 +21,8 @@ class DecoderModel:
         plan.validate()
         self.plan, self.dtype, self.device = plan, dtype, torch.device(device)
         self.blocks = [BLOCKS.build(lp.block) for lp in plan.layers]
-        self.final_norm = NORMS.build(plan.final_norm)
+        self.final_norm = NORMS.build(plan.final_norm) if plan.final_norm is not None else None
+        self.lm_head_bias = None         # [V] float32, when the plan names one
         self.embedding = None            # [V, D] in the compute dtype
         self.lm_head = None              # [V, D]; the embedding itself when tied
 
@@ -37,7 +38,11 @@ class DecoderModel:
             blk.load(local, self.device, self.dtype)
             del local
             done(lp.names.values())
-        self.final_norm.load({ln: tensors[fn] for ln, fn in p.final_norm_names.items()}, self.device, self.dtype)
+        if self.final_norm is not None:
+            self.final_norm.load({ln: tensors[fn] for ln, fn in p.final_norm_names.items()}, self.device, self.dtype)
+        if p.lm_head_bias_name is not None:
+            self.lm_head_bias = upload(tensors[p.lm_head_bias_name], self.device, torch.float32)
+            done([p.lm_head_bias_name])
         self.embedding = upload(tensors[p.embedding_name], self.device, self.dtype)
         done([p.embedding_name])
         if p.lm_head_name is None:
@@ -68,6 +73,7 @@ class DecoderModel:
             walk(blk)
         walk(self.final_norm)
         add(self.lm_head)
+        add(self.lm_head_bias)
         return total
 
     # ---- cache needs -------------------------------------------------------------------
@@ -85,8 +91,13 @@ class DecoderModel:
             ctx.entry = i
             self.blocks[e.layer].forward(stream, ctx, views[i])
         # final norm on the wanted rows only, then the output matrix (src/transformer/logits.c:249-314)
-        h = stream.normed(self.final_norm, self.dtype, rows=ctx.want_rows)
+        if self.final_norm is not None:
+            h = stream.normed(self.final_norm, self.dtype, rows=ctx.want_rows)
+        else:
+            h = ops.gather_rows(stream.flush(), ctx.want_rows, self.dtype)
         logits = ops.linear(h, self.lm_head, torch.float32)
+        if self.lm_head_bias is not None and logits.shape[0]:
+            ops.bias_add(logits, self.lm_head_bias)
         if self.plan.logit_softcap > 0:                            # src/transformer/logits.c:325-333
             ops.softcap_(logits, self.plan.logit_softcap)
         return logits

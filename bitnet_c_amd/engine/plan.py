@@ -35,7 +35,7 @@ class ModelPlan:
     hidden_size: int
     layers: List[LayerPlan]
     schedule: List[ScheduleEntry]
-    final_norm: PartSpec
+    final_norm: Optional[PartSpec]       # the norm in front of the output matrix; None: the architecture has none
     embedding_name: str
     final_norm_names: Dict[str, str]
     lm_head_name: Optional[str]          # None: the output matrix is the embedding matrix (tied)
@@ -45,6 +45,7 @@ class ModelPlan:
     # row, src/transformer/logits.c:325-333 bounds the logits); 1 and 0 leave this architecture's values as they are.
     embedding_multiplier: float = 1.0    # the embedding row times this before the first block
     logit_softcap: float = 0.0           # > 0: logits = cap * tanh(logits / cap)
+    lm_head_bias_name: Optional[str] = None   # a bias [vocab] added to the logits (before the soft-cap); None: none
 
     def validate(self) -> None:
         if not self.embedding_multiplier > 0 or self.logit_softcap < 0:
@@ -77,9 +78,12 @@ class ModelPlan:
                 if local not in lp.names:
                     raise ValueError(f"the plan gives no tensor name for {local!r}")
                 put(lp.names[local], spec.shape, spec.init, spec.optional)
-        norm = NORMS.build(self.final_norm)
-        for local, spec in norm.tensors().items():
-            put(self.final_norm_names[local], spec.shape, spec.init, spec.optional)
+        if self.final_norm is not None:
+            norm = NORMS.build(self.final_norm)
+            for local, spec in norm.tensors().items():
+                put(self.final_norm_names[local], spec.shape, spec.init, spec.optional)
         if self.lm_head_name is not None:
             put(self.lm_head_name, (self.vocab_size, self.hidden_size), "normal")
+        if self.lm_head_bias_name is not None:
+            put(self.lm_head_bias_name, (self.vocab_size,), "normal")
         return out

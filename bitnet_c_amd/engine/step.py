@@ -375,7 +375,7 @@ class Engine:
         # every later one is a replay.  Only when every part of the model says that its prompt work can be recorded
         # (Part.prompt_capturable); prompt_graphs False keeps prompt steps eager.
         self.prompt_graphs = (all(getattr(b, "prompt_capturable", False) for b in model.blocks)
-                              and getattr(model.final_norm, "prompt_capturable", False))
+                              and (model.final_norm is None or getattr(model.final_norm, "prompt_capturable", False)))
         self._prompt_graphs: Dict[tuple, _PromptGraph] = {}     # in order of last use
         self._prompt_seen: Dict[tuple, int] = {}
         self._prompt_lists = None                                # (tile sizes asked for, page tiles asked for) of an eager prompt step

@@ -31,6 +31,7 @@ _SIGNATURES = {
     "elementwise": {
         "bn_embed_gather": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
         "bn_softcap": [c_void_p, c_longlong, c_float, c_void_p],
+        "bn_gather_rows": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "bn_add_rmsnorm": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p],
         "bn_residual_add": [c_int, c_void_p, c_void_p, c_longlong, c_void_p],
         "bn_add_rmsnorm_parts": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
@@ -198,6 +199,21 @@ def embed_gather(table: torch.Tensor, tokens: torch.Tensor, scale: float = 1.0) 
                                                  tokens.data_ptr(), n, dim, table.shape[0], float(scale), _stream()),
            "embed_gather")
     return x
+
+
+def gather_rows(x: torch.Tensor, rows: torch.Tensor, out_dtype) -> torch.Tensor:
+    """The rows `rows` (int32) of the float32 stream x [T, D], in out_dtype: what an output matrix reads when the
+    architecture puts no norm in front of it."""
+    require_gpu()
+    _dev(x, "x", torch.float32, 2)
+    _dev(rows, "rows", torch.int32, 1)
+    if not x.is_contiguous() or not rows.is_contiguous():
+        raise KernelError("gather_rows: x and rows must be contiguous")
+    out = torch.empty((rows.numel(), x.shape[1]), dtype=out_dtype, device=x.device)
+    if rows.numel():
+        _check(_fn("elementwise", "bn_gather_rows")(_code(out_dtype), out.data_ptr(), x.data_ptr(), rows.data_ptr(), rows.numel(),
+                                                    x.shape[1], _stream()), "gather_rows")
+    return out
 
 
 def softcap_(logits: torch.Tensor, cap: float) -> None:

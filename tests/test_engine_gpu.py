@@ -786,6 +786,59 @@ def test_prompt_steps_are_replayed_from_graphs(model_folders, name, dtype, monke
             assert rel_err(a, b) < TOL[dtype], i
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_graph_row_that_changes_its_owner_holds_nothing_of_the_former_one(model_folders, dtype):
+    """A captured decode step keeps a block table at the engine's full width.  A long sequence decodes in row 0, ends, and a
+    short one takes the row (and later no one does: the batch shrinks): the row's entries beyond the new owner's pages are
+    zero, as the eager step's table has them, and a replayed step writes nothing but the new keys and values of the
+    sequences it holds: every other place of the cache, the former owner's pages among them, keeps its bits."""
+    import bitnet_c_amd as bn
+    from bitnet_c_amd.cache import PAGE
+    folder = model_folders("A", dtype)
+    eng = bn.Engine.from_folder(folder, dtype=dtype, max_tokens=64 * 16)
+    vocab = eng.vocab_size
+    long_, other, short = _requests(vocab, 55, [200, 70, 5])
+    a, b = eng.new_sequence(), eng.new_sequence()
+    eng.step([bn.StepEntry(a, long_, []), bn.StepEntry(b, other, [])])
+    eng.step([bn.StepEntry(a, [1], [0]), bn.StepEntry(b, [2], [0])])           # a graph of two rows; row 0 holds a's four pages
+    g = eng._graphs[2]
+    assert int((g.tables_np[0, 0] != 0).sum()) >= 3
+    eng.release(a)
+    c = eng.new_sequence()
+    eng.step([bn.StepEntry(c, short, [])])
+    grp = eng.cache.groups[0]
+
+    def step_and_diff(entries):
+        k0, v0 = grp.k.clone(), grp.v.clone()
+        out = eng.step(entries)
+        torch.cuda.synchronize()
+        changed = ((grp.k != k0) | (grp.k.isnan() != k0.isnan())).any(dim=0)      # [pages, Hkv, PAGE, hs] over the entries
+        return out, {(int(p), int(o)) for p, _, o, _ in changed.nonzero().tolist()}, v0
+
+    want = lambda slots: {(eng.cache.pages_of(0, s)[(eng.length(s) - 1) // PAGE], (eng.length(s) - 1) % PAGE) for s in slots}
+    out, places, _ = step_and_diff([bn.StepEntry(c, [3], [0]), bn.StepEntry(b, [4], [0])])   # c in the row that a had
+    assert places == want([c, b])
+    assert len(eng.cache.pages_of(0, c)) == 1 and int((g.tables_np[0, 0, 1:] != 0).sum()) == 0
+    # and the logits are those of the same sequences in an engine without graphs
+    ref = bn.Engine.from_folder(folder, dtype=dtype, max_tokens=64 * 16, use_graphs=False)
+    rc, rb = ref.new_sequence(), ref.new_sequence()
+    ref.step([bn.StepEntry(rc, short, []), bn.StepEntry(rb, other + [2], [])])
+    want_out = ref.step([bn.StepEntry(rc, [3], [0]), bn.StepEntry(rb, [4], [0])])
+    assert torch.equal(out, want_out) if dtype == torch.float32 else rel_err(out, want_out) < TOL[dtype]
+    # four sequences in a graph of four rows, then three: row 2 goes from a sequence of three pages to one of two, and
+    # row 3 to nobody
+    d, e = eng.new_sequence(), eng.new_sequence()
+    eng.step([bn.StepEntry(d, other[:60] + long_[:70], []), bn.StepEntry(e, long_[:100], [])])
+    eng.step([bn.StepEntry(s, [5 + i], [0]) for i, s in enumerate((c, b, d, e))])
+    g4 = eng._graphs[4]
+    assert int((g4.tables_np[0, 2] != 0).sum()) >= 2 and int((g4.tables_np[0, 3] != 0).sum()) >= 1
+    eng.release(d)
+    _, places, _ = step_and_diff([bn.StepEntry(s, [9 + i], [0]) for i, s in enumerate((c, b, e))])
+    assert places == want([c, b, e])
+    assert int((g4.tables_np[0, 2, 2:] != 0).sum()) == 0 and int((g4.tables_np[0, 3] != 0).sum()) == 0
+    eng.cache.check()
+
+
 def test_decode_steps_of_many_sequences_are_replayed_from_graphs(model_folders):
     """300 sequences decode together: more than the largest captured step holds (256 rows), so the step is replayed in
     two pieces (256 rows and 64 rows for the other 44); then 70 of them go on (a captured step of 128 rows).  float32:

@@ -547,6 +547,67 @@ def test_an_architecture_with_an_embedding_multiplier_and_a_logit_softcap(tmp_pa
         assert rel_err(pl.forward(c, W, r, rounded, softcap=cap), want) > 10 * TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_an_architecture_without_a_final_norm_and_with_a_bias_on_its_output_matrix(tmp_path, dtype):
+    """The model's skeleton is the plan's to say as well: a toy architecture's builder drops the norm in front of the
+    output matrix and names a bias for it.  The folder then holds no final norm and one bias tensor; prompts, decoded
+    tokens (from graphs) and a prompt step from its graph equal the plain layers followed by W x + b on the stream itself."""
+    from dataclasses import replace
+    from bitnet_c_amd import Engine, StepEntry
+    from bitnet_c_amd.config import Architecture, LlamaConfig, register_architecture
+    from bitnet_c_amd.config.base import _ARCHITECTURES
+    from bitnet_c_amd.config.llama_plan import build_llama_plan
+    from bitnet_c_amd.weights import write_model_folder
+    from conftest import TINY_A
+
+    class BareConfig(LlamaConfig):
+        def to_dict(self):
+            return dict(LlamaConfig.to_dict(self), model_type="toy_bare_head", architectures=["ToyBareHead"])
+
+    if "toy_bare_head" not in _ARCHITECTURES:
+        register_architecture(Architecture(
+            "toy_bare_head", BareConfig,
+            lambda c: replace(build_llama_plan(c), final_norm=None, final_norm_names={}, lm_head_bias_name="lm_head.bias")))
+    cfg = BareConfig.from_dict(dict(TINY_A, model_type="toy_bare_head"))
+    folder = write_model_folder(str(tmp_path / "bare"), cfg, 25, dtype)
+    from safetensors.torch import load_file
+    names = set(load_file(os.path.join(folder, "model.safetensors")))
+    assert "model.norm.weight" not in names and "lm_head.bias" in names
+    eng = Engine.from_folder(folder, dtype=dtype, max_tokens=1024)
+    assert eng.model.final_norm is None and eng.prompt_graphs
+    c, W = pl.read_config(folder), pl.read_weights(folder)
+    rt = torch.bfloat16 if dtype == torch.bfloat16 else None
+    r_ = (lambda x: x) if rt is None else (lambda x: x.to(rt).float())
+
+    def plain(toks):
+        x = W["model.embed_tokens.weight"][torch.tensor(toks)].float()
+        inv = pl.rope_inv_freq(c["head_dim"], c["theta"], c["rope_scaling"])
+        for l in range(c["layers"]):
+            x = pl.decoder_layer(x, torch.arange(len(toks)), W, l, c, inv, rt)
+        return pl.linear(r_(x), W["lm_head.weight"].float(), W["lm_head.bias"].float())
+
+    rnd = random.Random(26)
+    reqs = [[rnd.randrange(cfg.vocab_size) for _ in range(n)] for n in (30, 9)]
+    for round_ in range(3):                       # the third round's prompt step is a replay of the second's graph
+        slots = [eng.new_sequence() for _ in reqs]
+        out = eng.step([StepEntry(s, r[:-3], list(range(len(r) - 3))) for s, r in zip(slots, reqs)])
+        got, o = [[] for _ in reqs], 0
+        for i, r in enumerate(reqs):
+            got[i].append(out[o:o + len(r) - 3])
+            o += len(r) - 3
+        for k in range(3):
+            out = eng.step([StepEntry(s, [r[len(r) - 3 + k]], [0]) for s, r in zip(slots, reqs)])
+            for i in range(2):
+                got[i].append(out[i:i + 1].clone())
+        for i, r in enumerate(reqs):
+            want = plain(r)
+            assert rel_err(torch.cat(got[i]), want) < TOL[dtype], (round_, i)
+            assert rel_err(pl.forward(c, dict(W, **{"model.norm.weight": torch.ones(c["dim"])}), r, rt), want) > 10 * TOL[dtype]
+        for s in slots:
+            eng.release(s)
+    assert eng._prompt_graphs and eng._graphs
+
+
 def test_a_windowed_group_beside_a_full_one_through_the_engine(tmp_path):
     """A toy architecture whose odd layers see only the last 70 positions: two cache groups with
     storage of their own; the windowed one gives pages back while sequences grow, and the logits
