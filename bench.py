@@ -216,7 +216,8 @@ def main() -> int:
     model.load(tensors)
     del tensors
     torch.cuda.empty_cache()
-    print(f"[bench] model built in {time.time() - t0:.1f} s, weights {model.weight_bytes() / 1e9:.2f} GB",
+    print(f"[bench] model built in {time.time() - t0:.1f} s, weights {model.weight_bytes() / 1e9:.2f} GB"
+          + (f", and {model.streamed_bytes() / 1e9:.2f} GB of streamed copies" if model.has_streamed else ""),
           file=sys.stderr, flush=True)
 
     max_batch = max(args.batch, 1 if args.no_points else 64)
@@ -332,7 +333,7 @@ def main() -> int:
                    "vocab": cfg.vocab_size, "rope_theta": cfg.rope_theta, "rope_scaling": "llama3 f8 l1 h4 o8192" if cfg.rope_scaling else "none",
                    "rms_norm_eps": cfg.rms_norm_eps, "tied": cfg.tie_word_embeddings,
                    "global_batch": args.batch, "seq_len": CONTEXT, "prompt_lens": f"U[{len_lo},{len_hi}]",
-                   "prefill_tokens": PREFILL, "parallelism": "none (1 GPU)"},
+                   "prefill_tokens": PREFILL, "streamed_weights": model.has_streamed, "parallelism": "none (1 GPU)"},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBS, 4), "gb_per_step": round(bytes_step / 1e9, 3)},

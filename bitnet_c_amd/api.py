@@ -50,10 +50,13 @@ class LLM:
 
 
 def load(folder: str, dtype="bfloat16", max_tokens: int = 8192, device: str = "cuda:0", max_seq_len: int = 0,
-         use_graphs: bool = True, n_seqs: int = 1) -> LLM:
+         use_graphs: bool = True, n_seqs: int = 1, streamed_weights=None) -> LLM:
     """max_tokens: cached positions of all live sequences together (sizes the cache); 0: room for n_seqs sequences
     of the longest length there can be, or what fits into the device's free memory if that is less.
-    max_seq_len: the longest sequence (the reference's --maxseq), 0 = the model's limit."""
+    max_seq_len: the longest sequence (the reference's --maxseq), 0 = the model's limit.
+    streamed_weights: keep every weight matrix a second time in the order the decode kernels read it (faster decode
+    steps for the matrices' memory once more); None: where half of the device's memory stays free."""
     if dtype not in _DTYPES:
         raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}")
-    return LLM(Engine.from_folder(folder, _DTYPES[dtype], max_tokens, device, max_seq_len, 0, use_graphs, n_seqs))
+    return LLM(Engine.from_folder(folder, _DTYPES[dtype], max_tokens, device, max_seq_len, 0, use_graphs, n_seqs,
+                                  streamed_weights))

@@ -21,6 +21,11 @@
 // a row), parks it in a region of shared memory of its own (no workgroup barrier) and reads the
 // operand fragments from there; the vector memory pipe is left to the weights.
 //
+// TILED: W is the streamed copy of the matrix (common.h: tiles of 16 rows x 32 columns in the lanes' order, 1 KB each);
+// a load of a wave is then one tile, 1 KB of consecutive bytes, and ldw the number of tiles along K.  Measured against
+// the row-major matrix at 8 rows of an 8B shape: QKV 14.3 -> 13.2 us, output projection 10.7 -> 9.3, gate/up 49.5 ->
+// 43.9, down 28.0 -> 24.0.
+//
 // Needs K % 8 == 0 and 16-byte aligned rows; other shapes go to the tiled kernel.
 #include "common.h"
 
@@ -33,7 +38,7 @@ __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast
 
 #define SK_XROW 528           // bytes between rows of a wave's staged X chunk (512 + 16: conflict-free 16-byte reads)
 
-template <int MT, bool DUAL, typename TO, bool GLU8 = false, bool XS = false>
+template <int MT, bool DUAL, typename TO, bool GLU8 = false, bool XS = false, bool TILED = false>
 __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                            TO* __restrict__ Y, int M, int N, int K, int ldx,
                                                            int ldw, int ldy, int up_off, int act) {
@@ -44,7 +49,7 @@ __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_ke
     const int i = lane & 15, g = lane >> 4;
     const int n0 = blockIdx.x * 16;
     const int n = min(n0 + i, N - 1);                 // clamp: rows past N are computed and dropped
-    const bf16* wrow = W + (size_t)n * ldw;
+    const bf16* wrow = TILED ? W + (size_t)blockIdx.x * ldw * BN_STREAM_TILE + lane * 8 : W + (size_t)n * ldw;
     const bf16* urow = DUAL ? W + (size_t)(up_off + n) * ldw : nullptr;
 
     f32x4 acc[NA];
@@ -70,7 +75,11 @@ __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_ke
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int k = kb + j * 32;
-            wv[j] = (k < K) ? *reinterpret_cast<const uint4*>(wrow + k) : make_uint4(0, 0, 0, 0);
+            if (TILED)          // tile kc / 32 + j of this block of rows; its columns past K hold zeros
+                wv[j] = (kc + j * 32 < K) ? *reinterpret_cast<const uint4*>(wrow + (size_t)((kc >> 5) + j) * BN_STREAM_TILE)
+                                          : make_uint4(0, 0, 0, 0);
+            else
+                wv[j] = (k < K) ? *reinterpret_cast<const uint4*>(wrow + k) : make_uint4(0, 0, 0, 0);
             if (DUAL) uv[j] = (k < K) ? *reinterpret_cast<const uint4*>(urow + k) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
@@ -160,7 +169,7 @@ struct SkinnyFused {
     int ld_resid, ld_rb;
 };
 
-template <bool GLU8, bool PRE, bool RES, int SL>
+template <bool GLU8, bool PRE, bool RES, int SL, bool TILED>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, bf16* __restrict__ Y, int M, int N,
                               int K, int ldx, int ldw, int ldy, int tile_cols, int act, SkinnyFused f) {
@@ -173,7 +182,8 @@ void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict
     const int n0 = blockIdx.x * tile_cols;
     const bool col = i < tile_cols;
     const int n = min(n0 + i, N - 1);
-    const bf16* wrow = W + (size_t)n * ldw;
+    // tiled: tile_cols is 16 and the workgroup's rows are one row of tiles
+    const bf16* wrow = TILED ? W + (size_t)blockIdx.x * ldw * BN_STREAM_TILE + lane * 8 : W + (size_t)n * ldw;
     float* scale_s = red + NW * 256;
     unsigned char* xs = reinterpret_cast<unsigned char*>(red + NW * 256 + 16) + (size_t)wave * M * SK_XROW;
 
@@ -191,7 +201,11 @@ void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int k = kb + j * 32;
-            wv[j] = (col && k < K) ? *reinterpret_cast<const uint4*>(wrow + k) : make_uint4(0, 0, 0, 0);
+            if (TILED)
+                wv[j] = (kc + j * 32 < K) ? *reinterpret_cast<const uint4*>(wrow + (size_t)((kc >> 5) + j) * BN_STREAM_TILE)
+                                          : make_uint4(0, 0, 0, 0);
+            else
+                wv[j] = (col && k < K) ? *reinterpret_cast<const uint4*>(wrow + k) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
@@ -265,6 +279,7 @@ void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict
 }
 
 extern "C" int bn_skinny_gemm_supports(int M, int N, int K, int ldx, int ldw);
+static bool sk_tiled_ok(int K, int ldw) { return ldw == (K + BN_STREAM_TILE_COLS - 1) / BN_STREAM_TILE_COLS; }
 
 static int sk_compute_units() {
     static int cus = 0;
@@ -295,10 +310,11 @@ static int sk_fused_tile_cols(int N) {
     return pick;
 }
 
-// Column tiles (= slots per row that a RES call writes) of the fused kernel for N columns.
-extern "C" int bn_skinny_gemm_fused_tiles(int N) {
+// Column tiles (= slots per row that a RES call writes) of the fused kernel for N columns; over a streamed copy of W
+// (tiled) they are its rows of tiles.
+extern "C" int bn_skinny_gemm_fused_tiles(int N, int tiled) {
     if (N < 1) return 0;
-    const int tc = sk_fused_tile_cols(N);
+    const int tc = tiled ? 16 : sk_fused_tile_cols(N);
     return (N + tc - 1) / tc;
 }
 
@@ -309,11 +325,13 @@ extern "C" int bn_skinny_gemm_fused_tiles(int N) {
 // resid != null (RES): the product is added to resid [M, N] in place; resid_bf16 [M, N] becomes the new stream
 // times next_weight [N], slots_out [M, bn_skinny_gemm_fused_tiles(N)] the sums of squares of its column tiles
 // (glu8 == 0, no Y).
+// tiled: W is the streamed copy (common.h) of the matrix (of its 2N interleaved rows with glu8) and ldw its tiles along K.
 extern "C" int bn_skinny_gemm_fused(const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw, int ldy,
                                     int glu8, int act, const float* slots_in, int n_slots, int stream_width, float eps,
                                     float* resid, int ld_resid, void* resid_bf16, int ld_rb, const float* next_weight,
-                                    float* slots_out, hipStream_t s) {
-    if (!bn_skinny_gemm_supports(M, N, K, ldx, ldw) || M > 16 || act < 0 || act >= BN_ACT_KINDS) return BN_ERR_ARG;
+                                    float* slots_out, int tiled, hipStream_t s) {
+    if (!bn_skinny_gemm_supports(M, N, K, ldx, tiled ? 8 : ldw) || M > 16 || act < 0 || act >= BN_ACT_KINDS) return BN_ERR_ARG;
+    if (tiled && !sk_tiled_ok(K, ldw)) return BN_ERR_ARG;
     if (((uintptr_t)X | (uintptr_t)W) & 15) return BN_ERR_ARG;
     const bool pre = slots_in != nullptr, res = resid != nullptr;
     if (!pre && !res) return BN_ERR_ARG;
@@ -329,7 +347,7 @@ extern "C" int bn_skinny_gemm_fused(const void* X, const void* W, void* Y, int M
     f.resid = resid; f.resid_bf16 = (bf16*)resid_bf16; f.next_weight = next_weight; f.slots_out = slots_out;
     f.ld_resid = ld_resid; f.ld_rb = ld_rb;
     const size_t smem = (size_t)(8 * 256 + 16) * sizeof(float) + (size_t)8 * M * SK_XROW;
-    const int tile_cols = glu8 ? 16 : sk_fused_tile_cols(N);
+    const int tile_cols = (glu8 || tiled) ? 16 : sk_fused_tile_cols(N);
     const dim3 grid((N + tile_cols - 1) / tile_cols), block(8 * 64);
     auto go = [&](auto kernel) {
         if (smem > 64 * 1024) {
@@ -342,23 +360,29 @@ extern "C" int bn_skinny_gemm_fused(const void* X, const void* W, void* Y, int M
         return bn_launch_status();
     };
     const bool few = n_slots <= 256;                  // four slot loads per row and lane are enough
-    if (glu8) {
-        if (!pre) return BN_ERR_ARG;
-        return few ? go(skinny_gemm_fused_kernel<true, true, false, 4>) : go(skinny_gemm_fused_kernel<true, true, false, 8>);
-    }
-    if (pre && res)
-        return few ? go(skinny_gemm_fused_kernel<false, true, true, 4>) : go(skinny_gemm_fused_kernel<false, true, true, 8>);
-    if (pre) return few ? go(skinny_gemm_fused_kernel<false, true, false, 4>) : go(skinny_gemm_fused_kernel<false, true, false, 8>);
-    return go(skinny_gemm_fused_kernel<false, false, true, 4>);
+    if (glu8 && !pre) return BN_ERR_ARG;
+#define SK_FUSED(T)                                                                                                      \
+    do {                                                                                                                 \
+        if (glu8) return few ? go(skinny_gemm_fused_kernel<true, true, false, 4, T>)                                     \
+                             : go(skinny_gemm_fused_kernel<true, true, false, 8, T>);                                    \
+        if (pre && res) return few ? go(skinny_gemm_fused_kernel<false, true, true, 4, T>)                               \
+                                   : go(skinny_gemm_fused_kernel<false, true, true, 8, T>);                              \
+        if (pre) return few ? go(skinny_gemm_fused_kernel<false, true, false, 4, T>)                                     \
+                            : go(skinny_gemm_fused_kernel<false, true, false, 8, T>);                                    \
+        return go(skinny_gemm_fused_kernel<false, false, true, 4, T>);                                                   \
+    } while (0)
+    if (tiled) SK_FUSED(true);
+    SK_FUSED(false);
+#undef SK_FUSED
 }
 
-template <int MT, bool DUAL, typename TO, bool GLU8 = false>
+template <int MT, bool DUAL, typename TO, bool GLU8 = false, bool TILED = false>
 static int launch(const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw, int ldy,
                   int up_off, int act, int n_waves, hipStream_t s) {
     constexpr int NA = DUAL ? 2 * MT : MT;
     constexpr bool XS = MT == 1 && !DUAL;          // the two-block form has no registers to spare for it
     const size_t smem = (size_t)n_waves * NA * 64 * 4 * sizeof(float) + (XS ? (size_t)n_waves * M * SK_XROW : 0);
-    auto kernel = skinny_gemm_kernel<MT, DUAL, TO, GLU8, XS>;
+    auto kernel = skinny_gemm_kernel<MT, DUAL, TO, GLU8, XS, TILED>;
     if (smem > 64 * 1024) {                           // beyond the default limit of dynamic shared memory
         static bool raised = false;                   // per instantiation
         if (!raised) {
@@ -406,10 +430,20 @@ extern "C" int bn_skinny_gemm_supports(int M, int N, int K, int ldx, int ldw) {
 // the gate rows at [0, N) and the up rows at [up_off, up_off + N).  dual == 2: W has 2N rows, gate
 // and up interleaved in blocks of 8 (N a multiple of 8); the result has N columns.  act: the gate's activation
 // (BN_ACT_*), used when dual != 0.
+// tiled: W is the streamed copy (common.h) and ldw its tiles along K; up to 16 rows, dual == 0.
 extern "C" int bn_skinny_gemm(int out_dtype, const void* X, const void* W, void* Y, int M, int N, int K,
-                              int ldx, int ldw, int ldy, int dual, int up_off, int act, hipStream_t s) {
-    if (!bn_skinny_gemm_supports(M, N, K, ldx, ldw) || ldy < N || act < 0 || act >= BN_ACT_KINDS) return BN_ERR_ARG;
+                              int ldx, int ldw, int ldy, int dual, int up_off, int act, int tiled, hipStream_t s) {
+    if (!bn_skinny_gemm_supports(M, N, K, ldx, tiled ? 8 : ldw) || ldy < N || act < 0 || act >= BN_ACT_KINDS) return BN_ERR_ARG;
     if (((uintptr_t)X | (uintptr_t)W) & 15) return BN_ERR_ARG;
+    if (tiled) {
+        if (dual || M > 16 || !sk_tiled_ok(K, ldw)) return BN_ERR_ARG;
+        int n_waves = 8;                           // as the row-major form with staged activations
+        const int k_chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
+        while (n_waves > 1 && n_waves / 2 >= k_chunks) n_waves >>= 1;
+        if (out_dtype == BN_DT_BF16) return launch<1, false, bf16, false, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, act, n_waves, s);
+        if (out_dtype == BN_DT_F32) return launch<1, false, float, false, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, act, n_waves, s);
+        return BN_ERR_DTYPE;
+    }
     if (dual == 2) {
         if (N % 8) return BN_ERR_ARG;
         N *= 2;                                   // rows of W; the kernel halves the column index itself

@@ -404,14 +404,16 @@ class Engine:
 
     @staticmethod
     def from_folder(folder: str, dtype=torch.bfloat16, max_tokens: int = 4096, device="cuda:0",
-                    max_seq_len: int = 0, max_slots: int = 0, use_graphs: bool = True, n_seqs: int = 1) -> "Engine":
+                    max_seq_len: int = 0, max_slots: int = 0, use_graphs: bool = True, n_seqs: int = 1,
+                    streamed_weights=None) -> "Engine":
         """max_tokens: positions that the cache holds; 0: n_seqs sequences of the longest length there can be
         (the model's max_positions, or max_seq_len when that is less: the reference sizes its cache by
-        min(context length, --maxseq), src/model.c:256-257), or as many as fit into the free device memory."""
+        min(context length, --maxseq), src/model.c:256-257), or as many as fit into the free device memory.
+        streamed_weights: as DecoderModel's."""
         ops.require_gpu()
         arch, config = load_config(folder)
         plan = arch.build_plan(config)
-        model = DecoderModel(plan, dtype, device)
+        model = DecoderModel(plan, dtype, device, streamed_weights)
         with open_tensors(folder, plan.expected_tensors()) as tensors:      # views of the mapped file, uploaded one by one
             model.load(tensors)
         if max_tokens <= 0:

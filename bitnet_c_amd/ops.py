@@ -79,17 +79,18 @@ _SIGNATURES = {
     "skinny_gemm": {
         "bn_skinny_gemm_supports": [c_int, c_int, c_int, c_int, c_int],
         "bn_skinny_gemm": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                           c_int, c_int, c_void_p],
-        "bn_skinny_gemm_fused_tiles": [c_int],
+                           c_int, c_int, c_int, c_void_p],
+        "bn_skinny_gemm_fused_tiles": [c_int, c_int],
         "bn_skinny_gemm_fused": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                  c_void_p, c_int, c_int, c_float, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
-                                 c_void_p],
+                                 c_int, c_void_p],
     },
     "splitk_gemm": {
-        "bn_splitk_gemm_supports": [c_int, c_int, c_int, c_int, c_int],
+        "bn_splitk_gemm_supports": [c_int, c_int, c_int, c_int, c_int, c_int],
         "bn_splitk_gemm_splits": [c_int, c_int],
-        "bn_splitk_gemm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-        "bn_splitk_gemm_swiglu": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bn_splitk_gemm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bn_splitk_gemm_swiglu": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int,
+                                  c_int, c_float, c_int, c_void_p],
     },
     "sampling": {
         "bn_argmax": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
@@ -370,14 +371,78 @@ def skinny_supported(M: int, N: int, K: int, ldx: int, ldw: int) -> bool:
     return bool(_fn("skinny_gemm", "bn_skinny_gemm_supports")(M, N, K, ldx, ldw))
 
 
+# --------------------------------------------------------------------------------------
+# the streamed copy of a weight matrix
+# --------------------------------------------------------------------------------------
+STREAM_TILE_ROWS = _build.header_constant("BN_STREAM_TILE_ROWS")
+STREAM_TILE_COLS = _build.header_constant("BN_STREAM_TILE_COLS")
+
+
+@dataclass
+class StreamedWeight:
+    """A bf16 weight matrix [N, K] in the order in which the kernels that read it once per call load it (csrc/common.h):
+    tiles of 16 rows x 32 columns, each the 1 KB that one load of a wave takes (lane r + 16 g: columns 8 g .. 8 g + 7 of row
+    r), [ceil(N / 16), ceil(K / 32), 512], rows past N and columns past K zero.  A second copy beside the row-major matrix,
+    which the products of many rows (the library's) and everything else keep reading: the kernels of up to 128 rows take it
+    through their `streamed` argument and give the same result bit for bit, 5 to 15 % sooner."""
+    tiles: torch.Tensor
+    N: int
+    K: int
+
+    @property
+    def k_tiles(self) -> int:
+        return self.tiles.shape[1]
+
+    def nbytes(self) -> int:
+        return self.tiles.numel() * self.tiles.element_size()
+
+
+def stream_copy(w: torch.Tensor) -> StreamedWeight:
+    """The streamed copy of w [N, K] (bf16, on the device; made there)."""
+    require_gpu()
+    _dev(w, "w", torch.bfloat16, 2)
+    N, K = w.shape
+    R, C = STREAM_TILE_ROWS, STREAM_TILE_COLS
+    nt, kt = (N + R - 1) // R, (K + C - 1) // C
+    if nt * R != N or kt * C != K:
+        padded = torch.zeros((nt * R, kt * C), dtype=w.dtype, device=w.device)
+        padded[:N, :K] = w
+        w = padded
+    # [nt, r, kt, g, 8] -> [nt, kt, g, r, 8]: lane r + 16 g of tile (nt, kt)
+    tiles = w.view(nt, R, kt, C // 8, 8).permute(0, 2, 3, 1, 4).contiguous().view(nt, kt, R * C)
+    return StreamedWeight(tiles, N, K)
+
+
+def unstream(sw: StreamedWeight) -> torch.Tensor:
+    """The row-major matrix [N, K] that a streamed copy holds."""
+    R, C = STREAM_TILE_ROWS, STREAM_TILE_COLS
+    nt, kt = sw.tiles.shape[:2]
+    return sw.tiles.view(nt, kt, C // 8, R, 8).permute(0, 3, 1, 2, 4).reshape(nt * R, kt * C)[:sw.N, :sw.K].contiguous()
+
+
+def _weight_arg(w: torch.Tensor, streamed: Optional[StreamedWeight], what: str):
+    """(pointer, row stride or tiles along K, tiled) of the weights that a kernel is to read: the streamed copy if one is
+    given (checked against w), else w itself."""
+    if streamed is None:
+        return w.data_ptr(), _rows(w, "w"), 0
+    t = streamed.tiles
+    if (not isinstance(streamed, StreamedWeight) or (streamed.N, streamed.K) != tuple(w.shape) or t.device != w.device
+            or t.dtype != torch.bfloat16 or not t.is_contiguous() or t.dim() != 3
+            or tuple(t.shape) != ((streamed.N + STREAM_TILE_ROWS - 1) // STREAM_TILE_ROWS,
+                                  (streamed.K + STREAM_TILE_COLS - 1) // STREAM_TILE_COLS, STREAM_TILE_ROWS * STREAM_TILE_COLS)):
+        raise KernelError(f"{what}: the streamed copy does not belong to w {tuple(w.shape)}")
+    return t.data_ptr(), t.shape[1], 1
+
+
 # bf16 products with many rows: the library's matrix product (as the reference hands its batched
 # products to a library, src/gpu_cuda.cu:11571) unless this is False or BITNET_NO_LIBRARY is set;
 # then this library's own matrix-core kernel (gemm_mfma) does them.
 LIBRARY_PRODUCTS = os.environ.get("BITNET_NO_LIBRARY", "") in ("", "0")
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, *, allow_library: Optional[bool] = None) -> torch.Tensor:
-    """y[M, N] = x[M, K] . w[N, K]^T.
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, *, allow_library: Optional[bool] = None,
+           streamed: Optional[StreamedWeight] = None) -> torch.Tensor:
+    """y[M, N] = x[M, K] . w[N, K]^T.  streamed: w's streamed copy, which the kernel of up to 16 rows reads instead.
 
     float32: the tiled kernel (plain fmaf, a fixed order of summation).
     bf16: up to 16 rows (one MFMA tile of activations) the matrix-core kernel that streams
@@ -409,8 +474,9 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, *, allow_library: O
     small = M <= SKINNY_ROWS or (M <= 64 and not allow_library)
     if small and aligned and skinny_supported(M, N, K, ldx, ldw):
         y = torch.empty((M, N), dtype=out_dtype, device=x.device)
-        _check(_fn("skinny_gemm", "bn_skinny_gemm")(_code(out_dtype), x.data_ptr(), w.data_ptr(), y.data_ptr(),
-                                                    M, N, K, ldx, ldw, N, 0, 0, 0, _stream()), "skinny_gemm")
+        wp, wl, tiled = _weight_arg(w, streamed if M <= SKINNY_ROWS else None, "linear")
+        _check(_fn("skinny_gemm", "bn_skinny_gemm")(_code(out_dtype), x.data_ptr(), wp, y.data_ptr(),
+                                                    M, N, K, ldx, wl, N, 0, 0, 0, tiled, _stream()), "skinny_gemm")
         return y
     if M > SKINNY_ROWS and allow_library:
         if out_dtype == torch.bfloat16:
@@ -432,15 +498,64 @@ def interleave_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor) -> torch.Tensor
     return torch.stack([w_gate.reshape(F // 8, 8, K), w_up.reshape(F // 8, 8, K)], dim=1).reshape(2 * F, K).contiguous()
 
 
-# Without the library the interleaved gate/up product of 17 to 128 rows with its SwiGLU epilogue is the kernel that stages
-# the activations once per 64 columns (splitk_gemm.hip).  With the library it is not used: measured against the library's
-# product and the SwiGLU kernel after it, it is 5 to 10 % faster at 17 to 32 rows of the 8B shape (50 us against 55) and 10
-# to 30 % slower at the 13B and 70B shapes and at a hidden size of 3,072 (65 against 54, 200 against 184, 30 against 26).
+# The interleaved gate/up product with its SwiGLU epilogue in the kernel that stages the activations once per 64 or 112
+# columns (splitk_gemm.hip).  Without the library it is the kernel of 17 to 128 rows.  With the library it takes the row
+# counts at which it was measured faster than what else there is (the fused streaming kernel up to 16 rows, whose every
+# workgroup stages all rows for its 16 columns; above that the library's product and the kernel of the gated unit) on
+# matrices of at least STAGED_MIN_TILES_PER_CU column tiles per CU (smaller ones leave it too few waves): 13 to 16 rows,
+# and up to 64 rows over a streamed copy of the weights (us at 16 / 32 / 64 rows, streamed: 8B 45.6 / 45.7 / 50.9 against
+# 47.8 / 55.4 / 54.3; 13B 53.2 / 53.7 / 61.5 against 57.9 / 56.1 / 59.7; 70B 163 / 169 / 190 against 175 / 196 / 216;
+# at a hidden size of 3,072 and below the others win by 5 to 15 %).
 SWIGLU_STAGED_ROWS = (17, 128)
+SWIGLU_STAGED_LIBRARY_ROWS = (13, 16)
+SWIGLU_STAGED_STREAMED_ROWS = (13, 64)
+STAGED_MIN_TILES_PER_CU = 6
+
+
+def _compute_units() -> int:
+    global _CUS
+    if _CUS is None:
+        _CUS = int(torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count)
+    return _CUS
+
+
+_CUS = None
+
+
+def _staged_swiglu_rows(M: int, allow_library: bool, w_rows: int, streamed) -> bool:
+    if not allow_library:
+        lo, hi = SWIGLU_STAGED_ROWS
+        return lo <= M <= hi
+    lo, hi = SWIGLU_STAGED_STREAMED_ROWS if streamed is not None else SWIGLU_STAGED_LIBRARY_ROWS
+    return lo <= M <= hi and w_rows // 16 >= STAGED_MIN_TILES_PER_CU * _compute_units()
+
+
+def _staged_swiglu(x, w_gate_up, pre, activation, streamed=None):
+    """The staged kernel's gate/up product with the gated unit (and a deferred norm's factor) in its epilogue; None if
+    it does not take the shape."""
+    M, K = x.shape
+    F = w_gate_up.shape[0] // 2
+    ldx = _rows(x, "x")
+    wp, wl, tiled = _weight_arg(w_gate_up, streamed, "linear_swiglu")
+    if F % 8 or not _fn("splitk_gemm", "bn_splitk_gemm_supports")(M, 2 * F, K, ldx, wl, tiled):
+        return None
+    if pre is not None:          # what the kernel's passes over the parts of the sums of squares hold (SG_NORM_*)
+        n = pre.slots.shape[1]
+        per = min(64, 1 << max(0, n - 1).bit_length())
+        if -(-M // (4 * (64 // per))) > 4 or -(-n // per) > 8:
+            return None
+    y = torch.empty((M, F), dtype=x.dtype, device=x.device)
+    _check(_fn("splitk_gemm", "bn_splitk_gemm_swiglu")(
+        x.data_ptr(), wp, y.data_ptr(), M, F, K, ldx, wl, F, _act(activation),
+        pre.slots.data_ptr() if pre is not None else None, pre.slots.shape[1] if pre is not None else 0,
+        pre.stream.shape[1] if pre is not None else 0, float(pre.eps) if pre is not None else 0.0, tiled, _stream()),
+        "splitk_gemm(glu)")
+    return y
 
 
 def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = False, *,
-                  allow_library: Optional[bool] = None, activation: str = "silu") -> torch.Tensor:
+                  allow_library: Optional[bool] = None, activation: str = "silu",
+                  streamed: Optional[StreamedWeight] = None) -> torch.Tensor:
     """act(x.Wg^T) * (x.Wu^T) for w_gate_up = [Wg; Wu] ([2F, K]), or the two interleaved in
     blocks of 8 rows (interleave_gate_up); act is silu unless `activation` names another of
     ACTIVATIONS.  The decode-sized bf16 case is one kernel, and so is the interleaved case without
@@ -460,19 +575,16 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = 
         return torch.empty((0, F), dtype=x.dtype, device=x.device)
     ldx, ldw = _rows(x, "x"), _rows(w_gate_up, "w_gate_up")
     aligned = x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0
-    lo, hi = SWIGLU_STAGED_ROWS
-    if (x.dtype == torch.bfloat16 and interleaved and aligned and not allow_library and lo <= M <= hi
-            and _fn("splitk_gemm", "bn_splitk_gemm_supports")(M, 2 * F, K, ldx, ldw)):
-        y = torch.empty((M, F), dtype=x.dtype, device=x.device)
-        _check(_fn("splitk_gemm", "bn_splitk_gemm_swiglu")(x.data_ptr(), w_gate_up.data_ptr(), y.data_ptr(), M, F, K, ldx, ldw,
-                                                           F, _act(activation), _stream()), "splitk_gemm(glu)")
-        return y
+    if x.dtype == torch.bfloat16 and interleaved and aligned and _staged_swiglu_rows(M, allow_library, 2 * F, streamed):
+        y = _staged_swiglu(x, w_gate_up, None, activation, streamed)
+        if y is not None:
+            return y
     if (x.dtype == torch.bfloat16 and (M <= SKINNY_ROWS or (M <= 64 and not allow_library))
             and aligned and skinny_supported(M, F, K, ldx, ldw)):
         y = torch.empty((M, F), dtype=x.dtype, device=x.device)
         _check(_fn("skinny_gemm", "bn_skinny_gemm")(_code(x.dtype), x.data_ptr(), w_gate_up.data_ptr(),
                                                     y.data_ptr(), M, F, K, ldx, ldw, F, 2 if interleaved else 1, F,
-                                                    _act(activation), _stream()), "skinny_gemm(glu)")
+                                                    _act(activation), 0, _stream()), "skinny_gemm(glu)")
         return y
     if (x.dtype == torch.bfloat16 and interleaved and not allow_library and aligned
             and gemm_mfma_supported(M, 2 * F, K, ldx, ldw)):
@@ -519,22 +631,24 @@ def can_split_sums(M: int, N: int, K: int, dtype) -> bool:
     return K >= 2 * N or (K >= N and N <= SPLIT_SUM_SQUARE_WIDTH)
 
 
-def linear_partial_sums(x: torch.Tensor, w: torch.Tensor) -> PartialSums:
-    """x [M, K] . w[N, K]^T as float32 partial sums over ranges of K (bf16 operands, 1 to 128 rows)."""
+def linear_partial_sums(x: torch.Tensor, w: torch.Tensor, streamed: Optional[StreamedWeight] = None) -> PartialSums:
+    """x [M, K] . w[N, K]^T as float32 partial sums over ranges of K (bf16 operands, 1 to 128 rows).  streamed: w's
+    streamed copy, read instead of w."""
     require_gpu()
     _dev(x, "x", torch.bfloat16, 2)
     _dev(w, "w", torch.bfloat16, 2)
-    ldx, ldw = _rows(x, "x"), _rows(w, "w")
+    ldx = _rows(x, "x")
     M, K = x.shape
     N = w.shape[0]
     if w.shape[1] != K:
         raise KernelError(f"linear_partial_sums: x {tuple(x.shape)} and w {tuple(w.shape)} do not fit")
-    if not _fn("splitk_gemm", "bn_splitk_gemm_supports")(M, N, K, ldx, ldw) or (x.data_ptr() | w.data_ptr()) % 16:
+    wp, wl, tiled = _weight_arg(w, streamed, "linear_partial_sums")
+    if not _fn("splitk_gemm", "bn_splitk_gemm_supports")(M, N, K, ldx, wl, tiled) or (x.data_ptr() | wp) % 16:
         raise KernelError(f"linear_partial_sums: the kernel takes 1 to 128 rows, K a multiple of 8 and 16-byte aligned "
-                          f"operands, not x {tuple(x.shape)} (row stride {ldx}), w {tuple(w.shape)} (row stride {ldw})")
+                          f"operands, not x {tuple(x.shape)} (row stride {ldx}), w {tuple(w.shape)} (row stride {wl})")
     S = _fn("splitk_gemm", "bn_splitk_gemm_splits")(N, K)
     slabs = torch.empty((S, M, N), dtype=torch.float32, device=x.device)
-    _check(_fn("splitk_gemm", "bn_splitk_gemm")(x.data_ptr(), w.data_ptr(), slabs.data_ptr(), M, N, K, ldx, ldw, S,
+    _check(_fn("splitk_gemm", "bn_splitk_gemm")(x.data_ptr(), wp, slabs.data_ptr(), M, N, K, ldx, wl, S, tiled,
                                                 _stream()), "splitk_gemm")
     return PartialSums(slabs)
 
@@ -633,16 +747,17 @@ def can_fuse_norm(M: int, N: int, K: int, dtype) -> bool:
 
 
 def _fused_call(x, w, y, M, N, K, glu8, pre: Optional[DeferredNorm], resid, resid_bf16, next_weight, slots_out,
-                activation: str = "silu"):
+                activation: str = "silu", streamed: Optional[StreamedWeight] = None):
+    wp, wl, tiled = _weight_arg(w, streamed, "fused product")
     _check(_fn("skinny_gemm", "bn_skinny_gemm_fused")(
-        x.data_ptr(), w.data_ptr(), y.data_ptr() if y is not None else None, M, N, K, _rows(x, "x"), _rows(w, "w"),
+        x.data_ptr(), wp, y.data_ptr() if y is not None else None, M, N, K, _rows(x, "x"), wl,
         N if y is not None else 0, int(glu8), _act(activation),
         pre.slots.data_ptr() if pre is not None else None, pre.slots.shape[1] if pre is not None else 0,
         pre.stream.shape[1] if pre is not None else 0, float(pre.eps) if pre is not None else 0.0,
         resid.data_ptr() if resid is not None else None, _rows(resid, "resid") if resid is not None else 0,
         resid_bf16.data_ptr() if resid_bf16 is not None else None, N if resid_bf16 is not None else 0,
         next_weight.data_ptr() if next_weight is not None else None,
-        slots_out.data_ptr() if slots_out is not None else None, _stream()), "skinny_gemm(fused)")
+        slots_out.data_ptr() if slots_out is not None else None, tiled, _stream()), "skinny_gemm(fused)")
 
 
 def _check_deferred(pre: DeferredNorm, K: int) -> int:
@@ -656,8 +771,9 @@ def _check_deferred(pre: DeferredNorm, K: int) -> int:
     return M
 
 
-def linear_prenorm(pre: DeferredNorm, w: torch.Tensor) -> torch.Tensor:
-    """linear(rmsnorm(stream), w) for a deferred norm, in one kernel (bf16, up to 16 rows)."""
+def linear_prenorm(pre: DeferredNorm, w: torch.Tensor, streamed: Optional[StreamedWeight] = None) -> torch.Tensor:
+    """linear(rmsnorm(stream), w) for a deferred norm, in one kernel (bf16, up to 16 rows).  streamed: w's streamed
+    copy, read instead of w."""
     require_gpu()
     _dev(w, "w", torch.bfloat16, 2)
     N, K = w.shape
@@ -665,16 +781,23 @@ def linear_prenorm(pre: DeferredNorm, w: torch.Tensor) -> torch.Tensor:
     if not can_fuse_norm(M, N, K, torch.bfloat16) or w.data_ptr() % 16:
         raise KernelError(f"linear_prenorm: {M} rows, w {tuple(w.shape)} cannot be fused")
     y = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
-    _fused_call(pre.scaled, w, y, M, N, K, False, pre, None, None, None, None)
+    _fused_call(pre.scaled, w, y, M, N, K, False, pre, None, None, None, None, streamed=streamed)
     return y
 
 
-def linear_swiglu_prenorm(pre: DeferredNorm, w_gate_up: torch.Tensor, activation: str = "silu") -> torch.Tensor:
-    """linear_swiglu(rmsnorm(stream), w) for gate and up interleaved in blocks of 8, in one kernel."""
+def linear_swiglu_prenorm(pre: DeferredNorm, w_gate_up: torch.Tensor, activation: str = "silu",
+                          streamed: Optional[StreamedWeight] = None) -> torch.Tensor:
+    """linear_swiglu(rmsnorm(stream), w) for gate and up interleaved in blocks of 8, in one kernel.  streamed: w's
+    streamed copy, read instead of w."""
     require_gpu()
     _dev(w_gate_up, "w_gate_up", torch.bfloat16, 2)
     F, K = w_gate_up.shape[0] // 2, w_gate_up.shape[1]
     M = _check_deferred(pre, K)
+    if (w_gate_up.shape[0] % 16 == 0 and w_gate_up.data_ptr() % 16 == 0
+            and _staged_swiglu_rows(M, LIBRARY_PRODUCTS, w_gate_up.shape[0], streamed)):
+        y = _staged_swiglu(pre.scaled, w_gate_up, pre, activation, streamed)
+        if y is not None:
+            return y
     if M > FUSED_ROWS and w_gate_up.shape[0] % 16 == 0 and LIBRARY_PRODUCTS:
         # more rows than the fused kernel takes: the library's product of the copy, and the norm's factor in the
         # kernel of the gated unit, which runs anyway
@@ -682,13 +805,14 @@ def linear_swiglu_prenorm(pre: DeferredNorm, w_gate_up: torch.Tensor, activation
     if w_gate_up.shape[0] % 16 or not can_fuse_norm(M, F, K, torch.bfloat16) or w_gate_up.data_ptr() % 16:
         raise KernelError(f"linear_swiglu_prenorm: {M} rows, w {tuple(w_gate_up.shape)} cannot be fused")
     y = torch.empty((M, F), dtype=torch.bfloat16, device=w_gate_up.device)
-    _fused_call(pre.scaled, w_gate_up, y, M, F, K, True, pre, None, None, None, None, activation)
+    _fused_call(pre.scaled, w_gate_up, y, M, F, K, True, pre, None, None, None, None, activation, streamed)
     return y
 
 
-def _fused_tiles(N: int) -> int:
-    """Column tiles of the fused product kernel for N columns: one partial sum of squares per row and tile."""
-    return int(_fn("skinny_gemm", "bn_skinny_gemm_fused_tiles")(int(N)))
+def _fused_tiles(N: int, tiled: bool = False) -> int:
+    """Column tiles of the fused product kernel for N columns (over a streamed copy if tiled): one partial sum of
+    squares per row and tile."""
+    return int(_fn("skinny_gemm", "bn_skinny_gemm_fused_tiles")(int(N), int(tiled)))
 
 
 def can_defer_norm(M: int, N: int, K: int, dtype) -> bool:
@@ -697,7 +821,7 @@ def can_defer_norm(M: int, N: int, K: int, dtype) -> bool:
 
 
 def linear_into_stream(x: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, weight: torch.Tensor,
-                       eps: float) -> DeferredNorm:
+                       eps: float, streamed: Optional[StreamedWeight] = None) -> DeferredNorm:
     """stream += linear(x, w) (float32 stream [M, N], in place), and what the next norm (weights
     `weight`, `eps`) needs: the bf16 copy of the new stream times the weights and the rows' sums of
     squares in parts.  Returns that norm, deferred."""
@@ -714,8 +838,8 @@ def linear_into_stream(x: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, w
     if not can_defer_norm(M, N, K, torch.bfloat16) or x.data_ptr() % 16 or w.data_ptr() % 16:
         raise KernelError(f"linear_into_stream: {M} rows, w {tuple(w.shape)} cannot be fused")
     scaled = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-    slots = torch.empty((M, _fused_tiles(N)), dtype=torch.float32, device=x.device)
-    _fused_call(x, w, None, M, N, K, False, None, stream, scaled, weight, slots)
+    slots = torch.empty((M, _fused_tiles(N, streamed is not None)), dtype=torch.float32, device=x.device)
+    _fused_call(x, w, None, M, N, K, False, None, stream, scaled, weight, slots, streamed=streamed)
     return DeferredNorm(scaled, slots, stream, weight, float(eps))
 
 

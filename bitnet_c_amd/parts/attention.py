@@ -67,6 +67,9 @@ class Attention(Part):
         self.o.load(tensors["wo"], tensors.get("bo") if self.has_bias else None, device, dtype)
         self.position.prepare(device)
 
+    def linears(self):
+        return [self.qkv, self.o]
+
     def cache_need(self) -> CacheNeed:
         return CacheNeed(kv=KVNeed(self.Hkv, self.hs, self.window))
 

@@ -151,6 +151,11 @@ class Part:
     def load(self, tensors: Dict[str, torch.Tensor], device, dtype) -> None:
         pass
 
+    def linears(self) -> list:
+        """The part's weight matrices (parts.linear.Linear) that are read once per product: a model may ask each of them
+        to keep a streamed copy of its weight.  A part with kernels of its own returns none."""
+        return []
+
 
 @dataclass
 class KVView:

@@ -22,6 +22,9 @@ class PreNormBlock(Part):
     def children(self):
         return {"mixer": self.mixer, "ffn": self.ffn, "mixer_norm": self.mixer_norm, "ffn_norm": self.ffn_norm}
 
+    def linears(self):
+        return [l for part in self.children().values() for l in getattr(part, "linears", list)()]
+
     def tensors(self):
         return {f"{cn}.{tn}": spec for cn, c in self.children().items() for tn, spec in c.tensors().items()}
 

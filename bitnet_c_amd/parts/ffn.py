@@ -48,6 +48,9 @@ class SwiGLU(Part):
         self.gate_up.load(w, b, device, dtype)
         self.down.load(tensors["w_down"], tensors.get("b_down") if self.has_bias else None, device, dtype)
 
+    def linears(self):
+        return [self.gate_up, self.down]
+
     def forward(self, h, ctx, lazy_ok: bool = False):
         if isinstance(h, ops.DeferredNorm):
             w = self.gate_up.weight
@@ -55,11 +58,12 @@ class SwiGLU(Part):
             if (not self.has_bias and self.interleaved and w.dtype == torch.bfloat16
                     and (ops.can_fuse_norm(M, self.F, self.hidden, w.dtype)
                          or (M > ops.FUSED_ROWS and ops.LIBRARY_PRODUCTS and w.data_ptr() % 16 == 0))):
-                act = ops.linear_swiglu_prenorm(h, w, self.activation)
+                act = ops.linear_swiglu_prenorm(h, w, self.activation, self.gate_up.streamed)
                 return self.down.lazy(act) if lazy_ok else self.down(act)
             h = h.materialize()
         if self.has_bias:
             act = ops.swiglu(self.gate_up(h), self.interleaved, self.activation)
         else:
-            act = ops.linear_swiglu(h, self.gate_up.weight, self.interleaved, activation=self.activation)
+            act = ops.linear_swiglu(h, self.gate_up.weight, self.interleaved, activation=self.activation,
+                                    streamed=self.gate_up.streamed)
         return self.down.lazy(act) if lazy_ok else self.down(act)

@@ -108,6 +108,52 @@ def test_decode_steps_fold_their_norms_into_the_products(model_folders, name, gr
         assert rel_err(fused[i], plain_k[i]) < TOL[torch.bfloat16]
 
 
+@pytest.mark.parametrize("small_matrices", [False, True])
+@pytest.mark.parametrize("name", ["A", "B", "E"])
+def test_streamed_copies_of_the_weights_change_no_result(model_folders, name, small_matrices, monkeypatch):
+    """A bf16 engine with a second copy of every weight matrix in the order its decode kernels read it, and one
+    without: prompts (whole, and one of 100 tokens after 50, whose feed-forward ends in partial sums), decode steps of
+    3 sequences and of 20 (graphs of 4 and 32 rows) give the plain implementation's logits either way, and the copies
+    are no part of what a step is counted to read.  With small_matrices the staged gate/up kernel takes these tiny
+    matrices too (it is meant for matrices of at least six column tiles a CU), so that its path through the
+    feed-forward runs here at 13 to 64 rows."""
+    from bitnet_c_amd import StepEntry, ops
+    if small_matrices:
+        monkeypatch.setattr(ops, "STAGED_MIN_TILES_PER_CU", 0)
+    folder = model_folders(name, torch.bfloat16)
+    vocab = pl.read_config(folder)["vocab"]
+    reqs = _requests(vocab, 77, [150] + [40 + j for j in range(19)])
+    n_dec = 6
+    outs = {}
+    for streamed in (False, True):
+        eng = make_engine(folder, torch.bfloat16, max_tokens=4096, streamed_weights=streamed)
+        m = eng.model
+        assert m.has_streamed == streamed and (m.lm_head_streamed is not None) == streamed
+        assert all((l.streamed is not None) == (streamed and l.stream_bytes() > 0) for l in m.linears()) and m.linears()
+        assert m.streamed_bytes() >= m.weight_bytes() * 0.5           # every matrix once more (padded), norms aside
+        outs[streamed, "bytes"] = m.weight_bytes()
+        s = eng.new_sequence()
+        eng.step([StepEntry(s, reqs[0][:50], [])])
+        chunk = eng.step([StepEntry(s, reqs[0][50:], list(range(100)))])
+        eng.release(s)
+        assert rel_err(chunk, plain_logits(folder, reqs[0], torch.bfloat16)[50:]) < TOL[torch.bfloat16]
+        for group in (reqs[:3], reqs):
+            slots = [eng.new_sequence() for _ in group]
+            eng.step([StepEntry(q, r[:-n_dec], []) for q, r in zip(slots, group)])
+            got = torch.stack([eng.step([StepEntry(q, [r[len(r) - n_dec + t]], [0]) for q, r in zip(slots, group)])
+                               for t in range(n_dec)], dim=1)          # [request, step, vocab]
+            for q in slots:
+                eng.release(q)
+            for i, r in enumerate(group):
+                assert rel_err(got[i], plain_logits(folder, r, torch.bfloat16)[len(r) - n_dec:]) < TOL[torch.bfloat16], (streamed, i)
+            outs[streamed, len(group)] = got
+        eng.cache.check()
+        assert eng._graphs.keys() >= {4, 32}
+    assert outs[False, "bytes"] == outs[True, "bytes"]
+    for n in (3, len(reqs)):
+        assert rel_err(outs[True, n], outs[False, n]) < TOL[torch.bfloat16]
+
+
 @pytest.mark.parametrize("name", NAMES)
 def test_whole_requests_without_the_library(model_folders, name, monkeypatch):
     """bf16 with the library's matrix product switched off: prompts of more than 64 tokens then go

@@ -404,12 +404,118 @@ def test_swiglu_product_with_staged_activations(M, F, K):
     xd = x.cuda()
     y = torch.full((M, F), float("nan"), dtype=torch.bfloat16, device="cuda")
     rc = ops._fn("splitk_gemm", "bn_splitk_gemm_swiglu")(xd.data_ptr(), wi.data_ptr(), y.data_ptr(), M, F, K, K, K, F,
-                                                         ops.ACTIVATIONS["silu"], torch.cuda.current_stream().cuda_stream)
+                                                         ops.ACTIVATIONS["silu"], None, 0, 0, 0.0, 0,
+                                                         torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     assert close(y.float(), want, torch.bfloat16)
     lo, hi = ops.SWIGLU_STAGED_ROWS
     if lo <= M <= hi:                              # without the library this is the kernel of these row counts
         assert torch.equal(ops.linear_swiglu(xd, wi, True, allow_library=False), y)
+    # over the streamed copy of the weights (other workgroup sizes, the same sums): the same bits
+    ws = ops.stream_copy(wi)
+    y2 = torch.full((M, F), float("nan"), dtype=torch.bfloat16, device="cuda")
+    rc = ops._fn("splitk_gemm", "bn_splitk_gemm_swiglu")(xd.data_ptr(), ws.tiles.data_ptr(), y2.data_ptr(), M, F, K, K, ws.k_tiles,
+                                                         F, ops.ACTIVATIONS["silu"], None, 0, 0, 0.0, 1,
+                                                         torch.cuda.current_stream().cuda_stream)
+    assert rc == 0 and torch.equal(y2, y)
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 50, 64, 128])
+@pytest.mark.parametrize("D,F", [(264, 328), (4096, 520), (1000, 136), (5120, 64)])
+def test_staged_swiglu_product_applies_a_deferred_norm(M, D, F):
+    """The staged gate/up product takes a deferred norm: its activations are the stream's bf16 copy times the norm's
+    weights, and the rows' 1/sqrt(mean + eps), from sums of squares that arrive in parts (many parts of few columns as
+    the fused product of up to 16 rows leaves them, few parts of 1,024 columns as sum_deferred does), multiplies gate
+    and up in the epilogue.  Against the plain formulas on the same stream, over the row-major weights and over their
+    streamed copy (the same bits); and the dispatcher's own choice gives a result of the same accuracy."""
+    ops = _ops()
+    eps = 1e-5
+    stream = _rand((M, D), torch.float32, 91, 2.0)
+    norm_w = _rand((D,), torch.float32, 92) * 0.2 + 1.0
+    w = _rand((2 * F, D), torch.bfloat16, 93, 0.05)
+    x = stream.clone().cuda()
+    if M <= 16:
+        act, w_out = _rand((M, 64), torch.bfloat16, 94), _rand((D, 64), torch.bfloat16, 95, 0.1)
+        pre = ops.linear_into_stream(act.cuda(), w_out.cuda(), x, norm_w.cuda(), eps)
+        want_x = stream.double() + act.double() @ w_out.double().t()
+    else:
+        delta = _rand((M, D), torch.bfloat16, 94)
+        pre = ops.sum_deferred(x, delta.cuda(), norm_w.cuda(), eps)
+        want_x = stream.double() + delta.double()
+    h = pl.rmsnorm(want_x.float(), norm_w, eps).double()
+    g, u = h @ w[:F].double().t(), h @ w[F:].double().t()
+    exact = ((g / (1 + torch.exp(-g))) * u).float()
+    wi = ops.interleave_gate_up(w[:F].cuda(), w[F:].cuda())
+    got = ops._staged_swiglu(pre.scaled, wi, pre, "silu")
+    assert got is not None and got.dtype == torch.bfloat16
+    classic = ops.linear_swiglu(pre.materialize(), wi, True)
+    e_got, e_classic = rel_err(got.float(), exact), rel_err(classic.float(), exact)
+    assert e_got <= 2.0 * e_classic + 2.0 ** -7, (e_got, e_classic)
+    assert torch.equal(ops._staged_swiglu(pre.scaled, wi, pre, "silu", ops.stream_copy(wi)), got)
+    routed = ops.linear_swiglu_prenorm(pre, wi) if (M <= 16 or ops.LIBRARY_PRODUCTS) else got
+    assert rel_err(routed.float(), exact) <= 2.0 * e_classic + 2.0 ** -7
+
+
+def test_the_streamed_copy_is_the_lanes_order():
+    """The streamed copy of a weight matrix by its definition: tile (a, b) holds rows 16 a .. 16 a + 15 and columns
+    32 b .. 32 b + 31, lane l = r + 16 g of a wave gets elements 8 l .. 8 l + 7 of the tile, which are columns 8 g .. 8 g + 7
+    of row r; rows past N and columns past K are zero; unstream gives the matrix back."""
+    ops = _ops()
+    for N, K in ((31, 264), (48, 64), (100, 1000), (16, 8)):
+        w = _rand((N, K), torch.bfloat16, 71, 0.5).cuda()
+        sw = ops.stream_copy(w)
+        nt, kt = (N + 15) // 16, (K + 31) // 32
+        assert tuple(sw.tiles.shape) == (nt, kt, 512) and (sw.N, sw.K, sw.k_tiles) == (N, K, kt)
+        assert sw.nbytes() == nt * kt * 1024
+        assert torch.equal(ops.unstream(sw), w)
+        t, wc = sw.tiles.cpu(), w.cpu()
+        for a, b, lane in ((0, 0, 0), (nt - 1, kt - 1, 63), (nt - 1, 0, 17), (0, kt - 1, 40), (nt // 2, kt // 2, 5)):
+            r, g = lane % 16, lane // 16
+            row, col = 16 * a + r, 32 * b + 8 * g
+            want = torch.zeros(8, dtype=torch.bfloat16)
+            if row < N and col < K:
+                n = min(8, K - col)
+                want[:n] = wc[row, col:col + n]
+            assert torch.equal(t[a, b, 8 * lane:8 * lane + 8], want), (N, K, a, b, lane)
+    with pytest.raises(ops.KernelError):                   # a copy of another matrix
+        ops.linear(torch.zeros(4, 64, dtype=torch.bfloat16, device="cuda"), torch.zeros(32, 64, dtype=torch.bfloat16, device="cuda"),
+                   streamed=ops.stream_copy(torch.zeros(48, 64, dtype=torch.bfloat16, device="cuda")))
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 64, 128])
+@pytest.mark.parametrize("N,K", [(100, 64), (48, 1000), (264, 3592), (4104, 4096), (31, 264), (4096, 14336)])
+def test_products_over_the_streamed_copy_are_the_same_bits(M, N, K):
+    """Every product that takes a streamed copy of its weights forms the same sums in the same order as over the
+    row-major matrix: the plain product of up to 16 rows (bf16 and float32 results), the products with a norm folded
+    in (before, after, with the gated unit), and the partial sums of up to 128 rows.  N and K that are no multiples
+    of the tile's 16 and 32 among them."""
+    ops = _ops()
+    x, w = _rand((M, K), torch.bfloat16, 81).cuda(), _rand((N, K), torch.bfloat16, 82, 0.05).cuda()
+    sw = ops.stream_copy(w)
+    a, b = ops.linear_partial_sums(x, w), ops.linear_partial_sums(x, w, sw)
+    assert torch.equal(a.slabs, b.slabs)
+    if M > 16:
+        return
+    for out in (torch.bfloat16, torch.float32):
+        assert torch.equal(ops.linear(x, w, out), ops.linear(x, w, out, streamed=sw))
+    if N > 16 * 512:
+        return
+    eps = 1e-5
+    norm_w = (_rand((N,), torch.float32, 83) * 0.2 + 1.0).cuda()
+    s1, s2 = _rand((M, N), torch.float32, 84, 2.0).cuda(), _rand((M, N), torch.float32, 84, 2.0).cuda()
+    p1 = ops.linear_into_stream(x, w, s1, norm_w, eps)
+    p2 = ops.linear_into_stream(x, w, s2, norm_w, eps, sw)
+    assert torch.equal(s1, s2) and torch.equal(p1.scaled, p2.scaled)
+    assert p2.slots.shape[1] == (N + 15) // 16                      # one part per row of tiles
+    assert rel_err(p2.slots.sum(dim=1), p1.slots.sum(dim=1)) < 1e-6
+    # the next product reads either norm; its own weights streamed or not
+    F = 40 if N % 8 == 0 else 0
+    if N % 8 == 0:
+        w_in = _rand((2 * F, N), torch.bfloat16, 85, 0.05).cuda()
+        si = ops.stream_copy(w_in)
+        for pre in (p1, p2):
+            assert torch.equal(ops.linear_prenorm(pre, w_in), ops.linear_prenorm(pre, w_in, si))
+            assert torch.equal(ops.linear_swiglu_prenorm(pre, w_in), ops.linear_swiglu_prenorm(pre, w_in, streamed=si))
 
 
 @pytest.mark.parametrize("activation", ["gelu_tanh", "relu2", "silu"])
