@@ -73,6 +73,15 @@ class Attention(Part):
     def cache_need(self) -> CacheNeed:
         return CacheNeed(kv=KVNeed(self.Hkv, self.hs, self.window))
 
+    def wants_deferred_norm(self, ctx, rows: int) -> bool:
+        """With more rows than the fused product takes, the norm's factor can only go into the decode kernel that
+        rotates by itself (forward); a prompt step is better served by the plain norm."""
+        if rows <= ops.FUSED_ROWS:
+            return True
+        fuse_ok, inv_freq = self.position.fusable(self.hs)
+        return bool(ctx.is_decode and fuse_ok and inv_freq is not None and not self.has_bias and ops.LIBRARY_PRODUCTS
+                    and ops.can_fuse_decode(self.qkv.weight.dtype, self.H, self.Hkv, self.hs))
+
     def forward(self, h, ctx, kv, lazy_ok: bool = False):
         H, Hkv, hs = self.H, self.Hkv, self.hs
         last = self.o.lazy if lazy_ok else self.o

@@ -209,10 +209,12 @@ class ResidualStream:
             self.pending = None
         return self.x
 
-    def normed(self, norm, out_dtype, rows=None, consumer=None):
+    def normed(self, norm, out_dtype, rows=None, consumer=None, ctx=None):
         """The normed stream for the next part.  `consumer`: the part that will read it; when it
         declares `takes_deferred_norm` and the pending output is a LazyDelta that the norm can be
-        folded around, the result is an ops.DeferredNorm instead of a tensor."""
+        folded around, the result is an ops.DeferredNorm instead of a tensor.  With more rows than the fused
+        products take, a consumer that has a method wants_deferred_norm(ctx, rows) is asked first (ctx: the step's
+        context): one that would only apply the norm the plain way gets the plain norm, in one kernel instead of two."""
         if (rows is None and isinstance(self.pending, LazyDelta) and getattr(consumer, "takes_deferred_norm", False)
                 and getattr(norm, "deferrable", False)):
             deferred = self.pending.linear.into_stream(self.pending.act, self.x, norm.weight, norm.eps)
@@ -222,7 +224,9 @@ class ResidualStream:
         if (rows is None and getattr(consumer, "takes_deferred_norm", False) and getattr(norm, "deferrable", False)
                 and not isinstance(self.pending, LazyDelta)):
             from .. import ops
-            if ops.can_sum_deferred(self.x.shape[0], self.x.shape[1], out_dtype) and self.x.is_contiguous():
+            wants = getattr(consumer, "wants_deferred_norm", None)
+            if (ops.can_sum_deferred(self.x.shape[0], self.x.shape[1], out_dtype) and self.x.is_contiguous()
+                    and (wants is None or ctx is None or wants(ctx, self.x.shape[0]))):
                 # more rows than the fused products take: one kernel adds the pending output (a tensor or partial sums)
                 # and leaves the norm's factor to the consumer's own kernels
                 deferred = ops.sum_deferred(self.x, self.pending, norm.weight, norm.eps)

@@ -41,14 +41,14 @@ class PreNormBlock(Part):
         tap = getattr(ctx, "tap", None)        # diagnostics (StepContext.tap): the stream at the reference's three dump points
         if tap is not None:
             tap("layer_in", ctx.entry, stream, ctx)
-        h = stream.normed(self.mixer_norm, ctx.act_dtype, consumer=self.mixer)
+        h = stream.normed(self.mixer_norm, ctx.act_dtype, consumer=self.mixer, ctx=ctx)
         if getattr(self.mixer, "gives_lazy_delta", False):
             stream.add(self.mixer.forward(h, ctx, kv, lazy_ok=True))
         else:
             stream.add(self.mixer.forward(h, ctx, kv))
         if tap is not None:
             tap("ffn_in", ctx.entry, stream, ctx)
-        h = stream.normed(self.ffn_norm, ctx.act_dtype, consumer=self.ffn)
+        h = stream.normed(self.ffn_norm, ctx.act_dtype, consumer=self.ffn, ctx=ctx)
         if getattr(self.ffn, "gives_lazy_delta", False):
             stream.add(self.ffn.forward(h, ctx, lazy_ok=True))
         else:
