@@ -18,12 +18,13 @@
 
 // The streamed copy of a bf16 weight matrix W[N, K], for the kernels that read W once per call in the operand layout of
 // v_mfma_f32_16x16x32_bf16 (lane l = r + 16 g holds columns 8 g .. 8 g + 7 of row r of a 16 x 32 block): tile (a, b) is rows
-// 16 a .. 16 a + 15, columns 32 b .. 32 b + 31, stored as BN_STREAM_TILE elements of which lane l's eight are the
-// elements 8 l .. 8 l + 7; tiles in the order [ceil(N / 16)][ceil(K / 32)], rows past N and columns past K zero.  One
-// load of a wave reads one tile as 1 KB of consecutive bytes.  The Python side reads these lines too.
-#define BN_STREAM_TILE_ROWS 16
+// R a .. R a + R - 1, columns 32 b .. 32 b + 31, for a number R <= 16 of rows per tile that the copy names (16, or fewer
+// where that spreads the tiles more evenly over the CUs); its 32 R elements are stored so that the eight of lane
+// r + 16 g (r < R) are the elements 8 (R g + r) .. 8 (R g + r) + 7; tiles in the order [ceil(N / R)][ceil(K / 32)], rows
+// past N and columns past K zero.  One load of a wave reads one tile as 64 R consecutive bytes (the lanes r >= R idle).
+// The Python side reads these lines too.
+#define BN_STREAM_TILE_ROWS 16        // the most rows of a tile
 #define BN_STREAM_TILE_COLS 32
-#define BN_STREAM_TILE (BN_STREAM_TILE_ROWS * BN_STREAM_TILE_COLS)
 
 // error codes returned by the extern "C" entry points (0 = ok, >0 = hipError_t)
 #define BN_ERR_ARG   (-1)     // an argument the kernel cannot take (size, alignment)

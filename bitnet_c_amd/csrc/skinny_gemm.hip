@@ -21,8 +21,9 @@
 // a row), parks it in a region of shared memory of its own (no workgroup barrier) and reads the
 // operand fragments from there; the vector memory pipe is left to the weights.
 //
-// TILED: W is the streamed copy of the matrix (common.h: tiles of 16 rows x 32 columns in the lanes' order, 1 KB each);
-// a load of a wave is then one tile, 1 KB of consecutive bytes, and ldw the number of tiles along K.  Measured against
+// TILED: W is the streamed copy of the matrix (common.h: tiles of up to 16 rows x 32 columns in the lanes' order); a
+// load of a wave is then one tile, up to 1 KB of consecutive bytes, ldw the number of tiles along K, and a workgroup
+// owns the columns of one row of tiles.  Measured against
 // the row-major matrix at 8 rows of an 8B shape: QKV 14.3 -> 13.2 us, output projection 10.7 -> 9.3, gate/up 49.5 ->
 // 43.9, down 28.0 -> 24.0.
 //
@@ -44,12 +45,16 @@ __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_ke
                                                            int ldw, int ldy, int up_off, int act) {
     constexpr int NA = DUAL ? 2 * MT : MT;            // accumulator tiles per wave
     extern __shared__ __align__(16) float red[];      // [n_waves][NA][64][4]
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);      // a scalar
     const int n_waves = blockDim.x >> 6;
     const int i = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * 16;
+    const int CW = TILED ? up_off : 16;               // columns a workgroup owns; TILED: up_off carries the copy's rows per tile
+    const int n0 = blockIdx.x * CW;
     const int n = min(n0 + i, N - 1);                 // clamp: rows past N are computed and dropped
-    const bf16* wrow = TILED ? W + (size_t)blockIdx.x * ldw * BN_STREAM_TILE + lane * 8 : W + (size_t)n * ldw;
+    const int TS = CW * BN_STREAM_TILE_COLS;          // elements of a tile
+    // tiled: the row of tiles is the same for all lanes (a base in scalar registers), the lane adds its 16 bytes' place
+    const bf16* wrow = TILED ? W + (size_t)blockIdx.x * ldw * TS : W + (size_t)n * ldw;
+    const unsigned lane_at = (g * CW + i) * 8;
     const bf16* urow = DUAL ? W + (size_t)(up_off + n) * ldw : nullptr;
 
     f32x4 acc[NA];
@@ -76,8 +81,8 @@ __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_ke
         for (int j = 0; j < 8; ++j) {
             const int k = kb + j * 32;
             if (TILED)          // tile kc / 32 + j of this block of rows; its columns past K hold zeros
-                wv[j] = (kc + j * 32 < K) ? *reinterpret_cast<const uint4*>(wrow + (size_t)((kc >> 5) + j) * BN_STREAM_TILE)
-                                          : make_uint4(0, 0, 0, 0);
+                wv[j] = (i < CW && kc + j * 32 < K) ? *reinterpret_cast<const uint4*>(wrow + (size_t)((kc >> 5) + j) * TS + lane_at)
+                                                    : make_uint4(0, 0, 0, 0);
             else
                 wv[j] = (k < K) ? *reinterpret_cast<const uint4*>(wrow + k) : make_uint4(0, 0, 0, 0);
             if (DUAL) uv[j] = (k < K) ? *reinterpret_cast<const uint4*>(urow + k) : make_uint4(0, 0, 0, 0);
@@ -131,7 +136,7 @@ __global__ __launch_bounds__((DUAL && MT >= 3) ? 512 : 1024) void skinny_gemm_ke
             if (DUAL) u += red[(((size_t)w * NA + MT + mt) * 64 + l) * 4 + r];
         }
         const int m = mt * 16 + 4 * (l >> 4) + r;
-        const int nn = n0 + (l & 15);
+        const int nn = (l & 15) < CW ? n0 + (l & 15) : N;          // a column past the workgroup's own is nobody's
         if (GLU8) {
             // columns 0..7 of the tile are gates, 8..15 the ups of the same result columns
             const float up = __shfl_xor(v, 8, BN_WAVE);
@@ -175,23 +180,26 @@ void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict
                               int K, int ldx, int ldw, int ldy, int tile_cols, int act, SkinnyFused f) {
     constexpr int NW = 8;                              // always eight waves: wave w owns rows w and w + 8 of the norm
     extern __shared__ __align__(16) float red[];       // [NW][64][4], then 16 row scales, then the staging
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // the wave's number as a scalar: what depends on it alone (its chunks of K, a tile's address) stays in scalar registers
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, g = lane >> 4;
     // A workgroup owns tile_cols <= 16 columns (the rest of its MFMA tile is not loaded and not stored): the
     // host picks the width that spreads the column tiles evenly over the CUs.
     const int n0 = blockIdx.x * tile_cols;
     const bool col = i < tile_cols;
     const int n = min(n0 + i, N - 1);
-    // tiled: tile_cols is 16 and the workgroup's rows are one row of tiles
-    const bf16* wrow = TILED ? W + (size_t)blockIdx.x * ldw * BN_STREAM_TILE + lane * 8 : W + (size_t)n * ldw;
+    // tiled: tile_cols is the copy's rows per tile and the workgroup's rows are one row of tiles
+    const int TS = tile_cols * BN_STREAM_TILE_COLS;
+    // (the row of tiles is the same for all lanes, a base in scalar registers; the lane adds its 16 bytes' place)
+    const bf16* wrow = TILED ? W + (size_t)blockIdx.x * ldw * TS : W + (size_t)n * ldw;
+    const unsigned lane_at = (g * tile_cols + i) * 8;
     float* scale_s = red + NW * 256;
     unsigned char* xs = reinterpret_cast<unsigned char*>(red + NW * 256 + 16) + (size_t)wave * M * SK_XROW;
 
     f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
-    auto step = [&](int kc) {
+    auto fetch = [&](int kc, uint4* wv, uint4* xd) {
         const int kb = kc + g * 8;
         const int xk = kc + (lane & 31) * 8;
-        uint4 wv[8], xd[8], xv[8];
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
             const int row = 2 * r + (lane >> 5);
@@ -202,11 +210,14 @@ void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict
         for (int j = 0; j < 8; ++j) {
             const int k = kb + j * 32;
             if (TILED)
-                wv[j] = (kc + j * 32 < K) ? *reinterpret_cast<const uint4*>(wrow + (size_t)((kc >> 5) + j) * BN_STREAM_TILE)
-                                          : make_uint4(0, 0, 0, 0);
+                wv[j] = (col && kc + j * 32 < K) ? *reinterpret_cast<const uint4*>(wrow + (size_t)((kc >> 5) + j) * TS + lane_at)
+                                                 : make_uint4(0, 0, 0, 0);
             else
                 wv[j] = (col && k < K) ? *reinterpret_cast<const uint4*>(wrow + k) : make_uint4(0, 0, 0, 0);
         }
+    };
+    auto multiply = [&](const uint4* wv, const uint4* xd) {
+        uint4 xv[8];
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
             const int row = 2 * r + (lane >> 5);
@@ -220,6 +231,11 @@ void skinny_gemm_fused_kernel(const bf16* __restrict__ X, const bf16* __restrict
 #pragma unroll
         for (int j = 0; j < 8; ++j)
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xv[j]), as_bf16x8(wv[j]), acc, 0, 0, 0);
+    };
+    auto step = [&](int kc) {
+        uint4 wv[8], xd[8];
+        fetch(kc, wv, xd);
+        multiply(wv, xd);
     };
     // the slots of the norm are asked for first: they arrive while the wave waits for its first weights
     float sv[2][SL];                                   // PRE: this lane's slots of rows wave and wave + 8
@@ -310,11 +326,15 @@ static int sk_fused_tile_cols(int N) {
     return pick;
 }
 
+// Columns per workgroup that the fused kernel picks for a product of N columns over a row-major W: the rows per tile
+// that a streamed copy of W is best made with.
+extern "C" int bn_skinny_gemm_fused_tile_cols(int N) { return N < 1 ? 0 : sk_fused_tile_cols(N); }
+
 // Column tiles (= slots per row that a RES call writes) of the fused kernel for N columns; over a streamed copy of W
-// (tiled) they are its rows of tiles.
-extern "C" int bn_skinny_gemm_fused_tiles(int N, int tiled) {
-    if (N < 1) return 0;
-    const int tc = tiled ? 16 : sk_fused_tile_cols(N);
+// (tile_rows > 0) they are its rows of tiles.
+extern "C" int bn_skinny_gemm_fused_tiles(int N, int tile_rows) {
+    if (N < 1 || tile_rows < 0 || tile_rows > BN_STREAM_TILE_ROWS) return 0;
+    const int tc = tile_rows ? tile_rows : sk_fused_tile_cols(N);
     return (N + tc - 1) / tc;
 }
 
@@ -325,13 +345,16 @@ extern "C" int bn_skinny_gemm_fused_tiles(int N, int tiled) {
 // resid != null (RES): the product is added to resid [M, N] in place; resid_bf16 [M, N] becomes the new stream
 // times next_weight [N], slots_out [M, bn_skinny_gemm_fused_tiles(N)] the sums of squares of its column tiles
 // (glu8 == 0, no Y).
-// tiled: W is the streamed copy (common.h) of the matrix (of its 2N interleaved rows with glu8) and ldw its tiles along K.
+// tile_rows > 0: W is the streamed copy (common.h) of the matrix (of its 2N interleaved rows with glu8, then with 16 rows
+// a tile) with that many rows a tile and ldw its tiles along K; a RES call then writes a slot per row of tiles.
 extern "C" int bn_skinny_gemm_fused(const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw, int ldy,
                                     int glu8, int act, const float* slots_in, int n_slots, int stream_width, float eps,
                                     float* resid, int ld_resid, void* resid_bf16, int ld_rb, const float* next_weight,
-                                    float* slots_out, int tiled, hipStream_t s) {
+                                    float* slots_out, int tile_rows, hipStream_t s) {
+    const bool tiled = tile_rows != 0;
     if (!bn_skinny_gemm_supports(M, N, K, ldx, tiled ? 8 : ldw) || M > 16 || act < 0 || act >= BN_ACT_KINDS) return BN_ERR_ARG;
-    if (tiled && !sk_tiled_ok(K, ldw)) return BN_ERR_ARG;
+    if (tiled && (!sk_tiled_ok(K, ldw) || tile_rows < 1 || tile_rows > BN_STREAM_TILE_ROWS || (glu8 && tile_rows != 16)))
+        return BN_ERR_ARG;
     if (((uintptr_t)X | (uintptr_t)W) & 15) return BN_ERR_ARG;
     const bool pre = slots_in != nullptr, res = resid != nullptr;
     if (!pre && !res) return BN_ERR_ARG;
@@ -347,7 +370,7 @@ extern "C" int bn_skinny_gemm_fused(const void* X, const void* W, void* Y, int M
     f.resid = resid; f.resid_bf16 = (bf16*)resid_bf16; f.next_weight = next_weight; f.slots_out = slots_out;
     f.ld_resid = ld_resid; f.ld_rb = ld_rb;
     const size_t smem = (size_t)(8 * 256 + 16) * sizeof(float) + (size_t)8 * M * SK_XROW;
-    const int tile_cols = (glu8 || tiled) ? 16 : sk_fused_tile_cols(N);
+    const int tile_cols = tiled ? tile_rows : (glu8 ? 16 : sk_fused_tile_cols(N));
     const dim3 grid((N + tile_cols - 1) / tile_cols), block(8 * 64);
     auto go = [&](auto kernel) {
         if (smem > 64 * 1024) {
@@ -392,7 +415,8 @@ static int launch(const void* X, const void* W, void* Y, int M, int N, int K, in
             raised = true;
         }
     }
-    hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(n_waves * 64), smem, s,
+    const int cols = TILED ? up_off : 16;             // columns a workgroup owns
+    hipLaunchKernelGGL(kernel, dim3((N + cols - 1) / cols), dim3(n_waves * 64), smem, s,
                        (const bf16*)X, (const bf16*)W, (TO*)Y, M, N, K, ldx, ldw, ldy, up_off, act);
     return bn_launch_status();
 }
@@ -430,18 +454,23 @@ extern "C" int bn_skinny_gemm_supports(int M, int N, int K, int ldx, int ldw) {
 // the gate rows at [0, N) and the up rows at [up_off, up_off + N).  dual == 2: W has 2N rows, gate
 // and up interleaved in blocks of 8 (N a multiple of 8); the result has N columns.  act: the gate's activation
 // (BN_ACT_*), used when dual != 0.
-// tiled: W is the streamed copy (common.h) and ldw its tiles along K; up to 16 rows, dual == 0.
+// tile_rows > 0: W is the streamed copy (common.h) with that many rows a tile and ldw its tiles along K; up to 16 rows,
+// dual == 0.
 extern "C" int bn_skinny_gemm(int out_dtype, const void* X, const void* W, void* Y, int M, int N, int K,
-                              int ldx, int ldw, int ldy, int dual, int up_off, int act, int tiled, hipStream_t s) {
+                              int ldx, int ldw, int ldy, int dual, int up_off, int act, int tile_rows, hipStream_t s) {
+    const bool tiled = tile_rows != 0;
     if (!bn_skinny_gemm_supports(M, N, K, ldx, tiled ? 8 : ldw) || ldy < N || act < 0 || act >= BN_ACT_KINDS) return BN_ERR_ARG;
     if (((uintptr_t)X | (uintptr_t)W) & 15) return BN_ERR_ARG;
     if (tiled) {
-        if (dual || M > 16 || !sk_tiled_ok(K, ldw)) return BN_ERR_ARG;
+        if (dual || M > 16 || !sk_tiled_ok(K, ldw) || tile_rows < 1 || tile_rows > BN_STREAM_TILE_ROWS) return BN_ERR_ARG;
         int n_waves = 8;                           // as the row-major form with staged activations
         const int k_chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
         while (n_waves > 1 && n_waves / 2 >= k_chunks) n_waves >>= 1;
-        if (out_dtype == BN_DT_BF16) return launch<1, false, bf16, false, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, act, n_waves, s);
-        if (out_dtype == BN_DT_F32) return launch<1, false, float, false, true>(X, W, Y, M, N, K, ldx, ldw, ldy, 0, act, n_waves, s);
+        // the kernel's up_off carries the rows per tile; its grid is one workgroup per row of tiles
+        if (out_dtype == BN_DT_BF16)
+            return launch<1, false, bf16, false, true>(X, W, Y, M, N, K, ldx, ldw, ldy, tile_rows, act, n_waves, s);
+        if (out_dtype == BN_DT_F32)
+            return launch<1, false, float, false, true>(X, W, Y, M, N, K, ldx, ldw, ldy, tile_rows, act, n_waves, s);
         return BN_ERR_DTYPE;
     }
     if (dual == 2) {

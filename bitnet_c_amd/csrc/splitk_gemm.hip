@@ -18,11 +18,11 @@
 // without a test per load, and the two sets of weight registers swap roles from step to step instead of being
 // copied: a fifth of the vector instructions of the loop's first form.
 //
-// TILED: W is a copy laid out for this way of reading it (bn_stream_tile_*, common.h): tiles of 16 rows x 32 columns,
-// 1 KB each, a tile's 16 bytes of lane l = row + 16 g at byte 16 l, the tiles of 16 rows one after another along K.  A
-// load of a wave is then 1 KB of consecutive bytes and a wave's whole stream one run of memory, where the row-major
-// matrix gives 64 bytes in each of 16 rows: measured 5 to 15 % faster at every shape tried (8B down product, 64 rows: 29.2
-// -> 26.8 us; 70B gate/up, 17 rows: 192 -> 165).  ldw is then the number of tiles along K.
+// TILED: W is a copy laid out for this way of reading it (the streamed copy of common.h): tiles of tile_rows <= 16 rows x
+// 32 columns in the lanes' order, the tiles of one block of rows one after another along K.  A load of a wave is then
+// one run of 64 tile_rows bytes and a wave's whole stream one run of memory, where the row-major matrix gives 64 bytes
+// in each of 16 rows: measured 5 to 15 % faster at every shape tried (8B down product, 64 rows: 29.2 -> 26.8 us; 70B
+// gate/up, 17 rows: 192 -> 165).  ldw is then the number of tiles along K, and a wave owns tile_rows columns.
 //
 // The same loop with K unsplit and a SwiGLU epilogue is the gate/up product of a feed-forward, from one row on: W holds
 // gate and up rows interleaved in blocks of 8, a wave's 16 columns are 8 gate and 8 up columns of the same 8 outputs,
@@ -61,17 +61,25 @@ struct SgNorm {
 template <int MT, int NWV, bool GLU, bool TILED>
 __global__ __launch_bounds__(NWV * 64) void splitk_gemm_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                                float* __restrict__ P, bf16* __restrict__ Y, int M, int N, int K,
-                                                               int ldx, int ldw, int ldy, int k_per_split, int act, SgNorm nrm) {
+                                                               int ldx, int ldw, int ldy, int k_per_split, int act, SgNorm nrm,
+                                                               int tile_rows) {
     extern __shared__ __align__(16) unsigned char xs[];       // [2][MT * 16][SG_XROW], GLU: then MT * 16 row factors
     constexpr int ROWS = MT * 16;
     constexpr int RP = NWV * 2;                               // rows staged per pass of the workgroup (32 threads a row)
     constexpr int XL = (ROWS + RP - 1) / RP;                  // staging loads per thread and step
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int i = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * (NWV * 16) + wave * 16;
-    // row-major: this lane's row (rows past N are computed and dropped); tiled: this lane's 16 bytes of the wave's first tile
-    const bf16* wrow = TILED ? W + (size_t)min(n0 >> 4, (N - 1) >> 4) * ldw * BN_STREAM_TILE + lane * 8
+    const int CW = TILED ? tile_rows : 16;                    // columns of the result that a wave owns
+    const int n0 = (blockIdx.x * NWV + wave) * CW;
+    const bool col = i < CW;
+    // row-major: this lane's row (rows past N are computed and dropped); tiled: this lane's 16 bytes of the wave's first
+    // tile (the last block of rows stands in for a wave past the end)
+    const int TS = CW * BN_STREAM_TILE_COLS;                  // elements of a tile
+    // (the wave's row of tiles is a base in scalar registers, the lane adds its 16 bytes' place at the load)
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const bf16* wrow = TILED ? W + (size_t)min((int)(blockIdx.x * NWV + wave_u), (N - 1) / CW) * ldw * TS
                              : W + (size_t)min(n0 + i, N - 1) * ldw;
+    const unsigned lane_at = TILED ? (g * CW + i) * 8 : 0;
     const int k_begin = blockIdx.y * k_per_split;
     const int k_end = min(K, k_begin + k_per_split);
     const int n_steps = (k_end - k_begin + SG_STEP - 1) / SG_STEP;
@@ -96,16 +104,16 @@ __global__ __launch_bounds__(NWV * 64) void splitk_gemm_kernel(const bf16* __res
     auto load_w = [&](uint4* dst, int k0) {
         // load j: columns k0 + 32 j + 8 g .. + 7 of the lane's row; in the tiled copy that is tile k0 / 32 + j (whose
         // columns past K hold zeros, so a tile that begins below k_end is read whole)
-        constexpr int JS = TILED ? BN_STREAM_TILE : 32;
-        const bf16* p = TILED ? wrow + (size_t)(k0 >> 5) * BN_STREAM_TILE : wrow + k0 + g * 8;
+        const int JS = TILED ? TS : 32;
+        const bf16* p = TILED ? wrow + (size_t)(k0 >> 5) * TS + lane_at : wrow + k0 + g * 8;
         const int kl = TILED ? k0 : k0 + g * 8;
-        if (k0 + SG_STEP <= k_end) {
+        if (col && k0 + SG_STEP <= k_end) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) dst[j] = *reinterpret_cast<const uint4*>(p + j * JS);
         } else {
 #pragma unroll
             for (int j = 0; j < 8; ++j)
-                dst[j] = (kl + j * 32 < k_end) ? *reinterpret_cast<const uint4*>(p + j * JS) : make_uint4(0, 0, 0, 0);
+                dst[j] = (col && kl + j * 32 < k_end) ? *reinterpret_cast<const uint4*>(p + j * JS) : make_uint4(0, 0, 0, 0);
         }
     };
     auto store_x = [&](int buf) {
@@ -191,7 +199,7 @@ __global__ __launch_bounds__(NWV * 64) void splitk_gemm_kernel(const bf16* __res
         return;
     }
     float* out = P + (size_t)blockIdx.y * M * N;
-    if (n0 + i < N) {
+    if (col && n0 + i < N) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -213,26 +221,33 @@ static int sg_compute_units() {
     return cus;
 }
 
-// K per k-range for a product of N columns over K: as many ranges as make column groups x ranges about the
-// number of CUs, each a multiple of the step and at least two steps long.
-static int sg_k_per_split(int N, int K) {
-    const int groups = (N + SG_COLS - 1) / SG_COLS;
+// K per k-range for a product whose columns fall into `groups` workgroups: as many ranges as make groups x ranges about
+// the number of CUs, each a multiple of the step and at least two steps long.
+static int sg_k_per_split(int groups, int K) {
     int want = (sg_compute_units() + groups / 2) / groups;
     want = max(1, min(want, K / (2 * SG_STEP)));
     int kps = (K + want - 1) / want;
     return (kps + SG_STEP - 1) / SG_STEP * SG_STEP;
 }
+// workgroups along the columns: SG_WAVES waves of 16 columns each, or of tile_rows over a streamed copy
+static int sg_groups(int N, int tile_rows) {
+    const int cw = tile_rows > 0 ? tile_rows : 16;
+    return ((N + cw - 1) / cw + SG_WAVES - 1) / SG_WAVES;
+}
+static bool sg_tile_rows_ok(int tile_rows) { return tile_rows == 0 || (tile_rows >= 1 && tile_rows <= BN_STREAM_TILE_ROWS); }
 
-// 1 when the kernel takes this product.  tiled: W is the streamed copy (common.h) and ldw its tiles along K.
-extern "C" int bn_splitk_gemm_supports(int M, int N, int K, int ldx, int ldw, int tiled) {
+// 1 when the kernel takes this product.  tile_rows > 0: W is the streamed copy (common.h) with that many rows a tile and
+// ldw its tiles along K; 0: W is row-major with row stride ldw.
+extern "C" int bn_splitk_gemm_supports(int M, int N, int K, int ldx, int ldw, int tile_rows) {
     if (!(M >= 1 && M <= SG_MAX_ROWS && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldx >= K)) return 0;
-    return (tiled ? ldw == (K + BN_STREAM_TILE_COLS - 1) / BN_STREAM_TILE_COLS : (ldw % 8 == 0 && ldw >= K)) ? 1 : 0;
+    if (!sg_tile_rows_ok(tile_rows)) return 0;
+    return (tile_rows ? ldw == (K + BN_STREAM_TILE_COLS - 1) / BN_STREAM_TILE_COLS : (ldw % 8 == 0 && ldw >= K)) ? 1 : 0;
 }
 
-// number of k-ranges (= slabs of the result) for a product of N columns over K
-extern "C" int bn_splitk_gemm_splits(int N, int K) {
-    if (N < 1 || K < 1) return 0;
-    const int kps = sg_k_per_split(N, K);
+// number of k-ranges (= slabs of the result) for a product of N columns over K (tile_rows as above)
+extern "C" int bn_splitk_gemm_splits(int N, int K, int tile_rows) {
+    if (N < 1 || K < 1 || !sg_tile_rows_ok(tile_rows)) return 0;
+    const int kps = sg_k_per_split(sg_groups(N, tile_rows), K);
     return (K + kps - 1) / kps;
 }
 
@@ -266,20 +281,21 @@ static int sg_launch(int M, dim3 grid, hipStream_t s, Args... args) {
 }
 
 // P[splits, M, N] (float32, contiguous) = the partial products of X[M, K] (bf16, row stride ldx) and W[N, K] (bf16,
-// row stride ldw; tiled: the streamed copy, ldw its tiles along K) over bn_splitk_gemm_splits(N, K) ranges of K.
-// X and W 16-byte aligned.
+// row stride ldw; tile_rows > 0: the streamed copy, ldw its tiles along K) over bn_splitk_gemm_splits(N, K, tile_rows)
+// ranges of K.  X and W 16-byte aligned.
 extern "C" int bn_splitk_gemm(const void* X, const void* W, float* P, int M, int N, int K, int ldx, int ldw, int splits,
-                              int tiled, hipStream_t s) {
-    if (!bn_splitk_gemm_supports(M, N, K, ldx, ldw, tiled) || !X || !W || !P) return BN_ERR_ARG;
-    if ((((uintptr_t)X | (uintptr_t)W | (uintptr_t)P) & 15) || splits != bn_splitk_gemm_splits(N, K)) return BN_ERR_ARG;
-    const int kps = sg_k_per_split(N, K);
-    const dim3 grid((N + SG_COLS - 1) / SG_COLS, splits);
+                              int tile_rows, hipStream_t s) {
+    if (!bn_splitk_gemm_supports(M, N, K, ldx, ldw, tile_rows) || !X || !W || !P) return BN_ERR_ARG;
+    if ((((uintptr_t)X | (uintptr_t)W | (uintptr_t)P) & 15) || splits != bn_splitk_gemm_splits(N, K, tile_rows)) return BN_ERR_ARG;
+    const int groups = sg_groups(N, tile_rows);
+    const int kps = sg_k_per_split(groups, K);
+    const dim3 grid(groups, splits);
     const SgNorm none{nullptr, 0, 0.f, 0.f, 1};
-    if (tiled)
+    if (tile_rows)
         return sg_launch<SG_WAVES, false, true>(M, grid, s, (const bf16*)X, (const bf16*)W, P, (bf16*)nullptr, M, N, K, ldx, ldw,
-                                                0, kps, 0, none);
+                                                0, kps, 0, none, tile_rows);
     return sg_launch<SG_WAVES, false, false>(M, grid, s, (const bf16*)X, (const bf16*)W, P, (bf16*)nullptr, M, N, K, ldx, ldw, 0,
-                                             kps, 0, none);
+                                             kps, 0, none, 0);
 }
 
 // Whether workgroups of SG_GLU_WIDE_WAVES waves leave the busiest CU fewer of the N / 16 column tiles than workgroups of
@@ -291,14 +307,16 @@ static bool sg_glu_wide(int N) {
 }
 
 // Y[M, F] (bf16, row stride ldy) = act(c X . Wg^T) * (c X . Wu^T) for W [2F, K] with gate and up rows interleaved in blocks
-// of 8 (F a multiple of 8); X, W, tiled as above; act one of BN_ACT_*.  c is 1 with slots == null; else X is the copy of a
+// of 8 (F a multiple of 8); X, W as above; tiled: W is the streamed copy with 16 rows a tile (a tile then holds both halves
+// of 8 outputs) and ldw its tiles along K; act one of BN_ACT_*.  c is 1 with slots == null; else X is the copy of a
 // stream of stream_width columns that a deferred norm leaves, slots [M, n_slots] (contiguous) the parts of its rows' sums
 // of squares, and c the row's 1 / sqrt(sum / stream_width + eps).
 extern "C" int bn_splitk_gemm_swiglu(const void* X, const void* W, void* Y, int M, int F, int K, int ldx, int ldw, int ldy,
                                      int act, const float* slots, int n_slots, int stream_width, float eps, int tiled,
                                      hipStream_t s) {
     if (act < 0 || act >= BN_ACT_KINDS) return BN_ERR_ARG;
-    if (F < 8 || F % 8 || F > (1 << 29) || !bn_splitk_gemm_supports(M, 2 * F, K, ldx, ldw, tiled) || !X || !W || !Y || ldy < F)
+    const int tile_rows = tiled ? 16 : 0;
+    if (F < 8 || F % 8 || F > (1 << 29) || !bn_splitk_gemm_supports(M, 2 * F, K, ldx, ldw, tile_rows) || !X || !W || !Y || ldy < F)
         return BN_ERR_ARG;
     if (((uintptr_t)X | (uintptr_t)W) & 15) return BN_ERR_ARG;
     if (slots && (n_slots < 1 || stream_width < 1)) return BN_ERR_ARG;
@@ -314,10 +332,10 @@ extern "C" int bn_splitk_gemm_swiglu(const void* X, const void* W, void* Y, int 
     auto grid = [&](int waves) { return dim3((N + waves * 16 - 1) / (waves * 16), 1); };
     if (!tiled)
         return sg_launch<SG_GLU_WAVES, true, false>(M, grid(SG_GLU_WAVES), s, (const bf16*)X, (const bf16*)W, (float*)nullptr,
-                                                    (bf16*)Y, M, N, K, ldx, ldw, ldy, kps, act, nrm);
+                                                    (bf16*)Y, M, N, K, ldx, ldw, ldy, kps, act, nrm, 0);
     if (sg_glu_wide(N))
         return sg_launch<SG_GLU_WIDE_WAVES, true, true>(M, grid(SG_GLU_WIDE_WAVES), s, (const bf16*)X, (const bf16*)W,
-                                                        (float*)nullptr, (bf16*)Y, M, N, K, ldx, ldw, ldy, kps, act, nrm);
+                                                        (float*)nullptr, (bf16*)Y, M, N, K, ldx, ldw, ldy, kps, act, nrm, 16);
     return sg_launch<SG_GLU_WAVES, true, true>(M, grid(SG_GLU_WAVES), s, (const bf16*)X, (const bf16*)W, (float*)nullptr,
-                                               (bf16*)Y, M, N, K, ldx, ldw, ldy, kps, act, nrm);
+                                               (bf16*)Y, M, N, K, ldx, ldw, ldy, kps, act, nrm, 16);
 }

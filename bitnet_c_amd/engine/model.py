@@ -86,7 +86,7 @@ class DecoderModel:
             return 0
         head = 0
         if self.lm_head is not None and self.lm_head.shape[1] % 8 == 0:
-            R, C = ops.STREAM_TILE_ROWS, ops.STREAM_TILE_COLS
+            R, C = ops.stream_tile_rows(self.lm_head.shape[0]), ops.STREAM_TILE_COLS
             head = -(-self.lm_head.shape[0] // R) * R * -(-self.lm_head.shape[1] // C) * C * 2
         return head + sum(l.stream_bytes() for l in self.linears())
 

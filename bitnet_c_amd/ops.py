@@ -80,6 +80,7 @@ _SIGNATURES = {
         "bn_skinny_gemm_supports": [c_int, c_int, c_int, c_int, c_int],
         "bn_skinny_gemm": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                            c_int, c_int, c_int, c_void_p],
+        "bn_skinny_gemm_fused_tile_cols": [c_int],
         "bn_skinny_gemm_fused_tiles": [c_int, c_int],
         "bn_skinny_gemm_fused": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                  c_void_p, c_int, c_int, c_float, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
@@ -87,7 +88,7 @@ _SIGNATURES = {
     },
     "splitk_gemm": {
         "bn_splitk_gemm_supports": [c_int, c_int, c_int, c_int, c_int, c_int],
-        "bn_splitk_gemm_splits": [c_int, c_int],
+        "bn_splitk_gemm_splits": [c_int, c_int, c_int],
         "bn_splitk_gemm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "bn_splitk_gemm_swiglu": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int,
                                   c_int, c_float, c_int, c_void_p],
@@ -381,13 +382,16 @@ STREAM_TILE_COLS = _build.header_constant("BN_STREAM_TILE_COLS")
 @dataclass
 class StreamedWeight:
     """A bf16 weight matrix [N, K] in the order in which the kernels that read it once per call load it (csrc/common.h):
-    tiles of 16 rows x 32 columns, each the 1 KB that one load of a wave takes (lane r + 16 g: columns 8 g .. 8 g + 7 of row
-    r), [ceil(N / 16), ceil(K / 32), 512], rows past N and columns past K zero.  A second copy beside the row-major matrix,
-    which the products of many rows (the library's) and everything else keep reading: the kernels of up to 128 rows take it
-    through their `streamed` argument and give the same result bit for bit, 5 to 15 % sooner."""
+    tiles of tile_rows (at most 16) rows x 32 columns, each the run of bytes that one load of a wave takes (lane r + 16 g:
+    columns 8 g .. 8 g + 7 of row r), [ceil(N / tile_rows), ceil(K / 32), 32 tile_rows], rows past N and columns past K zero.
+    A second copy beside the row-major matrix, which the products of many rows (the library's) and everything else keep
+    reading: the kernels of up to 128 rows take it through their `streamed` argument and give the same result bit for
+    bit, 5 to 15 % sooner.  The kernel of up to 16 rows gives a workgroup one row of tiles, so fewer than 16 rows a tile
+    are chosen where that spreads the tiles more evenly over the CUs (stream_tile_rows)."""
     tiles: torch.Tensor
     N: int
     K: int
+    tile_rows: int = STREAM_TILE_ROWS
 
     @property
     def k_tiles(self) -> int:
@@ -397,12 +401,22 @@ class StreamedWeight:
         return self.tiles.numel() * self.tiles.element_size()
 
 
-def stream_copy(w: torch.Tensor) -> StreamedWeight:
-    """The streamed copy of w [N, K] (bf16, on the device; made there)."""
+def stream_tile_rows(N: int) -> int:
+    """The rows per tile with which a matrix of N rows is best streamed: the columns that the fused product of up to 16
+    rows gives a workgroup over the row-major matrix (16, or fewer when that leaves the busiest CU at least 15 % fewer
+    columns: 12 for 6,144 rows on 256 CUs, 10 for 5,120)."""
+    return int(_fn("skinny_gemm", "bn_skinny_gemm_fused_tile_cols")(int(N)))
+
+
+def stream_copy(w: torch.Tensor, tile_rows: Optional[int] = None) -> StreamedWeight:
+    """The streamed copy of w [N, K] (bf16, on the device; made there).  tile_rows None: stream_tile_rows(N); a matrix
+    with gate and up rows interleaved in blocks of 8 needs 16."""
     require_gpu()
     _dev(w, "w", torch.bfloat16, 2)
     N, K = w.shape
-    R, C = STREAM_TILE_ROWS, STREAM_TILE_COLS
+    R, C = (stream_tile_rows(N) if tile_rows is None else int(tile_rows)), STREAM_TILE_COLS
+    if not 1 <= R <= STREAM_TILE_ROWS:
+        raise KernelError(f"stream_copy: a tile has 1 to {STREAM_TILE_ROWS} rows, not {R}")
     nt, kt = (N + R - 1) // R, (K + C - 1) // C
     if nt * R != N or kt * C != K:
         padded = torch.zeros((nt * R, kt * C), dtype=w.dtype, device=w.device)
@@ -410,28 +424,32 @@ def stream_copy(w: torch.Tensor) -> StreamedWeight:
         w = padded
     # [nt, r, kt, g, 8] -> [nt, kt, g, r, 8]: lane r + 16 g of tile (nt, kt)
     tiles = w.view(nt, R, kt, C // 8, 8).permute(0, 2, 3, 1, 4).contiguous().view(nt, kt, R * C)
-    return StreamedWeight(tiles, N, K)
+    return StreamedWeight(tiles, N, K, R)
 
 
 def unstream(sw: StreamedWeight) -> torch.Tensor:
     """The row-major matrix [N, K] that a streamed copy holds."""
-    R, C = STREAM_TILE_ROWS, STREAM_TILE_COLS
+    R, C = sw.tile_rows, STREAM_TILE_COLS
     nt, kt = sw.tiles.shape[:2]
     return sw.tiles.view(nt, kt, C // 8, R, 8).permute(0, 3, 1, 2, 4).reshape(nt * R, kt * C)[:sw.N, :sw.K].contiguous()
 
 
-def _weight_arg(w: torch.Tensor, streamed: Optional[StreamedWeight], what: str):
-    """(pointer, row stride or tiles along K, tiled) of the weights that a kernel is to read: the streamed copy if one is
-    given (checked against w), else w itself."""
+def _weight_arg(w: torch.Tensor, streamed: Optional[StreamedWeight], what: str, need_rows: int = 0):
+    """(pointer, row stride or tiles along K, rows per tile or 0) of the weights that a kernel is to read: the streamed
+    copy if one is given (checked against w; need_rows: the only tile height the kernel takes, else w is read), else
+    w itself."""
+    if streamed is not None and need_rows and getattr(streamed, "tile_rows", 0) != need_rows:
+        streamed = None
     if streamed is None:
         return w.data_ptr(), _rows(w, "w"), 0
     t = streamed.tiles
+    R = streamed.tile_rows
     if (not isinstance(streamed, StreamedWeight) or (streamed.N, streamed.K) != tuple(w.shape) or t.device != w.device
-            or t.dtype != torch.bfloat16 or not t.is_contiguous() or t.dim() != 3
-            or tuple(t.shape) != ((streamed.N + STREAM_TILE_ROWS - 1) // STREAM_TILE_ROWS,
-                                  (streamed.K + STREAM_TILE_COLS - 1) // STREAM_TILE_COLS, STREAM_TILE_ROWS * STREAM_TILE_COLS)):
+            or t.dtype != torch.bfloat16 or not t.is_contiguous() or t.dim() != 3 or not 1 <= R <= STREAM_TILE_ROWS
+            or tuple(t.shape) != ((streamed.N + R - 1) // R, (streamed.K + STREAM_TILE_COLS - 1) // STREAM_TILE_COLS,
+                                  R * STREAM_TILE_COLS)):
         raise KernelError(f"{what}: the streamed copy does not belong to w {tuple(w.shape)}")
-    return t.data_ptr(), t.shape[1], 1
+    return t.data_ptr(), t.shape[1], R
 
 
 # bf16 products with many rows: the library's matrix product (as the reference hands its batched
@@ -536,7 +554,7 @@ def _staged_swiglu(x, w_gate_up, pre, activation, streamed=None):
     M, K = x.shape
     F = w_gate_up.shape[0] // 2
     ldx = _rows(x, "x")
-    wp, wl, tiled = _weight_arg(w_gate_up, streamed, "linear_swiglu")
+    wp, wl, tiled = _weight_arg(w_gate_up, streamed, "linear_swiglu", need_rows=STREAM_TILE_ROWS)
     if F % 8 or not _fn("splitk_gemm", "bn_splitk_gemm_supports")(M, 2 * F, K, ldx, wl, tiled):
         return None
     if pre is not None:          # what the kernel's passes over the parts of the sums of squares hold (SG_NORM_*)
@@ -548,7 +566,7 @@ def _staged_swiglu(x, w_gate_up, pre, activation, streamed=None):
     _check(_fn("splitk_gemm", "bn_splitk_gemm_swiglu")(
         x.data_ptr(), wp, y.data_ptr(), M, F, K, ldx, wl, F, _act(activation),
         pre.slots.data_ptr() if pre is not None else None, pre.slots.shape[1] if pre is not None else 0,
-        pre.stream.shape[1] if pre is not None else 0, float(pre.eps) if pre is not None else 0.0, tiled, _stream()),
+        pre.stream.shape[1] if pre is not None else 0, float(pre.eps) if pre is not None else 0.0, int(tiled != 0), _stream()),
         "splitk_gemm(glu)")
     return y
 
@@ -646,7 +664,7 @@ def linear_partial_sums(x: torch.Tensor, w: torch.Tensor, streamed: Optional[Str
     if not _fn("splitk_gemm", "bn_splitk_gemm_supports")(M, N, K, ldx, wl, tiled) or (x.data_ptr() | wp) % 16:
         raise KernelError(f"linear_partial_sums: the kernel takes 1 to 128 rows, K a multiple of 8 and 16-byte aligned "
                           f"operands, not x {tuple(x.shape)} (row stride {ldx}), w {tuple(w.shape)} (row stride {wl})")
-    S = _fn("splitk_gemm", "bn_splitk_gemm_splits")(N, K)
+    S = _fn("splitk_gemm", "bn_splitk_gemm_splits")(N, K, tiled)
     slabs = torch.empty((S, M, N), dtype=torch.float32, device=x.device)
     _check(_fn("splitk_gemm", "bn_splitk_gemm")(x.data_ptr(), wp, slabs.data_ptr(), M, N, K, ldx, wl, S, tiled,
                                                 _stream()), "splitk_gemm")
@@ -748,7 +766,7 @@ def can_fuse_norm(M: int, N: int, K: int, dtype) -> bool:
 
 def _fused_call(x, w, y, M, N, K, glu8, pre: Optional[DeferredNorm], resid, resid_bf16, next_weight, slots_out,
                 activation: str = "silu", streamed: Optional[StreamedWeight] = None):
-    wp, wl, tiled = _weight_arg(w, streamed, "fused product")
+    wp, wl, tiled = _weight_arg(w, streamed, "fused product", need_rows=STREAM_TILE_ROWS if glu8 else 0)
     _check(_fn("skinny_gemm", "bn_skinny_gemm_fused")(
         x.data_ptr(), wp, y.data_ptr() if y is not None else None, M, N, K, _rows(x, "x"), wl,
         N if y is not None else 0, int(glu8), _act(activation),
@@ -809,10 +827,10 @@ def linear_swiglu_prenorm(pre: DeferredNorm, w_gate_up: torch.Tensor, activation
     return y
 
 
-def _fused_tiles(N: int, tiled: bool = False) -> int:
-    """Column tiles of the fused product kernel for N columns (over a streamed copy if tiled): one partial sum of
-    squares per row and tile."""
-    return int(_fn("skinny_gemm", "bn_skinny_gemm_fused_tiles")(int(N), int(tiled)))
+def _fused_tiles(N: int, tile_rows: int = 0) -> int:
+    """Column tiles of the fused product kernel for N columns (over a streamed copy with tile_rows rows a tile if that
+    is not 0): one partial sum of squares per row and tile."""
+    return int(_fn("skinny_gemm", "bn_skinny_gemm_fused_tiles")(int(N), int(tile_rows)))
 
 
 def can_defer_norm(M: int, N: int, K: int, dtype) -> bool:
@@ -837,8 +855,11 @@ def linear_into_stream(x: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, w
                           f"weight {tuple(weight.shape)} do not agree")
     if not can_defer_norm(M, N, K, torch.bfloat16) or x.data_ptr() % 16 or w.data_ptr() % 16:
         raise KernelError(f"linear_into_stream: {M} rows, w {tuple(w.shape)} cannot be fused")
+    if streamed is not None and _fused_tiles(N, streamed.tile_rows) > FUSED_SLOTS:
+        streamed = None                       # more rows of tiles than a consumer adds up slots
     scaled = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-    slots = torch.empty((M, _fused_tiles(N, streamed is not None)), dtype=torch.float32, device=x.device)
+    slots = torch.empty((M, _fused_tiles(N, streamed.tile_rows if streamed is not None else 0)), dtype=torch.float32,
+                        device=x.device)
     _fused_call(x, w, None, M, N, K, False, None, stream, scaled, weight, slots, streamed=streamed)
     return DeferredNorm(scaled, slots, stream, weight, float(eps))
 

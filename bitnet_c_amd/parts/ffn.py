@@ -26,6 +26,7 @@ class SwiGLU(Part):
             raise ValueError(f"feed-forward: unknown activation {activation!r}; known: {sorted(ops.ACTIVATIONS)}")
         self.hidden, self.F, self.has_bias, self.activation = int(hidden), int(intermediate), bool(bias), activation
         self.gate_up, self.down = Linear(), Linear()
+        self.gate_up.stream_tile_rows = ops.STREAM_TILE_ROWS     # gate and up interleaved in blocks of 8: a tile holds both
 
     def tensors(self):
         t = {"w_gate": ParamSpec((self.F, self.hidden)), "w_up": ParamSpec((self.F, self.hidden)),

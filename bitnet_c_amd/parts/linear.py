@@ -18,6 +18,7 @@ class Linear:
         self.weight = None
         self.bias = None
         self.streamed = None     # ops.StreamedWeight: the weight once more, in the order the decode kernels read it
+        self.stream_tile_rows = None     # rows per tile of that copy; None: what suits the matrix (ops.stream_tile_rows)
 
     def load(self, weight: torch.Tensor, bias, device, dtype):
         self.weight = upload(weight, device, dtype)
@@ -29,12 +30,12 @@ class Linear:
         w = self.weight
         if w is None or w.dtype != torch.bfloat16 or w.dim() != 2 or not w.is_cuda or w.shape[1] % 8:
             return 0
-        R, C = ops.STREAM_TILE_ROWS, ops.STREAM_TILE_COLS
+        R, C = self.stream_tile_rows or ops.stream_tile_rows(w.shape[0]), ops.STREAM_TILE_COLS
         return -(-w.shape[0] // R) * R * -(-w.shape[1] // C) * C * 2
 
     def keep_streamed(self, keep: bool = True) -> None:
         """Makes (or drops) the streamed copy of the weight, which every product of up to 128 rows then reads."""
-        self.streamed = ops.stream_copy(self.weight) if keep and self.stream_bytes() else None
+        self.streamed = ops.stream_copy(self.weight, self.stream_tile_rows) if keep and self.stream_bytes() else None
 
     def __call__(self, x, out_dtype=None, rows: slice | None = None) -> torch.Tensor:
         """x: activations, or an ops.DeferredNorm whose norm this product applies itself when it can."""

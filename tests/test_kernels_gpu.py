@@ -412,7 +412,7 @@ def test_swiglu_product_with_staged_activations(M, F, K):
     if lo <= M <= hi:                              # without the library this is the kernel of these row counts
         assert torch.equal(ops.linear_swiglu(xd, wi, True, allow_library=False), y)
     # over the streamed copy of the weights (other workgroup sizes, the same sums): the same bits
-    ws = ops.stream_copy(wi)
+    ws = ops.stream_copy(wi, 16)
     y2 = torch.full((M, F), float("nan"), dtype=torch.bfloat16, device="cuda")
     rc = ops._fn("splitk_gemm", "bn_splitk_gemm_swiglu")(xd.data_ptr(), ws.tiles.data_ptr(), y2.data_ptr(), M, F, K, K, ws.k_tiles,
                                                          F, ops.ACTIVATIONS["silu"], None, 0, 0, 0.0, 1,
@@ -451,49 +451,60 @@ def test_staged_swiglu_product_applies_a_deferred_norm(M, D, F):
     classic = ops.linear_swiglu(pre.materialize(), wi, True)
     e_got, e_classic = rel_err(got.float(), exact), rel_err(classic.float(), exact)
     assert e_got <= 2.0 * e_classic + 2.0 ** -7, (e_got, e_classic)
-    assert torch.equal(ops._staged_swiglu(pre.scaled, wi, pre, "silu", ops.stream_copy(wi)), got)
+    assert torch.equal(ops._staged_swiglu(pre.scaled, wi, pre, "silu", ops.stream_copy(wi, 16)), got)
     routed = ops.linear_swiglu_prenorm(pre, wi) if (M <= 16 or ops.LIBRARY_PRODUCTS) else got
     assert rel_err(routed.float(), exact) <= 2.0 * e_classic + 2.0 ** -7
 
 
 def test_the_streamed_copy_is_the_lanes_order():
-    """The streamed copy of a weight matrix by its definition: tile (a, b) holds rows 16 a .. 16 a + 15 and columns
-    32 b .. 32 b + 31, lane l = r + 16 g of a wave gets elements 8 l .. 8 l + 7 of the tile, which are columns 8 g .. 8 g + 7
-    of row r; rows past N and columns past K are zero; unstream gives the matrix back."""
+    """The streamed copy of a weight matrix by its definition: tile (a, b) holds rows R a .. R a + R - 1 and columns
+    32 b .. 32 b + 31 (R rows a tile, at most 16), lane l = r + 16 g of a wave (r < R) gets elements 8 (R g + r) .. + 7 of the
+    tile, which are columns 8 g .. 8 g + 7 of row r; rows past N and columns past K are zero; unstream gives the matrix
+    back.  The height that a matrix gets unasked is the one that spreads its tiles evenly over the CUs."""
     ops = _ops()
-    for N, K in ((31, 264), (48, 64), (100, 1000), (16, 8)):
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    assert ops.stream_tile_rows(16 * cus) == 16 and ops.stream_tile_rows(16 * cus * 7) == 16
+    assert ops.stream_tile_rows(24 * cus) == 12 and ops.stream_tile_rows(20 * cus) == 10      # 6,144 and 5,120 on 256 CUs
+    for N, K, R in ((31, 264, 16), (48, 64, 12), (100, 1000, 10), (16, 8, 16), (50, 96, 7), (6144, 64, None)):
         w = _rand((N, K), torch.bfloat16, 71, 0.5).cuda()
-        sw = ops.stream_copy(w)
-        nt, kt = (N + 15) // 16, (K + 31) // 32
-        assert tuple(sw.tiles.shape) == (nt, kt, 512) and (sw.N, sw.K, sw.k_tiles) == (N, K, kt)
-        assert sw.nbytes() == nt * kt * 1024
+        sw = ops.stream_copy(w, R)
+        R = R or ops.stream_tile_rows(N)
+        nt, kt = (N + R - 1) // R, (K + 31) // 32
+        assert tuple(sw.tiles.shape) == (nt, kt, 32 * R) and (sw.N, sw.K, sw.k_tiles, sw.tile_rows) == (N, K, kt, R)
+        assert sw.nbytes() == nt * kt * 64 * R
         assert torch.equal(ops.unstream(sw), w)
         t, wc = sw.tiles.cpu(), w.cpu()
-        for a, b, lane in ((0, 0, 0), (nt - 1, kt - 1, 63), (nt - 1, 0, 17), (0, kt - 1, 40), (nt // 2, kt // 2, 5)):
-            r, g = lane % 16, lane // 16
-            row, col = 16 * a + r, 32 * b + 8 * g
+        for a, b, r, g in ((0, 0, 0, 0), (nt - 1, kt - 1, R - 1, 3), (nt - 1, 0, 1, 1), (0, kt - 1, R // 2, 2), (nt // 2, kt // 2, 5, 0)):
+            row, col = R * a + r, 32 * b + 8 * g
             want = torch.zeros(8, dtype=torch.bfloat16)
             if row < N and col < K:
                 n = min(8, K - col)
                 want[:n] = wc[row, col:col + n]
-            assert torch.equal(t[a, b, 8 * lane:8 * lane + 8], want), (N, K, a, b, lane)
+            at = 8 * (R * g + r)
+            assert torch.equal(t[a, b, at:at + 8], want), (N, K, R, a, b, r, g)
     with pytest.raises(ops.KernelError):                   # a copy of another matrix
         ops.linear(torch.zeros(4, 64, dtype=torch.bfloat16, device="cuda"), torch.zeros(32, 64, dtype=torch.bfloat16, device="cuda"),
                    streamed=ops.stream_copy(torch.zeros(48, 64, dtype=torch.bfloat16, device="cuda")))
+    with pytest.raises(ops.KernelError):
+        ops.stream_copy(torch.zeros(48, 64, dtype=torch.bfloat16, device="cuda"), 17)
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 64, 128])
-@pytest.mark.parametrize("N,K", [(100, 64), (48, 1000), (264, 3592), (4104, 4096), (31, 264), (4096, 14336)])
-def test_products_over_the_streamed_copy_are_the_same_bits(M, N, K):
+@pytest.mark.parametrize("N,K,R", [(100, 64, 16), (48, 1000, 12), (264, 3592, 10), (4104, 4096, 16), (31, 264, 7), (4096, 14336, None),
+                                   (6144, 512, None)])
+def test_products_over_the_streamed_copy_are_the_same_bits(M, N, K, R):
     """Every product that takes a streamed copy of its weights forms the same sums in the same order as over the
     row-major matrix: the plain product of up to 16 rows (bf16 and float32 results), the products with a norm folded
     in (before, after, with the gated unit), and the partial sums of up to 128 rows.  N and K that are no multiples
-    of the tile's 16 and 32 among them."""
+    of the tile's rows and 32 columns among them, tiles of 7 to 16 rows, and the height a matrix gets unasked."""
     ops = _ops()
     x, w = _rand((M, K), torch.bfloat16, 81).cuda(), _rand((N, K), torch.bfloat16, 82, 0.05).cuda()
-    sw = ops.stream_copy(w)
+    sw = ops.stream_copy(w, R)
     a, b = ops.linear_partial_sums(x, w), ops.linear_partial_sums(x, w, sw)
-    assert torch.equal(a.slabs, b.slabs)
+    if a.slabs.shape == b.slabs.shape:
+        assert torch.equal(a.slabs, b.slabs)
+    else:                           # narrower tiles, more workgroups along the columns, other ranges of K: the same sum
+        assert rel_err(b.slabs.sum(dim=0), a.slabs.sum(dim=0)) < 1e-6
     if M > 16:
         return
     for out in (torch.bfloat16, torch.float32):
@@ -506,16 +517,21 @@ def test_products_over_the_streamed_copy_are_the_same_bits(M, N, K):
     p1 = ops.linear_into_stream(x, w, s1, norm_w, eps)
     p2 = ops.linear_into_stream(x, w, s2, norm_w, eps, sw)
     assert torch.equal(s1, s2) and torch.equal(p1.scaled, p2.scaled)
-    assert p2.slots.shape[1] == (N + 15) // 16                      # one part per row of tiles
+    assert p2.slots.shape[1] == (N + sw.tile_rows - 1) // sw.tile_rows           # one part per row of tiles
     assert rel_err(p2.slots.sum(dim=1), p1.slots.sum(dim=1)) < 1e-6
+    if R is None:                                                  # the copy's own height is the row-major kernel's tile
+        assert torch.equal(p1.slots, p2.slots)
     # the next product reads either norm; its own weights streamed or not
-    F = 40 if N % 8 == 0 else 0
     if N % 8 == 0:
+        F = 40
         w_in = _rand((2 * F, N), torch.bfloat16, 85, 0.05).cuda()
-        si = ops.stream_copy(w_in)
+        si, si16 = ops.stream_copy(w_in, 10), ops.stream_copy(w_in, 16)
         for pre in (p1, p2):
             assert torch.equal(ops.linear_prenorm(pre, w_in), ops.linear_prenorm(pre, w_in, si))
-            assert torch.equal(ops.linear_swiglu_prenorm(pre, w_in), ops.linear_swiglu_prenorm(pre, w_in, streamed=si))
+            # gate and up interleaved: tiles of 16 rows are read, a copy of another height is passed over
+            want = ops.linear_swiglu_prenorm(pre, w_in)
+            assert torch.equal(want, ops.linear_swiglu_prenorm(pre, w_in, streamed=si16))
+            assert torch.equal(want, ops.linear_swiglu_prenorm(pre, w_in, streamed=si))
 
 
 @pytest.mark.parametrize("activation", ["gelu_tanh", "relu2", "silu"])
