@@ -138,21 +138,29 @@ def _kernel_attention_decode(H=32, Hkv=8, hs=128):
 
 def _kernel_mid(rows=64, copies=3):
     """The products of a decode step of 64 rows, every weight matrix read cold: gate/up through this library's own kernel
-    with the SwiGLU epilogue (what runs when the library may not be called) and through the library, the feed-forward's
-    last product and the output projection as partial sums."""
+    with the SwiGLU epilogue over the row-major matrix and over its streamed copy, and through the library; the
+    feed-forward's last product and the output projection as partial sums, row-major and streamed."""
     import torch
     from bitnet_c_amd import ops
     x = torch.randn(rows, 4096, device="cuda:0", dtype=torch.bfloat16)
     ws = [torch.randn(28672, 4096, device="cuda:0", dtype=torch.bfloat16) * 0.02 for _ in range(copies)]
+    streamed = [ops.stream_copy(w, ops.STREAM_TILE_ROWS) for w in ws]
     for w in ws:
-        ops.linear_swiglu(x, w, True, allow_library=False)
+        ops._staged_swiglu(x, w, None, "silu")
+    for w, sw in zip(ws, streamed):
+        ops._staged_swiglu(x, w, None, "silu", sw)
     for w in ws:
         ops.swiglu(torch.matmul(x, w.t()), True)
-    del ws
+    del ws, streamed
     for n, k in ((4096, 14336), (4096, 4096)):
         xs = torch.randn(rows, k, device="cuda:0", dtype=torch.bfloat16)
-        for _ in range(copies):
-            ops.linear_partial_sums(xs, torch.randn(n, k, device="cuda:0", dtype=torch.bfloat16) * 0.02)
+        ws = [torch.randn(n, k, device="cuda:0", dtype=torch.bfloat16) * 0.02 for _ in range(copies)]
+        streamed = [ops.stream_copy(w) for w in ws]
+        for w in ws:
+            ops.linear_partial_sums(xs, w)
+        for w, sw in zip(ws, streamed):
+            ops.linear_partial_sums(xs, w, sw)
+        del ws, streamed
     torch.cuda.synchronize()
 
 
