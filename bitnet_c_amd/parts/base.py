@@ -10,6 +10,8 @@ Interfaces (a new part implements the one of its kind and registers itself):
 
   every part     tensors() -> {local name: TensorSpec-like (shape, init, optional)}
                  load(tensors: {local name: host tensor}, device, dtype) -> None
+                 linears() -> [parts.linear.Linear] (optional: the weight matrices that the model may keep a
+                 second time in the order the decode kernels read them)
 
   norm           apply(x_f32 [T, D], delta or None, out_dtype, rows=None) -> [T or len(rows), D]
                  (adds delta into x in place when rows is None, then norms)
