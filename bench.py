@@ -146,9 +146,9 @@ def _kernel_mid(rows=64, copies=3):
     ws = [torch.randn(28672, 4096, device="cuda:0", dtype=torch.bfloat16) * 0.02 for _ in range(copies)]
     streamed = [ops.stream_copy(w, ops.STREAM_TILE_ROWS) for w in ws]
     for w in ws:
-        ops._staged_swiglu(x, w, None, "silu")
+        ops.linear_swiglu(x, w, True, allow_library=False)
     for w, sw in zip(ws, streamed):
-        ops._staged_swiglu(x, w, None, "silu", sw)
+        ops.linear_swiglu(x, w, True, streamed=sw)
     for w in ws:
         ops.swiglu(torch.matmul(x, w.t()), True)
     del ws, streamed
