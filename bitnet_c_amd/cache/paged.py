@@ -81,11 +81,22 @@ class _Group:
     pool: PagePool
     pages: Dict[int, List[int]]              # slot -> page of each PAGE positions (-1: given back)
     v_transposed: bool = False               # the layout of v that the group's need asks for
+    blocked: bool = False                    # keys and values in the matrix-core kernels' own order (sizes as v_transposed)
     k: Optional[torch.Tensor] = None         # [entries, pages, Hkv, PAGE, head_dim]
     v: Optional[torch.Tensor] = None         # [entries, pages, Hkv, PAGE, v_dim], or [.., v_dim, PAGE] when v_transposed
 
 
 class PagedCache:
+    @staticmethod
+    def _layout(need: KVNeed, dtype) -> str:
+        """The layout of a need's pages: what it names, else what this library's attention kernels read at the cache's
+        type (and, where the values are as wide as the keys, at the head size)."""
+        if need.v_layout:
+            if need.v_layout == "blocked" and dtype != torch.bfloat16:
+                raise CacheError("blocked pages are bf16 pages")
+            return need.v_layout
+        return kernel_v_layout(dtype, need.head_dim if need.v_dim == need.head_dim else 0)
+
     def __init__(self, needs: Sequence[CacheNeed], kv_from: Sequence[Optional[int]], max_tokens: int,
                  dtype=torch.bfloat16, device=None, max_slots: Optional[int] = None):
         """needs[i], kv_from[i]: what schedule entry i's mixer keeps, and the entry whose keys
@@ -110,8 +121,9 @@ class PagedCache:
             if gi is None:
                 gi = len(self.groups)
                 by_need[need.kv] = gi
-                layout = need.kv.v_layout or kernel_v_layout(dtype)      # the need says how its values lie
-                self.groups.append(_Group(need.kv, [], PagePool(self.n_pages), {}, v_transposed=layout == "transposed"))
+                layout = self._layout(need.kv, dtype)                    # the need says how its values lie
+                self.groups.append(_Group(need.kv, [], PagePool(self.n_pages), {}, v_transposed=layout != "rows",
+                                          blocked=layout == "blocked"))
             self._entry_group.append((gi, len(self.groups[gi].entries)))
             self.groups[gi].entries.append(i)
         for i, src in enumerate(kv_from):
@@ -121,7 +133,7 @@ class PagedCache:
                 a, b = needs[i].kv, needs[src].kv
                 if a is not None and b is not None and (
                         (a.n_kv_heads, a.head_dim, a.v_dim) != (b.n_kv_heads, b.head_dim, b.v_dim)
-                        or (a.v_layout or kernel_v_layout(dtype)) != (b.v_layout or kernel_v_layout(dtype))):
+                        or self._layout(a, dtype) != self._layout(b, dtype)):
                     raise CacheError(f"entry {i} reads the cache of entry {src} but their kv shapes or layouts differ")
                 self._entry_group[i] = self._entry_group[src]
         self._free_slots = list(range(self.max_slots - 1, -1, -1))
@@ -267,7 +279,7 @@ class PagedCache:
         g = self.groups[gi]
         return KVView(k_pages=g.k[idx] if g.k is not None else None,
                       v_pages=g.v[idx] if g.v is not None else None,
-                      v_transposed=g.v_transposed, block_table=block_tables.get(gi),
+                      v_transposed=g.v_transposed, blocked=g.blocked, block_table=block_tables.get(gi),
                       writes=self.kv_from[entry] is None, state=st, max_len=max_len)
 
     def check(self) -> None:

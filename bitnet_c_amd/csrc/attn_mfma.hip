@@ -48,8 +48,8 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 struct MfmaArgs {
     const bf16* q;            // [n_tokens, q_stride], head h at h*HS, rotated
     bf16* out;                // [n_tokens, out_stride]
-    const bf16* k_pages;      // [pages, Hkv, 64, HS]
-    const bf16* vt_pages;     // [pages, Hkv, HS, 64]
+    const bf16* k_pages;      // [pages, Hkv, 64 * HS]: keys in the blocked order of common.h
+    const bf16* vt_pages;     // [pages, Hkv, HS * 64]: values in the blocked order of common.h
     const int* block_table;   // [n_seqs, bt_stride]
     const int* seq_lens;      // decode: keys in the cache, the new one included; 0 = padding row
     const int* tiles;         // prompt: [n, 4] = seq, first token row, tokens, position of the first
@@ -151,7 +151,7 @@ __device__ __forceinline__ int v_swizzle(int row) {
 }
 
 // One 32-key block for NT column tiles, operands straight from the pages (the decode form).  kbase/vbase point at
-// the block's first key inside its page (row strides HS and BN_PAGE).  qpos/lo: per tile, this lane's column's
+// the block inside its page (blocked pages, common.h: every load below is 1 KB of consecutive bytes).  qpos/lo: per tile, this lane's column's
 // position and first visible key (qpos < 0: no such column).  key_hi: keys >= key_hi do not exist (split end /
 // length).  All operands are asked for up front: they come from memory, and the latency is paid once.
 // The prompt form below has code of its own on purpose: the decode kernel is sensitive to how the compiler lays
@@ -161,21 +161,22 @@ __device__ __forceinline__ void attend_block_direct_m(const bf16* __restrict__ k
                                                int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
                                                float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
                                                const int (&lo)[NT], int key_hi, float scale2, int lane) {
-    constexpr int DC = HS / 32, DT = HS / 16, KSTRIDE = HS, VSTRIDE = BN_PAGE;
-    const int i = lane & 15, g = lane >> 4;
-    const int krow0 = 8 * (i >> 2) + (i & 3);        // key row of tile 0; tile 1 is 4 further
+    constexpr int DC = HS / 32, DT = HS / 16;
+    const int g = lane >> 4;
     f32x4 st[NT][2];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) { st[nt][0] = (f32x4){0.f, 0.f, 0.f, 0.f}; st[nt][1] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
     bf16x8 ka[DC][2];
     bf16x8 va[DT];
+    // tile row i of key tile 0 is the block's key 8 (i / 4) + i % 4, tile 1 four further; lane i + 16 g of value tile t
+    // holds dimension 16 t + i of the block's keys 8 g .. 8 g + 7
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
-        ka[c][0] = ld16(kbase + (size_t)krow0 * KSTRIDE + c * 32 + g * 8);
-        ka[c][1] = ld16(kbase + (size_t)(krow0 + 4) * KSTRIDE + c * 32 + g * 8);
+        ka[c][0] = ld16(kbase + (2 * c) * 512 + lane * 8);
+        ka[c][1] = ld16(kbase + (2 * c + 1) * 512 + lane * 8);
     }
 #pragma unroll
-    for (int t = 0; t < DT; ++t) va[t] = ld16(vbase + (size_t)(t * 16 + i) * VSTRIDE + 8 * g);
+    for (int t = 0; t < DT; ++t) va[t] = ld16(vbase + t * 512 + lane * 8);
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
 #pragma unroll
@@ -457,12 +458,19 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
     int k_src[2], v_src[2], k_dst[2], v_dst[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
+        // A stage is one or two whole blocks of the blocked pages (common.h), and the threads fetch it in the pages' own
+        // order, 16 consecutive bytes a thread: piece idx of the keys is lane i + 16 g of tile (c, tile) of block b, which
+        // holds dimensions 32 c + 8 g .. + 7 of the block's key 8 (i / 4) + i % 4 + 4 tile; piece idx of the values is lane
+        // i + 16 g of tile t of block b: keys 8 g .. 8 g + 7 of dimension 16 t + i.  The staged copies keep their own
+        // (swizzled) order, and sixteen neighbouring lanes store the sixteen rows that sixteen lanes later read together.
         const int idx = threadIdx.x + h * 256 * NG;
+        const int b = idx / (4 * HS), rem = idx % (4 * HS);
+        const int li = rem & 15, lg = (rem >> 4) & 3, tl = rem >> 6;
         k_src[h] = idx * 16;
-        const int krow = (idx * 8) / HS, kchunk = ((idx * 8) % HS) / 8;
+        const int krow = 32 * b + 8 * (li >> 2) + (li & 3) + 4 * (tl & 1), kchunk = 4 * (tl >> 1) + lg;
         k_dst[h] = (krow * KS + ((kchunk ^ k_swizzle<HS>(krow)) * 8)) * 2;
-        const int vrow = idx / (KB / 8), vchunk = idx % (KB / 8);
-        v_src[h] = (vrow * BN_PAGE + vchunk * 8) * 2;
+        const int vrow = 16 * tl + li, vchunk = 4 * b + lg;
+        v_src[h] = idx * 16;
         v_dst[h] = (KB * KS + vrow * VS + ((vchunk ^ v_swizzle<KB>(vrow & 15)) * 8)) * 2;
         asm volatile("" : "+v"(k_src[h]), "+v"(v_src[h]), "+v"(k_dst[h]), "+v"(v_dst[h]));
     }
@@ -535,10 +543,10 @@ __global__ __launch_bounds__(256 * NG) __attribute__((amdgpu_waves_per_eu(2, 2))
     auto fetch = [&](int kb, Stage& st) {                 // a stage never crosses a page: KB divides BN_PAGE
         const int page = uniform_load(a.block_table, bt_row + kb / BN_PAGE);
         const int koff = kb % BN_PAGE;
-        // the same addresses in every lane: the page's keys of this kv head (KB rows of HS, contiguous) and its V^T
-        // rows (HS rows of 64 keys, KB of them wanted)
+        // the same addresses in every lane: the first of the stage's blocks of 32 keys in the page's keys of this kv
+        // head, and in its values
         const unsigned char* kg = reinterpret_cast<const unsigned char*>(a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS);
-        const unsigned char* vg = reinterpret_cast<const unsigned char*>(a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff);
+        const unsigned char* vg = reinterpret_cast<const unsigned char*>(a.vt_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS);
         st.k0 = *reinterpret_cast<const uint4*>(kg + (unsigned)k_src[0]);
         st.v0 = *reinterpret_cast<const uint4*>(vg + (unsigned)v_src[0]);
         if (KV4 > 1) {
@@ -757,8 +765,8 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
     if (a.write_kv && L > 0 && L - 1 >= k_lo && L - 1 < k_hi) {
         const int pos = L - 1;
         const int page = a.block_table[(size_t)seq * a.bt_stride + pos / BN_PAGE], off = pos % BN_PAGE;
-        bf16* kdst = const_cast<bf16*>(a.k_pages) + (((size_t)page * a.Hkv + kvh) * BN_PAGE + off) * HS;
-        bf16* vdst = const_cast<bf16*>(a.vt_pages) + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + off;
+        bf16* kdst = const_cast<bf16*>(a.k_pages) + ((size_t)page * a.Hkv + kvh) * BN_PAGE * HS;
+        bf16* vdst = const_cast<bf16*>(a.vt_pages) + ((size_t)page * a.Hkv + kvh) * BN_PAGE * HS;
         const int t = threadIdx.x;
         if (t < HALF) {
             float k0 = __bfloat162float(new_k0), k1 = __bfloat162float(new_k1);
@@ -767,11 +775,11 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
                 const float r0 = k0 * c - k1 * sv, r1 = k0 * sv + k1 * c;
                 k0 = r0; k1 = r1;
             }
-            kdst[t] = __float2bfloat16(k0);
-            kdst[t + HALF] = __float2bfloat16(k1);
+            kdst[bn_blocked_k_offset(off, t, HS)] = __float2bfloat16(k0);
+            kdst[bn_blocked_k_offset(off, t + HALF, HS)] = __float2bfloat16(k1);
         } else if (t < HALF + HS) {
             const int d = t - HALF;
-            vdst[(size_t)d * BN_PAGE] = a.row_ssq ? __float2bfloat16(__bfloat162float(new_v) * row_scale) : new_v;
+            vdst[bn_blocked_v_offset(off, d, HS)] = a.row_ssq ? __float2bfloat16(__bfloat162float(new_v) * row_scale) : new_v;
         }
         // only this workgroup reads what it has just stored: a fence of workgroup scope is enough
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
@@ -807,9 +815,9 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
             // the page index is the same for the whole wave: read through the scalar unit, so that it
             // does not queue behind the vector loads
             const int page = uniform_load(a.block_table, bt_row + __builtin_amdgcn_readfirstlane(kb / BN_PAGE));
-            const int koff = kb % BN_PAGE;
+            const int koff = kb % BN_PAGE;                 // 0 or 32: the page's first or second block
             const bf16* kbase = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS;
-            const bf16* vbase = a.vt_pages + ((size_t)page * a.Hkv + kvh) * HS * BN_PAGE + koff;
+            const bf16* vbase = a.vt_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + koff) * HS;
             const bool need_mask = (kb + 32 > k_hi) || (kb < k_lo);
             attend_block<HS, 1>(kbase, vbase, kb, q, acc, m, l, qpos, lo, k_hi, need_mask, scale2, lane);
         }
@@ -890,7 +898,7 @@ __global__ __launch_bounds__(64) void attn_mfma_combine_kernel(bf16* __restrict_
 }
 
 // 1 when the matrix-core kernels take this shape
-extern "C" int bn_attn_mfma_supports(int hs) { return (hs == 64 || hs == 128) ? 1 : 0; }
+extern "C" int bn_attn_mfma_supports(int hs) { return (hs == BN_MFMA_HEAD_DIM_SMALL || hs == BN_MFMA_HEAD_DIM_LARGE) ? 1 : 0; }
 
 // query tokens per tile of the prompt form, for GT heads per group
 extern "C" int bn_attn_mfma_prompt_tokens(int hs, int GT) { return (hs == 64 ? 256 : 128) / GT; }

@@ -26,6 +26,34 @@
 #define BN_STREAM_TILE_ROWS 16        // the most rows of a tile
 #define BN_STREAM_TILE_COLS 32
 
+// Cache pages in the matrix-core attention kernels' own order ("blocked"; bf16, head sizes that are multiples of 32).  A
+// page still holds BN_PAGE positions of hs elements for every kv head, keys and values each, but inside a (page, kv head)
+// they lie in blocks of 32 positions, and a block in the order in which a wave of the decode kernel loads it: one load
+// instruction takes 1 KB of consecutive bytes where pages that hold a row per position (or a row per dimension) give it
+// 64 bytes in each of 16 rows.  With position p = 32 b + r inside the page:
+//   keys:   the operand of the first product (S^T = K Q^T) is a tile of 16 positions x 32 dimensions, lane i + 16 g holding
+//           dimensions 8 g .. 8 g + 7 of tile row i; a block is two such row sets (tile 0: r = 8 (i / 4) + i % 4, tile 1:
+//           4 further) for each of hs / 32 dimension chunks c.  Element (p, d = 32 c + 8 g + e) lies at
+//           32 hs b + 8 (64 (2 c + tile) + 16 g + i) + e.
+//   values: the operand of the second product is a tile of 16 dimensions x 32 positions, lane i + 16 g holding positions
+//           8 g .. 8 g + 7 of dimension 16 t + i.  Element (p = 32 b + 8 g + e, d = 16 t + i) lies at
+//           32 hs b + 8 (64 t + 16 g + i) + e.
+// Eight consecutive dimensions of a key, and eight consecutive positions (from a multiple of 8) of a value's dimension,
+// stay 16 consecutive bytes, which is what the writers store at once.
+#define BN_KV_BLOCK 32
+// the head sizes that the matrix-core attention kernels are built for (the Python side reads these lines)
+#define BN_MFMA_HEAD_DIM_SMALL 64
+#define BN_MFMA_HEAD_DIM_LARGE 128
+__host__ __device__ __forceinline__ int bn_blocked_k_offset(int p, int d, int hs) {
+    const int b = p >> 5, r = p & 31;
+    const int tile = (r >> 2) & 1, i = ((r >> 3) << 2) | (r & 3);
+    return 32 * hs * b + 8 * (64 * (2 * (d >> 5) + tile) + 16 * ((d >> 3) & 3) + i) + (d & 7);
+}
+__host__ __device__ __forceinline__ int bn_blocked_v_offset(int p, int d, int hs) {
+    const int b = p >> 5;
+    return 32 * hs * b + 8 * (64 * (d >> 4) + 16 * ((p >> 3) & 3) + (d & 15)) + (p & 7);
+}
+
 // error codes returned by the extern "C" entry points (0 = ok, >0 = hipError_t)
 #define BN_ERR_ARG   (-1)     // an argument the kernel cannot take (size, alignment)
 #define BN_ERR_DTYPE (-2)

@@ -5,9 +5,16 @@
 // (src/transformer/cpu_backend.c:283-296).  angle = float(pos) * inv_freq[i], cos/sin
 // at full float32 accuracy (src/transformer.c:143-162 uses cosf/sinf).  The cache
 // holds rotated keys (src/transformer/cpu.c:893-898 rotates the cached row).
-// Cache layout per layer: K [page, kv_head, BN_PAGE, head_dim]; V the same, or transposed
-// [page, kv_head, head_dim, BN_PAGE] (v_transposed) for the matrix-core attention kernels.
+// Cache layout per layer (`layout` below): K [page, kv_head, BN_PAGE, head_dim] and V the same (BN_KV_ROWS), or V
+// transposed [page, kv_head, head_dim, BN_PAGE] (BN_KV_TRANSPOSED), or keys and values of a (page, kv head) in the
+// matrix-core attention kernels' own order (BN_KV_BLOCKED, common.h).  Adding BN_KV_V_BY_TILES says that the values are
+// stored by the page-tile kernel below (a prompt's tokens), not here.
 #include "common.h"
+
+#define BN_KV_ROWS 0
+#define BN_KV_TRANSPOSED 1
+#define BN_KV_BLOCKED 2
+#define BN_KV_V_BY_TILES 4
 
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
@@ -16,12 +23,14 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
                                      const int* __restrict__ block_table, int bt_stride,
                                      T* __restrict__ k_pages, T* __restrict__ v_pages,
                                      const float* __restrict__ inv_freq, int rope_dims,
-                                     int H, int Hkv, int hs, int v_transposed) {
+                                     int H, int Hkv, int hs, int layout) {
     extern __shared__ float cs[];            // cos[half], sin[half]
     const int t = blockIdx.x;
     const int pos = positions[t];
     if (pos < 0) return;                     // a padding row
     const int half = rope_dims / 2;
+    const int kind = layout & 3;
+    const bool v_elsewhere = (layout & BN_KV_V_BY_TILES) != 0;
     float* cos_s = cs;
     float* sin_s = cs + half;
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
@@ -57,11 +66,14 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
         } else {
             o = to_f32(hd[d]);
         }
-        const size_t dst = (((size_t)page * Hkv + kh) * BN_PAGE + off) * hs + d;
-        k_pages[dst] = from_f32<T>(o);
-        if (v_transposed == 2) continue;        // the page-tile kernel below stores V
-        if (v_transposed)       // V pages [page, kv_head, head_dim, BN_PAGE]
-            v_pages[(((size_t)page * Hkv + kh) * hs + d) * BN_PAGE + off] = vrow[idx];
+        const size_t head = ((size_t)page * Hkv + kh) * BN_PAGE * hs;       // this kv head's part of the page
+        const size_t dst = head + (size_t)off * hs + d;
+        k_pages[kind == BN_KV_BLOCKED ? head + bn_blocked_k_offset(off, d, hs) : dst] = from_f32<T>(o);
+        if (v_elsewhere) continue;              // the page-tile kernel below stores V
+        if (kind == BN_KV_BLOCKED)
+            v_pages[head + bn_blocked_v_offset(off, d, hs)] = vrow[idx];
+        else if (kind == BN_KV_TRANSPOSED)      // V pages [page, kv_head, head_dim, BN_PAGE]
+            v_pages[head + (size_t)d * BN_PAGE + off] = vrow[idx];
         else
             v_pages[dst] = vrow[idx];
     }
@@ -92,12 +104,14 @@ __global__ __launch_bounds__(256) void rope_kv_write_bf16x8_kernel(bf16* __restr
                                                                    const int* __restrict__ block_table, int bt_stride,
                                                                    bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
                                                                    const float* __restrict__ inv_freq, int rope_dims,
-                                                                   int H, int Hkv, int hs, int v_transposed) {
+                                                                   int H, int Hkv, int hs, int layout) {
     extern __shared__ float cs[];            // cos[half], sin[half]
     const int t = blockIdx.x;
     const int pos = positions[t];
     if (pos < 0) return;                     // a padding row
     const int half = rope_dims / 2;
+    const int kind = layout & 3;
+    const bool v_elsewhere = (layout & BN_KV_V_BY_TILES) != 0;
     float* cos_s = cs;
     float* sin_s = cs + half;
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
@@ -130,41 +144,49 @@ __global__ __launch_bounds__(256) void rope_kv_write_bf16x8_kernel(bf16* __restr
         uint4 a = *reinterpret_cast<const uint4*>(krow + kh * hs + c * 8);
         uint4 b = *reinterpret_cast<const uint4*>(krow + kh * hs + half + c * 8);
         rotate_groups(a, b, cos_s + c * 8, sin_s + c * 8);
-        bf16* dst = k_pages + (((size_t)page * Hkv + kh) * BN_PAGE + off) * hs;
-        *reinterpret_cast<uint4*>(dst + c * 8) = a;
-        *reinterpret_cast<uint4*>(dst + half + c * 8) = b;
+        // 8 consecutive dimensions of a key are 16 consecutive bytes in either order of a page
+        bf16* head = k_pages + ((size_t)page * Hkv + kh) * BN_PAGE * hs;
+        const bool blocked = kind == BN_KV_BLOCKED;
+        *reinterpret_cast<uint4*>(head + (blocked ? bn_blocked_k_offset(off, c * 8, hs) : off * hs + c * 8)) = a;
+        *reinterpret_cast<uint4*>(head + (blocked ? bn_blocked_k_offset(off, half + c * 8, hs) : off * hs + half + c * 8)) = b;
     }
     const int tail = (hs - rope_dims) / 8;
     for (int idx = threadIdx.x; idx < Hkv * tail; idx += blockDim.x) {
         const int kh = idx / tail, c = idx - kh * tail;
-        bf16* dst = k_pages + (((size_t)page * Hkv + kh) * BN_PAGE + off) * hs;
-        *reinterpret_cast<uint4*>(dst + rope_dims + c * 8) = *reinterpret_cast<const uint4*>(krow + kh * hs + rope_dims + c * 8);
+        bf16* head = k_pages + ((size_t)page * Hkv + kh) * BN_PAGE * hs;
+        const int d = rope_dims + c * 8;
+        *reinterpret_cast<uint4*>(head + (kind == BN_KV_BLOCKED ? bn_blocked_k_offset(off, d, hs) : off * hs + d)) =
+            *reinterpret_cast<const uint4*>(krow + kh * hs + d);
     }
-    // V (v_transposed == 2: the page-tile kernel below stores it)
+    // V (unless the page-tile kernel below stores it)
     const int vg = hs / 8;
-    for (int idx = threadIdx.x; v_transposed != 2 && idx < Hkv * vg; idx += blockDim.x) {
+    for (int idx = threadIdx.x; !v_elsewhere && idx < Hkv * vg; idx += blockDim.x) {
         const int kh = idx / vg, c = idx - kh * vg;
         const uint4 v = *reinterpret_cast<const uint4*>(vrow + kh * hs + c * 8);
-        if (v_transposed) {                  // V pages [page, kv_head, head_dim, BN_PAGE]
-            const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
-            uint16_t* dst = reinterpret_cast<uint16_t*>(v_pages) + (((size_t)page * Hkv + kh) * hs + c * 8) * BN_PAGE + off;
+        const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
+        uint16_t* head = reinterpret_cast<uint16_t*>(v_pages) + ((size_t)page * Hkv + kh) * BN_PAGE * hs;
+        if (kind == BN_KV_BLOCKED) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) dst[(size_t)j * BN_PAGE] = e[j];
+            for (int j = 0; j < 8; ++j) head[bn_blocked_v_offset(off, c * 8 + j, hs)] = e[j];
+        } else if (kind == BN_KV_TRANSPOSED) {      // V pages [page, kv_head, head_dim, BN_PAGE]
+#pragma unroll
+            for (int j = 0; j < 8; ++j) head[(size_t)(c * 8 + j) * BN_PAGE + off] = e[j];
         } else {
-            *reinterpret_cast<uint4*>(v_pages + (((size_t)page * Hkv + kh) * BN_PAGE + off) * hs + c * 8) = v;
+            *reinterpret_cast<uint4*>(head + (size_t)off * hs + c * 8) = v;
         }
     }
 }
 
-// V into transposed pages for the tokens of a prompt: a workgroup takes the rows of one sequence
+// V into transposed or blocked pages for the tokens of a prompt: a workgroup takes the rows of one sequence
 // that fall into one page (tile = sequence, first row, rows, position of the first) and one kv
 // head, turns the [rows, hs] block through shared memory and stores runs of 8 positions with
-// 16 bytes, instead of 2 bytes a position and dimension.
+// 16 bytes, instead of 2 bytes a position and dimension (8 positions from a multiple of 8 of one dimension are
+// 16 consecutive bytes in either order).
 #define VT_PAD 2
 __global__ __launch_bounds__(256) void v_transposed_write_kernel(const bf16* __restrict__ qkv, int row_stride,
                                                                  const int* __restrict__ tiles,
                                                                  const int* __restrict__ block_table, int bt_stride,
-                                                                 bf16* __restrict__ v_pages, int H, int Hkv, int hs) {
+                                                                 bf16* __restrict__ v_pages, int H, int Hkv, int hs, int blocked) {
     extern __shared__ uint16_t vt_s[];       // [hs][BN_PAGE + VT_PAD], column = position inside the page
     const int* tl = tiles + 4 * blockIdx.x;
     const int seq = tl[0], row0 = tl[1], n = tl[2], pos0 = tl[3];
@@ -187,47 +209,53 @@ __global__ __launch_bounds__(256) void v_transposed_write_kernel(const bf16* __r
         const int d = idx / (BN_PAGE / 8), p8 = (idx - d * (BN_PAGE / 8)) * 8;     // positions p8 .. p8+7 of the page
         if (p8 + 8 <= off || p8 >= off + n) continue;
         const uint16_t* src = vt_s + d * ld + p8;
+        uint16_t* run = dst + (blocked ? bn_blocked_v_offset(p8, d, hs) : d * BN_PAGE + p8);
         if (p8 >= off && p8 + 8 <= off + n) {
             uint4 w;
             w.x = src[0] | ((uint32_t)src[1] << 16);
             w.y = src[2] | ((uint32_t)src[3] << 16);
             w.z = src[4] | ((uint32_t)src[5] << 16);
             w.w = src[6] | ((uint32_t)src[7] << 16);
-            *reinterpret_cast<uint4*>(dst + (size_t)d * BN_PAGE + p8) = w;
+            *reinterpret_cast<uint4*>(run) = w;
         } else {
             for (int j = 0; j < 8; ++j)
-                if (p8 + j >= off && p8 + j < off + n) dst[(size_t)d * BN_PAGE + p8 + j] = src[j];
+                if (p8 + j >= off && p8 + j < off + n) run[j] = src[j];
         }
     }
 }
 
-// tiles: [n_tiles, 4] int32 as above; every tile lies inside one page.  V heads are read from qkv.
+// tiles: [n_tiles, 4] int32 as above; every tile lies inside one page.  V heads are read from qkv.  blocked: the pages
+// are in the blocked order (hs a multiple of 32), else transposed.
 extern "C" int bn_v_transposed_write(const void* qkv, int row_stride, const int* tiles, int n_tiles,
                                      const int* block_table, int bt_stride, void* v_pages, int H, int Hkv, int hs,
-                                     hipStream_t s) {
+                                     int blocked, hipStream_t s) {
     if (n_tiles <= 0 || H <= 0 || Hkv <= 0 || hs <= 0 || hs % 8 || row_stride % 8 || row_stride < (H + 2 * Hkv) * hs ||
-        !tiles || !block_table || !v_pages || n_tiles > 0x7fffffff / 4 || Hkv > 65535)
+        !tiles || !block_table || !v_pages || n_tiles > 0x7fffffff / 4 || Hkv > 65535 || (blocked && hs % 32))
         return BN_ERR_ARG;
     if (((uintptr_t)qkv | (uintptr_t)v_pages) & 15) return BN_ERR_ARG;
     const size_t smem = (size_t)hs * (BN_PAGE + VT_PAD) * sizeof(uint16_t);
     if (smem > 64 * 1024) return BN_ERR_ARG;
     hipLaunchKernelGGL(v_transposed_write_kernel, dim3(n_tiles, Hkv), dim3(256), smem, s, (const bf16*)qkv, row_stride,
-                       tiles, block_table, bt_stride, (bf16*)v_pages, H, Hkv, hs);
+                       tiles, block_table, bt_stride, (bf16*)v_pages, H, Hkv, hs, blocked);
     return bn_launch_status();
 }
 
 // qkv: [n_tokens, row_stride] with Q heads first, then K heads, then V heads.
 // k_pages == null: rotate Q only (a layer that reads another layer's cache).
 // rope_dims == 0: no rotation, the write alone.
-// v_transposed: 0 = V pages like K pages, 1 = transposed pages, 2 = transposed pages that
-// bn_v_transposed_write fills (V is left alone here).
+// layout: BN_KV_ROWS (0) = V pages like K pages, BN_KV_TRANSPOSED (1) = transposed V pages, BN_KV_BLOCKED (2) = keys and
+// values in the blocked order (hs a multiple of 32); + BN_KV_V_BY_TILES (4): bn_v_transposed_write fills the values (V is
+// left alone here).
 extern "C" int bn_rope_kv_write(int dtype, void* qkv, int row_stride, const int* positions,
                                 const int* seq_index, const int* block_table, int bt_stride,
                                 void* k_pages, void* v_pages, const float* inv_freq, int rope_dims,
-                                int n_tokens, int H, int Hkv, int hs, int v_transposed, hipStream_t s) {
+                                int n_tokens, int H, int Hkv, int hs, int layout, hipStream_t s) {
     if (n_tokens <= 0 || H <= 0 || Hkv < 0 || hs <= 0 || rope_dims < 0 || rope_dims > hs ||
         (rope_dims & 1) || row_stride < (H + 2 * Hkv) * hs)
         return BN_ERR_ARG;
+    if (layout < 0 || (layout & 3) > BN_KV_BLOCKED || (layout & ~7) || ((layout & 3) == BN_KV_BLOCKED && hs % 32))
+        return BN_ERR_ARG;
+    const int v_transposed = layout;
     if (rope_dims > 0 && inv_freq == nullptr) return BN_ERR_ARG;
     if (k_pages && (!v_pages || !block_table || !seq_index)) return BN_ERR_ARG;
     const size_t smem = (size_t)(rope_dims > 0 ? rope_dims : 2) * sizeof(float);

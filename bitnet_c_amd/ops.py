@@ -47,7 +47,7 @@ _SIGNATURES = {
     },
     "rope_kv": {
         "bn_v_transposed_write": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
-                                  c_void_p],
+                                  c_int, c_void_p],
         "bn_rope_kv_write": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                              c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
@@ -868,37 +868,98 @@ def linear_into_stream(x: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, w
 # position encoding + cache write, attention
 # --------------------------------------------------------------------------------------
 
-def kernel_v_layout(dtype) -> str:
-    """The value layout (KVNeed.v_layout) that the attention kernels of this library read fastest at a cache
-    type: bf16 values transposed inside a page ([pages, Hkv, hs, PAGE]) for the matrix-core kernels, float32
-    values like the keys ([pages, Hkv, PAGE, hs]).  The vector kernel and the cache write take either layout
-    at either type; the matrix-core kernels take the transposed one alone."""
-    return "transposed" if dtype == torch.bfloat16 else "rows"
+KV_BLOCK = _build.header_constant("BN_KV_BLOCK")       # positions in a block of a blocked page
 
 
-def _check_pages(k_pages, v_pages, Hkv, hs, dtype, v_transposed=None):
-    """Checks both page tensors against the layout that the caller names (None: kernel_v_layout of the type);
-    returns whether V is transposed.  The kernels here want values as wide as keys."""
-    vt = kernel_v_layout(dtype) == "transposed" if v_transposed is None else bool(v_transposed)
-    for t, nm, shape in ((k_pages, "k_pages", (Hkv, PAGE, hs)), (v_pages, "v_pages", (Hkv, hs, PAGE) if vt else (Hkv, PAGE, hs))):
+def kernel_v_layout(dtype, head_dim: int = 0) -> str:
+    """The page layout (KVNeed.v_layout) that the attention kernels of this library read fastest at a cache type and
+    head size: "blocked" for bf16 at the head sizes of the matrix-core kernels (keys and values of a page in those
+    kernels' own order, blocked_page_index), else bf16 values transposed inside a page ([pages, Hkv, hs, PAGE]) and
+    float32 values like the keys ([pages, Hkv, PAGE, hs]).  Without a head size: "transposed" or "rows".  The vector
+    kernel and the cache write take rows and transposed values at either type; the matrix-core kernels take blocked
+    pages alone."""
+    if dtype != torch.bfloat16:
+        return "rows"
+    return "blocked" if head_dim and mfma_attention(dtype, head_dim) else "transposed"
+
+
+def _page_layout(dtype, hs: int, v_transposed, blocked) -> str:
+    """The layout that a caller names with v_transposed (None, False, True) and blocked (None, False, True); neither:
+    kernel_v_layout."""
+    if blocked:
+        if v_transposed is False or dtype != torch.bfloat16 or hs % 32:
+            raise KernelError(f"blocked pages are bf16 pages of head sizes that are multiples of 32 (got {dtype}, {hs})")
+        return "blocked"
+    if v_transposed is None:
+        return kernel_v_layout(dtype, hs if blocked is None else 0)
+    return "transposed" if v_transposed else "rows"
+
+
+_LAYOUT_CODES = {"rows": 0, "transposed": 1, "blocked": 2}       # BN_KV_* of csrc/rope_kv.hip; + 4: values by page tiles
+
+
+def _check_pages(k_pages, v_pages, Hkv, hs, dtype, v_transposed=None, blocked=None) -> str:
+    """Checks both page tensors against the layout that the caller names (_page_layout) and returns it.  The kernels here
+    want values as wide as keys.  Blocked pages have the shapes of pages with transposed values."""
+    layout = _page_layout(dtype, hs, v_transposed, blocked)
+    v_shape = (Hkv, PAGE, hs) if layout == "rows" else (Hkv, hs, PAGE)
+    for t, nm, shape in ((k_pages, "k_pages", (Hkv, PAGE, hs)), (v_pages, "v_pages", v_shape)):
         _dev(t, nm, dtype, 4)
         if tuple(t.shape[1:]) != shape or not t.is_contiguous():
             raise KernelError(f"{nm}: expected contiguous [pages, {', '.join(map(str, shape))}], got {tuple(t.shape)}")
     if k_pages.shape[0] != v_pages.shape[0]:
         raise KernelError("k_pages and v_pages differ in their number of pages")
-    return vt
+    return layout
+
+
+def blocked_page_index(hs: int):
+    """Where the elements of a (page, kv head) lie in a blocked page (csrc/common.h), as two int64 tensors: k_index[p, d]
+    = the place of dimension d of the key at position p, v_index[d, p] = the place of dimension d of the value at
+    position p, both counted in elements from the beginning of the (page, kv head).  Position p = 32 b + r: the keys'
+    operand tiles hold the block's positions 8 (i / 4) + i % 4 (tile 0) and 4 further (tile 1) in tile row i, a lane
+    group g the dimensions 32 c + 8 g .. + 7; the values' tiles hold dimension 16 t + i in row i, a lane group the
+    positions 8 g .. 8 g + 7 of the block."""
+    if hs % 32:
+        raise KernelError(f"blocked pages need a head size that is a multiple of 32, got {hs}")
+    p = torch.arange(PAGE).view(PAGE, 1)
+    d = torch.arange(hs).view(1, hs)
+    b, r = p // 32, p % 32
+    tile, i = (r // 4) % 2, (r // 8) * 4 + r % 4
+    k_index = 32 * hs * b + 8 * (64 * (2 * (d // 32) + tile) + 16 * ((d // 8) % 4) + i) + d % 8
+    v_index = 32 * hs * b + 8 * (64 * (d // 16) + 16 * ((p // 8) % 4) + d % 16) + p % 8
+    return k_index.contiguous(), v_index.t().contiguous()
+
+
+def to_blocked_pages(k_rows: torch.Tensor, v_transposed: torch.Tensor):
+    """Pages [n, Hkv, PAGE, hs] of keys and [n, Hkv, hs, PAGE] of transposed values as blocked pages (the same shapes)."""
+    hs = k_rows.shape[-1]
+    ki, vi = (t.to(k_rows.device).reshape(-1) for t in blocked_page_index(hs))
+    k = torch.empty_like(k_rows).view(*k_rows.shape[:2], -1)
+    v = torch.empty_like(v_transposed).view(*v_transposed.shape[:2], -1)
+    k[..., ki] = k_rows.reshape(*k_rows.shape[:2], -1)
+    v[..., vi] = v_transposed.reshape(*v_transposed.shape[:2], -1)
+    return k.view(k_rows.shape), v.view(v_transposed.shape)
+
+
+def from_blocked_pages(k_blocked: torch.Tensor, v_blocked: torch.Tensor):
+    """The inverse of to_blocked_pages: keys as rows, values transposed."""
+    hs = k_blocked.shape[-1]
+    ki, vi = (t.to(k_blocked.device).reshape(-1) for t in blocked_page_index(hs))
+    k = k_blocked.reshape(*k_blocked.shape[:2], -1)[..., ki].view(k_blocked.shape)
+    v = v_blocked.reshape(*v_blocked.shape[:2], -1)[..., vi].view(v_blocked.shape)
+    return k.contiguous(), v.contiguous()
 
 
 def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, hs: int, *,
                   inv_freq=None, rope_dims: int = 0, seq_index=None, block_table=None,
-                  k_pages=None, v_pages=None, page_tiles=None, v_transposed=None) -> None:
+                  k_pages=None, v_pages=None, page_tiles=None, v_transposed=None, blocked=None) -> None:
     """Rotate the Q heads of qkv ([T, (H+2Hkv)*hs]) in place, rotate the K heads and store
     them and the V heads at each token's position of its sequence's pages.
     k_pages None: rotate Q only.  rope_dims 0: no rotation.  positions < 0: padding rows.
     page_tiles (optional, [n, 4] int32 = sequence, first row, rows, position of the first; each
-    tile inside one page, all rows covered): transposed V pages are then filled by a kernel
+    tile inside one page, all rows covered): transposed or blocked V pages are then filled by a kernel
     that stores runs of positions instead of single elements.
-    v_transposed: the layout of v_pages (None: kernel_v_layout of qkv's type)."""
+    v_transposed, blocked: the layout of the pages (neither: kernel_v_layout of qkv's type and hs)."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(positions, "positions", torch.int32, 1)
@@ -913,9 +974,9 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
             raise KernelError(f"rope_kv_write: rope_dims {rope_dims} does not fit hs={hs} / inv_freq "
                               f"{tuple(inv_freq.shape)}")
     bt_stride = 0
-    vt = False
+    layout = "rows"
     if k_pages is not None:
-        vt = _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype, v_transposed)
+        layout = _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype, v_transposed, blocked)
         _dev(seq_index, "seq_index", torch.int32, 1)
         _dev(block_table, "block_table", torch.int32, 2)
         if seq_index.numel() != T or not seq_index.is_contiguous() or not block_table.is_contiguous():
@@ -923,7 +984,7 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
         bt_stride = block_table.shape[1]
     if T == 0:
         return
-    tiled_v = (page_tiles is not None and k_pages is not None and vt and qkv.dtype == torch.bfloat16     # a bf16 kernel
+    tiled_v = (page_tiles is not None and k_pages is not None and layout != "rows" and qkv.dtype == torch.bfloat16     # a bf16 kernel
                and hs % 8 == 0 and stride % 8 == 0
                and qkv.data_ptr() % 16 == 0 and hs * (PAGE + 2) * 2 <= 65536 and Hkv <= 65535)
     if tiled_v:
@@ -936,12 +997,12 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
         block_table.data_ptr() if k_pages is not None else None, bt_stride,
         k_pages.data_ptr() if k_pages is not None else None,
         v_pages.data_ptr() if k_pages is not None else None,
-        inv_freq.data_ptr() if rope_dims else None, rope_dims, T, H, Hkv, hs, 2 if tiled_v else int(vt), _stream()),
-        "rope_kv_write")
+        inv_freq.data_ptr() if rope_dims else None, rope_dims, T, H, Hkv, hs,
+        _LAYOUT_CODES[layout] + (4 if tiled_v else 0), _stream()), "rope_kv_write")
     if tiled_v:
         _check(_fn("rope_kv", "bn_v_transposed_write")(
             qkv.data_ptr(), stride, page_tiles.data_ptr(), page_tiles.shape[0], block_table.data_ptr(), bt_stride,
-            v_pages.data_ptr(), H, Hkv, hs, _stream()), "v_transposed_write")
+            v_pages.data_ptr(), H, Hkv, hs, int(layout == "blocked"), _stream()), "v_transposed_write")
 
 
 MAX_HEAD_DIM = _build.header_constant("BN_MAX_HEAD_DIM")    # the attention kernels take every even head size up to this
@@ -954,9 +1015,13 @@ def _pow2_at_least(n: int) -> int:
     return p
 
 
+MFMA_HEAD_DIMS = (_build.header_constant("BN_MFMA_HEAD_DIM_SMALL"), _build.header_constant("BN_MFMA_HEAD_DIM_LARGE"))
+
+
 def mfma_attention(dtype, hs: int) -> bool:
-    """Whether the matrix-core attention kernels take this cache type and head size."""
-    return dtype == torch.bfloat16 and bool(_fn("attn_mfma", "bn_attn_mfma_supports")(int(hs)))
+    """Whether the matrix-core attention kernels take this cache type and head size (bn_attn_mfma_supports, answered
+    from the header so that asking loads no kernel)."""
+    return dtype == torch.bfloat16 and int(hs) in MFMA_HEAD_DIMS
 
 
 def attention_row_shape(H: int, Hkv: int, decode: bool, dtype=None, hs: int = 0):
@@ -1040,16 +1105,16 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
               block_table: torch.Tensor, H: int, Hkv: int, hs: int, scale: float, *, window: int = 0,
               tiles=None, qt: int = 0, seq_lens=None, n_splits: int = 1, chunk: int = 0,
               force_vector: bool = False, fused_rotate=None, fused_write: bool = False, by_length=None,
-              max_len_dev=None, v_transposed=None, row_scale: Optional["DeferredNorm"] = None) -> None:
+              max_len_dev=None, v_transposed=None, row_scale: Optional["DeferredNorm"] = None, blocked=None) -> None:
     """Causal attention of the (rotated) Q heads in qkv over the paged cache.
 
     Prompt form: `tiles` [n, 4] int32 = (sequence, first token row, tokens (<= qt), position of
     the first), qt = the QT of attention_row_shape(H, Hkv, False, dtype, hs).
     Decode form: tiles None, seq_lens [B] int32 (keys in the cache, the new one included; 0 for a
     padding row); row b of qkv is sequence b's token; n_splits/chunk from decode_splits.
-    bf16 with head size 64 or 128 runs on the matrix cores, everything else on the vector ALUs
-    (force_vector: the vector kernel also where the other would run; its qt then is that of
-    attention_row_shape without dtype).
+    bf16 with head size 64 or 128 over blocked pages runs on the matrix cores, everything else on the vector ALUs,
+    which read rows and transposed values (force_vector: say so where the pages are not blocked and the head size
+    would be the other kernel's; its qt then is that of attention_row_shape without dtype).
     Decode on the matrix cores can do the work of rope_kv_write itself (can_fuse_decode):
     fused_rotate = inv_freq [hs/2]: qkv arrives unrotated, Q and the new K are rotated inside;
     fused_write: the new K, V of every row (from qkv) are stored at position seq_lens - 1 first.
@@ -1059,15 +1124,15 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     max_len_dev (decode form, optional): a device int32 holding the longest sequence's key count; with
     n_splits > 1 the kernels then cut the keys into n_splits runs of split_chunk(max_len, n_splits) and
     `chunk` is not used, so that one captured launch serves every length up to the block table's width.
-    v_transposed: the layout of v_pages (None: kernel_v_layout of qkv's type); values that lie like the keys go to
-    the vector kernel whatever their type.
+    v_transposed, blocked: the layout of the pages (neither: kernel_v_layout of qkv's type and hs).
     row_scale (decode form on the matrix cores with fused_rotate): a DeferredNorm whose factor the rows of qkv still
     lack (qkv is the product of its bf16 copy with the stacked weights); the kernel multiplies q and the new key and
     value of every row by it."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(out, "out", qkv.dtype, 2)
-    vt = _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype, v_transposed)
+    layout = _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype, v_transposed, blocked)
+    vt = layout != "rows"
     _dev(block_table, "block_table", torch.int32, 2)
     T = qkv.shape[0]
     if H % Hkv or qkv.shape[1] < H * hs or out.shape != (T, H * hs) or not out.is_contiguous():
@@ -1077,7 +1142,12 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     if not block_table.is_contiguous():
         raise KernelError("attention: block_table must be contiguous")
     decode = tiles is None
-    use_mfma = mfma_attention(qkv.dtype, hs) and vt and not force_vector
+    use_mfma = layout == "blocked"
+    if use_mfma and (force_vector or not mfma_attention(qkv.dtype, hs)):
+        raise KernelError(f"attention: blocked pages are read by the matrix-core kernels alone (head size {hs}, "
+                          f"force_vector={force_vector})")
+    if not use_mfma and mfma_attention(qkv.dtype, hs) and not force_vector:
+        force_vector = True          # pages in another order than the matrix-core kernels': the vector kernel reads them
     RT, GT, QT = attention_row_shape(H, Hkv, decode, qkv.dtype if use_mfma else None, hs)
     if decode:
         _dev(seq_lens, "seq_lens", torch.int32, 1)

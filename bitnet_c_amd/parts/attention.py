@@ -86,9 +86,9 @@ class Attention(Part):
         H, Hkv, hs = self.H, self.Hkv, self.hs
         last = self.o.lazy if lazy_ok else self.o
         fuse_ok, inv_freq = self.position.fusable(hs)
-        vt = kv.v_transposed
+        vt, blocked = kv.v_transposed, bool(kv.blocked)
         decode_fused = (ctx.is_decode and fuse_ok and ops.can_fuse_decode(self.qkv.weight.dtype, H, Hkv, hs)
-                        and (vt is None or vt))                 # the matrix-core kernels read transposed values
+                        and blocked)                            # the matrix-core kernels read blocked pages
         row_scale = None
         if isinstance(h, ops.DeferredNorm) and h.shape[0] > ops.FUSED_ROWS:
             # More rows than the fused product takes.  When the decode kernel rotates by itself it can apply the norm's
@@ -115,7 +115,8 @@ class Attention(Part):
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
                           window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
                           fused_rotate=inv_freq, fused_write=kv.writes, by_length=ctx.by_length,
-                          max_len_dev=ctx.max_len_dev if n_splits > 1 else None, v_transposed=vt, row_scale=row_scale)
+                          max_len_dev=ctx.max_len_dev if n_splits > 1 else None, v_transposed=vt, blocked=blocked,
+                          row_scale=row_scale)
             return last(out)
         self.position.encode_and_store(qkv, ctx, H, Hkv, hs, kv)
         if ctx.is_decode:
@@ -126,10 +127,10 @@ class Attention(Part):
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
                           window=self.window, seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
                           by_length=ctx.by_length, max_len_dev=ctx.max_len_dev if n_splits > 1 else None,
-                          v_transposed=vt)
+                          v_transposed=vt, blocked=blocked)
         else:
-            mfma = vt is None or vt                             # values that lie like the keys: the vector kernel
-            _, _, qt = ops.attention_row_shape(H, Hkv, False, h.dtype if mfma else None, hs)
+            # pages in another order than the matrix-core kernels' own: the vector kernel, with its tiles
+            _, _, qt = ops.attention_row_shape(H, Hkv, False, h.dtype if blocked else None, hs)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale,
-                          window=self.window, tiles=ctx.tiles(qt), qt=qt, v_transposed=vt, force_vector=not mfma)
+                          window=self.window, tiles=ctx.tiles(qt), qt=qt, v_transposed=vt, blocked=blocked)
         return last(out)

@@ -66,23 +66,27 @@ class KVNeed:
     """Keys and values of every position (window 0) or of the last `window` positions, and how a page of the
     cache holds them.  A page keeps PAGE positions of every kv head: the keys as [kv head, PAGE, head_dim]; the
     values, v_head_dim wide (0: as wide as the keys), either the same way (v_layout "rows") or turned,
-    [kv head, v_head_dim, PAGE] ("transposed": 8 consecutive positions of one value column lie together, which is
-    what a kernel that multiplies weights by values on the matrix cores reads).  v_layout None asks for the layout
-    that this library's attention kernels read at the cache's type (ops.kernel_v_layout); a mixer with kernels or
-    torch code of its own names the layout it wants."""
+    [kv head, v_head_dim, PAGE] ("transposed": 8 consecutive positions of one value column lie together).  "blocked"
+    (bf16, values as wide as keys, a head size that is a multiple of 32) keeps the sizes of "transposed" but orders
+    the keys and the values inside a (page, kv head) as this library's matrix-core attention kernels load them
+    (ops.blocked_page_index); nothing else reads such pages.  v_layout None asks for the layout
+    that this library's attention kernels read at the cache's type and head size (ops.kernel_v_layout); a mixer with
+    kernels or torch code of its own names the layout it wants ("rows" or "transposed")."""
     n_kv_heads: int
     head_dim: int
     window: int = 0
     v_head_dim: int = 0
     v_layout: Optional[str] = None
 
-    V_LAYOUTS = ("rows", "transposed")
+    V_LAYOUTS = ("rows", "transposed", "blocked")
 
     def __post_init__(self):
         if self.v_layout is not None and self.v_layout not in self.V_LAYOUTS:
             raise ValueError(f"KVNeed: v_layout {self.v_layout!r} is not one of {self.V_LAYOUTS}")
         if self.n_kv_heads < 1 or self.head_dim < 1 or self.v_head_dim < 0 or self.window < 0:
             raise ValueError(f"KVNeed: sizes must be positive, got {self}")
+        if self.v_layout == "blocked" and (self.head_dim % 32 or self.v_head_dim not in (0, self.head_dim)):
+            raise ValueError(f"KVNeed: blocked pages need values as wide as keys and a head size that is a multiple of 32, got {self}")
 
     @property
     def v_dim(self) -> int:
@@ -165,6 +169,7 @@ class KVView:
     k_pages: Optional[torch.Tensor] = None      # [pages, Hkv, PAGE, head_dim]
     v_pages: Optional[torch.Tensor] = None      # [pages, Hkv, PAGE, v_dim], or [pages, Hkv, v_dim, PAGE] when v_transposed
     v_transposed: Optional[bool] = None         # the layout of v_pages (KVNeed.v_layout as the cache resolved it)
+    blocked: bool = False                       # keys and values in the matrix-core kernels' own order (v_layout "blocked")
     block_table: Optional[torch.Tensor] = None  # [B, W] int32, this step's sequences
     writes: bool = True                         # False: the entry reads another entry's cache
     state: Optional[torch.Tensor] = None        # [max_slots + 1, *shape] fixed-size state, by slot

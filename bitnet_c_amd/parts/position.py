@@ -61,7 +61,7 @@ class PositionEncoding(Part):
                           k_pages=kv.k_pages if kv.writes else None,
                           v_pages=kv.v_pages if kv.writes else None,
                           page_tiles=ctx.page_tiles() if kv.writes and not ctx.is_decode else None,
-                          v_transposed=kv.v_transposed)
+                          v_transposed=kv.v_transposed, blocked=bool(kv.blocked))
 
 
 @POSITION_ENCODINGS.register("rope")

@@ -665,9 +665,13 @@ def test_linear_odd_shapes_and_many_rows(dtype):
 
 
 # ---------------------------------------------------------------------------------------
-def _paged(seqs_k, seqs_v, dtype, n_pages, seed):
-    """Random distinct pages for every sequence; returns k_pages, v_pages, block_table."""
+def _paged(seqs_k, seqs_v, dtype, n_pages, seed, blocked=None):
+    """Random distinct pages for every sequence; returns k_pages, v_pages, block_table.  The pages lie as the kernels
+    read them unasked at this type and head size (ops.kernel_v_layout); blocked=False: bf16 values transposed, whatever
+    the head size (what the vector kernel reads)."""
     Hkv, hs = seqs_k[0].shape[1], seqs_k[0].shape[2]
+    if blocked is None:
+        blocked = _ops().kernel_v_layout(dtype, hs) == "blocked"
     rnd = random.Random(seed)
     free = list(range(n_pages))
     rnd.shuffle(free)
@@ -686,13 +690,26 @@ def _paged(seqs_k, seqs_v, dtype, n_pages, seed):
             v_pages[p, :, :n] = v[64 * i:64 * i + n].transpose(0, 1).to(dtype)
     if vt:
         v_pages = v_pages.transpose(2, 3).contiguous()
+    if blocked:
+        k_pages, v_pages = _ops().to_blocked_pages(k_pages, v_pages)
     return k_pages, v_pages, bt
+
+
+def _as_rows(ops, dtype, hs, kp, vp):
+    """Pages as the kernels wrote them unasked -> keys as rows, values as rows too (float32 on the host)."""
+    layout = ops.kernel_v_layout(dtype, hs)
+    if layout == "blocked":
+        kp, vp = ops.from_blocked_pages(kp, vp)
+    kp, vp = kp.cpu().float(), vp.cpu().float()
+    return kp, (vp.transpose(2, 3) if layout != "rows" else vp)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,Hkv,hs,rope_dims", [(4, 2, 16, 16), (6, 3, 40, 24), (5, 5, 24, 24), (8, 1, 128, 128),
                                                  (2, 2, 256, 64), (8, 2, 64, 32)])
 def test_rope_kv_write(dtype, H, Hkv, hs, rope_dims):
+    """Rotation and the write into the pages, in the layout that the kernels use unasked at each type and head size
+    (rows for float32, transposed values for bf16, blocked pages at the head sizes of the matrix-core kernels)."""
     ops = _ops()
     lens_before, n_new = [0, 70, 130], [5, 1, 66]
     T = sum(n_new)
@@ -718,9 +735,8 @@ def test_rope_kv_write(dtype, H, Hkv, hs, rope_dims):
     v_ref = q_in[:, (H + Hkv) * hs:].float().view(T, Hkv, hs)
     assert close(g[:, :H * hs].float().view(T, H, hs), q_ref, dtype)
     assert torch.equal(g[:, H * hs:].cpu(), q_in[:, H * hs:])            # K, V of the input stay as they are
-    kp, vp = kp.cpu().float(), vp.cpu().float()
-    if vt:
-        vp = vp.transpose(2, 3)
+    kp_raw, vp_raw = kp.cpu(), vp.cpu()
+    kp, vp = _as_rows(ops, dtype, hs, kp, vp)
     written = torch.zeros((n_pages, 64), dtype=torch.bool)
     for t in range(T):
         page, off = int(bt[seq_index[t], positions[t] // 64]), positions[t] % 64
@@ -751,14 +767,66 @@ def test_rope_kv_write(dtype, H, Hkv, hs, rope_dims):
     ops.rope_kv_write(g4, pos.cuda(), H, Hkv, hs, inv_freq=inv_freq.cuda(), rope_dims=rope_dims,
                       seq_index=torch.tensor(seq_index, dtype=torch.int32).cuda(), block_table=bt.cuda(),
                       k_pages=kp4, v_pages=vp4, page_tiles=torch.tensor(tiles, dtype=torch.int32).cuda())
-    vp_first = vp.transpose(2, 3) if vt else vp
-    assert torch.equal(g4.cpu(), g.cpu()) and torch.equal(kp4.cpu().float(), kp)
-    assert torch.equal(vp4.cpu().float(), vp_first.contiguous())
+    assert torch.equal(g4.cpu(), g.cpu()) and torch.equal(kp4.cpu(), kp_raw) and torch.equal(vp4.cpu(), vp_raw)
 
 
 FAR_POSITIONS = [8191, 8192, 65535, 131071]
 LLAMA3_8B_SCALING = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
                          original_max_position_embeddings=8192)
+
+
+def test_blocked_pages_by_their_definition():
+    """The order of a blocked page, written out from its definition: a (page, kv head) is two blocks of 32 positions; a
+    block's keys are, for each chunk c of 32 dimensions, two tiles of 16 key rows (tile row i: the block's position
+    8 (i / 4) + i % 4, and 4 further for the second tile) in which lane i + 16 g holds dimensions 32 c + 8 g .. + 7, 8
+    elements a lane and 64 lanes a tile; its values are, for each tile t of 16 dimensions, the lanes i + 16 g holding
+    positions 8 g .. 8 g + 7 of dimension 16 t + i.  Conversion there and back; and the kernels agree: what the cache
+    write stores into blocked pages reads back as the same keys and values that it stores into plain pages."""
+    ops = _ops()
+    for hs in (64, 128, 32):
+        ki, vi = ops.blocked_page_index(hs)
+        assert tuple(ki.shape) == (64, hs) and tuple(vi.shape) == (hs, 64)
+        assert sorted(ki.reshape(-1).tolist()) == list(range(64 * hs)) == sorted(vi.reshape(-1).tolist())
+        for p, d in ((0, 0), (63, hs - 1), (5, 9), (36, 17), (31, 31), (44, hs - 8), (12, 40 % hs)):
+            b, r = divmod(p, 32)
+            tile, i = (r // 4) % 2, 4 * (r // 8) + r % 4
+            assert 8 * (r // 8) + r % 4 + 4 * tile == r
+            c, g, e = d // 32, (d % 32) // 8, d % 8
+            assert int(ki[p, d]) == b * 32 * hs + ((2 * c + tile) * 64 + (i + 16 * g)) * 8 + e
+            t, i2 = d // 16, d % 16
+            g2, e2 = (p % 32) // 8, p % 8
+            assert int(vi[d, p]) == b * 32 * hs + (t * 64 + (i2 + 16 * g2)) * 8 + e2
+        k = _rand((3, 2, 64, hs), torch.bfloat16, 5)
+        v = _rand((3, 2, hs, 64), torch.bfloat16, 6)
+        kb, vb = ops.to_blocked_pages(k, v)
+        assert kb.shape == k.shape and vb.shape == v.shape and not torch.equal(kb, k)
+        k2, v2 = ops.from_blocked_pages(kb, vb)
+        assert torch.equal(k2, k) and torch.equal(v2, v)
+        assert float(kb[1, 1].reshape(-1)[int(ki[37, 11])]) == float(k[1, 1, 37, 11])
+        assert float(vb[2, 0].reshape(-1)[int(vi[13, 50])]) == float(v[2, 0, 13, 50])
+    assert ops.kernel_v_layout(torch.bfloat16, 128) == "blocked" and ops.kernel_v_layout(torch.bfloat16, 64) == "blocked"
+    assert ops.kernel_v_layout(torch.bfloat16, 96) == "transposed" and ops.kernel_v_layout(torch.bfloat16) == "transposed"
+    assert ops.kernel_v_layout(torch.float32, 128) == "rows"
+    # the writers: blocked pages hold what transposed pages hold (single tokens, and a prompt's tokens by page tiles)
+    from bitnet_c_amd.engine.step import _page_tiles
+    H, Hkv, hs, T = 4, 2, 64, 100
+    qkv = _rand((T, (H + 2 * Hkv) * hs), torch.bfloat16, 7).cuda()
+    pos = torch.arange(30, 30 + T, dtype=torch.int32).cuda()
+    seq = torch.zeros(T, dtype=torch.int32).cuda()
+    bt = torch.tensor([[2, 0, 3]], dtype=torch.int32).cuda()
+    inv = pl.rope_inv_freq(hs, 10000.0).cuda()
+    tiles = torch.tensor(_page_tiles([T], [30]), dtype=torch.int32).cuda()
+    got = {}
+    for blocked in (False, True):
+        for by_tiles in (False, True):
+            kp = torch.zeros((4, Hkv, 64, hs), dtype=torch.bfloat16).cuda()
+            vp = torch.zeros((4, Hkv, hs, 64), dtype=torch.bfloat16).cuda()
+            ops.rope_kv_write(qkv.clone(), pos, H, Hkv, hs, inv_freq=inv, rope_dims=hs, seq_index=seq, block_table=bt,
+                              k_pages=kp, v_pages=vp, page_tiles=tiles if by_tiles else None, v_transposed=True, blocked=blocked)
+            got[blocked, by_tiles] = ops.from_blocked_pages(kp, vp) if blocked else (kp, vp)
+    for key in ((False, True), (True, False), (True, True)):
+        assert torch.equal(got[key][0], got[False, False][0]) and torch.equal(got[key][1], got[False, False][1]), key
+    assert float(got[False, False][0].float().abs().sum()) > 0
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -787,9 +855,10 @@ def test_rope_kv_write_at_far_positions(dtype):
     q_ref, k_ref = pl.apply_rope(q_in, pos, inv), pl.apply_rope(k_in, pos, inv)
     got_q = g[:, :H * hs].float().view(T, H, hs).cpu()
     assert close(got_q, q_ref, dtype)
+    kp, _ = _as_rows(ops, dtype, hs, kp, vp)
     for t, p in enumerate(FAR_POSITIONS):
-        assert close(kp[t + 1, :, p % 64].float().cpu(), k_ref[t], dtype), p
-    assert float(kp[0].float().abs().sum()) == 0.0
+        assert close(kp[t + 1, :, p % 64], k_ref[t], dtype), p
+    assert float(kp[0].abs().sum()) == 0.0
     assert rel_err(pl.apply_rope(q_in, pos - 1, inv), q_ref) > 0.5                               # a position off by one
     assert rel_err(pl.apply_rope(q_in, pos, pl.rope_inv_freq(hs, 500000.0)), q_ref) > 0.5        # the table not rescaled
 
@@ -848,10 +917,11 @@ def test_decode_attention_rotates_and_stores_at_far_positions():
     ops.attention(qkv.cuda(), out, kp, vp, bt, H, Hkv, hs, scale, seq_lens=lens, n_splits=n_splits, chunk=chunk,
                   fused_rotate=inv.cuda(), fused_write=True)
     assert mfma_close(out.float(), torch.stack(refs))
+    kp_rows, vp_rows = _as_rows(ops, dtype, hs, kp, vp)
     for b, p in enumerate(FAR_POSITIONS):
         page = int(bt[b, p // 64])
-        assert close(kp[page, 0, p % 64].float().cpu(), new_keys[b], dtype), p
-        assert torch.equal(vp[page, 0, :, p % 64].cpu(), qkv[b, (H + 1) * hs:]), p
+        assert close(kp_rows[page, 0, p % 64], new_keys[b], dtype), p
+        assert torch.equal(vp_rows[page, 0, p % 64], qkv[b, (H + 1) * hs:].float()), p
     # the same query turned for the position before would have weighted the two keys otherwise
     q_off = pl.apply_rope(qkv[0, :hs].float().view(1, 1, hs), torch.tensor([FAR_POSITIONS[0] - 1]), inv)[0, 0]
     k_far = seqs_k[0][FAR_POSITIONS[0] - 1000, 0].float()
@@ -880,9 +950,9 @@ def mfma_close(got, ref) -> bool:
     return bool(((got - ref).abs() <= ref.abs() * 2.0 ** -8 + 5 * 2.0 ** -9).all())
 
 
-def _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, seed):
+def _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, seed, blocked=None):
     """Random sequences; returns the kernel's output and the plain implementation's, rows in
-    batch order."""
+    batch order.  blocked as _paged's."""
     ops = _ops()
     seqs_q, seqs_k, seqs_v = [], [], []
     for s, (p0, n) in enumerate(zip(lens_before, n_new)):
@@ -891,7 +961,7 @@ def _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, seed):
         seqs_k.append(_rand((L, Hkv, hs), dtype, seed + 3 * s + 1))
         seqs_v.append(_rand((L, Hkv, hs), dtype, seed + 3 * s + 2))
     n_pages = sum((p0 + n + 63) // 64 for p0, n in zip(lens_before, n_new)) + 3
-    kp, vp, bt = _paged(seqs_k, seqs_v, dtype, n_pages, seed)
+    kp, vp, bt = _paged(seqs_k, seqs_v, dtype, n_pages, seed, blocked)
     scale = 1.0 / math.sqrt(hs)
     qrows, ref = [], []
     for s, (p0, n) in enumerate(zip(lens_before, n_new)):
@@ -912,9 +982,12 @@ def _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, seed):
 @pytest.mark.parametrize("force_vector", [False, True])
 def test_attention_prompt_form(dtype, H, Hkv, hs, window, force_vector):
     lens_before, n_new = [0, 0, 64, 130, 5, 0], [1, 37, 64, 3, 70, 300]
-    ops, qkv, kp, vp, bt, ref, scale = _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, 100)
+    ops = _ops()
     if force_vector and not ops.mfma_attention(dtype, hs):
         pytest.skip("the vector kernel is what runs anyway")
+    # force_vector: pages with transposed values instead of blocked ones, which the vector kernel reads
+    ops, qkv, kp, vp, bt, ref, scale = _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, 100,
+                                                  blocked=False if force_vector else None)
     _, _, qt = ops.attention_row_shape(H, Hkv, False, None if force_vector else dtype, hs)
     tiles, r = [], 0
     for s, (p0, n) in enumerate(zip(lens_before, n_new)):
@@ -923,7 +996,8 @@ def test_attention_prompt_form(dtype, H, Hkv, hs, window, force_vector):
         r += n
     out = torch.full((qkv.shape[0], H * hs), float("nan"), dtype=dtype).cuda()
     ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, scale, window=window,
-                  tiles=torch.tensor(tiles, dtype=torch.int32).cuda(), qt=qt, force_vector=force_vector)
+                  tiles=torch.tensor(tiles, dtype=torch.int32).cuda(), qt=qt, force_vector=force_vector,
+                  blocked=False if force_vector else None)
     assert mfma_close(out.float(), ref) if ops.mfma_attention(dtype, hs) and not force_vector else close(out.float(), ref, dtype)
 
 
@@ -994,9 +1068,12 @@ def test_attention_prompt_form_paired_tiles_of_several_sequences(window):
 @pytest.mark.parametrize("force_vector", [False, True])
 def test_attention_decode_form(dtype, H, Hkv, hs, window, force_splits, force_vector):
     lens_before, n_new = [0, 63, 64, 700, 129, 300], [1] * 6
-    ops, qkv, kp, vp, bt, ref, scale = _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, 200)
+    ops = _ops()
     if force_vector and not ops.mfma_attention(dtype, hs):
         pytest.skip("the vector kernel is what runs anyway")
+    # force_vector: pages with transposed values instead of blocked ones, which the vector kernel reads
+    ops, qkv, kp, vp, bt, ref, scale = _attn_case(dtype, H, Hkv, hs, lens_before, n_new, window, 200,
+                                                  blocked=False if force_vector else None)
     B = len(n_new)
     # two padding rows at the end: length 0, their output is zero and nothing else changes
     qkv = torch.cat([qkv, torch.zeros((2, qkv.shape[1]), dtype=dtype).cuda()])
@@ -1016,7 +1093,7 @@ def test_attention_decode_form(dtype, H, Hkv, hs, window, force_splits, force_ve
         n_splits, chunk = 1, 0
     out = torch.full((B + 2, H * hs), float("nan"), dtype=dtype).cuda()
     ops.attention(qkv, out, kp, vp, bt, H, Hkv, hs, scale, window=window, seq_lens=lens,
-                  n_splits=n_splits, chunk=chunk, force_vector=force_vector)
+                  n_splits=n_splits, chunk=chunk, force_vector=force_vector, blocked=False if force_vector else None)
     if ops.mfma_attention(dtype, hs) and not force_vector:
         assert mfma_close(out[:B].float(), ref)
     else:

@@ -33,8 +33,8 @@ def _library() -> ctypes.CDLL:
 
 
 def _case(seed, lens, H, Hkv, hs):
-    """A paged bf16 cache with random keys and values for sequences of the given lengths (the new token
-    included), pages in random order, unused pages NaN; one query row per sequence."""
+    """A paged bf16 cache (blocked pages) with random keys and values for sequences of the given lengths (the new
+    token included), pages in random order, unused pages NaN; one query row per sequence."""
     g = torch.Generator().manual_seed(seed)
     rnd = random.Random(seed)
     B = len(lens)
@@ -58,6 +58,8 @@ def _case(seed, lens, H, Hkv, hs):
             kp[p, :, :n] = k[PAGE * i:PAGE * i + n].transpose(0, 1)
             vp[p, :, :, :n] = v[PAGE * i:PAGE * i + n].permute(1, 2, 0)
     q = torch.randn((B, H * hs), generator=g).to(torch.bfloat16)
+    from bitnet_c_amd import ops
+    kp, vp = ops.to_blocked_pages(kp, vp)          # the order in which the matrix-core kernels read a page
     return q.cuda(), kp.cuda(), vp.cuda(), bt.cuda(), torch.tensor(lens, dtype=torch.int32).cuda(), ks, vs
 
 
