@@ -18,6 +18,8 @@ extern "C" {
 // under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The reference has
 // no counterpart; its back-ends allocate their work buffers themselves.
 //
+// k_pages and vt_pages are blocked pages (common.h: [pages, Hkv, 64 * hs] each, keys and values of a page in the order in
+// which the kernel loads them), as everywhere in attn_mfma.hip.
 // Same arguments and the same result, bit for bit, as bn_attn_mfma with tiles == null, except that
 // the split partials (n_seqs * H * n_splits * (hs + 2) floats) live in a file-scope device array
 // of BN_ATTN_STATIC_SCRATCH_FLOATS floats instead of buffers the caller brings.  It calls no

@@ -12,9 +12,11 @@
 // The S^T tile leaves lane (col, g) with 4 keys per 16-key tile; the key rows fed to the two
 // tiles of a 32-key block are permuted (row i of tile sb is key 8*(i/4) + 4*sb + i%4) so
 // that each lane group g ends up with the 8 consecutive keys 8g..8g+7, which is exactly what
-// the B operand of the second product wants and what one 16-byte load of a V^T row holds.
-// Hence V is kept transposed in bf16 caches: K pages [page, kv_head, 64, hs], V pages
-// [page, kv_head, hs, 64].
+// the B operand of the second product wants and what 16 bytes of 8 consecutive positions of one
+// value dimension hold.  The pages are laid out for exactly these operands ("blocked" pages,
+// common.h): a (page, kv head) holds its 64 positions in two blocks of 32, and a block its keys and
+// its values tile by tile in the lanes' order, so that the decode form loads an operand tile as 1 KB of
+// consecutive bytes and the prompt form fetches a stage as one run.
 //
 // Prompt form: a workgroup of 4 waves owns 64*NT columns = consecutive query tokens x GT heads;
 // the keys and values it walks are staged through shared memory once for all four waves.
