@@ -530,14 +530,14 @@ SWIGLU_STAGED_STREAMED_ROWS = (13, 64)
 STAGED_MIN_TILES_PER_CU = 6
 
 
+_CUS = None
+
+
 def _compute_units() -> int:
     global _CUS
     if _CUS is None:
         _CUS = int(torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count)
     return _CUS
-
-
-_CUS = None
 
 
 def _staged_swiglu_rows(M: int, allow_library: bool, w_rows: int, streamed) -> bool:
