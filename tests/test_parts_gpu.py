@@ -249,6 +249,63 @@ def test_the_order_of_layers_is_data(tmp_path):
     assert rel_err(got, want) < TOL[torch.float32]
 
 
+def test_an_entry_reads_another_entry_s_blocked_pages(tmp_path):
+    """bfloat16 at the head size and grouping of the benchmark shape (128, four query heads per kv head): the cache keeps
+    blocked pages, which only the matrix-core kernels read.  A schedule whose third entry runs layer 1's weights again
+    over the keys and values of entry 0 (it writes nothing): a prompt of 150 tokens whole, and 100 of them followed by 50
+    one by one (the decode kernel then reads the pages without storing into them), against the plain computation."""
+    from bitnet_c_amd import Engine, StepEntry
+    from bitnet_c_amd.config import LlamaConfig, load_config
+    from bitnet_c_amd.engine import DecoderModel, ScheduleEntry
+    from bitnet_c_amd.weights import load_tensors, write_model_folder
+    from conftest import TINY_E
+    from dataclasses import replace
+    folder = str(tmp_path / "e")
+    write_model_folder(folder, LlamaConfig.from_dict(TINY_E), 21, torch.bfloat16)
+    arch, cfg = load_config(folder)
+    plan = arch.build_plan(cfg)
+    plan = replace(plan, schedule=[ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(1, kv_from=0)])
+    model = DecoderModel(plan, torch.bfloat16, DEV)
+    model.load(load_tensors(folder, plan.expected_tensors()))
+    eng = Engine(model, max_tokens=512)
+    assert eng.cache.groups[0].blocked and eng.cache.groups[0].k.shape[0] == 2
+    c, W = pl.read_config(folder), pl.read_weights(folder)
+    H, Hkv, hd, D = c["heads"], c["kv_heads"], c["head_dim"], c["dim"]
+    toks = [random.Random(6).randrange(c["vocab"]) for _ in range(150)]
+    s = eng.new_sequence()
+    whole = eng.step([StepEntry(s, toks, list(range(150)))])
+    eng.release(s)
+    s = eng.new_sequence()
+    first = eng.step([StepEntry(s, toks[:100], list(range(100)))])
+    rest = [eng.step([StepEntry(s, [t], [0])]) for t in toks[100:]]
+    eng.release(s)
+    eng.cache.check()
+    r = lambda x: x.to(torch.bfloat16).float()
+    x = W["model.embed_tokens.weight"].float()[toks]
+    pos = torch.arange(len(toks))
+    inv = pl.rope_inv_freq(hd, c["theta"])
+    keep = None
+    for e, l in enumerate([0, 1, 1]):
+        p = f"model.layers.{l}."
+        xb = r(pl.rmsnorm(x, W[p + "input_layernorm.weight"].float(), c["eps"]))
+        q = r(pl.apply_rope(r(pl.linear(xb, W[p + "self_attn.q_proj.weight"].float())).view(-1, H, hd), pos, inv))
+        if e < 2:
+            k = r(pl.apply_rope(r(pl.linear(xb, W[p + "self_attn.k_proj.weight"].float())).view(-1, Hkv, hd), pos, inv))
+            v = r(pl.linear(xb, W[p + "self_attn.v_proj.weight"].float())).view(-1, Hkv, hd)
+            if e == 0:
+                keep = (k, v)
+        else:
+            k, v = keep
+        o = r(pl.attention(q, k, v, hd ** -0.5).reshape(len(toks), H * hd))
+        x = x + pl.linear(o, W[p + "self_attn.o_proj.weight"].float())
+        xb = r(pl.rmsnorm(x, W[p + "post_attention_layernorm.weight"].float(), c["eps"]))
+        x = x + pl.feed_forward(xb, W[p + "mlp.gate_proj.weight"].float(), W[p + "mlp.up_proj.weight"].float(),
+                                W[p + "mlp.down_proj.weight"].float())
+    want = pl.linear(r(pl.rmsnorm(x, W["model.norm.weight"].float(), c["eps"])), W["model.embed_tokens.weight"].float())
+    assert rel_err(whole, want) < TOL[torch.bfloat16]
+    assert rel_err(torch.cat([first] + rest), want) < TOL[torch.bfloat16]
+
+
 # ---------------------------------------------------------------------------------------
 # a toy architecture, defined here: layers alternate between attention and a mixer that keeps
 # a running decayed sum of its inputs per sequence; nothing of it lives in the library
@@ -1122,12 +1179,13 @@ def test_a_toy_mixer_whose_values_are_wider_than_its_keys(tmp_path):
         reqs = reqs[::-1]
 
 
-@pytest.mark.parametrize("dtype,layout", [(torch.bfloat16, "rows"), (torch.float32, "transposed")])
+@pytest.mark.parametrize("dtype,layout", [(torch.bfloat16, "rows"), (torch.float32, "transposed"), (torch.bfloat16, "transposed")])
 @pytest.mark.parametrize("hs", [64, 24])
 def test_the_attention_part_over_the_layout_that_is_not_its_kernels_own(dtype, layout, hs):
-    """An attention whose need names the other layout of the values (bfloat16 values lying like the keys, float32
-    values turned): the cache write and the vector kernel take either, the matrix-core kernels are not used, and the
-    result is the plain attention's."""
+    """An attention whose need names another layout than its kernels would pick (bfloat16 values lying like the keys,
+    float32 values turned, bfloat16 values turned at a head size where the kernels would keep blocked pages): the cache
+    write and the vector kernel take either, the matrix-core kernels are not used, and the result is the plain
+    attention's."""
     from bitnet_c_amd.cache import PAGE, PagedCache
     from bitnet_c_amd.parts import MIXERS, CacheNeed, KVNeed, PartSpec
     from bitnet_c_amd.parts.attention import Attention
