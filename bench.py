@@ -224,13 +224,15 @@ def main() -> int:
     model.load(tensors)
     del tensors
     torch.cuda.empty_cache()
-    print(f"[bench] model built in {time.time() - t0:.1f} s, weights {model.weight_bytes() / 1e9:.2f} GB"
-          + (f", and {model.streamed_bytes() / 1e9:.2f} GB of streamed copies" if model.has_streamed else ""),
+    print(f"[bench] model built in {time.time() - t0:.1f} s, weights {model.weight_bytes() / 1e9:.2f} GB",
           file=sys.stderr, flush=True)
 
     max_batch = max(args.batch, 1 if args.no_points else 64)
     per_seq = ((len_hi + args.steps + args.warmup + 64 + 63) // 64) * 64
     engine = bn.Engine(model, max_tokens=max(max_batch * per_seq, 4096, PREFILL + 64), max_seq_len=CONTEXT)
+    kept = sum(l.streamed.nbytes() for l in model.linears() if l.streamed is not None)
+    print(f"[bench] streamed copies of the weight matrices: {kept / 1e9:.2f} of {model.streamed_bytes() / 1e9:.2f} GB",
+          file=sys.stderr, flush=True)
     L, H, Hkv, hs = cfg.num_hidden_layers, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
     kv_bytes_per_token = 2 * L * Hkv * hs * 2
     weight_bytes = model.weight_bytes()      # every weight a decode step reads once (no embedding table unless it is tied)

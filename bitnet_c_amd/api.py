@@ -55,7 +55,7 @@ def load(folder: str, dtype="bfloat16", max_tokens: int = 8192, device: str = "c
     of the longest length there can be, or what fits into the device's free memory if that is less.
     max_seq_len: the longest sequence (the reference's --maxseq), 0 = the model's limit.
     streamed_weights: keep every weight matrix a second time in the order the decode kernels read it (faster decode
-    steps for the matrices' memory once more); None: where half of the device's memory stays free."""
+    steps for the matrices' memory once more); None: as many as fit into what the cache leaves free."""
     if dtype not in _DTYPES:
         raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}")
     return LLM(Engine.from_folder(folder, _DTYPES[dtype], max_tokens, device, max_seq_len, 0, use_graphs, n_seqs,

@@ -11,35 +11,39 @@ import torch
 
 from .. import ops
 from ..parts import BLOCKS, NORMS, CacheNeed, ResidualStream
-from ..parts.linear import upload
+from ..parts.linear import Linear, upload
 from .plan import ModelPlan
 
 
-# Of the device's memory, the share that has to stay free after the streamed copies for a model to keep them unasked.
-STREAMED_FREE_SHARE = 0.5
+# Of the device's memory, the share that stays free when a model takes streamed copies unasked: activations of long
+# prompts, captured graphs and the libraries' work buffers live there.
+STREAMED_RESERVE_SHARE = 0.1
 
 
-def streamed_by_default(copy_bytes: int, free_bytes: int, total_bytes: int) -> bool:
-    """Whether a model keeps streamed copies of its weight matrices when nobody says: they cost the matrices' size once
-    more and make every decode step and short prompt step 5 to 12 % faster, so they are kept where memory is plentiful
-    (half of the device still free afterwards: on 288 GB every model up to some 70 GB of weights) and left out where the
-    cache needs the room."""
-    return copy_bytes > 0 and free_bytes - copy_bytes >= STREAMED_FREE_SHARE * total_bytes
+def streamed_budget(free_bytes: int, total_bytes: int) -> int:
+    """Bytes that a model's streamed copies may take when nobody says: what is free once the weights and the cache are in
+    place, but for a tenth of the device's memory.  The copies cost a matrix's size once more and make every decode step
+    and short prompt step 5 to 12 % faster, so what the cache does not ask for is spent on them, the largest matrices
+    first (a model of 16 GB on 288 GB keeps them all; one of 140 GB keeps those of its feed-forwards' first products as
+    far as the room goes)."""
+    return max(0, int(free_bytes - STREAMED_RESERVE_SHARE * total_bytes))
 
 
 class DecoderModel:
     def __init__(self, plan: ModelPlan, dtype=torch.bfloat16, device="cuda:0", streamed_weights=None):
         """streamed_weights: keep a second copy of every weight matrix in the order in which the kernels of up to 128
-        rows read it (ops.StreamedWeight); None: streamed_by_default decides after the weights are loaded
-        (BITNET_STREAMED_WEIGHTS=0 or 1 decides instead, for measurements)."""
+        rows read it (ops.StreamedWeight): True at load, False never; None: the engine that takes the model decides once
+        its cache is allocated (settle_streamed: as many copies as streamed_budget allows, the largest matrices first).
+        BITNET_STREAMED_WEIGHTS=0 or 1 decides instead, for measurements."""
         if dtype not in (torch.bfloat16, torch.float32):
             raise ValueError(f"compute dtype must be bfloat16 or float32, got {dtype}")
         plan.validate()
         self.plan, self.dtype, self.device = plan, dtype, torch.device(device)
         env = os.environ.get("BITNET_STREAMED_WEIGHTS", "")
         self.streamed_weights = streamed_weights if streamed_weights is not None or env == "" else env != "0"
-        self.lm_head_streamed = None     # ops.StreamedWeight of the output matrix
-        self.has_streamed = False
+        self.head = Linear()             # the output matrix as the parts hold theirs (weight = lm_head; its streamed copy)
+        self.has_streamed = False        # whether any matrix has a streamed copy
+        self.streamed_settled = False    # whether the copies have been decided (at load, or by settle_streamed)
         self.blocks = [BLOCKS.build(lp.block) for lp in plan.layers]
         self.final_norm = NORMS.build(plan.final_norm) if plan.final_norm is not None else None
         self.lm_head_bias = None         # [V] float32, when the plan names one
@@ -70,34 +74,46 @@ class DecoderModel:
         else:
             self.lm_head = upload(tensors[p.lm_head_name], self.device, self.dtype)
             done([p.lm_head_name])
-        keep = self.streamed_weights
-        if keep is None:
-            free, total = torch.cuda.mem_get_info(self.device) if self.device.type == "cuda" else (0, 0)
-            keep = streamed_by_default(self.streamed_bytes(), free, total)
-        self.keep_streamed(bool(keep))
+        self.head.weight = self.lm_head
+        if self.streamed_weights is not None:
+            self.keep_streamed(bool(self.streamed_weights))
+        else:
+            self.keep_streamed(False)
+            self.streamed_settled = False          # an engine decides, with its cache in place
 
     # ---- streamed copies ---------------------------------------------------------------
     def linears(self) -> list:
-        return [l for blk in self.blocks for l in getattr(blk, "linears", list)()]
+        """Every weight matrix that a product of few rows reads once: the parts' own and the output matrix."""
+        return [l for blk in self.blocks for l in getattr(blk, "linears", list)()] + [self.head]
 
     def streamed_bytes(self) -> int:
         """Bytes that the streamed copies of all weight matrices take (taken or not)."""
         if self.dtype != torch.bfloat16 or self.device.type != "cuda":
             return 0
-        head = 0
-        if self.lm_head is not None and self.lm_head.shape[1] % 8 == 0:
-            R, C = ops.stream_tile_rows(self.lm_head.shape[0]), ops.STREAM_TILE_COLS
-            head = -(-self.lm_head.shape[0] // R) * R * -(-self.lm_head.shape[1] // C) * C * 2
-        return head + sum(l.stream_bytes() for l in self.linears())
+        return sum(l.stream_bytes() for l in self.linears())
 
-    def keep_streamed(self, keep: bool = True) -> None:
-        """Makes (or drops) the streamed copy of every weight matrix of the parts and of the output matrix."""
-        keep = keep and self.streamed_bytes() > 0
-        for l in self.linears():
-            l.keep_streamed(keep)
-        head = keep and self.lm_head is not None and self.lm_head.shape[1] % 8 == 0
-        self.lm_head_streamed = ops.stream_copy(self.lm_head) if head else None
-        self.has_streamed = bool(keep)
+    def keep_streamed(self, keep: bool = True, budget: int = None) -> int:
+        """Makes (or drops) the streamed copies of the parts' weight matrices and of the output matrix; with a budget (in
+        bytes) only as many as fit into it, the largest matrices first.  Returns the bytes that the copies take."""
+        matrices = self.linears()
+        applies = self.dtype == torch.bfloat16 and self.device.type == "cuda"
+        sizes = [l.stream_bytes() if applies else 0 for l in matrices]
+        used = 0
+        for i in sorted(range(len(matrices)), key=lambda i: -sizes[i]):      # a stable order: equal sizes in model order
+            fits = bool(keep and sizes[i] > 0 and (budget is None or used + sizes[i] <= budget))
+            matrices[i].keep_streamed(fits)
+            used += sizes[i] if fits else 0
+        self.has_streamed = used > 0
+        self.streamed_settled = True
+        return used
+
+    def settle_streamed(self) -> None:
+        """Called by an engine once its cache is allocated: a model that was not told whether to keep streamed copies
+        takes as many as streamed_budget allows now."""
+        if self.streamed_settled:
+            return
+        free, total = torch.cuda.mem_get_info(self.device) if self.device.type == "cuda" else (0, 0)
+        self.keep_streamed(True, streamed_budget(free, total))
 
     def weight_bytes(self) -> int:
         """Bytes of every weight a decode step reads once (the embedding table only when it is
@@ -144,7 +160,7 @@ class DecoderModel:
             h = stream.normed(self.final_norm, self.dtype, rows=ctx.want_rows)
         else:
             h = ops.gather_rows(stream.flush(), ctx.want_rows, self.dtype)
-        logits = ops.linear(h, self.lm_head, torch.float32, streamed=self.lm_head_streamed)
+        logits = ops.linear(h, self.lm_head, torch.float32, streamed=self.head.streamed)
         if self.lm_head_bias is not None and logits.shape[0]:
             ops.bias_add(logits, self.lm_head_bias)
         if self.plan.logit_softcap > 0:                            # src/transformer/logits.c:325-333

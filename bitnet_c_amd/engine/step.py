@@ -354,6 +354,7 @@ class Engine:
         needs, kv_from = model.cache_needs()
         self.cache = PagedCache(needs, kv_from, max_tokens, dtype=model.dtype, device=self.device,
                                 max_slots=max_slots or None)
+        model.settle_streamed()             # the cache has its memory: what is left may go to streamed copies of the weights
         limit = self.cache.n_pages * PAGE
         if model.plan.max_positions:
             limit = min(limit, model.plan.max_positions)

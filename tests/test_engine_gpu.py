@@ -128,7 +128,7 @@ def test_streamed_copies_of_the_weights_change_no_result(model_folders, name, sm
     for streamed in (False, True):
         eng = make_engine(folder, torch.bfloat16, max_tokens=4096, streamed_weights=streamed)
         m = eng.model
-        assert m.has_streamed == streamed and (m.lm_head_streamed is not None) == streamed
+        assert m.has_streamed == streamed and (m.head.streamed is not None) == streamed
         assert all((l.streamed is not None) == (streamed and l.stream_bytes() > 0) for l in m.linears()) and m.linears()
         assert m.streamed_bytes() >= m.weight_bytes() * 0.5           # every matrix once more (padded), norms aside
         outs[streamed, "bytes"] = m.weight_bytes()

@@ -166,13 +166,12 @@ def test_prompt_tiles_are_paired_long_with_short_inside_a_sequence():
         assert len({t[0] for t in rest}) == len(rest)       # one middle tile per sequence with an odd count
 
 
-def test_streamed_copies_are_kept_where_memory_is_plentiful():
-    """The rule by which a model keeps a second copy of its weight matrices when nobody says: half of the device's
-    memory has to stay free afterwards."""
-    from bitnet_c_amd.engine.model import streamed_by_default
+def test_streamed_copies_take_what_the_cache_leaves():
+    """The rule by which a model takes streamed copies of its weight matrices when nobody says: what is free once the
+    weights and the cache are in place, but for a tenth of the device's memory."""
+    from bitnet_c_amd.engine.model import streamed_budget
     GB = 1 << 30
-    assert streamed_by_default(16 * GB, 270 * GB, 288 * GB)            # an 8B model on a fresh device
-    assert streamed_by_default(68 * GB, 218 * GB, 288 * GB)            # 34B: 150 GB stay free
-    assert not streamed_by_default(141 * GB, 145 * GB, 288 * GB)       # 70B: no room for a second copy
-    assert not streamed_by_default(16 * GB, 150 * GB, 288 * GB)        # a device that others already fill
-    assert not streamed_by_default(0, 270 * GB, 288 * GB)              # nothing to copy (a float32 model)
+    assert streamed_budget(250 * GB, 288 * GB) >= 16 * GB              # an 8B model with a cache of 20 GB: all of it
+    assert 60 * GB <= streamed_budget(100 * GB, 288 * GB) <= 75 * GB   # 70B with a cache of 46 GB: most feed-forwards
+    assert streamed_budget(20 * GB, 288 * GB) == 0                     # a device that the cache fills
+    assert streamed_budget(0, 0) == 0
