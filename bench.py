@@ -203,6 +203,7 @@ def main() -> int:
 
     import bitnet_c_amd as bn
     from bitnet_c_amd import ops
+    from bitnet_c_amd.sampling import SamplingParams, SequenceSampler, start_sampling
     from bitnet_c_amd.config import architecture_for
     from bitnet_c_amd.engine import DecoderModel
     from bitnet_c_amd.weights import random_tensors
@@ -286,12 +287,19 @@ def main() -> int:
                 last[j] = t
             i = k
 
-        def one():
-            nonlocal last
-            lg = engine.step([bn.StepEntry(slots[j], [last[j]], [0]) for j in range(batch)])
-            last = ops.argmax(lg).cpu().tolist()
-
+        # as the generation loop runs greedy decoding: the tokens stay on the device, a step is queued on them, then the
+        # host reads them (every token reaches the host, one step behind the device)
+        greedy = [SequenceSampler(SamplingParams())] * batch
+        entries = [bn.StepEntry(slots[j], [0], [0]) for j in range(batch)]
         engine.prepare_decode(batch)          # as generation does at a batch's start: no capture inside the clock
+        lg = engine.step([bn.StepEntry(slots[j], [last[j]], [0]) for j in range(batch)])
+
+        def one():
+            nonlocal last, lg
+            pending = start_sampling(lg, greedy)
+            lg = engine.step(entries, device_tokens=pending.device_tokens)
+            last = pending.tokens()
+
         for _ in range(warmup):
             one()
         sync()
@@ -300,7 +308,7 @@ def main() -> int:
             one()
         sync()
         dt = time.perf_counter() - t
-        ctx_mid = sum(lens) + batch * (warmup + steps / 2.0)          # cached tokens read by a mid step
+        ctx_mid = sum(lens) + batch * (1 + warmup + steps / 2.0)          # cached tokens read by a mid step
         for s in slots:
             engine.release(s)
         return dt / steps, ctx_mid

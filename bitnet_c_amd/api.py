@@ -25,8 +25,8 @@ class LLM:
     def new_sequence(self) -> int:
         return self.engine.new_sequence()
 
-    def step(self, entries) -> torch.Tensor:
-        return self.engine.step(entries)
+    def step(self, entries, device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return self.engine.step(entries, device_tokens)
 
     def release(self, slot: int) -> None:
         self.engine.release(slot)

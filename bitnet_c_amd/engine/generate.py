@@ -12,6 +12,16 @@ is emitted (the callback may cancel) -> when the budget is reached no further st
 -> otherwise the token is fed for the next logits.  Its loop detector, stop strings and
 chat templates are serving helpers and are not taken over.
 
+Decode steps are queued one ahead of the host where that is possible: when the sampler can
+leave its tokens on the device (`sample_fn.start(logits, samplers)` returns an object with
+device_tokens, rows(indices) and tokens(), or None when it needs the host first) and the engine
+takes them from there (`takes_device_tokens`, step(entries, device_tokens=...)), the next step
+is queued for every sequence that neither its budget nor the sequence limit ends, before the
+host has seen the tokens.  It then reads them and decides as above; a sequence that its token
+has ended (a stop token, a cancelling callback) has run one step for nothing, and its row of
+the new logits is dropped.  The device so never waits for the host between two steps; tokens,
+their order and the finish reasons are the same either way.
+
 Nothing here touches the GPU directly: `engine` needs new_sequence(), release(slot),
 step(entries) -> logits, max_seq_len and a cache that can tell how many tokens fit, and
 `sample_fn(logits, samplers)` picks the tokens, so the decisions run in tests with stand-ins.
@@ -23,7 +33,7 @@ from typing import Callable, List, Optional, Sequence
 
 from ..cache import PAGE
 from ..sampling.sampler import SamplingParams, SequenceSampler
-from .step import StepEntry
+from .step import StepEntry, StepError
 
 
 @dataclass
@@ -90,6 +100,9 @@ def generate(engine, requests: Sequence[Request], sample_fn: Callable, batch_siz
     for i, msg in errors.items():
         results[i].finish = msg
     prepare = getattr(engine, "prepare_decode", None)
+    # a sampler that can leave its tokens on the device and an engine that takes them from there: decode steps are
+    # queued one ahead of the tokens that the host has seen
+    start = getattr(sample_fn, "start", None) if getattr(engine, "takes_device_tokens", False) else None
     for batch in batches:
         live: List[_Live] = []
         if prepare is not None and any(requests[i].max_new_tokens > 1 for i in batch):
@@ -114,9 +127,26 @@ def generate(engine, requests: Sequence[Request], sample_fn: Callable, batch_siz
                     live = [s for s in live if s.req.max_new_tokens > 0]
                     if not live:
                         break
-                tokens = sample_fn(logits, [s.sampler for s in live])
-                nxt: List[_Live] = []
-                for s, tok in zip(live, tokens):
+                samplers = [s.sampler for s in live]
+                pending = start(logits, samplers) if start is not None else None
+                ahead = None
+                if pending is not None:
+                    # Whoever is neither at its budget nor at the limit goes on unless its token ends it.  The host
+                    # learns that a step late: the next step is queued for all of them on the tokens that lie on the
+                    # device, and a sequence that its token has ended leaves it unused.
+                    cont = [k for k, s in enumerate(live)
+                            if len(results[s.index].tokens) + 1 < s.req.max_new_tokens and s.length + 1 <= engine.max_seq_len]
+                    if cont:
+                        toks = pending.device_tokens if len(cont) == len(live) else pending.rows(cont)
+                        try:
+                            ahead = (cont, engine.step([StepEntry(live[k].slot, [0], [0]) for k in cont], device_tokens=toks))
+                        except StepError:
+                            ahead = None             # nothing has changed: decided below, with the tokens at hand
+                    tokens = pending.tokens()
+                else:
+                    tokens = sample_fn(logits, samplers)
+                nxt: List[int] = []
+                for k, (s, tok) in enumerate(zip(live, tokens)):
                     res = results[s.index]
                     if tok in s.req.stop_ids:
                         res.finish = "stop"                      # not emitted
@@ -132,11 +162,17 @@ def generate(engine, requests: Sequence[Request], sample_fn: Callable, batch_siz
                     if res.finish:
                         engine.release(s.slot)
                     else:
-                        nxt.append(s)
-                live = nxt
+                        nxt.append(k)
+                if ahead is not None:
+                    cont, logits = ahead
+                    if len(nxt) != len(cont):                    # rows of sequences that their token has ended
+                        row_of = {k: r for r, k in enumerate(cont)}
+                        logits = logits[[row_of[k] for k in nxt]]
+                live = [live[k] for k in nxt]
                 if not live:
                     break
-                logits = engine.step([StepEntry(s.slot, [results[s.index].tokens[-1]], [0]) for s in live])
+                if ahead is None:
+                    logits = engine.step([StepEntry(s.slot, [results[s.index].tokens[-1]], [0]) for s in live])
                 for s in live:
                     s.length += 1
         except Exception:

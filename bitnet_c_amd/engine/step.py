@@ -460,13 +460,28 @@ class Engine:
                 if not (0 <= int(w) < n):
                     raise StepError(f"slot {e.slot}: wanted place {w} is outside its {n} tokens")
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    takes_device_tokens = True        # step(..., device_tokens=...) is there
+
+    def step(self, entries: Sequence[StepEntry], device_tokens: torch.Tensor = None) -> torch.Tensor:
         """Runs the entries' tokens as one batch; returns float32 logits [wanted, vocab] in the
-        order of the entries and of each entry's `want`.  On an error nothing has changed."""
+        order of the entries and of each entry's `want`.  On an error nothing has changed.
+
+        device_tokens: for a step of one token a sequence, an int32 tensor [len(entries)] on the engine's device that
+        holds the tokens (what a sampling kernel has just written); the entries' own tokens are placeholders then.
+        The step is queued behind whatever writes that tensor, so the host can queue a decode step before it has
+        seen the tokens that the step consumes."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         self._validate(entries)
         slots = [e.slot for e in entries]
         n_new = [len(e.tokens) for e in entries]
+        if device_tokens is not None:
+            if any(n != 1 for n in n_new):
+                raise StepError("tokens on the device are taken by steps of one token a sequence only")
+            dev = torch.device(self.device)
+            there = device_tokens.device.type == dev.type and dev.index in (None, device_tokens.device.index)
+            if device_tokens.dtype != torch.int32 or not there or tuple(device_tokens.shape) != (len(entries),):
+                raise StepError(f"device_tokens must be int32 [{len(entries)}] on {self.device}, got "
+                                f"{device_tokens.dtype} {tuple(device_tokens.shape)} on {device_tokens.device}")
         pos0 = [self.cache.length(s) for s in slots]
         try:
             self.cache.reserve(slots, n_new)
@@ -478,13 +493,14 @@ class Engine:
             if is_decode and graphs:
                 # the sequences of a decode step do not depend on each other: more of them than the largest captured
                 # step holds are replayed in pieces
-                pieces = [self._step_graph(entries[i:i + MAX_GRAPH_ROWS], slots[i:i + MAX_GRAPH_ROWS], pos0[i:i + MAX_GRAPH_ROWS])
+                pieces = [self._step_graph(entries[i:i + MAX_GRAPH_ROWS], slots[i:i + MAX_GRAPH_ROWS], pos0[i:i + MAX_GRAPH_ROWS],
+                                           None if device_tokens is None else device_tokens[i:i + MAX_GRAPH_ROWS])
                           for i in range(0, len(entries), MAX_GRAPH_ROWS)]
                 logits = pieces[0] if len(pieces) == 1 else torch.cat(pieces)
             elif not is_decode and graphs and self.prompt_graphs and self._prompt_bucket_ready(entries, n_new):
                 logits = self._step_prompt_graph(entries, slots, n_new, pos0)
             else:
-                logits = self._step_eager(entries, slots, n_new, pos0, is_decode)
+                logits = self._step_eager(entries, slots, n_new, pos0, is_decode, device_tokens)
         except BaseException:
             self.cache.unreserve(slots)          # the step did not happen: its pages go back
             raise
@@ -492,7 +508,7 @@ class Engine:
         self.steps_run += 1
         return logits
 
-    def _step_eager(self, entries, slots, n_new, pos0, is_decode):
+    def _step_eager(self, entries, slots, n_new, pos0, is_decode, device_tokens=None):
         dev = self.device
         tokens, positions, seq_index, want = [], [], [], []
         row = 0
@@ -520,6 +536,8 @@ class Engine:
             return v
 
         d_tokens, d_pos, d_seq, d_lens, d_want, d_slots = take(T), take(T), take(T), take(B), take(len(want)), take(B)
+        if device_tokens is not None:
+            d_tokens.copy_(device_tokens)
         d_order = take(len(order)) if is_decode else None
         d_tables = {g: take(tables[g].numel()).view(tables[g].shape) for g in sorted(tables)}
         ctx = StepContext(dev, self.model.dtype, d_tokens, d_pos, d_seq, d_lens, d_want, d_slots, is_decode,
@@ -600,12 +618,14 @@ class Engine:
             self.graphs_built += 1
         return g
 
-    def _step_graph(self, entries, slots, pos0):
+    def _step_graph(self, entries, slots, pos0, device_tokens=None):
         B = len(entries)
         lens_after = [p + 1 for p in pos0]
         g = self._graph_for(_bucket(B))
         g.fill(slots, [int(e.tokens[0]) for e in entries], lens_after, self)
         g.upload()
+        if device_tokens is not None:
+            g.tokens[:B].copy_(device_tokens)            # behind the upload, before the replay
         logits = g.run()
         rows = [i for i, e in enumerate(entries) for _ in e.want]
         if rows == list(range(B)):

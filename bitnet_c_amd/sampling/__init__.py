@@ -1,1 +1,1 @@
-from .sampler import SamplingParams, SequenceSampler, XorShift64Star, sample_batch
+from .sampler import PendingTokens, SamplingParams, SequenceSampler, XorShift64Star, sample_batch, start_sampling

@@ -70,17 +70,17 @@ class SequenceSampler:
                 del self.recent[0]
 
 
-def sample_batch(logits: torch.Tensor, samplers: Sequence[SequenceSampler]) -> List[int]:
-    """One token per row of `logits` ([B, vocab] float32 on the GPU; changed in place when a
-    penalty applies).  Rows are grouped by their parameters; each group is one launch."""
+def _sample_rows(logits: torch.Tensor, samplers: Sequence[SequenceSampler]) -> torch.Tensor:
+    """One token per row of `logits`, left on the GPU (int32 [B]).  Rows are grouped by their parameters; each group
+    is one launch."""
     if logits.shape[0] != len(samplers):
         raise ValueError("one sampler per row of logits")
-    out = [0] * len(samplers)
     groups = {}
     for i, s in enumerate(samplers):
         p = s.params
         groups.setdefault((p.temperature, p.top_p, p.repeat_penalty, p.repeat_window), []).append(i)
     whole = len(groups) == 1
+    out = None if whole else torch.empty((len(samplers),), dtype=torch.int32, device=logits.device)
     for (temp, top_p, penalty, window), rows in groups.items():
         sub = logits if whole else logits[rows].contiguous()
         if penalty != 1.0 and any(samplers[i].recent for i in rows):
@@ -90,8 +90,53 @@ def sample_batch(logits: torch.Tensor, samplers: Sequence[SequenceSampler]) -> L
             ops.repeat_penalty_(sub, rec.to(sub.device), penalty)
         uniforms = None
         if temp != 0.0:
-            uniforms = torch.tensor([samplers[i].rng.next_float() for i in rows], dtype=torch.float32).to(sub.device)
-        toks = ops.sample(sub, temp, top_p, uniforms).tolist()
-        for i, t in zip(rows, toks):
-            out[i] = int(t)
+            # from pinned memory, so that the upload does not make the host wait for the device
+            uniforms = torch.tensor([samplers[i].rng.next_float() for i in rows], dtype=torch.float32)
+            uniforms = (uniforms.pin_memory() if sub.is_cuda else uniforms).to(sub.device, non_blocking=True)
+        toks = ops.sample(sub, temp, top_p, uniforms)
+        if whole:
+            return toks
+        out[torch.tensor(rows, dtype=torch.long).to(out.device)] = toks
     return out
+
+
+def sample_batch(logits: torch.Tensor, samplers: Sequence[SequenceSampler]) -> List[int]:
+    """One token per row of `logits` ([B, vocab] float32 on the GPU; changed in place when a
+    penalty applies)."""
+    return [int(t) for t in _sample_rows(logits, samplers).tolist()]
+
+
+class PendingTokens:
+    """Tokens that a sampling launch has left on the device and that are on their way to the host."""
+
+    def __init__(self, device_tokens: torch.Tensor):
+        self.device_tokens = device_tokens
+        self._host = torch.empty(device_tokens.shape, dtype=device_tokens.dtype, pin_memory=device_tokens.is_cuda)
+        self._host.copy_(device_tokens, non_blocking=True)
+        self._arrived = torch.cuda.Event() if device_tokens.is_cuda else None
+        if self._arrived is not None:
+            self._arrived.record()
+
+    def rows(self, indices: Sequence[int]) -> torch.Tensor:
+        """device_tokens of the given rows, still on the device."""
+        idx = torch.tensor(list(indices), dtype=torch.long)
+        return self.device_tokens[(idx.pin_memory() if self.device_tokens.is_cuda else idx).to(self.device_tokens.device,
+                                                                                           non_blocking=True)]
+
+    def tokens(self) -> List[int]:
+        """Waits for the copy (not for anything queued after it)."""
+        if self._arrived is not None:
+            self._arrived.synchronize()
+        return [int(t) for t in self._host.tolist()]
+
+
+def start_sampling(logits: torch.Tensor, samplers: Sequence[SequenceSampler]):
+    """sample_batch without the wait: queues the sampling and the tokens' copy to the host and returns PendingTokens,
+    whose device_tokens a decode step can consume (Engine.step(..., device_tokens=...)) before the host has seen them.
+    None when a sequence's penalty needs the host's list of recent tokens first: then sample_batch is the way."""
+    if any(s.params.repeat_penalty != 1.0 for s in samplers):
+        return None
+    return PendingTokens(_sample_rows(logits, samplers))
+
+
+sample_batch.start = start_sampling

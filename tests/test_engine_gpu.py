@@ -911,6 +911,46 @@ def test_decode_steps_of_many_sequences_are_replayed_from_graphs(model_folders):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("graphs", [True, False])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_decode_step_takes_its_tokens_from_the_device(model_folders, dtype, graphs):
+    """Tokens that a sampling kernel has left on the device are consumed from there: the same logits, bit for bit, as
+    a step that is given the same tokens by the host; 300 sequences are more than one captured step holds, so the
+    tensor is cut with the step.  A wrong tensor is refused and changes nothing."""
+    import bitnet_c_amd as bn
+    from bitnet_c_amd import ops
+    from bitnet_c_amd.engine import StepError
+    folder = model_folders("B", dtype)
+    for n in (5, 300):
+        reqs = _requests(389, 17 + n, [1 + i % 11 for i in range(n)])
+        outs = []
+        for on_device in (False, True):
+            eng = bn.Engine.from_folder(folder, dtype=dtype, max_tokens=64 * (n + 4), use_graphs=graphs)
+            slots = [eng.new_sequence() for _ in reqs]
+            lg = eng.step([bn.StepEntry(s, r, [len(r) - 1]) for s, r in zip(slots, reqs)])
+            got = []
+            for k in range(3):
+                toks = ops.argmax(lg)
+                if on_device:
+                    lg = eng.step([bn.StepEntry(s, [0], [0]) for s in slots], device_tokens=toks)
+                else:
+                    lg = eng.step([bn.StepEntry(s, [t], [0]) for s, t in zip(slots, toks.tolist())])
+                got.append(lg)
+                if k == 1:                      # the batch shrinks: rows of the token tensor are picked on the device
+                    slots, lg = slots[1::2], lg[1::2].contiguous()
+            if on_device:
+                good = ops.argmax(lg)
+                for bad, entries in ((good.to(torch.int64), None), (good[:-1], None), (good.cpu(), None),
+                                     (good, [bn.StepEntry(s, [0, 1], [0]) for s in slots])):
+                    with pytest.raises(StepError):
+                        eng.step(entries or [bn.StepEntry(s, [0], [0]) for s in slots], device_tokens=bad)
+                assert all(eng.length(s) == len(r) + 3 for s, r in zip(slots, reqs[1::2]))
+            eng.cache.check()
+            outs.append(got)
+        for a, b in zip(*outs):
+            assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("n_tokens", [2048, 2000, 128])
 def test_graph_replays_of_a_prompt_step_at_the_benchmark_layer_sizes(n_tokens):
     """A prompt step at the Llama-3.1-8B layer sizes (two layers, bfloat16) recorded into a graph: its products are the

@@ -75,6 +75,36 @@ def test_sampled_generation_follows_the_plain_sampler(model_folders, temperature
     assert alone[0] == want[2]
 
 
+@pytest.mark.parametrize("with_penalty", [False, True])
+def test_requests_of_one_batch_sample_each_in_their_own_way(model_folders, with_penalty):
+    """Greedy, temperature and top-p requests in one batch (with a penalty among them the host must see every token
+    before the next step; without, steps are queued on tokens that are still on the device), unequal budgets and a stop
+    token: every request gets the plain sampler's tokens."""
+    import bitnet_c_amd as bn
+    from bitnet_c_amd.engine import Request, generate
+    from bitnet_c_amd.sampling import SamplingParams, sample_batch
+    folder = model_folders("B", torch.float32)
+    llm = bn.load(folder, dtype="float32", max_tokens=2048)
+    c, W = pl.read_config(folder), pl.read_weights(folder)
+    prompts = _prompts(c["vocab"], 5, [4, 17, 2, 33, 9])
+    kinds = [(0.0, 0.9, 1.0), (0.8, 1.0, 1.0), (0.7, 0.9, 1.0), (0.0, 0.9, 1.0), (1.1, 0.5, 1.25 if with_penalty else 1.0)]
+    budgets = [9, 4, 12, 1, 7]
+    free = pl.generate(c, W, prompts[2], 12, 0.7, 0.9, 11, (), 1.0)
+    stops = [(), (), (free[5],), (), ()]
+    reqs = [Request(p, n, SamplingParams(temperature=t, top_p=tp, seed=11, repeat_penalty=pen), st)
+            for p, n, (t, tp, pen), st in zip(prompts, budgets, kinds, stops)]
+    steps_before = llm.engine.steps_run
+    res = generate(llm.engine, reqs, sample_batch, batch_size=8)
+    want = [pl.generate(c, W, p, n, t, tp, 11, st, pen) for p, n, (t, tp, pen), st in zip(prompts, budgets, kinds, stops)]
+    assert [r.tokens for r in res] == want
+    assert res[2].finish == "stop" and len(want[2]) < 12
+    # the steps that ran: one for the prompts, then one a token of the longest request; queued ahead, the request that
+    # its stop token ended had its row in one step more, which is no step more
+    assert llm.engine.steps_run - steps_before == max(len(w) for w in want)
+    assert not llm.engine.cache.live_slots()
+    llm.engine.cache.check()
+
+
 def test_bfloat16_generation_starts_like_the_plain_one(model_folders):
     import bitnet_c_amd as bn
     folder = model_folders("A", torch.bfloat16)

@@ -113,6 +113,91 @@ def test_an_error_in_a_step_gives_the_slots_back():
     assert not eng.live
 
 
+class AheadEngine(FakeEngine):
+    """A stand-in that takes a decode step's tokens from a tensor, as the engine takes them from the device."""
+    takes_device_tokens = True
+
+    def __init__(self, *a, fail_ahead_at=None, **kw):
+        super().__init__(*a, **kw)
+        self.ahead_steps, self.fail_ahead_at = 0, fail_ahead_at
+
+    def step(self, entries, device_tokens=None):
+        if device_tokens is not None:
+            from bitnet_c_amd.engine.step import StepError
+            self.ahead_steps += 1
+            if self.fail_ahead_at == self.ahead_steps:
+                raise StepError("no page left")
+            assert all(list(e.tokens) == [0] for e in entries) and device_tokens.shape == (len(entries),)
+            entries = [type(e)(e.slot, [int(t)], e.want) for e, t in zip(entries, device_tokens)]
+        return super().step(entries)
+
+
+class _Pending:
+    def __init__(self, toks):
+        self.device_tokens = toks
+
+    def rows(self, idx):
+        return self.device_tokens[list(idx)]
+
+    def tokens(self):
+        return [int(t) for t in self.device_tokens]
+
+
+def _greedy_ahead():
+    def fn(logits, samplers):
+        return greedy(logits, samplers)
+    fn.start = lambda logits, samplers: _Pending(logits.argmax(dim=1).to(torch.int32))
+    return fn
+
+
+def _mixed_requests():
+    return [Request([1, 2, 3], 5), Request([10], 2), Request([20, 21], 10, stop_ids=(24,)), Request([30], 0),
+            Request([40], 1), Request([41, 42], 7, stop_ids=(43,)), Request([7], 9, stop_ids=(12, 3))]
+
+
+@pytest.mark.parametrize("batch_size", [8, 3, 1])
+def test_steps_queued_ahead_decide_the_same(batch_size):
+    """With tokens that stay on the device a step is queued before the host has seen them: tokens, finish reasons and
+    the slots' fate are those of the plain loop; a sequence that its token has ended ran one step for nothing."""
+    a, b = FakeEngine(), AheadEngine()
+    want = generate(a, _mixed_requests(), greedy, batch_size=batch_size)
+    got = generate(b, _mixed_requests(), _greedy_ahead(), batch_size=batch_size)
+    assert [(r.tokens, r.finish) for r in got] == [(r.tokens, r.finish) for r in want]
+    assert not b.live and sorted(b.released) == sorted(a.released)
+    assert b.ahead_steps > 0
+    # the steps differ only by the rows of sequences that a stop token ended: those ran once more
+    fed = lambda eng: sorted((sl, t[0]) for st in eng.steps for sl, t in st if len(t) == 1)
+    extra = [x for x in fed(b) if x not in fed(a)]
+    stopped = sum(r.finish == "stop" for r in want)
+    assert len(fed(b)) - len(fed(a)) == len(extra) <= stopped
+    # nothing ran for a sequence at its budget or at the limit: those are counts, known without the token
+    eng = AheadEngine(max_seq_len=6)
+    res = generate(eng, [Request([1, 2, 3, 4], 10)], _greedy_ahead())
+    assert res[0].finish == "limit" and res[0].tokens == [5, 6, 7] and [len(s) for s in eng.steps] == [1, 1, 1]
+
+
+def test_a_cancelling_callback_and_a_refused_step_under_queued_steps():
+    eng = AheadEngine()
+    seen = []
+    res = generate(eng, [Request([1], 10), Request([5], 3)], _greedy_ahead(),
+                   on_token=lambda i, t: seen.append((i, t)) or i == 0)
+    assert res[0].tokens == [2] and res[0].finish == "cancelled" and res[1].tokens == [6, 7, 8]
+    assert seen == [(0, 2), (1, 6), (1, 7), (1, 8)] and not eng.live
+    # a step that the engine refuses when it is queued ahead changes nothing: the loop decides with the tokens at hand
+    # and asks again the plain way
+    eng = AheadEngine(fail_ahead_at=2)
+    res = generate(eng, [Request([1], 6), Request([9], 4)], _greedy_ahead())
+    assert res[0].tokens == [2, 3, 4, 5, 6, 7] and res[1].tokens == [10, 11, 12, 13] and not eng.live
+
+
+def test_a_sampler_that_needs_the_host_first_is_asked_the_plain_way():
+    fn = _greedy_ahead()
+    fn.start = lambda logits, samplers: None
+    eng = AheadEngine()
+    res = generate(eng, [Request([1], 3)], fn)
+    assert res[0].tokens == [2, 3, 4] and eng.ahead_steps == 0
+
+
 def test_host_rng_and_recent_ring_follow_the_plain_sampler():
     a, b = XorShift64Star(0), pl.XorShift64Star(42)
     assert [a.next_float() for _ in range(50)] == [b.next_float() for _ in range(50)]
