@@ -19,7 +19,9 @@ extern "C" {
 // no counterpart; its back-ends allocate their work buffers themselves.
 //
 // k_pages and vt_pages are blocked pages (common.h: [pages, Hkv, 64 * hs] each, keys and values of a page in the order in
-// which the kernel loads them), as everywhere in attn_mfma.hip.
+// which the kernel loads them), as everywhere in attn_mfma.hip.  block_table [n_seqs, bt_stride >= 1]: every entry names a
+// page of the pool, also those behind a sequence's last page (a workgroup asks for its first block of keys before it
+// knows the sequence's length, and drops it if the sequence ends before it).
 // Same arguments and the same result, bit for bit, as bn_attn_mfma with tiles == null, except that
 // the split partials (n_seqs * H * n_splits * (hs + 2) floats) live in a file-scope device array
 // of BN_ATTN_STATIC_SCRATCH_FLOATS floats instead of buffers the caller brings.  It calls no

@@ -22,7 +22,12 @@
 // the keys and values it walks are staged through shared memory once for all four waves.
 // Decode form: the 16 columns are the heads of one kv group for the sequence's one new token;
 // the 4 waves take 32-key blocks in turn and merge through shared memory; long contexts are
-// also split over gridDim.z and merged by attn_mfma_combine_kernel in a fixed order.
+// also split over gridDim.z and merged by attn_mfma_combine_kernel in a fixed order.  What a decode workgroup needs
+// before its first block (the query, the frequencies, the new key and value, the length, the first block itself) is
+// asked for at once, in straight-line code, with the length and the page numbers through the scalar unit: the first
+// block of keys is on its way before the length is known (see the kernel), so that a short launch is two trips to
+// memory instead of five.  Every entry of a block table must name a page of the pool for that, also the entries
+// behind a sequence's last page.
 #include "common.h"
 #include "attn_mfma.h"
 #include <mutex>
@@ -118,6 +123,20 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
     return (ua >> 16) | (ub & 0xffff0000u);
 }
 
+// A barrier of the workgroup that orders its shared memory only.  __syncthreads() also waits for everything that the wave
+// has asked from global memory; this one leaves such loads in flight (whoever needs their data waits for it there).
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// The float32 value of a bf16 bit pattern, widened where this stands and nowhere else: the compiler moves a plain shift
+// up to the load of the pattern, and the load's wait with it.
+__device__ __forceinline__ float widen_here(unsigned bits) {
+    float f;
+    asm volatile("v_lshlrev_b32 %0, 16, %1" : "=v"(f) : "v"(bits));
+    return f;
+}
+
 // A read of p[idx] for an index that is the same in every lane, through the scalar unit (the
 // constant address space makes the compiler pick a scalar load).  Only for memory that no kernel
 // writes while this one runs (block tables, lengths).
@@ -158,8 +177,22 @@ __device__ __forceinline__ int v_swizzle(int row) {
 // length).  All operands are asked for up front: they come from memory, and the latency is paid once.
 // The prompt form below has code of its own on purpose: the decode kernel is sensitive to how the compiler lays
 // this code out, and changes made for the staged form must not move it.
+// The operands of a block of 32 keys from blocked pages: tile row i of key tile 0 is the block's key 8 (i / 4) + i % 4,
+// tile 1 four further; lane i + 16 g of value tile t holds dimension 16 t + i of the block's keys 8 g .. 8 g + 7.
+template <int HS>
+__device__ __forceinline__ void load_block(const bf16* __restrict__ kbase, const bf16* __restrict__ vbase,
+                                           bf16x8 (&ka)[HS / 32][2], bf16x8 (&va)[HS / 16], int lane) {
+#pragma unroll
+    for (int c = 0; c < HS / 32; ++c) {
+        ka[c][0] = ld16(kbase + (2 * c) * 512 + lane * 8);
+        ka[c][1] = ld16(kbase + (2 * c + 1) * 512 + lane * 8);
+    }
+#pragma unroll
+    for (int t = 0; t < HS / 16; ++t) va[t] = ld16(vbase + t * 512 + lane * 8);
+}
+
 template <int HS, int NT, bool need_mask>
-__device__ __forceinline__ void attend_block_direct_m(const bf16* __restrict__ kbase, const bf16* __restrict__ vbase,
+__device__ __forceinline__ void attend_loaded_m(const bf16x8 (&ka)[HS / 32][2], bf16x8 (&va)[HS / 16],
                                                int kb, const bf16x8 (&q)[NT][HS / 32], f32x4 (&acc)[NT][HS / 16],
                                                float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
                                                const int (&lo)[NT], int key_hi, float scale2, int lane) {
@@ -168,17 +201,6 @@ __device__ __forceinline__ void attend_block_direct_m(const bf16* __restrict__ k
     f32x4 st[NT][2];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) { st[nt][0] = (f32x4){0.f, 0.f, 0.f, 0.f}; st[nt][1] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
-    bf16x8 ka[DC][2];
-    bf16x8 va[DT];
-    // tile row i of key tile 0 is the block's key 8 (i / 4) + i % 4, tile 1 four further; lane i + 16 g of value tile t
-    // holds dimension 16 t + i of the block's keys 8 g .. 8 g + 7
-#pragma unroll
-    for (int c = 0; c < DC; ++c) {
-        ka[c][0] = ld16(kbase + (2 * c) * 512 + lane * 8);
-        ka[c][1] = ld16(kbase + (2 * c + 1) * 512 + lane * 8);
-    }
-#pragma unroll
-    for (int t = 0; t < DT; ++t) va[t] = ld16(vbase + t * 512 + lane * 8);
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
 #pragma unroll
@@ -399,10 +421,13 @@ __device__ __forceinline__ void attend_block(const bf16* __restrict__ kbase, con
                                              float (&m)[NT], float (&l)[NT], const int (&qpos)[NT],
                                              const int (&lo)[NT], int key_hi, bool need_mask, float scale2,
                                              int lane) {
+    bf16x8 ka[HS / 32][2];
+    bf16x8 va[HS / 16];
+    load_block<HS>(kbase, vbase, ka, va, lane);
     if (need_mask)
-        attend_block_direct_m<HS, NT, true>(kbase, vbase, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
+        attend_loaded_m<HS, NT, true>(ka, va, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
     else
-        attend_block_direct_m<HS, NT, false>(kbase, vbase, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
+        attend_loaded_m<HS, NT, false>(ka, va, kb, q, acc, m, l, qpos, lo, key_hi, scale2, lane);
 }
 template <int HS, int NT, int VSTRIDE>
 __device__ __forceinline__ void block_weights_values(const f32x4 (&st)[NT][2], const unsigned char* __restrict__ stage, int voff, int kb,
@@ -707,41 +732,52 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
                 r = first + (last - r);
             }
         }
-        seq = a.by_length[r];
+        seq = uniform_load(a.by_length, r);
         if ((unsigned)seq >= gridDim.y) return;          // not a permutation: touch nothing
     }
-    // Everything that can be asked for before the sequence's length is known is asked for now (the query's heads, the
-    // frequencies, the new key and value): one wait for memory instead of one after the other.
+    // Everything that does not depend on the sequence's length is asked for now, in straight-line code with no lane left
+    // out of a load (a lane without a head, a thread without an element asks for a neighbour's and drops it), so that
+    // nothing waits for anything but its own data: the query's heads, the frequencies, the new key and value, the sums of
+    // squares of a deferred norm.  The length and the pages come through the scalar unit, beside those loads.
     const int hg = ht * GT + n;
-    const int head = kvh * G + hg;
+    const bool q_lane = n < GT && hg < G;
+    const int head = kvh * G + (q_lane ? hg : 0);
     const bf16* row = a.q + (size_t)seq * a.q_stride;
     uint4 z[DC];
 #pragma unroll
-    for (int c = 0; c < DC; ++c) {
-        z[c] = make_uint4(0, 0, 0, 0);
-        if (n < GT && hg < G) z[c] = *reinterpret_cast<const uint4*>(row + (size_t)head * HS + c * 32 + g * 8);
-    }
+    for (int c = 0; c < DC; ++c) z[c] = *reinterpret_cast<const uint4*>(row + (size_t)head * HS + c * 32 + g * 8);
     const int tid = threadIdx.x;
-    const float freq = (a.rotate && tid < HALF) ? a.inv_freq[tid] : 0.f;
-    float row_scale = 1.0f;
-    if (a.row_ssq) {                                     // the same few floats in every thread, added in piece order
-        float ss = 0.f;
-        for (int p = 0; p < a.n_pieces; ++p) ss += a.row_ssq[(size_t)seq * a.n_pieces + p];
-        row_scale = 1.0f / sqrtf(ss * a.inv_ssq_width + a.ssq_eps);
+    float freq = 0.f, piece = 0.f;
+    if (a.rotate) freq = a.inv_freq[tid & (HALF - 1)];
+    if (a.row_ssq) piece = a.row_ssq[(size_t)seq * a.n_pieces + min(lane, a.n_pieces - 1)];
+    unsigned new_k0 = 0, new_k1 = 0, new_v = 0;          // bf16 bit patterns, widened where they are used
+    if (a.write_kv) {        // threads below HALF hold a pair of the key, the HS behind them an element of the value
+        const unsigned short* kn = reinterpret_cast<const unsigned short*>(row + (size_t)(a.H + kvh) * HS);
+        const unsigned short* vn = reinterpret_cast<const unsigned short*>(row + (size_t)(a.H + a.Hkv + kvh) * HS);
+        new_k0 = kn[tid & (HALF - 1)];
+        new_k1 = kn[(tid & (HALF - 1)) + HALF];
+        new_v = vn[(tid - HALF) & (HS - 1)];
     }
-    bf16 new_k0 = __float2bfloat16(0.f), new_k1 = new_k0, new_v = new_k0;
-    if (a.write_kv) {
-        if (tid < HALF) {
-            new_k0 = row[(size_t)(a.H + kvh) * HS + tid];
-            new_k1 = row[(size_t)(a.H + kvh) * HS + tid + HALF];
-        } else if (tid < HALF + HS) {
-            new_v = row[(size_t)(a.H + a.Hkv + kvh) * HS + tid - HALF];
-        }
-    }
-    const int L = a.seq_lens[seq];
-    const bool ok = n < GT && hg < G && L > 0;
-    const int lo_key = a.window > 0 ? max(0, L - a.window) : 0;
+    const int L = uniform_load(a.seq_lens, seq);
     const int chunk = a.max_len ? bn_split_chunk(uniform_load(a.max_len, 0), a.n_splits) : a.chunk;
+    // So is the first block of keys that this wave will take, whose place does not depend on the length when no window
+    // cuts the keys: its page and its 16 KB are on their way while the rotation is worked out and the new token is
+    // stored, instead of after all that.  If the sequence turns out to end before the block, it is dropped unused (every
+    // entry of a block table names a page of the pool, also those behind a sequence's last page); if the block holds
+    // the new token's position, it is asked for again behind the store.
+    // (With a window, or a table that ends before the block, the loads go to the table's first page and are dropped:
+    // loads under a branch would make everything behind it wait for all of them.)
+    const int kb_first = split * chunk + 32 * __builtin_amdgcn_readfirstlane(wave);
+    const bool ahead = a.window == 0 && kb_first / BN_PAGE < a.bt_stride;
+    bf16x8 ka0[DC][2];
+    bf16x8 va0[DT];
+    const int page0 = uniform_load(a.block_table, (size_t)seq * a.bt_stride + (ahead ? kb_first / BN_PAGE : 0));
+    const size_t at0 = (((size_t)page0 * a.Hkv + kvh) * BN_PAGE + kb_first % BN_PAGE) * HS;
+    const bf16* kbase0 = a.k_pages + at0;
+    const bf16* vbase0 = a.vt_pages + at0;
+    load_block<HS>(kbase0, vbase0, ka0, va0, lane);
+    const bool ok = q_lane && L > 0;
+    const int lo_key = a.window > 0 ? max(0, L - a.window) : 0;
     const int k_lo = max(lo_key, split * chunk), k_hi = min(L, (split + 1) * chunk);       // [k_lo, k_hi)
     if (a.n_splits > 1 && k_lo >= k_hi) {
         // A split without keys (a sequence shorter than the launch's longest, a padding row): it leaves "nothing seen"
@@ -751,7 +787,15 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
             a.part_ml[prow * 2] = -INFINITY;
             a.part_ml[prow * 2 + 1] = 0.f;
         }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // what was asked for has arrived before the wave ends
         return;
+    }
+    float row_scale = 1.0f;
+    if (a.row_ssq) {                                     // the same few floats in every lane, added in piece order
+        float ss = 0.f;
+        for (int p = 0; p < a.n_pieces; ++p)
+            ss += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, piece), p));
+        row_scale = 1.0f / sqrtf(ss * a.inv_ssq_width + a.ssq_eps);
     }
 
     if (a.rotate && L > 0) {
@@ -760,18 +804,21 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
             sincosf((float)(L - 1) * freq, &sv, &cv);
             cos_s[tid] = cv * row_scale; sin_s[tid] = sv * row_scale;
         }
-        __syncthreads();
+        lds_barrier();                                   // the block that is on its way stays on its way
     }
     // the new token's key and value go into the cache before anyone reads them: the workgroup
     // that owns the new position does it (there is one per kv head: write_kv needs n_head_tiles == 1)
     if (a.write_kv && L > 0 && L - 1 >= k_lo && L - 1 < k_hi) {
         const int pos = L - 1;
-        const int page = a.block_table[(size_t)seq * a.bt_stride + pos / BN_PAGE], off = pos % BN_PAGE;
+        // through the scalar unit (the length is the same in every lane), so that it does not queue behind the block
+        // that is on its way
+        const int page = uniform_load(a.block_table, (size_t)seq * a.bt_stride + __builtin_amdgcn_readfirstlane(pos / BN_PAGE));
+        const int off = pos % BN_PAGE;
         bf16* kdst = const_cast<bf16*>(a.k_pages) + ((size_t)page * a.Hkv + kvh) * BN_PAGE * HS;
         bf16* vdst = const_cast<bf16*>(a.vt_pages) + ((size_t)page * a.Hkv + kvh) * BN_PAGE * HS;
         const int t = threadIdx.x;
         if (t < HALF) {
-            float k0 = __bfloat162float(new_k0), k1 = __bfloat162float(new_k1);
+            float k0 = widen_here(new_k0), k1 = widen_here(new_k1);
             if (a.rotate) {
                 const float c = cos_s[t], sv = sin_s[t];
                 const float r0 = k0 * c - k1 * sv, r1 = k0 * sv + k1 * c;
@@ -781,7 +828,9 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
             kdst[bn_blocked_k_offset(off, t + HALF, HS)] = __float2bfloat16(k1);
         } else if (t < HALF + HS) {
             const int d = t - HALF;
-            vdst[bn_blocked_v_offset(off, d, HS)] = a.row_ssq ? __float2bfloat16(__bfloat162float(new_v) * row_scale) : new_v;
+            reinterpret_cast<unsigned short*>(vdst)[bn_blocked_v_offset(off, d, HS)] =
+                a.row_ssq ? __builtin_bit_cast(unsigned short, __float2bfloat16(widen_here(new_v) * row_scale))
+                          : (unsigned short)new_v;
         }
         // only this workgroup reads what it has just stored: a fence of workgroup scope is enough
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
@@ -790,6 +839,10 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
 
     bf16x8 q[1][DC];
     {
+        if (!q_lane) {
+#pragma unroll
+            for (int c = 0; c < DC; ++c) z[c] = make_uint4(0, 0, 0, 0);
+        }
         if (a.rotate && L > 0) {
 #pragma unroll
             for (int c = 0; c < DC / 2; ++c)      // chunk c holds pair indices c*32 + g*8 .. +7, its partners are in chunk c + DC/2
@@ -813,7 +866,16 @@ __global__ __launch_bounds__(256) void attn_mfma_decode_kernel(MfmaArgs a) {
         // The waves take the blocks of 32 keys in turn, so that neighbouring waves ask for the two halves of a page at
         // the same time (a wave that takes whole pages by itself was measured 10 to 20 % slower, and so was splitting
         // the sequences of a large batch: the order by length with unsplit sequences keeps the CUs busiest).
-        for (int kb = (k_lo / 32) * 32 + 32 * wave; kb < k_hi; kb += 128) {
+        int kb = (k_lo / 32) * 32 + 32 * wave;
+        if (ahead && kb == kb_first && kb < k_hi) {        // the block that was asked for at the start
+            if (a.write_kv && L - 1 >= kb && L - 1 < kb + 32) load_block<HS>(kbase0, vbase0, ka0, va0, lane);
+            if ((kb + 32 > k_hi) || (kb < k_lo))
+                attend_loaded_m<HS, 1, true>(ka0, va0, kb, q, acc, m, l, qpos, lo, k_hi, scale2, lane);
+            else
+                attend_loaded_m<HS, 1, false>(ka0, va0, kb, q, acc, m, l, qpos, lo, k_hi, scale2, lane);
+            kb += 128;
+        }
+        for (; kb < k_hi; kb += 128) {
             // the page index is the same for the whole wave: read through the scalar unit, so that it
             // does not queue behind the vector loads
             const int page = uniform_load(a.block_table, bt_row + __builtin_amdgcn_readfirstlane(kb / BN_PAGE));
@@ -916,7 +978,7 @@ static int attn_mfma_launch(const void* q, int q_stride, void* out, int out_stri
     if (row_ssq && (tiles || !rotate || n_pieces < 1 || n_pieces > 64 || ssq_width < 1)) return BN_ERR_ARG;   // decode form, rotating
     if (GT <= 0 || GT > 16 || (GT & (GT - 1)) || window < 0 || n_splits < 1 || n_splits > 64) return BN_ERR_ARG;
     if (n_splits > 1 && (!part_o || !part_ml || (!max_len && (chunk <= 0 || chunk % BN_PAGE)))) return BN_ERR_ARG;
-    if (!tiles && !seq_lens) return BN_ERR_ARG;
+    if (!tiles && (!seq_lens || bt_stride < 1)) return BN_ERR_ARG;      // the decode form reads a row's first entry unasked
     if (max_len && tiles) return BN_ERR_ARG;                               // decode form only
     if (q_stride % 8 || out_stride % 4 || (((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)vt_pages) & 15) ||
         ((uintptr_t)out & 7))

@@ -9,7 +9,7 @@
 #define BN_PAGE 64            // tokens per cache page; the Python side reads this line (csrc/build.py: header_constant)
 // Decode attention splits a sequence's keys over workgroups in runs of at least this many pages: shorter
 // runs cost more in merging than they gain in parallelism (measured at batch 1, 8 and 64 of an 8B shape).
-#define BN_SPLIT_MIN_PAGES 4
+#define BN_SPLIT_MIN_PAGES 2
 // A float32 cache's keys are summed in runs of this many positions (whole pages, counted from position 0), each run by
 // itself and the runs folded in order: a decode step then spreads a long sequence's runs over workgroups and still forms
 // every sum in the order in which a prompt step forms it, so that float32 logits do not depend on how a sequence was cut.

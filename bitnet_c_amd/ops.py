@@ -1111,7 +1111,9 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     Prompt form: `tiles` [n, 4] int32 = (sequence, first token row, tokens (<= qt), position of
     the first), qt = the QT of attention_row_shape(H, Hkv, False, dtype, hs).
     Decode form: tiles None, seq_lens [B] int32 (keys in the cache, the new one included; 0 for a
-    padding row); row b of qkv is sequence b's token; n_splits/chunk from decode_splits.
+    padding row); row b of qkv is sequence b's token; n_splits/chunk from decode_splits.  Every entry of
+    block_table names a page of the pool, also those behind a sequence's last page (0 will do): the
+    matrix-core kernel asks for a workgroup's first block of keys before it knows the sequence's length.
     bf16 with head size 64 or 128 over blocked pages runs on the matrix cores, everything else on the vector ALUs,
     which read rows and transposed values (force_vector: say so where the pages are not blocked and the head size
     would be the other kernel's; its qt then is that of attention_row_shape without dtype).

@@ -1370,10 +1370,13 @@ def test_repeat_penalty_on_device():
 @pytest.mark.parametrize("force_splits", [1, 0, 7])
 def test_decode_attention_that_rotates_and_stores_itself(H, Hkv, hs, window, force_splits):
     """The decode kernel doing rope_kv_write's work: unrotated qkv in, the new key and value stored,
-    against rope_kv_write followed by the same attention; run twice in a row."""
+    against rope_kv_write followed by the same attention; run twice in a row.  Every wave of a workgroup asks for its
+    first block of 32 keys before it knows the length: the lengths put the new token's place into the first block of
+    each of the four waves (which must then be read again behind the store), into a later block, and behind a
+    sequence's end (a block that is dropped)."""
     ops = _ops()
     dtype = torch.bfloat16
-    lens_before = [0, 63, 64, 700, 129, 300, 31]
+    lens_before = [0, 63, 64, 700, 129, 300, 31, 100, 127, 32]
     B = len(lens_before)
     seqs_k = [_rand((p + 1, Hkv, hs), dtype, 700 + i) for i, p in enumerate(lens_before)]
     seqs_v = [_rand((p + 1, Hkv, hs), dtype, 800 + i) for i, p in enumerate(lens_before)]
