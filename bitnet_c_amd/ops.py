@@ -1066,8 +1066,10 @@ def pair_tiles(rows: list) -> list:
     return out
 
 
-# Workgroups that a decode attention launch aims for when it cuts the keys (two for every CU of this chip).
-DECODE_TARGET_WGS = int(os.environ.get("BITNET_DECODE_WGS", "512"))
+# Workgroups that a decode attention launch aims for when it cuts the keys: one for every CU of this chip.  (Measured at
+# 8,000 and 32,000 cached tokens a sequence and 1 to 8 sequences of the 8B shape: about 256 workgroups are fastest
+# whatever the batch, 29 us against 35 for 504 at one sequence of 32,000 tokens, 183 against 188 at eight.)
+DECODE_TARGET_WGS = int(os.environ.get("BITNET_DECODE_WGS", "256"))
 
 
 def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int, dtype=None):
@@ -1081,7 +1083,7 @@ def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int, dtype=None):
     G = H // Hkv
     wgs = max(1, n_seqs * Hkv * ((G + GT - 1) // GT))
     pages = max(1, (max_len + PAGE - 1) // PAGE)
-    # about 512 workgroups, but no split shorter than SPLIT_MIN_PAGES pages: below that the merging costs
+    # about DECODE_TARGET_WGS workgroups, but no split shorter than SPLIT_MIN_PAGES pages: below that the merging costs
     # more than the parallelism gains (measured at batch 1, 8 and 64 of the 8B shape)
     want = max(1, min(pages // SPLIT_MIN_PAGES, 64, (DECODE_TARGET_WGS + wgs - 1) // wgs))
     chunk = ((pages + want - 1) // want) * PAGE
