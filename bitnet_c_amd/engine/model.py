@@ -92,16 +92,29 @@ class DecoderModel:
             return 0
         return sum(l.stream_bytes() for l in self.linears())
 
-    def keep_streamed(self, keep: bool = True, budget: int = None) -> int:
+    def keep_streamed(self, keep: bool = True, budget: int = None, keep_free: int = 0) -> int:
         """Makes (or drops) the streamed copies of the parts' weight matrices and of the output matrix; with a budget (in
-        bytes) only as many as fit into it, the largest matrices first.  Returns the bytes that the copies take."""
+        bytes) only as many as fit into it, the largest matrices first.  keep_free: bytes of the device's memory that
+        must stay free; a copy that cuts into them (the allocator could not place it in what it holds) is dropped again
+        and no other of its size or larger is tried, and so is a copy that the device has no room for.  Returns the bytes that the copies
+        take."""
         matrices = self.linears()
         applies = self.dtype == torch.bfloat16 and self.device.type == "cuda"
         sizes = [l.stream_bytes() if applies else 0 for l in matrices]
-        used = 0
+        used, too_large = 0, None                # too_large: the size of a copy that found no place (smaller ones still may)
         for i in sorted(range(len(matrices)), key=lambda i: -sizes[i]):      # a stable order: equal sizes in model order
-            fits = bool(keep and sizes[i] > 0 and (budget is None or used + sizes[i] <= budget))
-            matrices[i].keep_streamed(fits)
+            fits = bool(keep and sizes[i] > 0 and (too_large is None or sizes[i] < too_large)
+                        and (budget is None or used + sizes[i] <= budget))
+            free_before = torch.cuda.mem_get_info(self.device)[0] if fits and keep_free else 0
+            try:
+                matrices[i].keep_streamed(fits)
+            except torch.cuda.OutOfMemoryError:
+                matrices[i].keep_streamed(False)
+                fits, too_large = False, sizes[i]
+            if fits and keep_free and torch.cuda.mem_get_info(self.device)[0] < min(keep_free, free_before):
+                matrices[i].keep_streamed(False)         # it was placed in memory that is to stay free
+                torch.cuda.empty_cache()
+                fits, too_large = False, sizes[i]
             used += sizes[i] if fits else 0
         self.has_streamed = used > 0
         self.streamed_settled = True
@@ -109,11 +122,17 @@ class DecoderModel:
 
     def settle_streamed(self) -> None:
         """Called by an engine once its cache is allocated: a model that was not told whether to keep streamed copies
-        takes as many as streamed_budget allows now."""
+        takes as many as streamed_budget allows now.  What the allocator holds without using it counts as free (after
+        loading a model of 140 GB that is tens of GB, in pieces: a copy that finds no piece large enough is placed in the
+        device's free memory, of which a tenth of the device is kept back)."""
         if self.streamed_settled:
             return
-        free, total = torch.cuda.mem_get_info(self.device) if self.device.type == "cuda" else (0, 0)
-        self.keep_streamed(True, streamed_budget(free, total))
+        free, total, held = 0, 0, 0
+        if self.device.type == "cuda":
+            torch.cuda.empty_cache()
+            free, total = torch.cuda.mem_get_info(self.device)
+            held = max(0, torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device))
+        self.keep_streamed(True, streamed_budget(free + held, total), keep_free=int(STREAMED_RESERVE_SHARE * total))
 
     def weight_bytes(self) -> int:
         """Bytes of every weight a decode step reads once (the embedding table only when it is
