@@ -98,15 +98,14 @@ __device__ __forceinline__ void rotate_groups(uint4& lo, uint4& hi, const float*
     }
 }
 
-__global__ __launch_bounds__(256) void rope_kv_write_bf16x8_kernel(bf16* __restrict__ qkv, int row_stride,
-                                                                   const int* __restrict__ positions,
-                                                                   const int* __restrict__ seq_index,
-                                                                   const int* __restrict__ block_table, int bt_stride,
-                                                                   bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
-                                                                   const float* __restrict__ inv_freq, int rope_dims,
-                                                                   int H, int Hkv, int hs, int layout) {
-    extern __shared__ float cs[];            // cos[half], sin[half]
-    const int t = blockIdx.x;
+// The work of one workgroup on token row t; cs: shared memory for cos[half], sin[half].
+__device__ __forceinline__ void rope_kv_write_bf16x8_row(int t, float* cs, bf16* __restrict__ qkv, int row_stride,
+                                                         const int* __restrict__ positions,
+                                                         const int* __restrict__ seq_index,
+                                                         const int* __restrict__ block_table, int bt_stride,
+                                                         bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
+                                                         const float* __restrict__ inv_freq, int rope_dims,
+                                                         int H, int Hkv, int hs, int layout) {
     const int pos = positions[t];
     if (pos < 0) return;                     // a padding row
     const int half = rope_dims / 2;
@@ -177,20 +176,31 @@ __global__ __launch_bounds__(256) void rope_kv_write_bf16x8_kernel(bf16* __restr
     }
 }
 
+__global__ __launch_bounds__(256) void rope_kv_write_bf16x8_kernel(bf16* __restrict__ qkv, int row_stride,
+                                                                   const int* __restrict__ positions,
+                                                                   const int* __restrict__ seq_index,
+                                                                   const int* __restrict__ block_table, int bt_stride,
+                                                                   bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
+                                                                   const float* __restrict__ inv_freq, int rope_dims,
+                                                                   int H, int Hkv, int hs, int layout) {
+    extern __shared__ __align__(16) unsigned char dyn_s[];
+    rope_kv_write_bf16x8_row(blockIdx.x, reinterpret_cast<float*>(dyn_s), qkv, row_stride, positions, seq_index, block_table,
+                             bt_stride, k_pages, v_pages, inv_freq, rope_dims, H, Hkv, hs, layout);
+}
+
 // V into transposed or blocked pages for the tokens of a prompt: a workgroup takes the rows of one sequence
 // that fall into one page (tile = sequence, first row, rows, position of the first) and one kv
 // head, turns the [rows, hs] block through shared memory and stores runs of 8 positions with
 // 16 bytes, instead of 2 bytes a position and dimension (8 positions from a multiple of 8 of one dimension are
 // 16 consecutive bytes in either order).
 #define VT_PAD 2
-__global__ __launch_bounds__(256) void v_transposed_write_kernel(const bf16* __restrict__ qkv, int row_stride,
-                                                                 const int* __restrict__ tiles,
-                                                                 const int* __restrict__ block_table, int bt_stride,
-                                                                 bf16* __restrict__ v_pages, int H, int Hkv, int hs, int blocked) {
-    extern __shared__ uint16_t vt_s[];       // [hs][BN_PAGE + VT_PAD], column = position inside the page
-    const int* tl = tiles + 4 * blockIdx.x;
+// The work of one workgroup on (tile, kv head kh); vt_s: shared memory [hs][BN_PAGE + VT_PAD], column = position inside the page.
+__device__ __forceinline__ void v_transposed_write_tile(int tile, int kh, uint16_t* vt_s, const bf16* __restrict__ qkv,
+                                                        int row_stride, const int* __restrict__ tiles,
+                                                        const int* __restrict__ block_table, int bt_stride,
+                                                        bf16* __restrict__ v_pages, int H, int Hkv, int hs, int blocked) {
+    const int* tl = tiles + 4 * tile;
     const int seq = tl[0], row0 = tl[1], n = tl[2], pos0 = tl[3];
-    const int kh = blockIdx.y;
     const int off = pos0 % BN_PAGE;
     if (n <= 0 || off + n > BN_PAGE) return;
     const int page = block_table[(size_t)seq * bt_stride + pos0 / BN_PAGE];
@@ -222,6 +232,36 @@ __global__ __launch_bounds__(256) void v_transposed_write_kernel(const bf16* __r
                 if (p8 + j >= off && p8 + j < off + n) run[j] = src[j];
         }
     }
+}
+
+__global__ __launch_bounds__(256) void v_transposed_write_kernel(const bf16* __restrict__ qkv, int row_stride,
+                                                                 const int* __restrict__ tiles,
+                                                                 const int* __restrict__ block_table, int bt_stride,
+                                                                 bf16* __restrict__ v_pages, int H, int Hkv, int hs, int blocked) {
+    extern __shared__ __align__(16) unsigned char dyn_s[];
+    v_transposed_write_tile(blockIdx.x, blockIdx.y, reinterpret_cast<uint16_t*>(dyn_s), qkv, row_stride, tiles, block_table,
+                            bt_stride, v_pages, H, Hkv, hs, blocked);
+}
+
+// Both at once: the first n_v_blocks workgroups (the longer ones) store the values of a (tile, kv head) each, the others
+// rotate a token row and store its keys.  One launch instead of two that do not depend on each other.
+__global__ __launch_bounds__(256) void rope_kv_write_tiles_kernel(bf16* __restrict__ qkv, int row_stride,
+                                                                  const int* __restrict__ positions,
+                                                                  const int* __restrict__ seq_index,
+                                                                  const int* __restrict__ block_table, int bt_stride,
+                                                                  bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
+                                                                  const float* __restrict__ inv_freq, int rope_dims,
+                                                                  int H, int Hkv, int hs, int layout,
+                                                                  const int* __restrict__ tiles, int n_v_blocks) {
+    extern __shared__ __align__(16) unsigned char dyn_s[];
+    const int b = blockIdx.x;
+    if (b < n_v_blocks)
+        v_transposed_write_tile(b / Hkv, b % Hkv, reinterpret_cast<uint16_t*>(dyn_s), qkv, row_stride, tiles, block_table,
+                                bt_stride, v_pages, H, Hkv, hs, (layout & 3) == BN_KV_BLOCKED);
+    else
+        rope_kv_write_bf16x8_row(b - n_v_blocks, reinterpret_cast<float*>(dyn_s), qkv, row_stride, positions, seq_index,
+                                 block_table, bt_stride, k_pages, v_pages, inv_freq, rope_dims, H, Hkv, hs,
+                                 layout | BN_KV_V_BY_TILES);
 }
 
 // tiles: [n_tiles, 4] int32 as above; every tile lies inside one page.  V heads are read from qkv.  blocked: the pages
@@ -274,5 +314,30 @@ extern "C" int bn_rope_kv_write(int dtype, void* qkv, int row_stride, const int*
                            (bf16*)k_pages, (bf16*)v_pages, inv_freq, rope_dims, H, Hkv, hs, v_transposed);
     else
         return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+// bn_rope_kv_write and bn_v_transposed_write in one launch, for bf16 rows that the 16-byte kernel takes (rope_dims a
+// positive multiple of 16, hs and row_stride multiples of 8, 16-byte aligned pointers) and transposed or blocked pages.
+// Returns BN_ERR_ARG for anything else: the caller then makes the two calls.
+extern "C" int bn_rope_kv_write_tiles(void* qkv, int row_stride, const int* positions, const int* seq_index,
+                                      const int* block_table, int bt_stride, void* k_pages, void* v_pages,
+                                      const float* inv_freq, int rope_dims, int n_tokens, int H, int Hkv, int hs, int layout,
+                                      const int* tiles, int n_tiles, hipStream_t s) {
+    if (n_tokens <= 0 || n_tiles <= 0 || H <= 0 || Hkv <= 0 || Hkv > 65535 || hs <= 0 || hs % 8 || rope_dims <= 0 ||
+        rope_dims > hs || rope_dims % 16 || row_stride % 8 || row_stride < (H + 2 * Hkv) * hs)
+        return BN_ERR_ARG;
+    const int kind = layout & 3;
+    if ((layout & ~7) || (kind != BN_KV_TRANSPOSED && kind != BN_KV_BLOCKED) || (kind == BN_KV_BLOCKED && hs % 32)) return BN_ERR_ARG;
+    if (!qkv || !positions || !seq_index || !block_table || !k_pages || !v_pages || !inv_freq || !tiles) return BN_ERR_ARG;
+    if (((uintptr_t)qkv | (uintptr_t)k_pages | (uintptr_t)v_pages) & 15) return BN_ERR_ARG;
+    const long long n_v_blocks = (long long)n_tiles * Hkv;
+    if (n_v_blocks + n_tokens > 0x7fffffff) return BN_ERR_ARG;
+    const size_t smem_v = (size_t)hs * (BN_PAGE + VT_PAD) * sizeof(uint16_t), smem_r = (size_t)rope_dims * sizeof(float);
+    const size_t smem = smem_v > smem_r ? smem_v : smem_r;
+    if (smem > 64 * 1024) return BN_ERR_ARG;
+    hipLaunchKernelGGL(rope_kv_write_tiles_kernel, dim3((unsigned)(n_v_blocks + n_tokens)), dim3(256), smem, s, (bf16*)qkv,
+                       row_stride, positions, seq_index, block_table, bt_stride, (bf16*)k_pages, (bf16*)v_pages, inv_freq,
+                       rope_dims, H, Hkv, hs, layout, tiles, (int)n_v_blocks);
     return bn_launch_status();
 }

@@ -50,6 +50,8 @@ _SIGNATURES = {
                                   c_int, c_void_p],
         "bn_rope_kv_write": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                              c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bn_rope_kv_write_tiles": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                                   c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p],
     },
     "attn_rows": {
         "bn_attn_rows_key_tile": [c_int, c_int],
@@ -991,6 +993,14 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
         _dev(page_tiles, "page_tiles", torch.int32, 2)
         if page_tiles.shape[1] != 4 or not page_tiles.is_contiguous() or page_tiles.shape[0] == 0:
             raise KernelError("rope_kv_write: page_tiles must be a contiguous [n, 4] tensor")
+    if (tiled_v and rope_dims > 0 and rope_dims % 16 == 0
+            and (k_pages.data_ptr() | v_pages.data_ptr()) % 16 == 0):
+        # the rows that the 16-byte kernel takes: rotation, keys and the values' tiles in one launch
+        _check(_fn("rope_kv", "bn_rope_kv_write_tiles")(
+            qkv.data_ptr(), stride, positions.data_ptr(), seq_index.data_ptr(), block_table.data_ptr(), bt_stride,
+            k_pages.data_ptr(), v_pages.data_ptr(), inv_freq.data_ptr(), rope_dims, T, H, Hkv, hs, _LAYOUT_CODES[layout],
+            page_tiles.data_ptr(), page_tiles.shape[0], _stream()), "rope_kv_write(tiles)")
+        return
     _check(_fn("rope_kv", "bn_rope_kv_write")(
         _code(qkv.dtype), qkv.data_ptr(), stride, positions.data_ptr(),
         seq_index.data_ptr() if k_pages is not None else None,
