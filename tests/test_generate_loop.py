@@ -198,6 +198,14 @@ def test_a_sampler_that_needs_the_host_first_is_asked_the_plain_way():
     assert res[0].tokens == [2, 3, 4] and eng.ahead_steps == 0
 
 
+def test_sampling_that_needs_the_host_first_says_so():
+    """A repetition penalty reads the host's ring of recent tokens before it can sample: tokens cannot stay on the device."""
+    from bitnet_c_amd.sampling import start_sampling
+    logits = torch.zeros(2, 10)
+    with_penalty = [SequenceSampler(SamplingParams(repeat_penalty=1.3), [1, 2]), SequenceSampler(SamplingParams(), [3])]
+    assert start_sampling(logits, with_penalty) is None
+
+
 def test_host_rng_and_recent_ring_follow_the_plain_sampler():
     a, b = XorShift64Star(0), pl.XorShift64Star(42)
     assert [a.next_float() for _ in range(50)] == [b.next_float() for _ in range(50)]
