@@ -127,11 +127,17 @@ def _by_length(lens) -> List[int]:
 MAX_GRAPH_ROWS = 256      # rows of the largest captured decode step; a step of more sequences is replayed in pieces of this size
 
 
+# Rows of the captured decode steps: the powers of two, and between them the counts at which the kernels' work takes a
+# step (twelve rows of the sixteen of a matrix-core tile, three and six tiles of rows), so that a batch that has shrunk
+# to 40 sequences does not pay for 64.
+DECODE_BUCKETS = (1, 2, 4, 8, 12, 16, 32, 48, 64, 96, 128, 192, 256)
+
+
 def _bucket(n: int) -> int:
-    b = 1
-    while b < n:
-        b *= 2
-    return b
+    for b in DECODE_BUCKETS:
+        if b >= n:
+            return b
+    return DECODE_BUCKETS[-1]
 
 
 class _DecodeGraph:
@@ -366,7 +372,7 @@ class Engine:
         # host's slot list cannot, and a model with such a mixer runs its decode steps eagerly.
         self.use_graphs = use_graphs and all(n.state is None or n.state.device_addressed for n in needs)
         self.tap = None                     # see StepContext.tap; while it is set, steps run without graphs
-        # One captured step per number of rows (1, 2, 4 .. MAX_GRAPH_ROWS): at most nine, made at a batch's
+        # One captured step per number of rows (DECODE_BUCKETS, up to MAX_GRAPH_ROWS): at most thirteen, made at a batch's
         # start (prepare_decode) or at first use.  They share one memory pool: what a capture frees, the next
         # reuses, and each keeps only its own inputs and logits ([rows, vocab] float32).
         self._graphs: Dict[int, _DecodeGraph] = {}
@@ -605,10 +611,9 @@ class Engine:
         shrinks as sequences end), so that no later step waits for a capture.  Does nothing for what is there."""
         if not self.use_graphs or self.tap is not None:
             return
-        rows = _bucket(min(max(n_seqs, 1), MAX_GRAPH_ROWS))
-        while rows >= 1:
+        top = _bucket(min(max(n_seqs, 1), MAX_GRAPH_ROWS))
+        for rows in reversed([b for b in DECODE_BUCKETS if b <= top]):
             self._graph_for(rows)
-            rows //= 2
 
     def _graph_for(self, rows: int) -> _DecodeGraph:
         g = self._graphs.get(rows)
